@@ -1,0 +1,346 @@
+/*
+ * m40llm C ABI, MI355X (gfx950) implementation.
+ *
+ * The drop-in boundary of the decode-step hot path: the `m40llm_*` symbols the
+ * reference's Rust FFI block declares (src/cuda.rs:87-682) and its native side
+ * defines (cuda/kernels.cu, C view in cuda/stub.c), with the same names, argument
+ * meaning, stream behaviour and negative error codes.  Plain pointers and sizes
+ * only.  Each declaration cites the reference definition it replaces.
+ *
+ * Conventions (all from the reference):
+ *   - every function returns int (0 = ok, distinct negative code per failure
+ *     site) or a handle (NULL = failure);
+ *   - buffers are device pointers unless the name says host;
+ *   - stream_kind: 0 = prefill stream, 1 = decode stream, anything else is an error
+ *     (cuda/kernels.cu:287-292);
+ *   - rope_layout: 0 = adjacent pairs (2i,2i+1), 1 = NeoX split half (i,i+hd/2);
+ *   - weight_dtype: 0 = f16, 1 = f32;  exact_old_backing: 0 dense, 1 q8, 2 fp16-K/q4-V;
+ *   - `_async` = enqueue on the decode stream and return; the GEMMs and
+ *     f16_to_f32 / q80_to_f32 run on the prefill stream and block until done.
+ *   - calls on one context are serialised by the caller (the reference holds a
+ *     mutex around every FFI call, src/cuda.rs:1121-1137).
+ *
+ * Symbols of the reference that lie outside the decode hot path (staged / q8 /
+ * lossy-summary attention modes, prefill attention, cuBLAS-only GEMM, persistent
+ * decode prototype, telemetry readers) are exported and return their
+ * "unavailable" code exactly as cuda/stub.c does (-1), so a binding that declares
+ * all of them still links.  They are listed at the end of this header.
+ *
+ * Entry points that have no counterpart in the reference are prefixed
+ * `m40llm_ext_` and say so.
+ */
+#ifndef M40LLM_H
+#define M40LLM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct M40llmCudaContext M40llmCudaContext;     /* src/cuda.rs:30-33   */
+typedef struct M40llmKVCache M40llmKVCache;             /* src/cuda.rs:35-38   */
+typedef struct M40llmCudaGraphExec M40llmCudaGraphExec; /* src/cuda.rs:40-42   */
+typedef struct M40llmCudaEvent M40llmCudaEvent;         /* src/cuda.rs:43-45   */
+typedef struct M40llmAttentionTelemetry M40llmAttentionTelemetry;
+
+#define M40LLM_STREAM_PREFILL 0u
+#define M40LLM_STREAM_DECODE 1u
+#define M40LLM_ROPE_LAYOUT_ADJACENT 0u
+#define M40LLM_ROPE_LAYOUT_NEOX 1u
+
+/* ---- context, memory, streams (cuda/kernels.cu:276-514, 1245-1292, 7960ff) ---- */
+M40llmCudaContext* m40llm_create_context(int device_id);                         /* kernels.cu:366-474 */
+void m40llm_destroy_context(M40llmCudaContext* ctx);
+int m40llm_current_device_props(char* name_buf, size_t buf_len, int* major, int* minor,
+                                int* device_id);                                  /* kernels.cu:1245-1263 */
+int m40llm_device_malloc(M40llmCudaContext* ctx, size_t bytes, void** out_ptr);   /* kernels.cu:302-310 */
+int m40llm_device_free(M40llmCudaContext* ctx, void* ptr);                        /* kernels.cu:312-319 */
+int m40llm_memcpy_h2d(M40llmCudaContext* ctx, void* dst_device, const void* src_host, size_t bytes);
+int m40llm_memcpy_d2h(M40llmCudaContext* ctx, void* dst_host, const void* src_device, size_t bytes);
+int m40llm_memcpy_d2d_async(M40llmCudaContext* ctx, void* dst_device, const void* src_device,
+                            size_t bytes, uint32_t stream_kind);                  /* kernels.cu:337-355 */
+int m40llm_validate_device_ptr(const void* ptr);                                  /* kernels.cu:357-364 */
+int m40llm_upload_weights(M40llmCudaContext* ctx, const void* host_ptr, size_t num_bytes,
+                          void** out_device_ptr);                                 /* kernels.cu:1268-1292 */
+int m40llm_stream_synchronize(M40llmCudaContext* ctx, uint32_t stream_kind);      /* kernels.cu:476-484 */
+int m40llm_stream_wait_for_stream(M40llmCudaContext* ctx, uint32_t waiting_stream_kind,
+                                  uint32_t signal_stream_kind);                   /* kernels.cu:486-514 */
+
+/* events and graphs (cuda/kernels.cu:516-680) */
+int m40llm_cuda_event_create(M40llmCudaContext* ctx, M40llmCudaEvent** out_event);
+int m40llm_cuda_event_record(M40llmCudaContext* ctx, M40llmCudaEvent* event, uint32_t stream_kind);
+int m40llm_cuda_event_elapsed_sync(M40llmCudaContext* ctx, M40llmCudaEvent* start,
+                                   M40llmCudaEvent* stop, float* elapsed_ms);
+void m40llm_cuda_event_destroy(M40llmCudaEvent* event);
+int m40llm_cuda_graph_begin_capture(M40llmCudaContext* ctx, uint32_t stream_kind);
+int m40llm_cuda_graph_end_capture(M40llmCudaContext* ctx, uint32_t stream_kind,
+                                  M40llmCudaGraphExec** out_graph);
+int m40llm_cuda_graph_cancel_capture(M40llmCudaContext* ctx, uint32_t stream_kind);
+int m40llm_cuda_graph_launch(M40llmCudaContext* ctx, M40llmCudaGraphExec* graph, uint32_t stream_kind);
+int m40llm_cuda_graph_launch_timed_sync(M40llmCudaContext* ctx, M40llmCudaGraphExec* graph,
+                                        uint32_t stream_kind, float* elapsed_ms);
+void m40llm_cuda_graph_destroy(M40llmCudaGraphExec* graph);
+
+/* ---- GEMV / GEMM: C[M,N] f32 row-major (cuda/kernels.cu:4981-5302) ------------- */
+/* A f32 [M,K] x B f16 GGUF layout B[n*K + k]: the decode projection (kernels.cu:5158-5195) */
+int m40llm_gemm_f32xf16_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16,
+                                 void* d_C_f32, int M, int N, int K);
+/* A f32 x B f16 row-major B[k*N + n] (kernels.cu:5106-5155) */
+int m40llm_gemm_f32xf16_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16,
+                            void* d_C_f32, int M, int N, int K);
+/* A f16 x B f16 row-major -> f32 (kernels.cu:5267-5302) */
+int m40llm_gemm_f16xf16_f32(M40llmCudaContext* ctx, const void* d_A_f16, const void* d_B_f16,
+                            void* d_C_f32, int M, int N, int K);
+/* A f16 x B f16 row-major -> f16, f32 accumulate (kernels.cu:5068-5103) */
+int m40llm_gemm_f16_storage_f32_compute(M40llmCudaContext* ctx, const void* d_A, const void* d_B,
+                                        void* d_C, int M, int N, int K);
+int m40llm_f16_to_f32(M40llmCudaContext* ctx, const void* d_in_f16, void* d_out_f32, size_t n);   /* :1129-1158 */
+int m40llm_q80_to_f32(M40llmCudaContext* ctx, const void* d_in_q80, void* d_out_f32, size_t n);   /* :1160-1173 */
+
+/* ---- elementwise, decode stream (cuda/kernels.cu:1036-1241, 7370-7546) ---------- */
+int m40llm_rms_norm_f32(M40llmCudaContext* ctx, const void* d_in, void* d_out, uint32_t rows,
+                        uint32_t dim, float eps);
+int m40llm_rms_norm_f32_async(M40llmCudaContext* ctx, const void* d_in, void* d_out, uint32_t rows,
+                              uint32_t dim, float eps);
+int m40llm_rms_norm_f32_weighted(M40llmCudaContext* ctx, const void* d_in, const void* d_weight,
+                                 void* d_out, uint32_t rows, uint32_t dim, float eps,
+                                 uint32_t weight_dtype);
+int m40llm_rms_norm_f32_weighted_async(M40llmCudaContext* ctx, const void* d_in, const void* d_weight,
+                                       void* d_out, uint32_t rows, uint32_t dim, float eps,
+                                       uint32_t weight_dtype);
+int m40llm_rope_f32(M40llmCudaContext* ctx, void* d_q, void* d_k, uint32_t rows, uint32_t num_heads,
+                    uint32_t head_dim, uint32_t past_len, float freq_base, float freq_scale);
+int m40llm_rope_f32_async(M40llmCudaContext* ctx, void* d_q, void* d_k, uint32_t rows,
+                          uint32_t num_heads, uint32_t head_dim, uint32_t past_len, float freq_base,
+                          float freq_scale);
+int m40llm_rope_f32_layout_async(M40llmCudaContext* ctx, void* d_q, void* d_k, uint32_t rows,
+                                 uint32_t num_heads, uint32_t head_dim, uint32_t past_len,
+                                 float freq_base, float freq_scale, uint32_t rope_layout);
+int m40llm_rope_f32_inplace(M40llmCudaContext* ctx, void* d_x, uint32_t rows, uint32_t num_heads,
+                            uint32_t head_dim, uint32_t past_len, float freq_base, float freq_scale);
+int m40llm_rope_f32_inplace_async(M40llmCudaContext* ctx, void* d_x, uint32_t rows,
+                                  uint32_t num_heads, uint32_t head_dim, uint32_t past_len,
+                                  float freq_base, float freq_scale);
+int m40llm_rope_f32_inplace_layout_async(M40llmCudaContext* ctx, void* d_x, uint32_t rows,
+                                         uint32_t num_heads, uint32_t head_dim, uint32_t past_len,
+                                         float freq_base, float freq_scale, uint32_t rope_layout);
+int m40llm_rope_f32_inplace_position_dev_async(M40llmCudaContext* ctx, void* d_x, uint32_t rows,
+                                               uint32_t num_heads, uint32_t head_dim,
+                                               const uint32_t* past_len_dev, float freq_base,
+                                               float freq_scale);
+int m40llm_rope_f32_inplace_position_dev_layout_async(M40llmCudaContext* ctx, void* d_x, uint32_t rows,
+                                                      uint32_t num_heads, uint32_t head_dim,
+                                                      const uint32_t* past_len_dev, float freq_base,
+                                                      float freq_scale, uint32_t rope_layout);
+int m40llm_residual_add_f32(M40llmCudaContext* ctx, const void* d_a, const void* d_b, void* d_out, size_t n);
+int m40llm_residual_add_f32_async(M40llmCudaContext* ctx, const void* d_a, const void* d_b, void* d_out, size_t n);
+int m40llm_swiglu_f32(M40llmCudaContext* ctx, const void* d_gate, const void* d_up, void* d_out, size_t n);
+int m40llm_swiglu_f32_async(M40llmCudaContext* ctx, const void* d_gate, const void* d_up, void* d_out, size_t n);
+
+/* ---- KV cache (cuda/kernels.cu:5304-5543, 5793-6379) ---------------------------- */
+M40llmKVCache* m40llm_kvcache_create(M40llmCudaContext* ctx, uint32_t max_seq_len,
+                                     uint32_t max_batch_size, uint32_t num_heads, uint32_t head_dim);
+/* Only exact_old_backing 0 (ring only) and 2 (fp16-K/q4-V) allocate usable
+ * storage here; backing 1 (q8) returns NULL. */
+M40llmKVCache* m40llm_kvcache_create_compressed(M40llmCudaContext* ctx, uint32_t max_seq_len,
+                                                uint32_t max_batch_size, uint32_t num_heads,
+                                                uint32_t head_dim, uint32_t recent_window,
+                                                uint32_t block_size, uint32_t top_blocks,
+                                                uint32_t representatives,
+                                                uint32_t representative_policy,
+                                                uint32_t exact_old_backing);
+void m40llm_kvcache_destroy(M40llmKVCache* kv);
+int m40llm_kvcache_reset(M40llmCudaContext* ctx, M40llmKVCache* kv);               /* :6308-6358 */
+int m40llm_kvcache_append_token(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
+                                const void* k_dev_f16, const void* v_dev_f16);     /* :5793-5823 */
+int m40llm_kvcache_append_token_f32(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
+                                    const void* k_dev_f32, const void* v_dev_f32);
+int m40llm_kvcache_append_token_f32_async(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
+                                          const void* k_dev_f32, const void* v_dev_f32); /* :5837-5907 */
+int m40llm_kvcache_append_token_f32_rope_k(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
+                                           const void* k_dev_f32, const void* v_dev_f32,
+                                           uint32_t past_len, float freq_base, float freq_scale);
+int m40llm_kvcache_append_token_f32_rope_k_async(M40llmCudaContext* ctx, M40llmKVCache* kv,
+                                                 uint32_t seq_id, const void* k_dev_f32,
+                                                 const void* v_dev_f32, uint32_t past_len,
+                                                 float freq_base, float freq_scale);
+int m40llm_kvcache_append_token_f32_rope_k_layout_async(M40llmCudaContext* ctx, M40llmKVCache* kv,
+                                                        uint32_t seq_id, const void* k_dev_f32,
+                                                        const void* v_dev_f32, uint32_t past_len,
+                                                        float freq_base, float freq_scale,
+                                                        uint32_t rope_layout);     /* :5976-6029 */
+int m40llm_kvcache_append_token_f32_rope_k_at_async(M40llmCudaContext* ctx, M40llmKVCache* kv,
+                                                    uint32_t seq_id, const void* k_dev_f32,
+                                                    const void* v_dev_f32, uint32_t position,
+                                                    uint32_t past_len, float freq_base,
+                                                    float freq_scale);
+/* dispatches to the compressed append/evict path when the cache is compressed (:6045-6093) */
+int m40llm_kvcache_append_token_f32_rope_k_at_layout_async(M40llmCudaContext* ctx, M40llmKVCache* kv,
+                                                           uint32_t seq_id, const void* k_dev_f32,
+                                                           const void* v_dev_f32, uint32_t position,
+                                                           uint32_t past_len, float freq_base,
+                                                           float freq_scale, uint32_t rope_layout);
+int m40llm_kvcache_append_token_f32_rope_k_compressed_at_async(M40llmCudaContext* ctx, M40llmKVCache* kv,
+                                                               uint32_t seq_id, const void* k_dev_f32,
+                                                               const void* v_dev_f32, uint32_t position,
+                                                               float freq_base, float freq_scale);
+int m40llm_kvcache_append_token_f32_rope_k_compressed_at_layout_async(
+    M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id, const void* k_dev_f32,
+    const void* v_dev_f32, uint32_t position, float freq_base, float freq_scale,
+    uint32_t rope_layout);                                                         /* :6108-6250 */
+int m40llm_kvcache_append_token_f32_rope_k_position_dev_async(M40llmCudaContext* ctx, M40llmKVCache* kv,
+                                                              uint32_t seq_id, const void* k_dev_f32,
+                                                              const void* v_dev_f32,
+                                                              const uint32_t* position_dev,
+                                                              float freq_base, float freq_scale);
+int m40llm_kvcache_append_token_f32_rope_k_position_dev_layout_async(
+    M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id, const void* k_dev_f32,
+    const void* v_dev_f32, const uint32_t* position_dev, float freq_base, float freq_scale,
+    uint32_t rope_layout);                                                         /* :6265-6306 */
+/* one token as [kv_heads*head_dim] f16 K then V, host buffers (:6360-6379) */
+int m40llm_kvcache_debug_read_token(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
+                                    uint32_t token, void* out_k_host, void* out_v_host);
+/* telemetry twin of the block ranking: q-head 0 / kv-head 0 only (:6449-6677) */
+int m40llm_kvcache_debug_select_old_blocks(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                           uint32_t seq_id, const void* q_dev_f32, uint32_t q_heads,
+                                           uint32_t seq_len, uint32_t recent_window,
+                                           uint32_t block_size, uint32_t top_blocks,
+                                           uint32_t* out_blocks_host, float* out_scores_host,
+                                           uint32_t* out_start_host, uint32_t* out_end_host,
+                                           uint32_t* out_count, uint32_t max_out,
+                                           uint32_t* out_total_old_blocks);
+
+/* ---- attention, decode stream (cuda/kernels.cu:3837-4070, 4504-4577, 4694-4832) -- */
+int m40llm_attention_last_token_f32(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,
+                                    const void* q_dev_f32, uint32_t seq_len, void* out_dev_f32);
+int m40llm_attention_last_token_f32_gqa(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                        uint32_t seq_id, const void* q_dev_f32, uint32_t q_heads,
+                                        uint32_t seq_len, void* out_dev_f32);
+int m40llm_attention_last_token_f32_gqa_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                              uint32_t seq_id, const void* q_dev_f32, uint32_t q_heads,
+                                              uint32_t seq_len, void* out_dev_f32);
+int m40llm_attention_last_token_f32_gqa_seq_len_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                          uint32_t seq_id, const void* q_dev_f32,
+                                                          uint32_t q_heads, const uint32_t* seq_len_dev,
+                                                          void* out_dev_f32);
+int m40llm_attention_last_token_f32_gqa_dense_recent_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                           uint32_t seq_id, const void* q_dev_f32,
+                                                           uint32_t q_heads, uint32_t seq_len,
+                                                           uint32_t recent_window, void* out_dev_f32);
+/* Variable-length batch: Q and Out packed [batch][q_heads][head_dim]; seq_ids / seq_lens are
+ * device u32 arrays.  The reference accepts head_dim 64 and lengths <= 8192 only
+ * (kernels.cu:4707, :4743); this implementation also takes head_dim 128 and any
+ * length <= max_seq_len. */
+int m40llm_attention_last_token_f32_gqa_batched(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                const uint32_t* seq_ids_dev, const uint32_t* seq_lens_dev,
+                                                uint32_t batch_size, const void* q_dev_f32,
+                                                uint32_t q_heads, void* out_dev_f32);
+int m40llm_attention_last_token_f32_gqa_batched_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                      const uint32_t* seq_ids_dev,
+                                                      const uint32_t* seq_lens_dev, uint32_t batch_size,
+                                                      const void* q_dev_f32, uint32_t q_heads,
+                                                      void* out_dev_f32);
+/* block-select over a dense cache (reference: head_dim 64 only; 128 accepted here) */
+int m40llm_attention_last_token_f32_gqa_block_select_exact_async(
+    M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q_dev_f32,
+    uint32_t q_heads, uint32_t seq_len, uint32_t recent_window, uint32_t block_size,
+    uint32_t top_blocks, void* out_dev_f32);
+/* block-select over the fp16-K / q4-V compressed cache, head_dim 64 or 128 */
+int m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async(
+    M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q_dev_f32,
+    uint32_t q_heads, uint32_t seq_len, uint32_t recent_window, uint32_t block_size,
+    uint32_t top_blocks, void* out_dev_f32);
+
+/* ---- additions with no counterpart in the reference -------------------------------- */
+/* q8_0 weights (34-byte blocks along K, GGUF order) -> C[M,N] f32.  The reference only
+ * dequantises q8_0 elementwise (kernels.cu:856-867); this is that dequant followed by
+ * the semantics of m40llm_gemm_f32xf16_gguf_f32.  Blocking, prefill stream. */
+int m40llm_ext_gemm_f32xq80_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_q80,
+                                     void* d_C_f32, int M, int N, int K);
+/* out[M,d_model] = down(swiglu(gate(x), up(x))) with q8_0 matrices; d_scratch_f32 holds
+ * 2*M*ffn floats.  Decode stream, asynchronous. */
+int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_f32,
+                                        const void* d_w_gate_q80, const void* d_w_up_q80,
+                                        const void* d_w_down_q80, void* d_scratch_f32,
+                                        void* d_out_f32, int M, int d_model, int ffn);
+/* same contraction as m40llm_gemm_f32xf16_gguf_f32, enqueued on `stream_kind` without blocking */
+int m40llm_ext_gemm_f32xf16_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32,
+                                           const void* d_B_f16, void* d_C_f32, int M, int N, int K,
+                                           uint32_t stream_kind);
+/* Per-q-head selection of the block-select path, computed by the same kernels that the
+ * attention entry points run (the reference's debug selector covers q-head 0 only).
+ * out_blocks_host: [q_heads][64] (0xffffffff beyond the count), out_counts_host: [q_heads],
+ * out_scores_host (may be NULL): [q_heads][64]. Works on dense and compressed caches. */
+int m40llm_ext_block_select_read_selection(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                           uint32_t seq_id, const void* q_dev_f32, uint32_t q_heads,
+                                           uint32_t seq_len, uint32_t recent_window,
+                                           uint32_t block_size, uint32_t top_blocks,
+                                           uint32_t* out_blocks_host, uint32_t* out_counts_host,
+                                           float* out_scores_host);
+/* Fill positions [0, seq_len) of one sequence from f16 K/V rows [seq_len][kv_heads][head_dim]
+ * on the device, leaving the cache exactly as seq_len ordered appends of those (already
+ * rotated) rows would: dense caches get the rows, compressed caches get old-K copies,
+ * q4 V + scales for positions < seq_len - recent_window and ring rows for the rest. */
+int m40llm_ext_kvcache_bulk_fill_f16(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
+                                     const void* k_dev_f16, const void* v_dev_f16, uint32_t seq_len);
+/* raw views of the compressed cache for tests: which = 0 old_k, 1 q4_v, 2 q4_scale, 3 recent_k,
+ * 4 recent_v, 5 seq_map; copies `bytes` from byte offset `offset` to the host */
+int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t which,
+                                      size_t offset, size_t bytes, void* out_host);
+/* first index of the maximum of each row of logits [rows][n] -> out_idx_dev u32 [rows]; also
+ * writes the top-1 minus top-2 gap to out_gap_dev (may be NULL).  Decode stream. */
+int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t rows,
+                                size_t n, uint32_t* out_idx_dev, float* out_gap_dev);
+const char* m40llm_ext_build_info(void);
+
+/* ---- present but unavailable (return -1, as cuda/stub.c does) ---------------------- */
+int m40llm_gemm_f32xf32_f32(M40llmCudaContext*, const void*, const void*, void*, int, int, int);
+int m40llm_gemm_f32xf32_f32_async(M40llmCudaContext*, const void*, const void*, void*, int, int, int);
+int m40llm_materialize_gguf_f16_to_f32_colmajor_nt(M40llmCudaContext*, const void*, void*, int, int);
+int m40llm_kvcache_build_q8_old_from_dense(M40llmCudaContext*, M40llmKVCache*, uint32_t, uint32_t, uint32_t);
+int m40llm_kvcache_build_compressed_from_dense(M40llmCudaContext*, M40llmKVCache*, const M40llmKVCache*, uint32_t);
+int m40llm_kvcache_debug_read_compressed_state(M40llmCudaContext*, M40llmKVCache*, uint32_t, uint32_t*,
+                                               uint32_t*, void*, void*, float*, float*, void*, void*,
+                                               void*, void*, uint32_t*);
+int m40llm_kvcache_debug_attention_telemetry(M40llmCudaContext*, const M40llmKVCache*, uint32_t, uint32_t,
+                                             const void*, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                                             uint32_t, M40llmAttentionTelemetry*);
+int m40llm_attention_last_token_f32_gqa_block_select_exact_staged_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
+    uint32_t, uint32_t, void*);
+int m40llm_attention_last_token_f32_gqa_block_select_exact_staged_with_buffers_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
+    uint32_t, uint32_t, void*, void*, void*, void*, uint32_t, void*);
+int m40llm_attention_last_token_f32_gqa_block_select_exact_staged_q8_old_with_buffers_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
+    uint32_t, uint32_t, void*, void*, void*, void*, uint32_t, void*);
+int m40llm_attention_last_token_f32_gqa_block_select_exact_staged_fp16_k_q4_v_old_with_buffers_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
+    uint32_t, uint32_t, void*, void*, void*, void*, uint32_t, void*);
+int m40llm_attention_last_token_f32_gqa_block_select_exact_q8_old_direct_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
+    uint32_t, uint32_t, void*);
+int m40llm_attention_last_token_f32_gqa_block_summary_lossy_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, uint32_t,
+    uint32_t, uint32_t, void*);
+int m40llm_attention_last_token_f32_gqa_compressed_recent_only_async(
+    M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, void*);
+int m40llm_attention_prefill_f32_gqa_varlen(M40llmCudaContext*, const void*, const void*, const void*,
+                                            const uint32_t*, const uint32_t*, const uint32_t*,
+                                            const uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t, void*);
+int m40llm_attention_prefill_f32_gqa_varlen_async(M40llmCudaContext*, const void*, const void*, const void*,
+                                                  const uint32_t*, const uint32_t*, const uint32_t*,
+                                                  const uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t,
+                                                  void*);
+int m40llm_start_persistent_decode(M40llmCudaContext*);
+int m40llm_stop_persistent_decode(M40llmCudaContext*);
+int m40llm_persistent_decode_submit_vec(M40llmCudaContext*, const void*, void*, uint32_t, float, float,
+                                        uint32_t, uint32_t*);
+int m40llm_persistent_decode_poll(M40llmCudaContext*, uint32_t*, uint32_t*);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* M40LLM_H */

@@ -1,0 +1,470 @@
+// Last-token GQA attention over the dense f16 KV cache for gfx950 (single sequence, device
+// length, recent-window and variable-length batched forms share one kernel).
+//
+// Work split: grid = (kv_head x q-head subgroup, token chunk, batch row).  A workgroup streams its
+// chunk of K and V exactly once with 128-bit loads and serves every q head of the GQA group
+// from it, so K/V traffic is 1/group of a per-q-head kernel.  Per chunk it produces the
+// softmax partial (max, sum, weighted V); a small second kernel merges chunks in ascending
+// order.  With a single chunk the first kernel writes the final output itself.
+//
+// Reference semantics: three-pass softmax per q head, kv head = qh / (q_heads / kv_heads),
+// scale literals for head_dim 64 / 128: cuda/kernels.cu:1367-1655, entry points :3837-4023,
+// batched :1740-1823 and :4694-4832.
+#include "common.hpp"
+
+namespace {
+
+constexpr int kAttnThreads = 256;
+constexpr int kWaves = kAttnThreads / 64;
+
+struct AttnParams {
+    const uint16_t* K;
+    const uint16_t* V;
+    const float* Q;
+    float* Out;
+    float* ws;                    // partials: [batch][q_heads][nchunks][hd + 2]
+    const uint32_t* seq_ids_dev;  // may be null
+    const uint32_t* seq_lens_dev; // may be null
+    uint32_t seq_id, seq_len;
+    uint32_t max_seq_len, kv_heads, q_heads, window;
+    uint32_t chunk, nchunks;
+    uint32_t subgroups;           // q-head subgroups per kv head
+};
+
+// HD in {64, 128}; G = q heads handled per workgroup (<= 8)
+template <int HD, int G>
+__global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p) {
+    constexpr int LPT = HD / 8;      // lanes per token row
+    constexpr int TPW = 64 / LPT;    // token rows per wave step
+    extern __shared__ float lds[];
+    float* sc = lds;                              // [G][chunk]
+    float* red = sc + (size_t)G * p.chunk;        // [kWaves][G][HD]
+    float* wmax = red + (size_t)kWaves * G * HD;  // [kWaves][G]
+    float* wsum = wmax + kWaves * G;              // [kWaves][G]
+
+    const uint32_t b = blockIdx.z;
+    const uint32_t seq_id = p.seq_ids_dev ? p.seq_ids_dev[b] : p.seq_id;
+    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] : p.seq_len;
+    if (len == 0 || len > p.max_seq_len) return;
+    const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    const uint32_t cbeg = t0 + blockIdx.y * p.chunk;
+    if (cbeg >= len) return;
+    const uint32_t cend = cbeg + p.chunk < len ? cbeg + p.chunk : len;
+
+    const uint32_t kvh = blockIdx.x / p.subgroups;
+    const uint32_t sub = blockIdx.x % p.subgroups;
+    const uint32_t group = p.q_heads / p.kv_heads;
+    const uint32_t qh0 = kvh * group + sub * G;          // first q head of this workgroup
+    const uint32_t gcount = (sub * G + G <= group) ? G : group - sub * G;
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int c = lane % LPT, tg = lane / LPT;
+    const size_t row_stride = (size_t)p.kv_heads * HD;
+    const uint16_t* Kb = p.K + ((size_t)seq_id * p.max_seq_len) * row_stride + (size_t)kvh * HD + 8 * c;
+    const uint16_t* Vb = p.V + ((size_t)seq_id * p.max_seq_len) * row_stride + (size_t)kvh * HD + 8 * c;
+    const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
+
+    // q slice of this lane for every head of the subgroup
+    float q[G][8];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        const uint32_t qh = qh0 + (h < (int)gcount ? h : 0);
+        const float* qp = p.Q + ((size_t)b * p.q_heads + qh) * HD + 8 * c;
+        const float4 q0 = *reinterpret_cast<const float4*>(qp);
+        const float4 q1 = *reinterpret_cast<const float4*>(qp + 4);
+        q[h][0] = q0.x; q[h][1] = q0.y; q[h][2] = q0.z; q[h][3] = q0.w;
+        q[h][4] = q1.x; q[h][5] = q1.y; q[h][6] = q1.z; q[h][7] = q1.w;
+    }
+
+    const uint32_t per_wave = p.chunk / kWaves;           // chunk is a multiple of kWaves*TPW
+    const uint32_t wbeg = cbeg + wave * per_wave;
+
+    // ---- pass A: scores ---------------------------------------------------------------
+    float lmax[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) lmax[h] = -INFINITY;
+    for (uint32_t it = 0; it < per_wave; it += TPW) {
+        const uint32_t t = wbeg + it + tg;
+        const bool valid = t < cend;
+        uint4 kw = make_uint4(0, 0, 0, 0);
+        if (valid) kw = *reinterpret_cast<const uint4*>(Kb + (size_t)t * row_stride);
+        float kf[8];
+        m40_unpack8(kw, kf);
+        const uint32_t tl = wave * per_wave + it + tg;
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            float d = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) d = fmaf(q[h][j], kf[j], d);
+            d = LPT == 8 ? m40_sum8(d) : m40_sum16(d);
+            const float s = valid ? d * inv_sqrt : -INFINITY;
+            lmax[h] = fmaxf(lmax[h], s);
+            if (c == 0) sc[h * p.chunk + tl] = s;
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        const float m = m40_max64(lmax[h]);
+        if (lane == 0) wmax[wave * G + h] = m;
+    }
+    __syncthreads();
+    float mh[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        float m = wmax[h];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, wmax[w * G + h]);
+        mh[h] = m;
+    }
+
+    // ---- pass B0: p = exp(s - max), row sums ---------------------------------------------
+    float lsum[G];
+#pragma unroll
+    for (int h = 0; h < G; ++h) lsum[h] = 0.0f;
+    for (uint32_t tl = tid; tl < p.chunk; tl += kAttnThreads) {
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            const float s = sc[h * p.chunk + tl];
+            const float e = s == -INFINITY ? 0.0f : expf(s - mh[h]);
+            sc[h * p.chunk + tl] = e;
+            lsum[h] += e;
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+        const float s = m40_sum64(lsum[h]);
+        if (lane == 0) wsum[wave * G + h] = s;
+    }
+    __syncthreads();
+
+    // ---- pass B: weighted V -----------------------------------------------------------------
+    float acc[G][8];
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[h][j] = 0.0f;
+    for (uint32_t it = 0; it < per_wave; it += TPW) {
+        const uint32_t t = wbeg + it + tg;
+        if (t < cend) {
+            const uint4 vw = *reinterpret_cast<const uint4*>(Vb + (size_t)t * row_stride);
+            float vf[8];
+            m40_unpack8(vw, vf);
+            const uint32_t tl = wave * per_wave + it + tg;
+#pragma unroll
+            for (int h = 0; h < G; ++h) {
+                const float pw = sc[h * p.chunk + tl];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[h][j] = fmaf(pw, vf[j], acc[h][j]);
+            }
+        }
+    }
+    // join the TPW token rows of the wave (lanes with equal c), then the waves
+#pragma unroll
+    for (int h = 0; h < G; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float v = acc[h][j];
+#pragma unroll
+            for (int o = LPT; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+            acc[h][j] = v;
+        }
+    if (tg == 0) {
+#pragma unroll
+        for (int h = 0; h < G; ++h)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) red[((size_t)wave * G + h) * HD + 8 * c + j] = acc[h][j];
+    }
+    __syncthreads();
+
+    const bool final_out = p.nchunks == 1;
+    for (uint32_t e = tid; e < gcount * HD; e += kAttnThreads) {
+        const uint32_t h = e / HD, d = e % HD;
+        float v = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            v += red[((size_t)w * G + h) * HD + d];
+            l += wsum[w * G + h];
+        }
+        const uint32_t qh = qh0 + h;
+        if (final_out) {
+            const float denom = l > 0.0f ? l : 1.0f;
+            p.Out[((size_t)b * p.q_heads + qh) * HD + d] = v / denom;
+        } else {
+            float* w = p.ws + (((size_t)b * p.q_heads + qh) * p.nchunks + blockIdx.y) * (HD + 2);
+            w[2 + d] = v;
+            if (d == 0) {
+                w[0] = mh[h];
+                w[1] = l;
+            }
+        }
+    }
+}
+
+// Merge chunk partials in ascending chunk order: grid (q_heads, batch), HD threads.
+template <int HD>
+__global__ __launch_bounds__(HD) void attn_combine_kernel(AttnParams p) {
+    const uint32_t qh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] : p.seq_len;
+    if (len == 0 || len > p.max_seq_len) return;
+    const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    const uint32_t n = (len - t0 + p.chunk - 1) / p.chunk;
+    const float* w = p.ws + (((size_t)b * p.q_heads + qh) * p.nchunks) * (HD + 2);
+    float M = -INFINITY;
+    for (uint32_t c = 0; c < n; ++c) M = fmaxf(M, w[(size_t)c * (HD + 2)]);
+    float num = 0.0f, den = 0.0f;
+    for (uint32_t c = 0; c < n; ++c) {
+        const float* wc = w + (size_t)c * (HD + 2);
+        const float f = expf(wc[0] - M);
+        num = fmaf(wc[2 + d], f, num);
+        den = fmaf(wc[1], f, den);
+    }
+    den = den > 0.0f ? den : 1.0f;
+    p.Out[((size_t)b * p.q_heads + qh) * HD + d] = num / den;
+}
+
+// Any head_dim: one thread per output element, the reference's three passes verbatim
+// (cuda/kernels.cu:1367-1426).  Used for head_dim other than 64 / 128 only.
+__global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p, uint32_t head_dim) {
+    const uint32_t b = blockIdx.z, qh = blockIdx.y;
+    const uint32_t d = blockIdx.x * 64 + threadIdx.x;
+    if (d >= head_dim) return;
+    const uint32_t seq_id = p.seq_ids_dev ? p.seq_ids_dev[b] : p.seq_id;
+    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] : p.seq_len;
+    if (len == 0 || len > p.max_seq_len) return;
+    const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    const uint32_t kvh = qh / (p.q_heads / p.kv_heads);
+    const size_t ept = (size_t)p.kv_heads * head_dim;
+    const float inv_sqrt = m40_inv_sqrt_head_dim(head_dim);
+    const float* q = p.Q + ((size_t)b * p.q_heads + qh) * head_dim;
+    const uint16_t* Kb = p.K + ((size_t)seq_id * p.max_seq_len) * ept + (size_t)kvh * head_dim;
+    const uint16_t* Vb = p.V + ((size_t)seq_id * p.max_seq_len) * ept + (size_t)kvh * head_dim;
+    float mx = -1e30f;
+    for (uint32_t t = t0; t < len; ++t) {
+        float dot = 0.0f;
+        for (uint32_t k = 0; k < head_dim; ++k) dot += q[k] * m40_h2f(Kb[(size_t)t * ept + k]);
+        mx = fmaxf(mx, dot * inv_sqrt);
+    }
+    float den = 0.0f, acc = 0.0f;
+    for (uint32_t t = t0; t < len; ++t) {
+        float dot = 0.0f;
+        for (uint32_t k = 0; k < head_dim; ++k) dot += q[k] * m40_h2f(Kb[(size_t)t * ept + k]);
+        const float e = expf(dot * inv_sqrt - mx);
+        den += e;
+        acc += e * m40_h2f(Vb[(size_t)t * ept + d]);
+    }
+    den = den > 0.0f ? den : 1.0f;
+    p.Out[((size_t)b * p.q_heads + qh) * head_dim + d] = acc / den;
+}
+
+template <int HD, int G>
+int launch_partial(hipStream_t stream, const AttnParams& p, uint32_t batch) {
+    const size_t lds = ((size_t)G * p.chunk + (size_t)kWaves * G * HD + 2 * kWaves * G) * sizeof(float);
+    dim3 grid(p.kv_heads * p.subgroups, p.nchunks, batch);
+    attn_partial_kernel<HD, G><<<grid, kAttnThreads, lds, stream>>>(p);
+    return 0;
+}
+
+template <int HD>
+int launch_hd(hipStream_t stream, AttnParams& p, uint32_t batch, uint32_t group) {
+    int G = group >= 8 ? 8 : (group >= 4 ? 4 : (group >= 2 ? 2 : 1));
+    if (group % G != 0) {
+        // uneven group sizes (3, 5, 6, 7...) run with the largest subgroup that fits
+        G = group >= 8 ? 8 : (group > 4 ? 8 : (group > 2 ? 4 : 2));
+    }
+    p.subgroups = (group + G - 1) / G;
+    switch (G) {
+        case 8: launch_partial<HD, 8>(stream, p, batch); break;
+        case 4: launch_partial<HD, 4>(stream, p, batch); break;
+        case 2: launch_partial<HD, 2>(stream, p, batch); break;
+        default: launch_partial<HD, 1>(stream, p, batch); break;
+    }
+    if (p.nchunks > 1) {
+        dim3 grid(p.q_heads, batch);
+        attn_combine_kernel<HD><<<grid, HD, 0, stream>>>(p);
+    }
+    return 0;
+}
+
+}  // namespace
+
+int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
+                               const M40AttnArgs& a) {
+    AttnParams p{};
+    p.K = a.K; p.V = a.V; p.Q = a.Q; p.Out = a.Out;
+    p.seq_ids_dev = a.seq_ids_dev; p.seq_lens_dev = a.seq_lens_dev;
+    p.seq_id = a.seq_id; p.seq_len = a.seq_len;
+    p.max_seq_len = a.max_seq_len; p.kv_heads = a.kv_heads; p.q_heads = a.q_heads; p.window = a.window;
+    p.subgroups = 1;
+    (void)hipGetLastError();
+    const uint32_t group = a.q_heads / a.kv_heads;
+    uint32_t span = a.max_len_hint;
+    if (a.window != 0 && span > a.window) span = a.window;
+    if (span == 0) span = 1;
+
+    if ((a.head_dim == 64 || a.head_dim == 128) && m40_aligned16(a.Q) && m40_aligned16(a.K) && m40_aligned16(a.V)) {
+        // chunk: small when there is little work so that more CUs take part; the per-row
+        // partial buffer bounds the chunk count.
+        const uint64_t rows = (uint64_t)a.batch * a.kv_heads;
+        uint32_t chunk = 512;
+        while (chunk > 64 && rows * ((span + chunk - 1) / chunk) < 2u * (uint32_t)ctx->num_cus) chunk >>= 1;
+        M40StreamScratch& sc = ctx->scratch[stream_kind];
+        for (;;) {
+            p.chunk = chunk;
+            p.nchunks = (span + chunk - 1) / chunk;
+            const size_t need = (size_t)a.batch * a.q_heads * p.nchunks * (a.head_dim + 2) * sizeof(float);
+            if (p.nchunks == 1 || need <= sc.attn_partial_bytes) break;
+            if (chunk >= 1024) return -7;   // LDS holds G x chunk scores
+            chunk <<= 1;
+        }
+        p.ws = static_cast<float*>(sc.attn_partial);
+        if (a.head_dim == 64) launch_hd<64>(stream, p, a.batch, group);
+        else launch_hd<128>(stream, p, a.batch, group);
+    } else {
+        p.chunk = span; p.nchunks = 1;
+        dim3 grid((a.head_dim + 63) / 64, a.q_heads, a.batch);
+        attn_generic_kernel<<<grid, 64, 0, stream>>>(p, a.head_dim);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+// Reads the (ids, lens) pair of a batched call back to the host for validation, as the reference
+// does before launching (cuda/kernels.cu:4721-4754); returns the largest length.
+static int validate_batch(const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
+                          uint32_t batch, uint32_t* max_len) {
+    uint32_t stack_ids[64], stack_lens[64];
+    uint32_t* ids = batch <= 64 ? stack_ids : new uint32_t[batch];
+    uint32_t* lens = batch <= 64 ? stack_lens : new uint32_t[batch];
+    int rc = 0;
+    if (hipMemcpy(lens, lens_dev, (size_t)batch * 4, hipMemcpyDeviceToHost) != hipSuccess ||
+        hipMemcpy(ids, ids_dev, (size_t)batch * 4, hipMemcpyDeviceToHost) != hipSuccess) {
+        (void)hipGetLastError();
+        rc = -7;
+    }
+    uint32_t mx = 0;
+    for (uint32_t i = 0; rc == 0 && i < batch; ++i) {
+        if (ids[i] >= kv->max_batch_size) rc = -8;
+        else if (lens[i] == 0 || lens[i] > kv->max_seq_len) rc = -8;
+        else if (lens[i] > mx) mx = lens[i];
+    }
+    if (batch > 64) { delete[] ids; delete[] lens; }
+    *max_len = mx;
+    return rc;
+}
+
+extern "C" {
+
+int m40llm_attention_last_token_f32_gqa_async(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,
+                                              const void* q_dev_f32, uint32_t q_heads, uint32_t seq_len,
+                                              void* out_dev_f32) {
+    if (!ctx || !kv || !q_dev_f32 || !out_dev_f32) return -1;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (seq_len == 0 || seq_len > kv->max_seq_len) return -3;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -6;
+    if (!kv->d_k || !kv->d_v) return -4;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = seq_len;
+    a.max_len_hint = seq_len;
+    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+}
+
+int m40llm_attention_last_token_f32_gqa(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,
+                                        const void* q_dev_f32, uint32_t q_heads, uint32_t seq_len,
+                                        void* out_dev_f32) {
+    int rc = m40llm_attention_last_token_f32_gqa_async(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, out_dev_f32);
+    if (rc != 0) return rc;
+    return hipStreamSynchronize(ctx->decode_stream) == hipSuccess ? 0 : -5;
+}
+
+// MHA form: q heads == kv heads (cuda/kernels.cu:3837-3861), synchronous.
+int m40llm_attention_last_token_f32(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,
+                                    const void* q_dev_f32, uint32_t seq_len, void* out_dev_f32) {
+    if (!ctx || !kv || !q_dev_f32 || !out_dev_f32) return -1;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (seq_len == 0 || seq_len > kv->max_seq_len) return -3;
+    if (!kv->d_k || !kv->d_v || kv->num_heads == 0) return -4;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = kv->num_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = seq_len;
+    a.max_len_hint = seq_len;
+    int rc = m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+    if (rc != 0) return -4;
+    return hipStreamSynchronize(ctx->decode_stream) == hipSuccess ? 0 : -5;
+}
+
+int m40llm_attention_last_token_f32_gqa_seq_len_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                          uint32_t seq_id, const void* q_dev_f32,
+                                                          uint32_t q_heads, const uint32_t* seq_len_dev,
+                                                          void* out_dev_f32) {
+    if (!ctx || !kv || !q_dev_f32 || !seq_len_dev || !out_dev_f32) return -1;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -3;
+    if (!kv->d_k || !kv->d_v) return -4;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = 0;
+    a.seq_lens_dev = seq_len_dev;            // row 0 of a one-row batch
+    a.max_len_hint = kv->max_seq_len;        // the length is unknown on the host: size for the maximum
+    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+}
+
+int m40llm_attention_last_token_f32_gqa_dense_recent_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                           uint32_t seq_id, const void* q_dev_f32,
+                                                           uint32_t q_heads, uint32_t seq_len,
+                                                           uint32_t recent_window, void* out_dev_f32) {
+    if (!ctx || !kv || !q_dev_f32 || !out_dev_f32) return -1;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (seq_len == 0 || seq_len > kv->max_seq_len) return -3;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -4;
+    if (kv->head_dim != 64 && kv->head_dim != 128) return -5;
+    if (recent_window == 0) return -6;
+    if (!kv->d_k || !kv->d_v) return -7;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = seq_len;
+    a.max_len_hint = seq_len; a.window = recent_window;
+    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a) == 0 ? 0 : -7;
+}
+
+static int batched_impl(M40llmCudaContext* ctx, const M40llmKVCache* kv, const uint32_t* seq_ids_dev,
+                        const uint32_t* seq_lens_dev, uint32_t batch_size, const void* q_dev_f32,
+                        uint32_t q_heads, void* out_dev_f32, bool synchronize) {
+    if (!ctx || !kv || !seq_ids_dev || !seq_lens_dev || !q_dev_f32 || !out_dev_f32) return -1;
+    if (batch_size == 0) return -2;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -3;
+    if (kv->head_dim != 64 && kv->head_dim != 128) return -6;
+    if (!kv->d_k || !kv->d_v) return -6;
+    uint32_t max_len = 0;
+    int rc = validate_batch(kv, seq_ids_dev, seq_lens_dev, batch_size, &max_len);
+    if (rc != 0) return rc;
+    if (max_len == 0) return -8;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = batch_size;
+    a.seq_ids_dev = seq_ids_dev; a.seq_lens_dev = seq_lens_dev; a.max_len_hint = max_len;
+    rc = m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+    if (rc != 0) return -4;
+    if (synchronize && hipStreamSynchronize(ctx->decode_stream) != hipSuccess) return -5;
+    return 0;
+}
+
+int m40llm_attention_last_token_f32_gqa_batched(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                const uint32_t* seq_ids_dev, const uint32_t* seq_lens_dev,
+                                                uint32_t batch_size, const void* q_dev_f32, uint32_t q_heads,
+                                                void* out_dev_f32) {
+    return batched_impl(ctx, kv, seq_ids_dev, seq_lens_dev, batch_size, q_dev_f32, q_heads, out_dev_f32, true);
+}
+
+int m40llm_attention_last_token_f32_gqa_batched_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                      const uint32_t* seq_ids_dev, const uint32_t* seq_lens_dev,
+                                                      uint32_t batch_size, const void* q_dev_f32,
+                                                      uint32_t q_heads, void* out_dev_f32) {
+    return batched_impl(ctx, kv, seq_ids_dev, seq_lens_dev, batch_size, q_dev_f32, q_heads, out_dev_f32, false);
+}
+
+}  // extern "C"

@@ -1,0 +1,472 @@
+// Block-select "exact old" attention for gfx950: exact recent window + top-k old blocks chosen
+// by mean-K block scores, over (a) the fp16-K / q4-V compressed cache and (b) a dense cache.
+//
+//   1. score  : one wave per (old block, kv head) streams the block's K rows once (128-bit
+//               loads), sums them per dimension in f32, and takes the dot of that sum with every
+//               q head of the GQA group, so old K is read once per kv head, not once per q head.
+//               score = (q . sum_t K[t]) / len * inv_sqrt.
+//   2. select : per q head, rank blocks by (score desc, block id asc) and keep the first
+//               min(top_blocks, old_blocks) whose score exceeds -1e30: the result of the
+//               reference's strict-'>' insertion into a list initialised to -1e30.
+//   3. attend : per q head, softmax attention over [tokens of the selected blocks in rank
+//               order] ++ [recent window], split into chunks; old V is unpacked from 4 bits in
+//               registers (value = nibble * scale, rounded through f16 as the reference does).
+//   4. combine: chunk partials merged in ascending order.
+//
+// Reference: kernel cuda/kernels.cu:2832-3096 (compressed) and :1825-1983 (dense), entry points
+// :4504-4577 and :4025-4070.  Only the plain top-k policy and score-rank block order are built.
+#include "common.hpp"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace {
+
+struct BsParams {
+    // K sources: tokens < old_len come from old_k_base (indexed by absolute position); tokens
+    // >= old_len from the ring (ring != 0) or from the same dense array.
+    const uint16_t* old_k;     // [max_seq_len][kvh][hd] of this sequence
+    const uint16_t* new_k;     // ring [W][kvh][hd] of this sequence, or dense K of this sequence
+    const uint16_t* dense_v;   // dense V of this sequence (dense backing) or ring V (compressed)
+    const uint8_t* q4_v;       // [max_seq_len][kvh][hd/2] of this sequence (compressed only)
+    const float* q4_scale;     // [max_seq_len][kvh]
+    const float* Q;            // [q_heads][hd]
+    float* Out;
+    float* scores;             // [q_heads][nblk]
+    uint32_t* sel;             // [q_heads][64]
+    float* sel_scores;         // [q_heads][64]
+    uint32_t* counts;          // [q_heads] selected blocks
+    uint32_t* ntok;            // [q_heads] attended tokens
+    float* partial;            // [q_heads][nchunks][hd+2]
+    uint32_t kv_heads, q_heads, seq_len, recent_window, block_size, top_n;
+    uint32_t old_len, nblk, chunk, nchunks, compressed;
+};
+
+// ---- 1. block scores ------------------------------------------------------------------------
+template <int HD, int G>
+__global__ __launch_bounds__(256) void bs_score_kernel(BsParams p) {
+    constexpr int C = HD / 8;   // 16-byte chunks per K row
+    constexpr int R = 64 / C;   // rows per wave step
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t blk = blockIdx.x * 4 + wave;
+    if (blk >= p.nblk) return;
+    const uint32_t kvh = blockIdx.y;
+    const int g = lane / C, c = lane % C;
+    const uint32_t start = blk * p.block_size;
+    const uint32_t end = start + p.block_size < p.old_len ? start + p.block_size : p.old_len;
+    const size_t row_stride = (size_t)p.kv_heads * HD;
+    const uint16_t* kb = p.old_k + (size_t)kvh * HD + 8 * c;
+
+    float sum[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sum[j] = 0.0f;
+#pragma unroll 4
+    for (uint32_t t = start + g; t < end; t += R) {
+        const uint4 kw = m40_load_stream(reinterpret_cast<const uint4*>(kb + (size_t)t * row_stride));
+        float kf[8];
+        m40_unpack8(kw, kf);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sum[j] += kf[j];
+    }
+    // join the R row groups: lanes with equal c, strides R/2*C ... C
+#pragma unroll
+    for (int stride = (R / 2) * C; stride >= C; stride >>= 1) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sum[j] += __shfl_xor(sum[j], stride, 64);
+    }
+    const uint32_t group = p.q_heads / p.kv_heads;
+    const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
+    const float len = (float)(end - start);
+    for (uint32_t h0 = 0; h0 < group; h0 += G) {
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            if (h0 + h < group) {
+                const uint32_t qh = kvh * group + h0 + h;
+                const float* qp = p.Q + (size_t)qh * HD + 8 * c;
+                float part = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) part = fmaf(qp[j], sum[j], part);
+                part = C == 8 ? m40_sum8(part) : m40_sum16(part);
+                if (lane == 0) p.scores[(size_t)qh * p.nblk + blk] = (part / len) * inv_sqrt;
+            }
+        }
+    }
+}
+
+// ---- 2. top-k selection per q head -----------------------------------------------------------
+__global__ __launch_bounds__(1024) void bs_select_kernel(BsParams p) {
+    extern __shared__ float s_sc[];  // [nblk]
+    const uint32_t qh = blockIdx.x;
+    const float* sc = p.scores + (size_t)qh * p.nblk;
+    for (uint32_t b = threadIdx.x; b < p.nblk; b += blockDim.x) s_sc[b] = sc[b];
+    for (uint32_t i = threadIdx.x; i < 64; i += blockDim.x) {
+        p.sel[qh * 64 + i] = 0xffffffffu;
+        p.sel_scores[qh * 64 + i] = -1e30f;
+    }
+    __shared__ uint32_t s_count, s_tok;
+    if (threadIdx.x == 0) { s_count = 0; s_tok = 0; }
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < p.nblk; b += blockDim.x) {
+        const float s = s_sc[b];
+        if (!(s > -1e30f)) continue;       // NaN and anything <= -1e30 never enter the list
+        uint32_t rank = 0;
+        for (uint32_t o = 0; o < p.nblk; ++o) {
+            const float so = s_sc[o];
+            rank += (so > s || (so == s && o < b)) ? 1u : 0u;
+        }
+        if (rank < p.top_n) {
+            p.sel[qh * 64 + rank] = b;
+            p.sel_scores[qh * 64 + rank] = s;
+            const uint32_t start = b * p.block_size;
+            const uint32_t end = start + p.block_size < p.old_len ? start + p.block_size : p.old_len;
+            atomicAdd(&s_count, 1u);
+            atomicAdd(&s_tok, end - start);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        p.counts[qh] = s_count;
+        p.ntok[qh] = s_tok + (p.seq_len - p.old_len);
+    }
+}
+
+// ---- 3. attention over the token list ---------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(256) void bs_attend_kernel(BsParams p) {
+    constexpr int LPT = HD / 8, TPW = 64 / LPT, kWaves = 4;
+    extern __shared__ float lds[];
+    float* sc = lds;                                                   // [chunk]
+    uint32_t* tok = reinterpret_cast<uint32_t*>(sc + p.chunk);         // [chunk]
+    float* red = reinterpret_cast<float*>(tok + p.chunk);              // [kWaves][HD]
+    float* wred = red + kWaves * HD;                                   // [2*kWaves]
+    __shared__ uint32_t pre[65];
+
+    const uint32_t qh = blockIdx.x;
+    const uint32_t n = p.ntok[qh];
+    const uint32_t cbeg = blockIdx.y * p.chunk;
+    if (cbeg >= n) return;
+    const uint32_t cend = cbeg + p.chunk < n ? cbeg + p.chunk : n;
+    const uint32_t count = p.counts[qh];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+
+    // list position -> token id.  pre[r] = first list position of the r-th selected block.
+    if (tid == 0) {
+        uint32_t acc = 0;
+        for (uint32_t r = 0; r < count; ++r) {
+            pre[r] = acc;
+            const uint32_t b = p.sel[qh * 64 + r];
+            const uint32_t start = b * p.block_size;
+            const uint32_t end = start + p.block_size < p.old_len ? start + p.block_size : p.old_len;
+            acc += end - start;
+        }
+        pre[count] = acc;
+    }
+    __syncthreads();
+    const uint32_t old_tokens = pre[count];
+    for (uint32_t i = tid; i < p.chunk; i += 256) {
+        const uint32_t pos = cbeg + i;
+        uint32_t t = 0xffffffffu;
+        if (pos < cend) {
+            if (pos >= old_tokens) {
+                t = p.old_len + (pos - old_tokens);
+            } else {
+                uint32_t r = 0;
+                while (r + 1 < count && pre[r + 1] <= pos) ++r;
+                t = p.sel[qh * 64 + r] * p.block_size + (pos - pre[r]);
+            }
+        }
+        tok[i] = t;
+    }
+    __syncthreads();
+
+    const uint32_t kvh = qh / (p.q_heads / p.kv_heads);
+    const int c = lane % LPT, tg = lane / LPT;
+    const size_t row_stride = (size_t)p.kv_heads * HD;
+    const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
+    float q[8];
+    {
+        const float* qp = p.Q + (size_t)qh * HD + 8 * c;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) q[j] = qp[j];
+    }
+    const uint32_t per_wave = p.chunk / kWaves;
+
+    // pass A: scores
+    float lmax = -INFINITY;
+    for (uint32_t it = 0; it < per_wave; it += TPW) {
+        const uint32_t tl = wave * per_wave + it + tg;
+        const uint32_t t = tok[tl];
+        const bool valid = t != 0xffffffffu;
+        uint4 kw = make_uint4(0, 0, 0, 0);
+        if (valid) {
+            const uint16_t* kp;
+            if (t < p.old_len) kp = p.old_k + (size_t)t * row_stride;
+            else kp = p.new_k + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
+            kw = *reinterpret_cast<const uint4*>(kp + (size_t)kvh * HD + 8 * c);
+        }
+        float kf[8];
+        m40_unpack8(kw, kf);
+        float d = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) d = fmaf(q[j], kf[j], d);
+        d = LPT == 8 ? m40_sum8(d) : m40_sum16(d);
+        const float s = valid ? d * inv_sqrt : -INFINITY;
+        lmax = fmaxf(lmax, s);
+        if (c == 0) sc[tl] = s;
+    }
+    lmax = m40_max64(lmax);
+    if (lane == 0) wred[wave] = lmax;
+    __syncthreads();
+    const float m = fmaxf(fmaxf(wred[0], wred[1]), fmaxf(wred[2], wred[3]));
+
+    // pass B0: exp and row sum
+    float lsum = 0.0f;
+    for (uint32_t tl = tid; tl < p.chunk; tl += 256) {
+        const float s = sc[tl];
+        const float e = s == -INFINITY ? 0.0f : expf(s - m);
+        sc[tl] = e;
+        lsum += e;
+    }
+    lsum = m40_sum64(lsum);
+    if (lane == 0) wred[kWaves + wave] = lsum;
+    __syncthreads();
+
+    // pass B: weighted V
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    for (uint32_t it = 0; it < per_wave; it += TPW) {
+        const uint32_t tl = wave * per_wave + it + tg;
+        const uint32_t t = tok[tl];
+        if (t == 0xffffffffu) continue;
+        const float pw = sc[tl];
+        float vf[8];
+        if (p.compressed && t < p.old_len) {
+            const uint32_t packed = *reinterpret_cast<const uint32_t*>(
+                p.q4_v + ((size_t)t * p.kv_heads + kvh) * (HD / 2) + 4 * c);
+            const float scale = p.q4_scale[(size_t)t * p.kv_heads + kvh];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int nib = (int)((packed >> (4 * j)) & 0xfu);
+                const int sv = nib >= 8 ? nib - 16 : nib;
+                vf[j] = m40_h2f(m40_f2h((float)sv * scale));
+            }
+        } else {
+            const uint16_t* vp = p.dense_v + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
+            const uint4 vw = *reinterpret_cast<const uint4*>(vp + (size_t)kvh * HD + 8 * c);
+            m40_unpack8(vw, vf);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = fmaf(pw, vf[j], acc[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float v = acc[j];
+#pragma unroll
+        for (int o = LPT; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+        acc[j] = v;
+    }
+    if (tg == 0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) red[wave * HD + 8 * c + j] = acc[j];
+    }
+    __syncthreads();
+    if (tid < HD) {
+        float v = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            v += red[w * HD + tid];
+            l += wred[kWaves + w];
+        }
+        if (p.nchunks == 1) {
+            p.Out[(size_t)qh * HD + tid] = v / (l > 0.0f ? l : 1.0f);
+        } else {
+            float* w = p.partial + ((size_t)qh * p.nchunks + blockIdx.y) * (HD + 2);
+            w[2 + tid] = v;
+            if (tid == 0) { w[0] = m; w[1] = l; }
+        }
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__(HD) void bs_combine_kernel(BsParams p) {
+    const uint32_t qh = blockIdx.x, d = threadIdx.x;
+    const uint32_t n = (p.ntok[qh] + p.chunk - 1) / p.chunk;
+    if (n == 0) return;
+    const float* w = p.partial + (size_t)qh * p.nchunks * (HD + 2);
+    float M = -INFINITY;
+    for (uint32_t c = 0; c < n; ++c) M = fmaxf(M, w[(size_t)c * (HD + 2)]);
+    float num = 0.0f, den = 0.0f;
+    for (uint32_t c = 0; c < n; ++c) {
+        const float* wc = w + (size_t)c * (HD + 2);
+        const float f = expf(wc[0] - M);
+        num = fmaf(wc[2 + d], f, num);
+        den = fmaf(wc[1], f, den);
+    }
+    p.Out[(size_t)qh * HD + d] = num / (den > 0.0f ? den : 1.0f);
+}
+
+uint32_t policy_from_env() {
+    const char* v = std::getenv("M40LLM_KV_BLOCK_SELECT_POLICY");
+    if (!v || !v[0] || std::strcmp(v, "topk") == 0) return 0u;
+    return 1u;  // any other policy name
+}
+uint32_t order_from_env() {
+    const char* v = std::getenv("M40LLM_KV_SELECTED_BLOCK_ORDER");
+    if (!v || !v[0]) return 0u;
+    if (std::strcmp(v, "chronological") == 0 || std::strcmp(v, "descending") == 0) return 1u;
+    return 0u;
+}
+
+// Fills the parameter block and checks scratch capacity.  Returns 0 or a negative code.
+int prepare(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q, uint32_t q_heads,
+            uint32_t seq_len, uint32_t W, uint32_t bs, uint32_t top, void* out, bool compressed, BsParams* p) {
+    std::memset(p, 0, sizeof(*p));
+    const uint32_t hd = kv->head_dim, kvh = kv->num_heads;
+    const size_t ept = (size_t)kvh * hd;
+    const uint32_t old_len = seq_len > W ? seq_len - W : 0;
+    const uint32_t nblk = old_len == 0 ? 0 : (old_len + bs - 1) / bs;
+    const uint32_t sel_old = top < nblk ? top : nblk;
+    const uint32_t recent_count = seq_len < W ? seq_len : W;
+    uint32_t old_cap = sel_old * bs;
+    if (old_cap > old_len) old_cap = old_len;
+    const uint32_t capacity = recent_count + old_cap;
+    if (capacity == 0 || capacity > seq_len) return -7;
+    p->kv_heads = kvh; p->q_heads = q_heads; p->seq_len = seq_len; p->recent_window = W; p->block_size = bs;
+    p->top_n = sel_old; p->old_len = old_len; p->nblk = nblk; p->compressed = compressed ? 1u : 0u;
+    p->Q = static_cast<const float*>(q);
+    p->Out = static_cast<float*>(out);
+    if (compressed) {
+        p->old_k = kv->d_fp16_old_k + (size_t)seq_id * kv->max_seq_len * ept;
+        p->new_k = kv->d_recent_k + (size_t)seq_id * kv->recent_window * ept;
+        p->dense_v = kv->d_recent_v + (size_t)seq_id * kv->recent_window * ept;
+        p->q4_v = kv->d_q4_old_v + (size_t)seq_id * kv->max_seq_len * kvh * (hd / 2u);
+        p->q4_scale = kv->d_q4_old_v_scale + (size_t)seq_id * kv->max_seq_len * kvh;
+    } else {
+        p->old_k = kv->d_k + (size_t)seq_id * kv->max_seq_len * ept;
+        p->new_k = p->old_k;
+        p->dense_v = kv->d_v + (size_t)seq_id * kv->max_seq_len * ept;
+    }
+    M40StreamScratch& sc = ctx->scratch[1];
+    // select scratch: scores | sel | sel_scores | counts | ntok
+    const size_t scores_bytes = ((size_t)q_heads * (nblk ? nblk : 1) * 4 + 255) & ~(size_t)255;
+    const size_t fixed = (size_t)q_heads * (64 * 4 + 64 * 4 + 4 + 4) + 1024;
+    if (scores_bytes + fixed > sc.select_bytes) return -7;
+    char* base = static_cast<char*>(sc.select);
+    p->scores = reinterpret_cast<float*>(base);
+    p->sel = reinterpret_cast<uint32_t*>(base + scores_bytes);
+    p->sel_scores = reinterpret_cast<float*>(p->sel + (size_t)q_heads * 64);
+    p->counts = reinterpret_cast<uint32_t*>(p->sel_scores + (size_t)q_heads * 64);
+    p->ntok = p->counts + q_heads;
+    uint32_t chunk = 128;
+    while (chunk < 1024 && (size_t)q_heads * ((capacity + chunk - 1) / chunk) * (hd + 2) * 4 > sc.attn_partial_bytes)
+        chunk <<= 1;
+    p->chunk = chunk;
+    p->nchunks = (capacity + chunk - 1) / chunk;
+    if ((size_t)q_heads * p->nchunks * (hd + 2) * 4 > sc.attn_partial_bytes) return -7;
+    p->partial = static_cast<float*>(sc.attn_partial);
+    if ((size_t)nblk * 4 > 60 * 1024) return -7;  // block scores of one q head live in LDS
+    return 0;
+}
+
+template <int HD>
+int launch_all(hipStream_t s, const BsParams& p, bool selection_only) {
+    (void)hipGetLastError();
+    const uint32_t group = p.q_heads / p.kv_heads;
+    if (p.nblk > 0) {
+        dim3 grid((p.nblk + 3) / 4, p.kv_heads);
+        if (group >= 4) bs_score_kernel<HD, 4><<<grid, 256, 0, s>>>(p);
+        else if (group >= 2) bs_score_kernel<HD, 2><<<grid, 256, 0, s>>>(p);
+        else bs_score_kernel<HD, 1><<<grid, 256, 0, s>>>(p);
+    }
+    bs_select_kernel<<<p.q_heads, 1024, (size_t)(p.nblk ? p.nblk : 1) * 4, s>>>(p);
+    if (!selection_only) {
+        const size_t lds = ((size_t)2 * p.chunk + 4 * HD + 8) * sizeof(float);
+        dim3 grid(p.q_heads, p.nchunks);
+        bs_attend_kernel<HD><<<grid, 256, lds, s>>>(p);
+        if (p.nchunks > 1) bs_combine_kernel<HD><<<p.q_heads, HD, 0, s>>>(p);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -8;
+}
+
+int common_checks(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q, uint32_t q_heads,
+                  uint32_t seq_len, uint32_t W, uint32_t bs, uint32_t top, const void* out, bool compressed) {
+    if (!ctx || !kv || !q || !out) return -1;
+    if (compressed) {
+        if (!kv->fp16_k_q4_v_old_backing || !kv->d_fp16_old_k || !kv->d_q4_old_v || !kv->d_q4_old_v_scale ||
+            !kv->d_recent_k || !kv->d_recent_v)
+            return -16;
+    } else if (!kv->d_k || !kv->d_v) {
+        return -16;
+    }
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (seq_len == 0 || seq_len > kv->max_seq_len) return -3;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -4;
+    if (kv->head_dim != 64 && kv->head_dim != 128) return -5;
+    if (W == 0 || bs == 0 || top == 0 || top > 64) return -6;
+    // Only the plain top-k policy in score-rank order is built; refuse the environment knobs of
+    // the reference's experimental policies instead of silently computing something else.
+    if (policy_from_env() != 0u || order_from_env() != 0u) return -17;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async(
+    M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q_dev_f32, uint32_t q_heads,
+    uint32_t seq_len, uint32_t recent_window, uint32_t block_size, uint32_t top_blocks, void* out_dev_f32) {
+    int rc = common_checks(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, recent_window, block_size, top_blocks,
+                           out_dev_f32, true);
+    if (rc != 0) return rc;
+    BsParams p;
+    rc = prepare(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, recent_window, block_size, top_blocks, out_dev_f32,
+                 true, &p);
+    if (rc != 0) return rc;
+    return kv->head_dim == 64 ? launch_all<64>(ctx->decode_stream, p, false)
+                              : launch_all<128>(ctx->decode_stream, p, false);
+}
+
+int m40llm_attention_last_token_f32_gqa_block_select_exact_async(
+    M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q_dev_f32, uint32_t q_heads,
+    uint32_t seq_len, uint32_t recent_window, uint32_t block_size, uint32_t top_blocks, void* out_dev_f32) {
+    if (kv && kv->compressed) return -16;
+    int rc = common_checks(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, recent_window, block_size, top_blocks,
+                           out_dev_f32, false);
+    if (rc != 0) return rc;
+    BsParams p;
+    rc = prepare(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, recent_window, block_size, top_blocks, out_dev_f32,
+                 false, &p);
+    if (rc != 0) return rc;
+    return kv->head_dim == 64 ? launch_all<64>(ctx->decode_stream, p, false)
+                              : launch_all<128>(ctx->decode_stream, p, false);
+}
+
+int m40llm_ext_block_select_read_selection(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,
+                                           const void* q_dev_f32, uint32_t q_heads, uint32_t seq_len,
+                                           uint32_t recent_window, uint32_t block_size, uint32_t top_blocks,
+                                           uint32_t* out_blocks_host, uint32_t* out_counts_host,
+                                           float* out_scores_host) {
+    if (!out_blocks_host || !out_counts_host) return -1;
+    const bool compressed = kv && kv->compressed;
+    int rc = common_checks(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, recent_window, block_size, top_blocks,
+                           out_blocks_host, compressed);
+    if (rc != 0) return rc;
+    BsParams p;
+    rc = prepare(ctx, kv, seq_id, q_dev_f32, q_heads, seq_len, recent_window, block_size, top_blocks,
+                 nullptr, compressed, &p);
+    if (rc != 0) return rc;
+    rc = kv->head_dim == 64 ? launch_all<64>(ctx->decode_stream, p, true)
+                            : launch_all<128>(ctx->decode_stream, p, true);
+    if (rc != 0) return rc;
+    if (hipStreamSynchronize(ctx->decode_stream) != hipSuccess) return -9;
+    if (hipMemcpy(out_blocks_host, p.sel, (size_t)q_heads * 64 * 4, hipMemcpyDeviceToHost) != hipSuccess) return -9;
+    if (hipMemcpy(out_counts_host, p.counts, (size_t)q_heads * 4, hipMemcpyDeviceToHost) != hipSuccess) return -9;
+    if (out_scores_host &&
+        hipMemcpy(out_scores_host, p.sel_scores, (size_t)q_heads * 64 * 4, hipMemcpyDeviceToHost) != hipSuccess)
+        return -9;
+    return 0;
+}
+
+}  // extern "C"

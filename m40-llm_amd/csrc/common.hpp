@@ -1,0 +1,224 @@
+// Shared host/device definitions of the gfx950 implementation of the m40llm C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/m40llm.h"
+
+// ---------------------------------------------------------------------------------
+// Opaque handles.  Layout is private to this library (the reference declares them
+// zero-sized on the Rust side, src/cuda.rs:30-45).
+// ---------------------------------------------------------------------------------
+struct M40llmCudaEvent {
+    hipEvent_t event;
+};
+
+struct M40llmCudaGraphExec {
+    hipGraph_t graph;
+    hipGraphExec_t exec;
+};
+
+// Per-stream scratch owned by the context.  Two streams may run a GEMM or an
+// attention call at the same time, so each stream kind has its own copy.
+struct M40StreamScratch {
+    void* gemm_pack;         // packed f16 hi/lo activation fragments for the MFMA GEMM
+    size_t gemm_pack_bytes;
+    void* attn_partial;      // split-KV partial results (m, l, acc[hd]) of the attention kernels
+    size_t attn_partial_bytes;
+    void* select;            // block scores / selected ids / counts of the block-select path
+    size_t select_bytes;
+};
+
+struct M40llmCudaContext {
+    int device_id;
+    hipStream_t prefill_stream;
+    hipStream_t decode_stream;
+    hipEvent_t prefill_waits_decode_event;
+    hipEvent_t decode_waits_prefill_event;
+    M40StreamScratch scratch[2];   // [stream_kind]
+    int num_cus;
+};
+
+struct M40llmKVCache {
+    // dense storage, f16 [seq][token][kv_head][head_dim]
+    uint16_t* d_k;
+    uint16_t* d_v;
+    uint32_t* d_seq_map;           // tokens appended per sequence
+    // compressed storage
+    uint16_t* d_recent_k;          // ring [seq][W][kvh][hd], slot = pos % W
+    uint16_t* d_recent_v;
+    uint16_t* d_fp16_old_k;        // [seq][max_seq_len][kvh][hd], index = pos - W
+    uint8_t* d_q4_old_v;           // [seq][max_seq_len][kvh][hd/2]
+    float* d_q4_old_v_scale;       // [seq][max_seq_len][kvh]
+    uint32_t max_seq_len;
+    uint32_t max_batch_size;
+    uint32_t num_heads;            // kv heads
+    uint32_t head_dim;
+    uint32_t compressed;
+    uint32_t recent_window;
+    uint32_t block_size;
+    uint32_t max_blocks;
+    uint32_t top_blocks;
+    uint32_t representatives;
+    uint32_t representative_policy;
+    uint32_t fp16_k_q4_v_old_backing;
+    int device_id;
+};
+
+// ---------------------------------------------------------------------------------
+// Host helpers
+// ---------------------------------------------------------------------------------
+static inline int m40_ensure_device(M40llmCudaContext* ctx) {
+    if (!ctx) return -1;
+    return hipSetDevice(ctx->device_id) == hipSuccess ? 0 : -2;
+}
+
+static inline hipStream_t m40_select_stream(M40llmCudaContext* ctx, uint32_t stream_kind) {
+    if (!ctx) return nullptr;
+    if (stream_kind == 0) return ctx->prefill_stream;
+    if (stream_kind == 1) return ctx->decode_stream;
+    return nullptr;
+}
+
+#ifdef __HIPCC__
+#define M40_HD __host__ __device__
+#else
+#define M40_HD
+#endif
+M40_HD static inline bool m40_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Internal launch entry points shared between translation units ------------------
+// GEMM family (gemm.hip)
+int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
+                                 const float* A, const uint16_t* B, float* C, int M, int N, int K);
+// attention over an explicit dense range (attention.hip)
+struct M40AttnArgs {
+    const uint16_t* K;       // base of the cache (sequence 0)
+    const uint16_t* V;
+    uint32_t max_seq_len, kv_heads, head_dim, q_heads;
+    const float* Q;          // [batch][q_heads][hd]
+    float* Out;
+    uint32_t batch;
+    // one of: fixed (seq_id, seq_len) for batch==1, or device arrays
+    uint32_t seq_id, seq_len;
+    const uint32_t* seq_ids_dev;
+    const uint32_t* seq_lens_dev;   // also used alone for the seq_len_dev variant (batch==1)
+    uint32_t max_len_hint;          // upper bound of any row's length (sizes the grid)
+    uint32_t window;                // 0 = whole sequence, else only the last `window` tokens
+};
+int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
+                               const M40AttnArgs& a);
+
+// ---------------------------------------------------------------------------------
+// Device helpers
+// ---------------------------------------------------------------------------------
+#ifdef __HIPCC__
+#include <hip/hip_fp16.h>
+
+typedef _Float16 m40_half;
+typedef _Float16 m40_half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 m40_half4 __attribute__((ext_vector_type(4)));
+typedef float m40_float4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float m40_h2f(uint16_t bits) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, bits));
+}
+// round-to-nearest-even f32 -> f16 (v_cvt_f16_f32 in the default rounding mode)
+__device__ __forceinline__ uint16_t m40_f2h(float x) {
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
+}
+
+// Streaming (read-once) 128-bit load: keeps weights / old K out of the way of data that is reused.
+typedef uint32_t m40_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 m40_load_stream(const uint4* p) {
+    const m40_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const m40_u32x4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// 8 halves packed in a uint4 -> 8 floats
+__device__ __forceinline__ void m40_unpack8(const uint4& w, float (&f)[8]) {
+    const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = m40_h2f(static_cast<uint16_t>(u[i] & 0xffffu));
+        f[2 * i + 1] = m40_h2f(static_cast<uint16_t>(u[i] >> 16));
+    }
+}
+
+// Cross-lane add through DPP (row = 16 lanes).  ctrl: quad_perm / row_* selector.
+template <int CTRL>
+__device__ __forceinline__ float m40_dpp_f(float x) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+#define M40_DPP_XOR1 0xB1        // quad_perm [1,0,3,2]
+#define M40_DPP_XOR2 0x4E        // quad_perm [2,3,0,1]
+#define M40_DPP_HALF_MIRROR 0x141  // lane i <-> 7-i inside each group of 8
+#define M40_DPP_MIRROR 0x140       // lane i <-> 15-i inside each row of 16
+
+// Butterfly sums.  After the xor-1/xor-2 steps every lane of a quad holds the quad
+// sum, so the mirrors act as xor-4 / xor-8 on those sums; additions are commutative,
+// hence every lane ends with the bits of the halving tree
+//   ((x0+x1)+(x2+x3)) + ((x4+x5)+(x6+x7)) ...
+__device__ __forceinline__ float m40_sum8(float x) {   // over aligned groups of 8 lanes
+    x += m40_dpp_f<M40_DPP_XOR1>(x);
+    x += m40_dpp_f<M40_DPP_XOR2>(x);
+    x += m40_dpp_f<M40_DPP_HALF_MIRROR>(x);
+    return x;
+}
+__device__ __forceinline__ float m40_sum16(float x) {  // over rows of 16 lanes
+    x = m40_sum8(x);
+    x += m40_dpp_f<M40_DPP_MIRROR>(x);
+    return x;
+}
+__device__ __forceinline__ float m40_sum64(float x) {  // whole wave
+    x = m40_sum16(x);
+    x += __shfl_xor(x, 16, 64);
+    x += __shfl_xor(x, 32, 64);
+    return x;
+}
+__device__ __forceinline__ float m40_max64(float x) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+    return x;
+}
+
+__device__ __forceinline__ float m40_inv_sqrt_head_dim(uint32_t hd) {
+    return hd == 64u ? 0.125f : (hd == 128u ? 0.08838834764831845f : 1.0f / sqrtf((float)hd));
+}
+
+// RoPE pair addressing and rotation shared by every kernel that rotates, so the
+// fused append and the standalone RoPE produce identical bits.
+__device__ __forceinline__ void m40_rope_pair(uint32_t head, uint32_t off, uint32_t head_dim,
+                                              uint32_t layout, size_t* i0, size_t* i1) {
+    const size_t hb = (size_t)head * head_dim;
+    if (layout == M40LLM_ROPE_LAYOUT_NEOX) {
+        *i0 = hb + off;
+        *i1 = *i0 + head_dim / 2u;
+    } else {
+        *i0 = hb + 2u * off;
+        *i1 = *i0 + 1u;
+    }
+}
+__device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off, uint32_t head_dim,
+                                                float base, float scale, float x0, float x1,
+                                                float* y0, float* y1) {
+    const float pos = static_cast<float>(position) * scale;
+    const float theta = pos * powf(base, -2.0f * static_cast<float>(off) / static_cast<float>(head_dim));
+    const float c = cosf(theta);
+    const float s = sinf(theta);
+    *y0 = x0 * c - x1 * s;
+    *y1 = x0 * s + x1 * c;
+}
+
+// q4 V pair, two's-complement nibbles, even dim in the low nibble
+__device__ __forceinline__ uint8_t m40_pack_q4_pair(float a, float b, float scale) {
+    int qa = (int)lrintf(a / scale);
+    int qb = (int)lrintf(b / scale);
+    qa = qa < -7 ? -7 : (qa > 7 ? 7 : qa);
+    qb = qb < -7 ? -7 : (qb > 7 ? 7 : qb);
+    return (uint8_t)((qa & 0x0f) | ((qb & 0x0f) << 4));
+}
+#endif  // __HIPCC__

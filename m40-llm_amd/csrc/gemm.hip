@@ -1,0 +1,453 @@
+// GEMV / skinny GEMM family for gfx950: C[M,N] f32 = A[M,K] x B, f32 accumulation.
+//
+//   M == 1      : wave-per-column GEMV.  64 lanes stride the K dimension with 128-bit loads of
+//                 the f16 weights (GGUF layout: K contiguous per output column), f32 FMA per
+//                 lane, one DPP/shuffle butterfly per column.  HBM-bound; bytes = 2*N*K.
+//   2 <= M <= 16: MFMA (v_mfma_f32_16x16x32_f16).  The f32 activations are split exactly into
+//                 f16 hi + f16 lo parts (after a per-row power-of-two scale), the f16 weights go
+//                 from HBM to the B operand registers without passing LDS: lane (n, g) loads the
+//                 32 contiguous bytes k = 64t+16g .. +15 of column n, which are the B fragments
+//                 of two MFMAs.  Weights are read once for all rows.
+//   otherwise   : a plain wave-per-output kernel (any shape, any alignment).
+//
+// Reference semantics: gemm_f32xf16_gguf_f32_kernel cuda/kernels.cu:5037-5052 and the entry
+// points :5068-5302 (which run on the prefill stream and block until done).
+#include "common.hpp"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------
+// M == 1
+// ---------------------------------------------------------------------------------------
+template <int COLS>
+__global__ __launch_bounds__(256) void gemv_f32xf16_gguf_kernel(const float* __restrict__ A,
+                                                                const uint16_t* __restrict__ B,
+                                                                float* __restrict__ C, int N, int K) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int col0 = (blockIdx.x * 4 + wave) * COLS;
+    if (col0 >= N) return;
+    const int nchunks = K >> 3;  // 8 halves = 16 bytes per chunk
+    const uint4* bp[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        const int col = col0 + c < N ? col0 + c : N - 1;
+        bp[c] = reinterpret_cast<const uint4*>(B + (size_t)col * K);
+    }
+    const float4* a4 = reinterpret_cast<const float4*>(A);
+    float acc[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[c] = 0.0f;
+
+#pragma unroll 2
+    for (int kc = lane; kc < nchunks; kc += 64) {
+        const float4 a0 = a4[2 * kc], a1 = a4[2 * kc + 1];
+        const float av[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        uint4 w[COLS];
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) w[c] = m40_load_stream(bp[c] + kc);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            float f[8];
+            m40_unpack8(w[c], f);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[c] = fmaf(av[j], f[j], acc[c]);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        const float s = m40_sum64(acc[c]);
+        if (lane == 0 && col0 + c < N) C[col0 + c] = s;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// 2 <= M <= 16: activation packing + MFMA
+// ---------------------------------------------------------------------------------------
+// Packed layout: for k-tile t (64 values of k) and half s in {0,1}, lane l of the wave finds
+// its A fragment (8 halves = 16 bytes) at P[((t*2+s)*64 + l)]:
+//     row = l % 16,  k = 64t + 16*(l/16) + 8s + 0..7
+// which pairs with the B fragment "column n, same k" that the GEMM kernel loads.
+// STACKED (M <= 8): rows 0..7 carry hi(A[row]), rows 8..15 carry lo(A[row-8]).
+// Otherwise two fragment sets are written: hi at P, lo at P + K/64*2*64.
+// One workgroup per (padded) row; row_scale[row] = 2^e receives the factor to undo.
+__global__ __launch_bounds__(256) void pack_a_hilo_kernel(const float* __restrict__ A, int M, int K,
+                                                          int stacked, uint4* __restrict__ P,
+                                                          float* __restrict__ row_scale) {
+    __shared__ float wave_max[4];
+    const int row = blockIdx.x;  // 0..7 (stacked) or 0..15
+    const int tid = threadIdx.x;
+    const bool live = row < M;
+    float inv_scale = 1.0f, scale = 1.0f;
+    if (live) {
+        float mx = 0.0f;
+        for (int k = tid; k < K; k += 256) mx = fmaxf(mx, fabsf(A[(size_t)row * K + k]));
+        mx = m40_max64(mx);
+        if ((tid & 63) == 0) wave_max[tid >> 6] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+        if (mx > 0.0f && mx < INFINITY) {
+            int e;
+            (void)frexpf(mx, &e);         // mx = f * 2^e, f in [0.5, 1)
+            e -= 11;                      // scaled max in [2^10, 2^11)
+            e = e < -100 ? -100 : (e > 100 ? 100 : e);
+            scale = ldexpf(1.0f, e);
+            inv_scale = ldexpf(1.0f, -e);
+        }
+    }
+    if (tid == 0) row_scale[row] = scale;
+    const int frags = (K >> 6) * 2;  // (t, s) pairs
+    uint4* P_lo = P + (size_t)frags * 64;
+    // each thread produces whole 8-half fragments of this row: one per (t, s, g)
+    for (int f = tid; f < frags * 4; f += 256) {
+        const int g = f & 3, ts = f >> 2;
+        const int t = ts >> 1, s = ts & 1;
+        const int k0 = 64 * t + 16 * g + 8 * s;
+        uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float a = A[(size_t)row * K + k0 + j] * inv_scale;
+                const _Float16 h = static_cast<_Float16>(a);
+                const _Float16 l = static_cast<_Float16>(a - static_cast<float>(h));
+                hi[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (j & 1));
+                lo[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, l) << (16 * (j & 1));
+            }
+        }
+        const size_t frag_base = (size_t)ts * 64 + (size_t)g * 16;
+        if (stacked) {
+            P[frag_base + row] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            P[frag_base + row + 8] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        } else {
+            P[frag_base + row] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            P_lo[frag_base + row] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        }
+    }
+}
+
+__device__ __forceinline__ m40_float4 mfma16x16x32(const uint4& a, const uint4& b, m40_float4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(m40_half8, a),
+                                                  __builtin_bit_cast(m40_half8, b), c, 0, 0, 0);
+}
+
+// Grid: ceil(ntiles / T) workgroups of T*S waves.  Wave (t, s) owns output columns
+// [16*ntile, 16*ntile+16) and k-tiles [s*KT/S, (s+1)*KT/S); slices are summed through LDS in
+// ascending s, so the result does not depend on timing.
+template <bool STACKED>
+__global__ __launch_bounds__(1024) void gemm_mfma_f32xf16_gguf_kernel(
+    const uint4* __restrict__ P, const float* __restrict__ row_scale, const uint16_t* __restrict__ B,
+    float* __restrict__ C, int M, int N, int K, int T, int S) {
+    extern __shared__ float red[];  // [S][T][16][16]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t_in = wave % T, s = wave / T;
+    const int ntiles = (N + 15) >> 4;
+    int ntile = blockIdx.x * T + t_in;
+    const bool tile_live = ntile < ntiles;
+    if (!tile_live) ntile = ntiles - 1;
+    const int j = lane & 15, g = lane >> 4;
+    const int col = ntile * 16 + j;
+    const int col_c = col < N ? col : N - 1;
+    const int KT = K >> 6;
+    const int t_begin = (int)(((long long)s * KT) / S), t_end = (int)(((long long)(s + 1) * KT) / S);
+    const uint16_t* bcol = B + (size_t)col_c * K + 16 * g;
+    const uint4* P_lo = P + (size_t)KT * 2 * 64;
+
+    m40_float4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int t = t_begin; t < t_end; ++t) {
+        const uint4* bp = reinterpret_cast<const uint4*>(bcol + 64 * t);
+        const uint4 b0 = m40_load_stream(bp);
+        const uint4 b1 = m40_load_stream(bp + 1);
+        const uint4 a0 = P[(size_t)(t * 2 + 0) * 64 + lane];
+        const uint4 a1 = P[(size_t)(t * 2 + 1) * 64 + lane];
+        acc = mfma16x16x32(a0, b0, acc);
+        acc = mfma16x16x32(a1, b1, acc);
+        if (!STACKED) {
+            const uint4 l0 = P_lo[(size_t)(t * 2 + 0) * 64 + lane];
+            const uint4 l1 = P_lo[(size_t)(t * 2 + 1) * 64 + lane];
+            acc = mfma16x16x32(l0, b0, acc);
+            acc = mfma16x16x32(l1, b1, acc);
+        }
+    }
+    // lane (j, g) holds D[4g + r][j], r = 0..3
+    if (STACKED) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], 32, 64);  // hi rows + lo rows
+    }
+    float* my = red + ((size_t)(s * T + t_in) * 256);
+    if (!STACKED || g < 2) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) my[(4 * g + r) * 16 + j] = acc[r];
+    }
+    __syncthreads();
+    if (s == 0 && tile_live && (!STACKED || g < 2)) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 4 * g + r;
+            float v = 0.0f;
+            for (int ss = 0; ss < S; ++ss) v += red[((size_t)(ss * T + t_in) * 256) + row * 16 + j];
+            if (row < M && col < N) C[(size_t)row * N + col] = v * row_scale[row];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Any shape: one wave per output element, lanes stride k.
+// ---------------------------------------------------------------------------------------
+template <typename AT, bool GGUF>
+__global__ __launch_bounds__(256) void gemm_generic_kernel(const AT* __restrict__ A,
+                                                           const uint16_t* __restrict__ B,
+                                                           float* __restrict__ C, int M, int N, int K) {
+    const long long out = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (out >= (long long)M * N) return;
+    const int row = (int)(out / N), col = (int)(out % N);
+    const int lane = threadIdx.x & 63;
+    float acc = 0.0f;
+    for (int k = lane; k < K; k += 64) {
+        float a;
+        if constexpr (sizeof(AT) == 2) a = m40_h2f(A[(size_t)row * K + k]);
+        else a = A[(size_t)row * K + k];
+        const float b = m40_h2f(GGUF ? B[(size_t)col * K + k] : B[(size_t)k * N + col]);
+        acc = fmaf(a, b, acc);
+    }
+    acc = m40_sum64(acc);
+    if (lane == 0) C[(size_t)row * N + col] = acc;
+}
+
+// Row-major B[k*N + n]: a thread owns one output column for four rows, k ascending with one
+// accumulator per output (the reference's own order, kernels.cu:4999-5032); lanes read
+// consecutive n, so every B load is one contiguous 128-byte line per wave.
+template <typename AT, typename CT>
+__global__ __launch_bounds__(256) void gemm_rowmajor_kernel(const AT* __restrict__ A,
+                                                            const uint16_t* __restrict__ B,
+                                                            CT* __restrict__ C, int M, int N, int K) {
+    const int col = blockIdx.x * 256 + threadIdx.x;
+    const int row0 = blockIdx.y * 4;
+    if (col >= N) return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < K; ++k) {
+        const float b = m40_h2f(B[(size_t)k * N + col]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = row0 + r < M ? row0 + r : M - 1;
+            float a;
+            if constexpr (sizeof(AT) == 2) a = m40_h2f(A[(size_t)row * K + k]);
+            else a = A[(size_t)row * K + k];
+            acc[r] = fmaf(a, b, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (row0 + r < M) {
+            if constexpr (sizeof(CT) == 2) C[(size_t)(row0 + r) * N + col] = m40_f2h(acc[r]);
+            else C[(size_t)(row0 + r) * N + col] = acc[r];
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// q8_0 weights, native GGUF blocks {f16 d; int8 qs[32]} (34 bytes) along K.
+// One wave per output column; lane handles blocks lane, lane+64, ...; per block the partial
+// sum of a*q is formed first and scaled by d once.
+// ---------------------------------------------------------------------------------------
+template <int ROWS>
+__global__ __launch_bounds__(256) void gemm_f32xq80_kernel(const float* __restrict__ A,
+                                                           const uint8_t* __restrict__ B,
+                                                           float* __restrict__ C, int M, int N, int K,
+                                                           int row0) {
+    const int col = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (col >= N) return;
+    const int lane = threadIdx.x & 63;
+    const int nblk = K >> 5;
+    const uint8_t* colp = B + (size_t)col * nblk * 34;
+    float acc[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
+    for (int b = lane; b < nblk; b += 64) {
+        const uint16_t* p16 = reinterpret_cast<const uint16_t*>(colp + (size_t)b * 34);  // 2-byte aligned
+        const float d = m40_h2f(p16[0]);
+        float part[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) part[r] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint16_t two = p16[1 + i];
+            const float q0 = (float)(int8_t)(two & 0xff), q1 = (float)(int8_t)(two >> 8);
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const int row = row0 + r < M ? row0 + r : M - 1;
+                const float* a = A + (size_t)row * K + b * 32 + 2 * i;
+                part[r] = fmaf(a[0], q0, part[r]);
+                part[r] = fmaf(a[1], q1, part[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) acc[r] = fmaf(d, part[r], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        const float s = m40_sum64(acc[r]);
+        if (lane == 0 && row0 + r < M) C[(size_t)(row0 + r) * N + col] = s;
+    }
+}
+
+int pick_mfma_shape(int ntiles, int KT, int* T, int* S) {
+    // Aim for a few thousand waves in flight and >= 512 workgroups where N allows it.
+    int s = 1;
+    while (s < 16 && (long long)ntiles * s < 4096 && KT / (s * 2) >= 2) s *= 2;
+    int t = 1;
+    while (t * s < 16 && t < 4 && ntiles / (t * 2) >= 1024) t *= 2;
+    *T = t;
+    *S = s;
+    return 0;
+}
+
+}  // namespace
+
+int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
+                                 const float* A, const uint16_t* B, float* C, int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return -2;
+    (void)hipGetLastError();
+    const bool fast = (K % 8 == 0) && m40_aligned16(A) && m40_aligned16(B);
+    if (fast && M == 1) {
+        // columns per wave: keep >= ~2048 waves, give each lane several loads in flight
+        const long long waves1 = N;
+        if (waves1 >= 16384) {
+            gemv_f32xf16_gguf_kernel<4><<<(N + 15) / 16, 256, 0, stream>>>(A, B, C, N, K);
+        } else if (waves1 >= 6144) {
+            gemv_f32xf16_gguf_kernel<2><<<(N + 7) / 8, 256, 0, stream>>>(A, B, C, N, K);
+        } else {
+            gemv_f32xf16_gguf_kernel<1><<<(N + 3) / 4, 256, 0, stream>>>(A, B, C, N, K);
+        }
+    } else if (fast && K % 64 == 0 && (size_t)K * 64 <= ctx->scratch[stream_kind].gemm_pack_bytes - 256) {
+        M40StreamScratch& sc = ctx->scratch[stream_kind];
+        const int KT = K >> 6;
+        const int ntiles = (N + 15) >> 4;
+        int T, S;
+        pick_mfma_shape(ntiles, KT, &T, &S);
+        // scratch: [row_scale: 16 floats (64 B, padded to 256)] [P hi (+lo)]
+        float* row_scale = static_cast<float*>(sc.gemm_pack);
+        uint4* P = reinterpret_cast<uint4*>(static_cast<char*>(sc.gemm_pack) + 256);
+        for (int r0 = 0; r0 < M; r0 += 16) {
+            const int m = M - r0 < 16 ? M - r0 : 16;
+            const bool stacked = m <= 8;
+            pack_a_hilo_kernel<<<stacked ? 8 : 16, 256, 0, stream>>>(A + (size_t)r0 * K, m, K, stacked ? 1 : 0,
+                                                                     P, row_scale);
+            const size_t lds = (size_t)S * T * 256 * sizeof(float);
+            const int blocks = (ntiles + T - 1) / T;
+            if (stacked) {
+                gemm_mfma_f32xf16_gguf_kernel<true><<<blocks, T * S * 64, lds, stream>>>(
+                    P, row_scale, B, C + (size_t)r0 * N, m, N, K, T, S);
+            } else {
+                gemm_mfma_f32xf16_gguf_kernel<false><<<blocks, T * S * 64, lds, stream>>>(
+                    P, row_scale, B, C + (size_t)r0 * N, m, N, K, T, S);
+            }
+        }
+    } else {
+        const long long outs = (long long)M * N;
+        gemm_generic_kernel<float, true><<<(unsigned)((outs + 3) / 4), 256, 0, stream>>>(A, B, C, M, N, K);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+static int launch_q80(hipStream_t stream, const float* A, const uint8_t* B, float* C, int M, int N, int K) {
+    (void)hipGetLastError();
+    for (int r0 = 0; r0 < M; r0 += 4) {
+        const int m = M - r0;
+        if (m >= 4) gemm_f32xq80_kernel<4><<<(N + 3) / 4, 256, 0, stream>>>(A, B, C, M, N, K, r0);
+        else if (m == 3) gemm_f32xq80_kernel<3><<<(N + 3) / 4, 256, 0, stream>>>(A, B, C, M, N, K, r0);
+        else if (m == 2) gemm_f32xq80_kernel<2><<<(N + 3) / 4, 256, 0, stream>>>(A, B, C, M, N, K, r0);
+        else gemm_f32xq80_kernel<1><<<(N + 3) / 4, 256, 0, stream>>>(A, B, C, M, N, K, r0);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+extern "C" {
+
+int m40llm_gemm_f32xf16_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16,
+                                 void* d_C_f32, int M, int N, int K) {
+    if (!ctx || !d_A_f32 || !d_B_f16 || !d_C_f32) return -1;
+    int rc = m40_launch_gemm_f32xf16_gguf(ctx, ctx->prefill_stream, 0, static_cast<const float*>(d_A_f32),
+                                          static_cast<const uint16_t*>(d_B_f16), static_cast<float*>(d_C_f32),
+                                          M, N, K);
+    if (rc != 0) return rc;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_gemm_f32xf16_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16,
+                                           void* d_C_f32, int M, int N, int K, uint32_t stream_kind) {
+    if (!ctx || !d_A_f32 || !d_B_f16 || !d_C_f32) return -1;
+    hipStream_t stream = m40_select_stream(ctx, stream_kind);
+    if (!stream) return -4;
+    return m40_launch_gemm_f32xf16_gguf(ctx, stream, stream_kind, static_cast<const float*>(d_A_f32),
+                                        static_cast<const uint16_t*>(d_B_f16), static_cast<float*>(d_C_f32),
+                                        M, N, K);
+}
+
+int m40llm_gemm_f32xf16_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16, void* d_C_f32,
+                            int M, int N, int K) {
+    if (!ctx || !d_A_f32 || !d_B_f16 || !d_C_f32) return -1;
+    if (M <= 0 || N <= 0 || K <= 0) return -2;
+    (void)hipGetLastError();
+    dim3 grid((N + 255) / 256, (M + 3) / 4);
+    gemm_rowmajor_kernel<float, float><<<grid, 256, 0, ctx->prefill_stream>>>(
+        static_cast<const float*>(d_A_f32), static_cast<const uint16_t*>(d_B_f16), static_cast<float*>(d_C_f32),
+        M, N, K);
+    if (hipGetLastError() != hipSuccess) return -2;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_gemm_f16xf16_f32(M40llmCudaContext* ctx, const void* d_A_f16, const void* d_B_f16, void* d_C_f32,
+                            int M, int N, int K) {
+    if (!ctx || !d_A_f16 || !d_B_f16 || !d_C_f32) return -1;
+    if (M <= 0 || N <= 0 || K <= 0) return -2;
+    (void)hipGetLastError();
+    dim3 grid((N + 255) / 256, (M + 3) / 4);
+    gemm_rowmajor_kernel<uint16_t, float><<<grid, 256, 0, ctx->prefill_stream>>>(
+        static_cast<const uint16_t*>(d_A_f16), static_cast<const uint16_t*>(d_B_f16),
+        static_cast<float*>(d_C_f32), M, N, K);
+    if (hipGetLastError() != hipSuccess) return -2;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_gemm_f16_storage_f32_compute(M40llmCudaContext* ctx, const void* d_A, const void* d_B, void* d_C,
+                                        int M, int N, int K) {
+    if (!ctx || !d_A || !d_B || !d_C) return -1;
+    if (M <= 0 || N <= 0 || K <= 0) return -2;
+    (void)hipGetLastError();
+    dim3 grid((N + 255) / 256, (M + 3) / 4);
+    gemm_rowmajor_kernel<uint16_t, uint16_t><<<grid, 256, 0, ctx->prefill_stream>>>(
+        static_cast<const uint16_t*>(d_A), static_cast<const uint16_t*>(d_B), static_cast<uint16_t*>(d_C), M, N, K);
+    if (hipGetLastError() != hipSuccess) return -2;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_gemm_f32xq80_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_q80,
+                                     void* d_C_f32, int M, int N, int K) {
+    if (!ctx || !d_A_f32 || !d_B_q80 || !d_C_f32) return -1;
+    if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return -2;
+    int rc = launch_q80(ctx->prefill_stream, static_cast<const float*>(d_A_f32),
+                        static_cast<const uint8_t*>(d_B_q80), static_cast<float*>(d_C_f32), M, N, K);
+    if (rc != 0) return rc;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_w_gate_q80,
+                                        const void* d_w_up_q80, const void* d_w_down_q80,
+                                        void* d_scratch_f32, void* d_out_f32, int M, int d_model, int ffn) {
+    if (!ctx || !d_x_f32 || !d_w_gate_q80 || !d_w_up_q80 || !d_w_down_q80 || !d_scratch_f32 || !d_out_f32)
+        return -1;
+    if (M <= 0 || d_model <= 0 || ffn <= 0 || d_model % 32 != 0 || ffn % 32 != 0) return -2;
+    float* gate = static_cast<float*>(d_scratch_f32);
+    float* up = gate + (size_t)M * ffn;
+    const float* x = static_cast<const float*>(d_x_f32);
+    int rc = launch_q80(ctx->decode_stream, x, static_cast<const uint8_t*>(d_w_gate_q80), gate, M, ffn, d_model);
+    if (rc != 0) return rc;
+    rc = launch_q80(ctx->decode_stream, x, static_cast<const uint8_t*>(d_w_up_q80), up, M, ffn, d_model);
+    if (rc != 0) return rc;
+    rc = m40llm_swiglu_f32_async(ctx, gate, up, gate, (size_t)M * ffn);
+    if (rc != 0) return -3;
+    return launch_q80(ctx->decode_stream, gate, static_cast<const uint8_t*>(d_w_down_q80),
+                      static_cast<float*>(d_out_f32), M, d_model, ffn);
+}
+
+}  // extern "C"

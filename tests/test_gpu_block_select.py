@@ -1,0 +1,257 @@
+"""fp16-K / q4-V compressed cache and block-select attention: HIP path vs the CPU oracle (through the C-ABI)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from gpu_common import close, f16bits, m40  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from gpu_common import Dev
+    d = Dev()
+    yield d
+    d.sync()
+
+
+def _read_state(kv, seq):
+    B, S, H, D, W = kv.max_batch, kv.max_seq_len, kv.kv_heads, kv.head_dim, kv.compressed["recent_window"]
+    return dict(
+        old_k=kv.read_raw(0, np.uint16, (B, S, H, D))[seq],
+        q4_v=kv.read_raw(1, np.uint8, (B, S, H, D // 2))[seq],
+        q4_scale=kv.read_raw(2, np.float32, (B, S, H))[seq],
+        recent_k=kv.read_raw(3, np.uint16, (B, W, H, D))[seq],
+        recent_v=kv.read_raw(4, np.uint16, (B, W, H, D))[seq],
+        seq_map=kv.read_raw(5, np.uint32, (B,))[seq])
+
+
+def _oracle_state(c, seq):
+    return dict(old_k=c.old_k[seq], q4_v=c.q4_v[seq], q4_scale=c.q4_scale[seq], recent_k=c.recent_k[seq],
+                recent_v=c.recent_v[seq], seq_map=c.seq_map[seq])
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+def test_compressed_append_evict_bit_exact(dev, orc, hd):
+    rng = np.random.default_rng(hd)
+    kvh, W, bs, L, S = 2, 4, 4, 11, 16
+    kv = m40.KVCache(dev.ctx, S, 2, kvh, hd, dict(recent_window=W, block_size=bs, top_blocks=3))
+    c = orc.CompressedKV(S, 2, kvh, hd, W, bs)
+    for p in range(L):
+        k = rng.standard_normal(kvh * hd).astype(np.float32); v = rng.standard_normal(kvh * hd).astype(np.float32)
+        if p == 3:
+            v[:hd] = 0.0                       # all-zero V row: scale 1/7
+        dk, dv = dev.up(k), dev.up(v)
+        # freq_scale 0 makes RoPE the identity, as the reference's own q4 tests do
+        dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv.h, 1, dk.ptr, dv.ptr, p, 0, 1e4, 0.0, 0)
+        assert c.append(1, p, k, v, 1e4, 0.0, 0) == 0
+    got, want = _read_state(kv, 1), _oracle_state(c, 1)
+    for name in want:
+        assert np.array_equal(got[name], want[name]), name
+    assert not _read_state(kv, 0)["old_k"].any()
+    # byte accounting literals of tests/attention_parity_cuda_grid.rs:726-843 (hd 128, max_seq 16, 1 seq, 2 heads)
+    if hd == 128:
+        assert (S * 1 * kvh * hd * 2, S * 1 * kvh * hd // 2, S * 1 * kvh * 4) == (8192, 2048, 128)
+    # with rotation: ring rows within f16 tolerance of the oracle's rotation, V exact
+    kv2 = m40.KVCache(dev.ctx, S, 1, kvh, hd, dict(recent_window=W, block_size=bs))
+    c2 = orc.CompressedKV(S, 1, kvh, hd, W, bs)
+    for layout in (0, 1):
+        for p in range(6):
+            k = rng.standard_normal(kvh * hd).astype(np.float32); v = rng.standard_normal(kvh * hd).astype(np.float32)
+            dk, dv = dev.up(k), dev.up(v)
+            dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv2.h, 0, dk.ptr, dv.ptr, p, 0, 1e4, 1.0, layout)
+            c2.append(0, p, k, v, 1e4, 1.0, layout)
+        g, w = _read_state(kv2, 0), _oracle_state(c2, 0)
+        assert np.array_equal(g["recent_v"], w["recent_v"]) and g["seq_map"] == w["seq_map"]
+        close(g["recent_k"].view(np.float16).astype(np.float32), w["recent_k"].view(np.float16).astype(np.float32), 2e-3, 2e-3)
+    dk, dv = dev.up(k), dev.up(v)
+    dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv.h, 2, dk.ptr, dv.ptr, 0, 0, 1e4, 1.0, 0, expect=-3)
+    dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv.h, 0, dk.ptr, dv.ptr, S, 0, 1e4, 1.0, 0, expect=-5)
+    dense = m40.KVCache(dev.ctx, S, 1, kvh, hd)
+    dev.call("m40llm_kvcache_append_token_f32_rope_k_compressed_at_layout_async", dense.h, 0, dk.ptr, dv.ptr, 0, 1e4, 1.0, 0, expect=-2)
+
+
+def test_bulk_fill_equals_ordered_appends(dev, orc):
+    rng = np.random.default_rng(2)
+    kvh, hd, W, bs, S = 2, 64, 8, 4, 64
+    for L in (5, 8, 9, 40):
+        k16 = f16bits(rng.standard_normal((L, kvh, hd))); v16 = f16bits(rng.standard_normal((L, kvh, hd)))
+        a = m40.KVCache(dev.ctx, S, 1, kvh, hd, dict(recent_window=W, block_size=bs))
+        b = m40.KVCache(dev.ctx, S, 1, kvh, hd, dict(recent_window=W, block_size=bs))
+        dk, dv = dev.up(k16), dev.up(v16)
+        dev.call("m40llm_ext_kvcache_bulk_fill_f16", a.h, 0, dk.ptr, dv.ptr, L)
+        for p in range(L):
+            kf = k16[p].view(np.float16).astype(np.float32).reshape(-1); vf = v16[p].view(np.float16).astype(np.float32).reshape(-1)
+            dkp, dvp = dev.up(kf), dev.up(vf)
+            dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", b.h, 0, dkp.ptr, dvp.ptr, p, 0, 1e4, 0.0, 0)
+        ga, gb = _read_state(a, 0), _read_state(b, 0)
+        for name in ga:
+            assert np.array_equal(ga[name], gb[name]), (L, name)
+        c = orc.CompressedKV(S, 1, kvh, hd, W, bs)
+        c.bulk_fill(0, k16, v16)
+        wo = _oracle_state(c, 0)
+        for name in ga:
+            assert np.array_equal(ga[name], wo[name]), (L, name)
+
+
+def _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, S=None, seed=0, scale_k=1.0):
+    rng = np.random.default_rng(seed)
+    S = S or L
+    k16 = f16bits(rng.standard_normal((L, kvh, hd)) * scale_k); v16 = f16bits(rng.standard_normal((L, kvh, hd)))
+    q = rng.standard_normal((qh, hd)).astype(np.float32)
+    kv = m40.KVCache(dev.ctx, S, 1, kvh, hd, dict(recent_window=W, block_size=bs, top_blocks=top))
+    dk, dv = dev.up(k16), dev.up(v16)
+    dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, 0, dk.ptr, dv.ptr, L)
+    c = orc.CompressedKV(S, 1, kvh, hd, W, bs)
+    c.bulk_fill(0, k16, v16)
+    dq, out = dev.up(q), dev.zeros(qh * hd * 4)
+    dev.call("m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async",
+             kv.h, 0, dq.ptr, qh, L, W, bs, top, out.ptr)
+    dev.sync()
+    got = out.download(np.float32, (qh * hd,))
+    sel = np.zeros((qh, 64), dtype=np.uint32); cnt = np.zeros(qh, dtype=np.uint32); ssc = np.zeros((qh, 64), dtype=np.float32)
+    dev.call("m40llm_ext_block_select_read_selection", kv.h, 0, dq.ptr, qh, L, W, bs, top,
+             sel.ctypes.data, cnt.ctypes.data, ssc.ctypes.data)
+    orc.set_threads(8)
+    rc, want, wsel, wcnt = c.attention(0, q, qh, L, top, score_order=2)
+    assert rc == 0
+    return dict(got=got, want=want, sel=sel, cnt=cnt, ssc=ssc, wsel=wsel, wcnt=wcnt, c=c, q=q, kv=kv, k16=k16, v16=v16)
+
+
+@pytest.mark.parametrize("qh,kvh,hd,L,W,bs,top", [
+    (4, 2, 128, 16, 4, 4, 3),          # tests/attention_parity_cuda_grid.rs:726-843
+    (4, 2, 128, 5, 4, 32, 8),          # :608-723, one partial old block
+    (8, 2, 64, 300, 32, 16, 4),
+    (8, 2, 64, 20, 32, 16, 4),         # shorter than the window: no old blocks
+    (32, 8, 128, 4096, 512, 64, 64),   # BASELINE config 5 geometry at 4K context
+    (16, 4, 64, 2100, 1024, 32, 8),    # the reference's default window / block / top
+    (6, 2, 128, 777, 100, 48, 5),      # ragged everything, partial last block
+])
+def test_block_select_indices_exact_and_output(dev, orc, qh, kvh, hd, L, W, bs, top):
+    r = _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top)
+    assert np.array_equal(r["cnt"], r["wcnt"])
+    assert np.array_equal(r["sel"], r["wsel"])            # block ids bit-exact, in rank order
+    close(r["got"], r["want"], 2e-3, 2e-4)                # q4-V path tolerance of the reference: 2e-3
+    # scores of the selected blocks are the oracle's bits (same summation order)
+    c, q = r["c"], r["q"]
+    for h in range(qh):
+        s2 = c.block_scores(0, q[h], h // (qh // kvh), L, 2, W, bs)
+        n = int(r["cnt"][h])
+        assert np.array_equal(r["ssc"][h, :n], s2[r["sel"][h, :n]])
+    # report how far the selection is from flipping under the other summation orders
+    flips = 0
+    for h in range(qh):
+        s0 = c.block_scores(0, q[h], h // (qh // kvh), L, 0, W, bs)
+        b0, _ = orc.select_top_blocks(s0, top)
+        flips += int(not np.array_equal(b0, r["sel"][h, :len(b0)]))
+    print(f"[block-select] heads whose ranking differs under the device-kernel summation order: {flips}/{qh}")
+
+
+def test_block_select_all_blocks_equals_dense(dev, orc):
+    # property of tests/attention_parity_cuda_grid.rs:182-486: top >= old_blocks -> every token attended
+    qh, kvh, hd, L, W, bs = 8, 2, 64, 200, 40, 8
+    r = _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, 64, seed=3)
+    assert list(r["cnt"]) == [20] * qh
+    k = r["k16"].view(np.float16).astype(np.float64); q = r["q"].astype(np.float64)
+    # dequantised V via the oracle cache
+    c = r["c"]
+    vq = np.zeros((L, kvh, hd))
+    for t in range(L):
+        for h in range(kvh):
+            if t < L - W:
+                p = c.q4_v[0, t, h]; s = c.q4_scale[0, t, h]
+                nib = np.stack([p & 15, p >> 4], axis=1).reshape(-1).astype(np.int32)
+                nib = np.where(nib >= 8, nib - 16, nib)
+                vq[t, h] = (nib.astype(np.float32) * s).astype(np.float16).astype(np.float64)
+            else:
+                vq[t, h] = r["v16"][t, h].view(np.float16).astype(np.float64)
+    for h in range(qh):
+        kvhh = h // (qh // kvh)
+        s = (k[:, kvhh] @ q[h]) * 0.125
+        p = np.exp(s - s.max()); p /= p.sum()
+        close(r["got"][h * hd:(h + 1) * hd], p @ vq[:, kvhh], 2e-3, 2e-4)
+
+
+def test_block_select_ties_and_degenerate_scores(dev, orc):
+    # identical K rows everywhere -> every block scores the same -> lowest block ids win, in ascending order
+    qh, kvh, hd, L, W, bs, top = 4, 2, 64, 8 + 16 * 6, 8, 16, 3
+    rng = np.random.default_rng(4)
+    row = rng.standard_normal((1, kvh, hd))
+    k16 = f16bits(np.repeat(row, L, axis=0)); v16 = f16bits(rng.standard_normal((L, kvh, hd)))
+    q = rng.standard_normal((qh, hd)).astype(np.float32)
+    kv = m40.KVCache(dev.ctx, L, 1, kvh, hd, dict(recent_window=W, block_size=bs))
+    dk, dv = dev.up(k16), dev.up(v16)
+    dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, 0, dk.ptr, dv.ptr, L)
+    dq = dev.up(q)
+    sel = np.zeros((qh, 64), dtype=np.uint32); cnt = np.zeros(qh, dtype=np.uint32)
+    dev.call("m40llm_ext_block_select_read_selection", kv.h, 0, dq.ptr, qh, L, W, bs, top, sel.ctypes.data, cnt.ctypes.data, None)
+    assert list(cnt) == [3] * qh and all(list(sel[h, :3]) == [0, 1, 2] for h in range(qh))
+    c = orc.CompressedKV(L, 1, kvh, hd, W, bs); c.bulk_fill(0, k16, v16)
+    _, _, wsel, _ = c.attention(0, q, qh, L, top, score_order=2)
+    assert np.array_equal(sel, wsel)
+
+
+def test_block_select_argument_checks(dev, orc):
+    qh, kvh, hd, L, W, bs = 4, 2, 64, 64, 16, 8
+    kv = m40.KVCache(dev.ctx, L, 1, kvh, hd, dict(recent_window=W, block_size=bs))
+    dense = m40.KVCache(dev.ctx, L, 1, kvh, hd)
+    q = dev.up(np.zeros(qh * hd, dtype=np.float32)); out = dev.zeros(qh * hd * 4)
+    f = "m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async"
+    dev.call(f, kv.h, 0, None, qh, L, W, bs, 4, out.ptr, expect=-1)
+    dev.call(f, dense.h, 0, q.ptr, qh, L, W, bs, 4, out.ptr, expect=-16)      # missing backing
+    dev.call(f, kv.h, 1, q.ptr, qh, L, W, bs, 4, out.ptr, expect=-2)
+    dev.call(f, kv.h, 0, q.ptr, qh, 0, W, bs, 4, out.ptr, expect=-3)
+    dev.call(f, kv.h, 0, q.ptr, qh, L + 1, W, bs, 4, out.ptr, expect=-3)
+    dev.call(f, kv.h, 0, q.ptr, 3, L, W, bs, 4, out.ptr, expect=-4)
+    dev.call(f, kv.h, 0, q.ptr, qh, L, 0, bs, 4, out.ptr, expect=-6)
+    dev.call(f, kv.h, 0, q.ptr, qh, L, W, 0, 4, out.ptr, expect=-6)
+    dev.call(f, kv.h, 0, q.ptr, qh, L, W, bs, 0, out.ptr, expect=-6)
+    dev.call(f, kv.h, 0, q.ptr, qh, L, W, bs, 65, out.ptr, expect=-6)          # top_blocks > 64
+    assert dev.lib.m40llm_kvcache_create_compressed(dev.h, 16, 1, 2, 64, 0, 4, 1, 0, 0, 2) is None
+    assert dev.lib.m40llm_kvcache_create_compressed(dev.h, 16, 1, 2, 80, 4, 4, 1, 0, 0, 2) is None
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+def test_dense_backed_block_select(dev, orc, hd):
+    rng = np.random.default_rng(5 + hd)
+    qh, kvh, L, W, bs, top, S = 8, 2, 500, 64, 16, 6, 512
+    k16 = f16bits(rng.standard_normal((L, kvh, hd))); v16 = f16bits(rng.standard_normal((L, kvh, hd)))
+    q = rng.standard_normal((qh, hd)).astype(np.float32)
+    kv = m40.KVCache(dev.ctx, S, 1, kvh, hd)
+    dev.fill_dense(kv, 0, k16, v16)
+    dq, out = dev.up(q), dev.zeros(qh * hd * 4)
+    dev.call("m40llm_attention_last_token_f32_gqa_block_select_exact_async", kv.h, 0, dq.ptr, qh, L, W, bs, top, out.ptr)
+    dev.sync()
+    Kc = np.zeros((1, S, kvh, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
+    Kc[0, :L] = k16; Vc[0, :L] = v16
+    rc, want, wsel, wcnt = orc.dense_block_select(Kc, Vc, S, kvh, hd, 0, q, qh, L, W, bs, top, 2)
+    assert rc == 0
+    close(out.download(np.float32, (qh * hd,)), want)
+    sel = np.zeros((qh, 64), dtype=np.uint32); cnt = np.zeros(qh, dtype=np.uint32)
+    dev.call("m40llm_ext_block_select_read_selection", kv.h, 0, dq.ptr, qh, L, W, bs, top, sel.ctypes.data, cnt.ctypes.data, None)
+    assert np.array_equal(sel, wsel) and np.array_equal(cnt, wcnt)
+    # every block selected -> dense attention
+    dev.call("m40llm_attention_last_token_f32_gqa_block_select_exact_async", kv.h, 0, dq.ptr, qh, L, W, bs, 64, out.ptr)
+    dev.sync()
+    close(out.download(np.float32, (qh * hd,)), dev.attention(kv, 0, q, qh, L))
+
+
+def test_debug_select_old_blocks_host_twin(dev, orc):
+    rng = np.random.default_rng(6)
+    kvh, hd, W, bs, L = 2, 64, 8, 4, 8 + 4 * 9 + 2
+    k16 = f16bits(rng.standard_normal((L, kvh, hd)))
+    kv = m40.KVCache(dev.ctx, 64, 1, kvh, hd, dict(recent_window=W, block_size=bs))
+    dk = dev.up(k16)
+    dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, 0, dk.ptr, dk.ptr, L)
+    c = orc.CompressedKV(64, 1, kvh, hd, W, bs); c.bulk_fill(0, k16, k16)
+    q = rng.standard_normal(4 * hd).astype(np.float32); dq = dev.up(q)
+    blocks = np.zeros(2048, dtype=np.uint32); scores = np.zeros(2048, dtype=np.float32)
+    start = np.zeros(2048, dtype=np.uint32); end = np.zeros(2048, dtype=np.uint32)
+    count = np.zeros(1, dtype=np.uint32); total = np.zeros(1, dtype=np.uint32)
+    dev.call("m40llm_kvcache_debug_select_old_blocks", kv.h, 0, dq.ptr, 4, L, 999, 999, 3,
+             blocks.ctypes.data, scores.ctypes.data, start.ctypes.data, end.ctypes.data, count.ctypes.data, 2048, total.ctypes.data)
+    rc, wb, ws, wst, wen, wtot = c.debug_select(0, q[:hd], L, 3)
+    n = int(count[0])
+    assert rc == 0 and n == len(wb) == 3 and total[0] == wtot == 10
+    assert np.array_equal(blocks[:n], wb) and np.array_equal(scores[:n], ws)
+    assert np.array_equal(start[:n], wst) and np.array_equal(end[:n], wen)

@@ -1,0 +1,433 @@
+"""Parity of the HIP path against the CPU oracle, called through the C-ABI on a real GPU."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from gpu_common import Dev
+    d = Dev()
+    yield d
+    d.sync()
+
+
+from gpu_common import close, f16bits, m40  # noqa: E402
+
+
+# ------------------------------------------------------------------ elementwise
+def test_rms_norm(dev, orc):
+    rng = np.random.default_rng(0)
+    for rows, dim in ((2, 8), (1, 2048), (8, 2048), (3, 4096), (2, 37)):
+        x = rng.standard_normal((rows, dim)).astype(np.float32)
+        if (rows, dim) == (2, 8):
+            x = (np.arange(16, dtype=np.float32) * 0.25 - 3.0).reshape(2, 8)   # tests/rmsnorm_rope.rs:85-89
+        dx, dy = dev.up(x), dev.zeros(x.nbytes)
+        dev.call("m40llm_rms_norm_f32", dx.ptr, dy.ptr, rows, dim, 1e-5)
+        close(dy.download(np.float32, x.shape), orc.rms_norm(x, 1e-5), 1e-4, 1e-5)
+        w = (0.5 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+        for wd, wbits in ((1, w), (0, w.astype(np.float16).view(np.uint16))):
+            dw = dev.up(wbits)
+            dev.call("m40llm_rms_norm_f32_weighted", dx.ptr, dw.ptr, dy.ptr, rows, dim, 1e-5, wd)
+            close(dy.download(np.float32, x.shape), orc.rms_norm(x, 1e-5, wbits, wd), 1e-4, 1e-5)
+    dev.call("m40llm_rms_norm_f32_weighted_async", dx.ptr, dw.ptr, dy.ptr, 1, 8, 1e-5, 2, expect=-4)
+    dev.call("m40llm_rms_norm_f32_async", None, dy.ptr, 1, 8, 1e-5, expect=-1)
+    dev.call("m40llm_rms_norm_f32_async", dx.ptr, dy.ptr, 1, 0, 1e-5, expect=-1)
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_rope(dev, orc, layout):
+    rng = np.random.default_rng(1)
+    for rows, heads, hd, past, base in ((1, 2, 4, 3, 1e4), (2, 2, 4, 5, 1e4), (1, 32, 64, 159, 1e4),
+                                        (8, 16, 128, 4100, 1e6), (3, 4, 128, 32767, 1e6)):
+        x = rng.standard_normal((rows, heads * hd)).astype(np.float32)
+        dx = dev.up(x)
+        dev.call("m40llm_rope_f32_inplace_layout_async", dx.ptr, rows, heads, hd, past, base, 1.0, layout)
+        dev.sync()
+        close(dx.download(np.float32, x.shape), orc.rope(x, heads, hd, past, base, 1.0, layout), 1e-4, 1e-4)
+        # q&k form
+        dq, dk = dev.up(x), dev.up(x * 2)
+        dev.call("m40llm_rope_f32_layout_async", dq.ptr, dk.ptr, rows, heads, hd, past, base, 1.0, layout)
+        dev.sync()
+        close(dk.download(np.float32, x.shape), orc.rope(x * 2, heads, hd, past, base, 1.0, layout), 1e-4, 1e-4)
+        # position read from the device
+        dpos = dev.up(np.array([past], dtype=np.uint32))
+        dx2 = dev.up(x)
+        dev.call("m40llm_rope_f32_inplace_position_dev_layout_async", dx2.ptr, rows, heads, hd, dpos.ptr, base, 1.0, layout)
+        dev.sync()
+        assert np.array_equal(dx2.download(np.float32, x.shape), dx.download(np.float32, x.shape))
+    dev.call("m40llm_rope_f32_inplace_layout_async", dx.ptr, 1, 2, 5, 0, 1e4, 1.0, layout, expect=-2)
+    dev.call("m40llm_rope_f32_inplace_layout_async", dx.ptr, 1, 0, 4, 0, 1e4, 1.0, layout, expect=-1)
+
+
+def test_swiglu_residual_casts(dev, orc):
+    rng = np.random.default_rng(2)
+    n = 5632 * 3 + 1
+    g = (rng.standard_normal(n) * 4).astype(np.float32); u = rng.standard_normal(n).astype(np.float32)
+    dg, du, do = dev.up(g), dev.up(u), dev.zeros(n * 4)
+    dev.call("m40llm_swiglu_f32", dg.ptr, du.ptr, do.ptr, n)
+    close(do.download(np.float32, (n,)), orc.swiglu(g, u), 1e-5, 1e-6)        # tests/cuda_elementwise.rs: 1e-5
+    dev.call("m40llm_residual_add_f32", dg.ptr, du.ptr, do.ptr, n)
+    assert np.array_equal(do.download(np.float32, (n,)), g + u)
+    dev.call("m40llm_swiglu_f32_async", dg.ptr, du.ptr, do.ptr, 0)
+    dev.call("m40llm_residual_add_f32_async", None, du.ptr, do.ptr, 4, expect=-1)
+    h = rng.standard_normal(1000).astype(np.float16)
+    dh, df = dev.up(h.view(np.uint16)), dev.zeros(4000)
+    dev.call("m40llm_f16_to_f32", dh.ptr, df.ptr, 1000)
+    assert np.array_equal(df.download(np.float32, (1000,)), h.astype(np.float32))
+
+
+def _q80_pack(d_f16, qs):
+    nblk = qs.shape[0]
+    out = np.zeros((nblk, 34), dtype=np.uint8)
+    out[:, :2] = d_f16.view(np.uint8).reshape(nblk, 2)
+    out[:, 2:] = qs.view(np.uint8)
+    return out
+
+
+def test_q80_dequant_reference_fixture(dev, orc):
+    rows, blks = 3, 2     # tests/embedding_dequant_cuda.rs:189-206
+    for row in range(rows):
+        d = np.array([0.25 + 0.125 * row + 0.0625 * b for b in range(blks)], dtype=np.float32).astype(np.float16)
+        qs = np.array([[((17 * row + 5 * b + i) % 23) - 11 for i in range(32)] for b in range(blks)], dtype=np.int8)
+        blob = _q80_pack(d, qs)
+        din, dout = dev.up(blob), dev.zeros(blks * 32 * 4)
+        dev.call("m40llm_q80_to_f32", din.ptr, dout.ptr, blks * 32)
+        assert np.array_equal(dout.download(np.float32, (blks * 32,)), orc.q80_to_f32(blob, blks * 32))
+
+
+# ------------------------------------------------------------------ KV append
+def test_kv_append_cast_bit_exact(dev, orc):
+    # fixtures of tests/kv_f32_to_f16_append.rs (odd element count included)
+    for heads, hd in ((1, 3), (2, 8), (4, 64)):
+        elems = heads * hd
+        kv = m40.KVCache(dev.ctx, 4, 2, heads, hd)
+        i = np.arange(elems, dtype=np.float32)
+        toks = [((i + 0.25).astype(np.float32), (100 + i + 0.5).astype(np.float32)),
+                ((-10 + 0.125 * i).astype(np.float32), (np.float32(np.pi) + 0.25 * i).astype(np.float32))]
+        for t, (k, v) in enumerate(toks):
+            dk, dv = dev.up(k), dev.up(v)
+            dev.call("m40llm_kvcache_append_token_f32", kv.h, 1, dk.ptr, dv.ptr)
+            gk, gv = kv.read_token(1, t)
+            assert np.array_equal(gk, k.astype(np.float16).view(np.uint16))
+            assert np.array_equal(gv, v.astype(np.float16).view(np.uint16))
+        gk, _ = kv.read_token(0, 0)
+        assert not gk.any()
+        # cache full after max_seq_len appends -> -4; reset -> position 0 again
+        for _ in range(2):
+            dev.call("m40llm_kvcache_append_token_f32_async", kv.h, 1, dk.ptr, dv.ptr)
+        dev.call("m40llm_kvcache_append_token_f32_async", kv.h, 1, dk.ptr, dv.ptr, expect=-4)
+        dev.call("m40llm_kvcache_append_token_f32_async", kv.h, 2, dk.ptr, dv.ptr, expect=-2)
+        dev.call("m40llm_kvcache_reset", kv.h)
+        dev.call("m40llm_kvcache_append_token_f32", kv.h, 1, dk.ptr, dv.ptr)
+        gk, _ = kv.read_token(1, 0)
+        assert np.array_equal(gk, toks[1][0].astype(np.float16).view(np.uint16))
+        # f16 D2D append
+        kv2 = m40.KVCache(dev.ctx, 4, 1, heads, hd)
+        hk = dev.up(toks[0][0].astype(np.float16).view(np.uint16)); hv = dev.up(toks[0][1].astype(np.float16).view(np.uint16))
+        dev.call("m40llm_kvcache_append_token", kv2.h, 0, hk.ptr, hv.ptr)
+        gk, gv = kv2.read_token(0, 0)
+        assert np.array_equal(gv, toks[0][1].astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_kv_append_rope_k_fused_equals_standalone(dev, orc, layout):
+    # tests/kv_f32_to_f16_append.rs:297-384: fused RoPE-K append must be bit-identical (u16) to
+    # standalone rope_f32_inplace + cast append on the same device
+    rng = np.random.default_rng(3)
+    for heads, hd, base in ((4, 64, 1e4), (2, 128, 1e6)):
+        elems = heads * hd
+        kv_a = m40.KVCache(dev.ctx, 64, 1, heads, hd)
+        kv_b = m40.KVCache(dev.ctx, 64, 1, heads, hd)
+        kv_c = m40.KVCache(dev.ctx, 64, 1, heads, hd)
+        for pos in (0, 1, 7, 40):
+            k = rng.standard_normal(elems).astype(np.float32); v = rng.standard_normal(elems).astype(np.float32)
+            dk, dv = dev.up(k), dev.up(v)
+            dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv_a.h, 0, dk.ptr, dv.ptr, pos, 999, base, 1.0, layout)
+            dk2 = dev.up(k)
+            dev.call("m40llm_rope_f32_inplace_layout_async", dk2.ptr, 1, heads, hd, pos, base, 1.0, layout)
+            dev.call("m40llm_kvcache_reset", kv_b.h)
+            dev.call("m40llm_kvcache_append_token_f32", kv_b.h, 0, dk2.ptr, dv.ptr)
+            dpos = dev.up(np.array([pos], dtype=np.uint32))
+            dev.call("m40llm_kvcache_append_token_f32_rope_k_position_dev_layout_async", kv_c.h, 0, dk.ptr, dv.ptr, dpos.ptr, base, 1.0, layout)
+            dev.sync()
+            ka, va = kv_a.read_token(0, pos)
+            kb, vb = kv_b.read_token(0, 0)
+            kc, vc = kv_c.read_token(0, pos)
+            assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+            assert np.array_equal(ka, kc) and np.array_equal(va, vc)
+            assert np.array_equal(va, v.astype(np.float16).view(np.uint16))
+            # against the oracle: rotation within tolerance of f16 storage
+            Ko = np.zeros((1, 64, heads, hd), dtype=np.uint16); Vo = np.zeros_like(Ko)
+            orc.lib().orc_kv_append_f32_rope_k(orc.ptr(Ko), orc.ptr(Vo), 64, heads, hd, 0, pos, orc.ptr(k), orc.ptr(v), base, 1.0, layout)
+            close(ka.view(np.float16).astype(np.float32), Ko[0, pos].reshape(-1).view(np.float16).astype(np.float32), 2e-3, 2e-3)
+            assert kv_a.read_raw(5, np.uint32, (1,))[0] == pos + 1      # seq_map = position + 1
+        # non-"at" variant stores at the current length and rotates for past_len
+        kv_d = m40.KVCache(dev.ctx, 64, 1, heads, hd)
+        dev.call("m40llm_kvcache_append_token_f32_rope_k_layout_async", kv_d.h, 0, dk.ptr, dv.ptr, 40, base, 1.0, layout)
+        dev.sync()
+        kd, _ = kv_d.read_token(0, 0)
+        assert np.array_equal(kd, ka)
+        dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv_a.h, 0, dk.ptr, dv.ptr, 64, 0, base, 1.0, layout, expect=-5)
+        dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv_a.h, 1, dk.ptr, dv.ptr, 0, 0, base, 1.0, layout, expect=-2)
+
+
+# ------------------------------------------------------------------ GEMM family
+def test_gemm_known_answers(dev, orc):
+    A = f16bits([[1, 2], [3, 4]]); B = f16bits([[5, 6], [7, 8]])
+    dA, dB, dC = dev.up(A), dev.up(B), dev.zeros(16)
+    dev.call("m40llm_gemm_f16xf16_f32", dA.ptr, dB.ptr, dC.ptr, 2, 2, 2)
+    assert np.array_equal(dC.download(np.float32, (2, 2)), [[19, 22], [43, 50]])
+    A = f16bits([[1, 2, 3]]); B = f16bits([[4, 5], [6, 7], [8, 9]])
+    dA, dB = dev.up(A), dev.up(B)
+    dev.call("m40llm_gemm_f16xf16_f32", dA.ptr, dB.ptr, dC.ptr, 1, 2, 3)
+    assert np.array_equal(dC.download(np.float32, (1, 2)), [[40, 46]])
+    Af = dev.up(np.array([[1, 2, 3]], dtype=np.float32))
+    dev.call("m40llm_gemm_f32xf16_f32", Af.ptr, dB.ptr, dC.ptr, 1, 2, 3)
+    assert np.array_equal(dC.download(np.float32, (1, 2)), [[40, 46]])
+    Bg = dev.up(f16bits(np.array([[4, 5], [6, 7], [8, 9]]).T))
+    dev.call("m40llm_gemm_f32xf16_gguf_f32", Af.ptr, Bg.ptr, dC.ptr, 1, 2, 3)
+    assert np.array_equal(dC.download(np.float32, (1, 2)), [[40, 46]])
+    dC16 = dev.zeros(8)
+    dA = dev.up(f16bits([[1, 2], [3, 4]])); dB = dev.up(f16bits([[5, 6], [7, 8]]))
+    dev.call("m40llm_gemm_f16_storage_f32_compute", dA.ptr, dB.ptr, dC16.ptr, 2, 2, 2)
+    assert np.array_equal(dC16.download(np.uint16, (2, 2)).view(np.float16).astype(np.float32), [[19, 22], [43, 50]])
+    assert dev.lib.m40llm_gemm_f32xf16_gguf_f32(None, Af.ptr, Bg.ptr, dC.ptr, 1, 2, 3) == -1
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (1, 2048, 2048), (1, 256, 2048), (1, 5632, 2048), (1, 2048, 5632), (1, 32000, 2048),   # TinyLlama shapes
+    (1, 11008, 2048), (1, 2048, 11008),                                                        # Qwen2.5-3B shapes
+    (2, 2048, 2048), (4, 256, 2048), (8, 2048, 2048), (8, 11008, 2048), (8, 2048, 11008),     # batched (MFMA, stacked)
+    (16, 2048, 2048), (9, 4096, 4096), (16, 300, 14336),                                       # MFMA, two fragment sets
+    (20, 520, 1024),                                                                           # more than one row tile
+    (1, 37, 300), (3, 37, 300), (5, 7, 8), (1, 50, 2056),                                      # odd shapes: generic / tails
+])
+def test_gemm_gguf_vs_oracle(dev, orc, M, N, K):
+    rng = np.random.default_rng(M * 1000003 + N * 101 + K)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    if M > 1:
+        A[1] *= 1e-3          # rows of very different magnitude (per-row scaling of the hi/lo split)
+    if M > 2:
+        A[2] *= 3e4
+    B = f16bits(rng.standard_normal((N, K)) * 0.02)
+    got = dev.gemm_gguf(A, B, M, N, K)
+    want = orc.gemm("f32xf16_gguf", A, B, M, N, K)
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    # relative 1e-3 / absolute 1e-4 on rows normalised to unit scale
+    close(got / scale, want / scale)
+    f64 = A.astype(np.float64) @ B.view(np.float16).astype(np.float64).T
+    close(got / scale, f64 / scale, 1e-4, 1e-5)
+
+
+def test_gemm_batched_rows_match_single_row(dev, orc):
+    """Each row of the batched (MFMA) GEMM is the same dot product as the M=1 GEMV within tolerance, and does
+    not depend on which other rows share the batch."""
+    rng = np.random.default_rng(5)
+    N, K = 2048, 2048
+    B = f16bits(rng.standard_normal((N, K)) * 0.02)
+    A = rng.standard_normal((8, K)).astype(np.float32)
+    full = dev.gemm_gguf(A, B, 8, N, K)
+    A2 = A.copy(); A2[[0, 2, 4]] = rng.standard_normal((3, K)).astype(np.float32) * 100
+    part = dev.gemm_gguf(A2, B, 8, N, K)
+    assert np.array_equal(full[[1, 3, 5, 6, 7]], part[[1, 3, 5, 6, 7]])
+    single = dev.gemm_gguf(A[3:4], B, 1, N, K)
+    close(full[3:4], single, 1e-4, 1e-5)
+
+
+def test_gemm_async_extension_matches_blocking(dev, orc):
+    rng = np.random.default_rng(6)
+    M, N, K = 1, 4096, 2048
+    A = rng.standard_normal((M, K)).astype(np.float32); B = f16bits(rng.standard_normal((N, K)) * 0.02)
+    dA, dB, dC = dev.up(A), dev.up(B), dev.zeros(M * N * 4)
+    dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_async", dA.ptr, dB.ptr, dC.ptr, M, N, K, 1)
+    dev.sync()
+    assert np.array_equal(dC.download(np.float32, (M, N)), dev.gemm_gguf(A, B, M, N, K))
+    dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_async", dA.ptr, dB.ptr, dC.ptr, M, N, K, 2, expect=-4)
+
+
+def test_gemm_rowmajor_vs_oracle(dev, orc):
+    rng = np.random.default_rng(7)
+    M, N, K = 5, 300, 129
+    A = rng.standard_normal((M, K)).astype(np.float32); B = f16bits(rng.standard_normal((K, N)) * 0.1)
+    dA, dB, dC = dev.up(A), dev.up(B), dev.zeros(M * N * 4)
+    dev.call("m40llm_gemm_f32xf16_f32", dA.ptr, dB.ptr, dC.ptr, M, N, K)
+    close(dC.download(np.float32, (M, N)), orc.gemm("f32xf16_rowmajor", A, B, M, N, K), 1e-4, 1e-5)
+    A16 = f16bits(A); dA16 = dev.up(A16)
+    dev.call("m40llm_gemm_f16xf16_f32", dA16.ptr, dB.ptr, dC.ptr, M, N, K)
+    close(dC.download(np.float32, (M, N)), orc.gemm("f16xf16_rowmajor", A16, B, M, N, K), 1e-4, 1e-5)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_q80_gemm_and_ffn_vs_oracle(dev, orc, M):
+    rng = np.random.default_rng(11 + M)
+    d_model, ffn = 256, 512
+    def qmat(n, k):
+        d = rng.uniform(0.001, 0.01, size=(n, k // 32)).astype(np.float16)
+        qs = rng.integers(-127, 128, size=(n, k // 32, 32)).astype(np.int8)
+        return np.ascontiguousarray(np.stack([_q80_pack(d[i], qs[i]) for i in range(n)]))
+    wg, wu, wd = qmat(ffn, d_model), qmat(ffn, d_model), qmat(d_model, ffn)
+    x = rng.standard_normal((M, d_model)).astype(np.float32)
+    dx, dwg, dC = dev.up(x), dev.up(wg), dev.zeros(M * ffn * 4)
+    dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dx.ptr, dwg.ptr, dC.ptr, M, ffn, d_model)
+    want = orc.gemm("f32xq80_gguf", x, wg, M, ffn, d_model)
+    close(dC.download(np.float32, (M, ffn)), want, 1e-3, 1e-4 * np.abs(want).max())
+    dwu, dwd = dev.up(wu), dev.up(wd)
+    scratch, out = dev.zeros(2 * M * ffn * 4), dev.zeros(M * d_model * 4)
+    dev.call("m40llm_ext_ffn_swiglu_q80_f32_async", dx.ptr, dwg.ptr, dwu.ptr, dwd.ptr, scratch.ptr, out.ptr, M, d_model, ffn)
+    dev.sync()
+    want = orc.ffn_swiglu_q80(x, wg, wu, wd, M, d_model, ffn)
+    close(out.download(np.float32, (M, d_model)), want, 1e-3, 1e-4 * max(np.abs(want).max(), 1.0))
+
+
+# ------------------------------------------------------------------ dense attention
+def _attention_case(dev, orc, qh, kvh, hd, L, k, v, q, max_seq=None, seq=0, batch=1):
+    max_seq = max_seq or L
+    kv = m40.KVCache(dev.ctx, max_seq, batch, kvh, hd)
+    K16 = f16bits(k).reshape(L, kvh, hd); V16 = f16bits(v).reshape(L, kvh, hd)
+    dev.fill_dense(kv, seq, K16, V16)
+    got = dev.attention(kv, seq, q, qh, L)
+    Kc = np.zeros((batch, max_seq, kvh, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
+    Kc[seq, :L] = K16; Vc[seq, :L] = V16
+    want = orc.attention(Kc, Vc, max_seq, kvh, hd, seq, q, qh, L)
+    return got, want, kv
+
+
+def test_attention_mha_grid_fixture(dev, orc):
+    # grid + closed-form data of tests/attention_parity_cpu_grid.rs:74-118, via the MHA entry point
+    for heads in (1, 2, 3, 4):
+        for hd in (1, 5, 7, 8, 16, 31, 32, 63, 64):
+            dim = heads * hd
+            for L in (1, 2, 3, 4, 7, 8, 16):
+                t = np.arange(L)[:, None]; i = np.arange(dim)[None, :]
+                k = ((t * dim + i).astype(np.float32) * np.float32(0.01) - 1)
+                v = ((t * dim + (dim - 1 - i)).astype(np.float32) * np.float32(0.02) - 2)
+                q = (np.arange(dim, dtype=np.float32) * np.float32(0.003) - np.float32(0.5))
+                kv = m40.KVCache(dev.ctx, 16, 1, heads, hd)
+                for tt in range(L):
+                    dk, dv = dev.up(k[tt].astype(np.float32)), dev.up(v[tt].astype(np.float32))
+                    dev.call("m40llm_kvcache_append_token_f32_async", kv.h, 0, dk.ptr, dv.ptr)
+                dq, out = dev.up(q), dev.zeros(dim * 4)
+                dev.call("m40llm_attention_last_token_f32", kv.h, 0, dq.ptr, L, out.ptr)
+                Kc = np.zeros((1, 16, heads, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
+                Kc[0, :L] = f16bits(k).reshape(L, heads, hd); Vc[0, :L] = f16bits(v).reshape(L, heads, hd)
+                want = orc.attention(Kc, Vc, 16, heads, hd, 0, q, heads, L)
+                close(out.download(np.float32, (dim,)), want, 1e-3, 1e-4)   # tests/attention_last_token.rs:203
+                kv.destroy()
+
+
+@pytest.mark.parametrize("L", [128, 512])
+def test_attention_gqa_config1_reference_fixture(dev, orc, L):
+    qh, kvh, hd = 32, 4, 64           # tests/attention_parity_cuda_grid.rs:1737-1772
+    kv_dim = kvh * hd
+    t = np.arange(L)[:, None]; i = np.arange(kv_dim)[None, :]
+    k = ((t * kv_dim + i).astype(np.float32) * np.float32(0.0003) - np.float32(0.25))
+    v = ((t * kv_dim + (kv_dim - 1 - i)).astype(np.float32) * np.float32(0.0002) - np.float32(0.1))
+    q = (np.arange(qh * hd, dtype=np.float32) * np.float32(0.0004) - np.float32(0.2))
+    got, want, _ = _attention_case(dev, orc, qh, kvh, hd, L, k, v, q)
+    close(got, want)
+
+
+@pytest.mark.parametrize("qh,kvh,hd,L", [
+    (32, 4, 64, 512),        # BASELINE config 1 (seed 0, N(0,1))
+    (32, 4, 64, 1), (32, 4, 64, 33), (32, 4, 64, 160),
+    (16, 2, 128, 2176), (16, 2, 128, 4096),
+    (32, 8, 128, 9000),      # beyond the reference's 8192 fast-path cap
+    (6, 2, 64, 100), (3, 3, 128, 70), (12, 1, 64, 257), (5, 1, 128, 31),   # uneven groups
+])
+def test_attention_random_vs_oracle(dev, orc, qh, kvh, hd, L):
+    rng = np.random.default_rng(0)
+    q = rng.standard_normal(qh * hd).astype(np.float32)
+    k = rng.standard_normal((L, kvh * hd)).astype(np.float32)
+    v = rng.standard_normal((L, kvh * hd)).astype(np.float32)
+    got, want, kv = _attention_case(dev, orc, qh, kvh, hd, L, k, v, q, max_seq=L + 3, seq=1, batch=2)
+    close(got, want)
+    if L == 1:
+        vf = f16bits(v).view(np.float16).astype(np.float32).reshape(kvh, hd)
+        assert np.array_equal(got.reshape(qh, hd), np.repeat(vf, qh // kvh, axis=0))
+    # error codes
+    dq, out = dev.up(q), dev.zeros(qh * hd * 4)
+    dev.call("m40llm_attention_last_token_f32_gqa_async", kv.h, 2, dq.ptr, qh, L, out.ptr, expect=-2)
+    dev.call("m40llm_attention_last_token_f32_gqa_async", kv.h, 0, dq.ptr, qh, 0, out.ptr, expect=-3)
+    dev.call("m40llm_attention_last_token_f32_gqa_async", kv.h, 0, dq.ptr, qh, L + 4, out.ptr, expect=-3)
+    dev.call("m40llm_attention_last_token_f32_gqa_async", kv.h, 0, dq.ptr, qh + 1 if kvh > 1 else 0, L, out.ptr, expect=-6)
+    # device-side length and recent-window forms agree with the plain call
+    dlen = dev.up(np.array([L], dtype=np.uint32))
+    dev.call("m40llm_attention_last_token_f32_gqa_seq_len_dev_async", kv.h, 1, dq.ptr, qh, dlen.ptr, out.ptr)
+    dev.sync()
+    close(out.download(np.float32, (qh * hd,)), want)
+    W = max(1, L // 3)
+    dev.call("m40llm_attention_last_token_f32_gqa_dense_recent_async", kv.h, 1, dq.ptr, qh, L, W, out.ptr)
+    dev.sync()
+    Kc = np.zeros((1, W, kvh, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
+    Kc[0] = f16bits(k).reshape(L, kvh, hd)[L - W:]; Vc[0] = f16bits(v).reshape(L, kvh, hd)[L - W:]
+    close(out.download(np.float32, (qh * hd,)), orc.attention(Kc, Vc, W, kvh, hd, 0, q, qh, W))
+
+
+def test_attention_batched_varlen_reference_fixture(dev, orc):
+    # tests/attention_batched_varlen.rs:36-69: qh 4, kvh 2, hd 64, lens [1,3,5], ids [0,1,2]
+    qh, kvh, hd, maxL = 4, 2, 64, 8
+    kv = m40.KVCache(dev.ctx, maxL, 3, kvh, hd)
+    Kc = np.zeros((3, maxL, kvh, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
+    lens, ids = [1, 3, 5], [0, 1, 2]
+    for s, L in zip(ids, lens):
+        t = np.arange(L)[:, None]; i = np.arange(kvh * hd)[None, :]
+        k = ((s * 7 + t * 3 + i) % 17).astype(np.float32) * np.float32(0.05) - np.float32(0.4)
+        v = ((s * 5 + t * 11 + i) % 13).astype(np.float32) * np.float32(0.07) - np.float32(0.3)
+        Kc[s, :L] = f16bits(k).reshape(L, kvh, hd); Vc[s, :L] = f16bits(v).reshape(L, kvh, hd)
+        dev.fill_dense(kv, s, Kc[s, :L], Vc[s, :L])
+    q = ((np.arange(3 * qh * hd) % 19).astype(np.float32) * np.float32(0.03) - np.float32(0.25)).reshape(3, qh * hd)
+    dq, out = dev.up(q), dev.zeros(q.nbytes)
+    dids, dlens = dev.up(np.array(ids, dtype=np.uint32)), dev.up(np.array(lens, dtype=np.uint32))
+    dev.call("m40llm_attention_last_token_f32_gqa_batched", kv.h, dids.ptr, dlens.ptr, 3, dq.ptr, qh, out.ptr)
+    got = out.download(np.float32, q.shape)
+    close(got, orc.attention_batched(Kc, Vc, maxL, kvh, hd, ids, lens, q, qh), 1e-4, 1e-5)   # reference: 1e-4
+    for b in range(3):      # batched == individual calls
+        close(got[b], dev.attention(kv, ids[b], q[b], qh, lens[b]), 1e-4, 1e-5)
+    # validation codes
+    dev.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, dids.ptr, dlens.ptr, 0, dq.ptr, qh, out.ptr, expect=-2)
+    dev.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, dids.ptr, dlens.ptr, 3, dq.ptr, 3, out.ptr, expect=-3)
+    bad = dev.up(np.array([1, 0, 5], dtype=np.uint32))
+    dev.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, dids.ptr, bad.ptr, 3, dq.ptr, qh, out.ptr, expect=-8)
+    bad = dev.up(np.array([0, 1, 3], dtype=np.uint32))
+    dev.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, bad.ptr, dlens.ptr, 3, dq.ptr, qh, out.ptr, expect=-8)
+
+
+def test_attention_batched_head128_qwen_shape(dev, orc):
+    # BASELINE config 3 attention shape: 16 q / 2 kv heads, hd 128, 8 sequences, lengths U[256, 4096]
+    rng = np.random.default_rng(0)
+    qh, kvh, hd, B, maxL = 16, 2, 128, 8, 4160
+    lens = rng.integers(256, 4097, size=B).astype(np.uint32)
+    ids = rng.permutation(B).astype(np.uint32)
+    kv = m40.KVCache(dev.ctx, maxL, B, kvh, hd)
+    Kc = np.zeros((B, maxL, kvh, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
+    for b in range(B):
+        L = int(lens[b]); s = int(ids[b])
+        Kc[s, :L] = f16bits(rng.standard_normal((L, kvh, hd))); Vc[s, :L] = f16bits(rng.standard_normal((L, kvh, hd)))
+        dev.fill_dense(kv, s, Kc[s, :L], Vc[s, :L])
+    q = rng.standard_normal((B, qh * hd)).astype(np.float32)
+    dq, out = dev.up(q), dev.zeros(q.nbytes)
+    dids, dlens = dev.up(ids), dev.up(lens)
+    dev.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, dids.ptr, dlens.ptr, B, dq.ptr, qh, out.ptr)
+    dev.sync()
+    orc.set_threads(8)
+    close(out.download(np.float32, q.shape), orc.attention_batched(Kc, Vc, maxL, kvh, hd, ids, lens, q, qh))
+
+
+def test_argmax_extension(dev, orc):
+    rng = np.random.default_rng(9)
+    rows, n = 8, 151936
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    x[3, 77] = x[3, 100000] = 9.0        # tie: first index wins
+    dx, di, dg = dev.up(x), dev.zeros(rows * 4), dev.zeros(rows * 4)
+    dev.call("m40llm_ext_argmax_f32_async", dx.ptr, rows, n, di.ptr, dg.ptr)
+    dev.sync()
+    idx = di.download(np.uint32, (rows,)); gap = dg.download(np.float32, (rows,))
+    for r in range(rows):
+        assert idx[r] == orc.sample_greedy(x[r]) == int(np.argmax(x[r]))
+        srt = np.sort(x[r])
+        assert gap[r] == srt[-1] - srt[-2]
+    assert idx[3] == 77 and gap[3] == 0.0
