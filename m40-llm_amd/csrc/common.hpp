@@ -206,7 +206,13 @@ __device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off,
                                                 float base, float scale, float x0, float x1,
                                                 float* y0, float* y1) {
     const float pos = static_cast<float>(position) * scale;
-    const float theta = pos * powf(base, -2.0f * static_cast<float>(off) / static_cast<float>(head_dim));
+    // The per-pair frequency is evaluated in double and rounded once: theta multiplies it by
+    // the position, so a one-ulp difference in a float powf would grow to ~position * 2^-23
+    // radians.  The rounded double result equals the host libm's powf for the bases and
+    // exponents in use.
+    const float exponent = -2.0f * static_cast<float>(off) / static_cast<float>(head_dim);
+    const float inv_freq = static_cast<float>(pow(static_cast<double>(base), static_cast<double>(exponent)));
+    const float theta = pos * inv_freq;
     const float c = cosf(theta);
     const float s = sinf(theta);
     *y0 = x0 * c - x1 * s;
