@@ -1,0 +1,153 @@
+/*
+ * C view of the C++ host layer that sits above the m40llm C ABI (libm40llm_host.so).
+ *
+ * The reference's host side is Rust (src/decode.rs, src/decode_batch.rs, src/kv_compression.rs,
+ * src/kv_selection.rs, src/sampling.rs and the decode part of src/infer/forward.rs); no Rust
+ * toolchain exists in this build environment, so the same modules are written in C++
+ * (m40-llm_amd/host/*.hpp) and exposed here so that tests and bindings in any language can drive
+ * them.  Every function that can fail returns a negative value and leaves a message for
+ * m40host_last_error().
+ */
+#ifndef M40LLM_HOST_H
+#define M40LLM_HOST_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "m40llm.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* m40host_last_error(void);
+
+/* ---- sampling (src/sampling.rs) ---------------------------------------------------------- */
+/* top_k < 0 = none, top_p <= 0 = none */
+void* m40host_sampler_create(float temperature, int64_t top_k, float top_p, uint64_t seed);
+void* m40host_greedy_sampler(uint64_t seed);                                  /* src/decode.rs:111-117 */
+int64_t m40host_sampler_sample(void* sampler, const float* logits, size_t n);
+int64_t m40host_sampler_sample_greedy(void* sampler, const float* logits, size_t n);
+void m40host_sampler_destroy(void* sampler);
+
+/* ---- stopping criteria and decode loop (src/decode.rs) ----------------------------------------- */
+/* max_tokens < 0 = none, eos_id < 0 = none.  with_stop_ids != 0 builds the criteria from stop_ids
+ * (first id doubles as eos), else from eos_id alone. */
+int m40host_should_stop(int64_t max_tokens, int64_t eos_id, const uint32_t* stop_ids, size_t n_stop,
+                        int with_stop_ids, const uint32_t* generated, size_t n_generated);
+/* logits callback: fill logits_out[vocab] for the ids so far; return 0, or nonzero to abort */
+typedef int (*m40host_logits_fn)(void* user, const uint32_t* ids, size_t n_ids, float* logits_out, size_t vocab);
+/* returns the total number of ids written to ids_out (prompt + generated), or a negative value */
+int64_t m40host_decode_loop(const uint32_t* prompt, size_t n_prompt, void* sampler, int64_t max_tokens,
+                            int64_t eos_id, const uint32_t* stop_ids, size_t n_stop, int with_stop_ids,
+                            size_t vocab, m40host_logits_fn logits_fn, void* user, uint32_t* ids_out,
+                            size_t ids_capacity);
+
+/* ---- sequence-slot pool (src/decode_batch.rs:14-85) ------------------------------------------------ */
+void* m40host_pool_create(uint32_t capacity);
+void m40host_pool_destroy(void* pool);
+uint32_t m40host_pool_capacity(void* pool);
+size_t m40host_pool_available(void* pool);
+void* m40host_pool_try_lease(void* pool);             /* NULL when no slot is free */
+uint32_t m40host_lease_sequence_id(void* lease);
+void m40host_lease_release(void* lease);              /* returns the slot to the back of the free list */
+
+/* ---- batch metadata and decode batch plan (src/infer/batch.rs:276-355, src/decode_batch.rs:142-355) */
+/* status: 0 active, 1 completed, 2 cancelled.  NULL on error. */
+void* m40host_batch_plan_from_requests(const uint64_t* request_ids, const uint32_t* sequence_ids,
+                                       const uint32_t* kv_lens, const uint32_t* status, size_t n);
+void m40host_batch_plan_destroy(void* plan);
+uint32_t m40host_batch_plan_size(void* plan);
+void m40host_batch_plan_sequence_ids(void* plan, uint32_t* out);
+void m40host_batch_plan_sequence_lens(void* plan, uint32_t* out);
+uint32_t m40host_batch_plan_total_q_tokens(void* plan);
+uint32_t m40host_batch_plan_total_kv_tokens(void* plan);
+uint64_t m40host_batch_plan_total_attention_cells(void* plan);
+uint32_t m40host_batch_plan_query_len(void* plan, size_t index);
+int64_t m40host_batch_plan_index_for_request(void* plan, uint64_t request_id);   /* -1 = none */
+int64_t m40host_batch_plan_output_offset_f32(void* plan, uint64_t request_id, uint32_t q_heads, uint32_t head_dim);
+/* uploads ids/lens and calls the batched attention entry point; Q/Out packed in plan order */
+int m40host_batch_plan_dispatch_attention(void* plan, M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                          const void* d_q_f32, uint32_t q_heads, void* d_out_f32, int async);
+/* validation only: 0 ok, -1 rejected (message in m40host_last_error) */
+int m40host_batch_metadata_check(const uint32_t* seq_lens, const uint32_t* kv_lens, const uint32_t* query_lens,
+                                 size_t n, uint32_t* total_q, uint32_t* total_kv, uint64_t* attention_cells);
+
+/* ---- KV-compression configuration (src/kv_compression.rs) ------------------------------------------ */
+typedef struct M40HostKvConfig {
+    uint32_t mode;                   /* 0 off, 1 dense-recent-only, 2 block-select-exact, 3 recent-only,
+                                        4 block-summary, 5 block-select-lossy */
+    uint32_t recent_window, block_size, top_blocks, representatives;
+    uint32_t representative_policy;  /* 0 last, 1 stride */
+    uint32_t exact_old_backing;      /* 0 dense, 1 q8, 2 fp16-k-q4-v */
+    uint32_t exact_old_attention;    /* 0 staged, 1 q8-direct, 2 fp16-k-q4-v-direct */
+} M40HostKvConfig;
+void m40host_kvcfg_default(M40HostKvConfig* out);
+void m40host_kvcfg_dense_reference(M40HostKvConfig* out);
+void m40host_kvcfg_for_mode(uint32_t mode, M40HostKvConfig* out);
+int m40host_kvcfg_validate(const M40HostKvConfig* cfg, char* err, size_t err_len);
+int m40host_kvcfg_validate_runtime_support(const M40HostKvConfig* cfg, uint32_t max_seq_len, uint32_t head_dim,
+                                           char* err, size_t err_len);
+uint32_t m40host_kvcfg_effective_backing(const M40HostKvConfig* cfg);
+uint32_t m40host_kvcfg_effective_attention(const M40HostKvConfig* cfg);
+void m40host_kvcfg_set_runtime(const M40HostKvConfig* cfg);
+void m40host_kvcfg_get_runtime(M40HostKvConfig* out);
+void* m40host_kvcfg_scoped_push(const M40HostKvConfig* cfg);   /* shadows the runtime config on this thread */
+void m40host_kvcfg_scoped_pop(void* guard);
+
+/* ---- selection telemetry (src/kv_selection.rs) ------------------------------------------------------ */
+int m40host_kvsel_enabled(void);
+void m40host_kvsel_reset(void);
+void m40host_kvsel_set_attention_context(int64_t layer, int64_t token);   /* < 0 = none */
+void m40host_kvsel_record(const uint32_t* blocks, size_t n, uint32_t total_old_blocks, uint32_t top_blocks);
+void m40host_kvsel_record_scored_timed(const uint32_t* blocks, const float* scores, const uint32_t* starts,
+                                       const uint32_t* ends, size_t n, uint32_t total_old_blocks,
+                                       uint32_t top_blocks, float elapsed_ms /* < 0 = none */);
+/* returns 0 when nothing was recorded, else 1 and fills the summary */
+int m40host_kvsel_snapshot(uint32_t* selected_out, size_t capacity, size_t* n_selected, uint32_t* total_old_blocks,
+                           uint32_t* top_blocks, size_t* n_records);
+int m40host_kvsel_snapshot_record(size_t index, int64_t* layer, int64_t* token, uint32_t* ranks, uint32_t* blocks,
+                                  float* scores, uint32_t* starts, uint32_t* ends, size_t capacity, size_t* n,
+                                  uint32_t* total_old_blocks, uint32_t* top_blocks, float* elapsed_ms);
+int m40host_kvsel_should_capture_attention(void);
+void m40host_kvsel_record_attention(float recent_mass, float selected_old_mass);
+size_t m40host_kvsel_attention_count(void);
+
+/* ---- model step (decode part of src/infer/forward.rs, src/infer/logits.rs, src/decode_session.rs) --- */
+typedef struct M40HostModel M40HostModel;
+typedef struct M40HostModelConfig {
+    uint32_t n_layers, d_model, q_heads, kv_heads, head_dim, ffn, vocab;
+    float rms_eps, rope_base, rope_scale;
+    uint32_t rope_layout, has_qkv_bias, norm_weight_dtype;
+    uint32_t max_seq_len, max_sequences;
+} M40HostModelConfig;
+typedef struct M40HostLayerWeights {
+    const void *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;   /* device, f16 GGUF layout */
+    const void *bq, *bk, *bv;                              /* device f32 or NULL */
+    const void *attn_norm, *ffn_norm;                      /* device, dtype = norm_weight_dtype */
+} M40HostLayerWeights;
+/* kv_cfg NULL = dense cache (mode off) */
+M40HostModel* m40host_model_create(M40llmCudaContext* ctx, const M40HostModelConfig* cfg,
+                                   const M40HostLayerWeights* layers, const void* out_norm, const void* lm_head,
+                                   const void* tok_emb, const M40HostKvConfig* kv_cfg);
+void m40host_model_destroy(M40HostModel* model);
+M40llmKVCache* m40host_model_kv(M40HostModel* model);
+uint32_t m40host_model_kv_slot(M40HostModel* model, uint32_t sequence_id, uint32_t layer);
+/* mode 0 = the reference's call sequence, 1 = fused single-stream path, 2 = fused + graph replay */
+int m40host_model_set_mode(M40HostModel* model, uint32_t mode);
+/* one token through all layers; either output may be NULL */
+int m40host_model_forward_token(M40HostModel* model, uint32_t sequence_id, uint32_t position, uint32_t token_id,
+                                float* hidden_host, float* logits_host);
+int m40host_model_decode_greedy(M40HostModel* model, uint32_t sequence_id, const uint32_t* prompt, uint32_t n_prompt,
+                                uint32_t n_gen, uint32_t start_pos, uint32_t* ids_out, float* gaps_out);
+/* one batched step: hidden_host [rows][d_model] and logits_host [rows][vocab] may be NULL */
+int m40host_model_forward_batched(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
+                                  const uint32_t* token_ids, uint32_t rows, float* hidden_host, float* logits_host);
+int m40host_model_decode_batch_greedy(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
+                                      const uint32_t* first_tokens, uint32_t rows, uint32_t steps, uint32_t* ids_out,
+                                      float* gaps_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

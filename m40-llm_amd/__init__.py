@@ -32,7 +32,7 @@ def _ctype_of(decl: str):
     base = d.replace("const", "").strip().split()
     ty = base[0] if base else ""
     return {"size_t": C.c_size_t, "uint32_t": C.c_uint32, "uint64_t": C.c_uint64, "int": C.c_int,
-            "float": C.c_float, "void": None, "int32_t": C.c_int32}.get(ty, C.c_void_p)
+            "float": C.c_float, "void": None, "int32_t": C.c_int32, "int64_t": C.c_int64, "double": C.c_double}.get(ty, C.c_void_p)
 
 
 def parse_header(path: str):

@@ -1,0 +1,403 @@
+// One-token decoder step orchestration above the C ABI: single-sequence and row-batched
+// variable-length decode, logits, greedy decode loops.
+//
+// Mirrors, for the decode path only:
+//   forward_one_token_minimal_with_norms          src/infer/forward.rs:246-667  (14 FFI calls / layer)
+//   forward_one_token_all_layers_for_sequence     src/infer/forward.rs:1659-1716 (ping-pong buffers)
+//   forward_one_token_all_layers_batched_...      src/infer/forward.rs:1729-2140
+//   KV slot addressing slot = seq * layers + layer src/infer/kv.rs:77-121
+//   run_attention_async mode dispatch              src/infer/kv.rs:433-765 (Off and block-select-exact
+//                                                  with the fp16-K/q4-V direct backing)
+//   logits_from_hidden_into                        src/infer/logits.rs:57-116
+//   load_token_embedding_to_f32 (F16 rows)         src/infer/embeddings.rs:64-79
+//   DecodeSession::logits_for_ids token loop       src/decode_session.rs:637-703
+//
+// Two execution modes share the same arithmetic contract:
+//   mode 0 "reference calls": exactly the reference's sequence of m40llm_* calls, GEMMs on the
+//           prefill stream, everything else on the decode stream, ordered by stream waits.
+//   mode 1 "fused": single decode stream, fused entry points (m40llm_ext_*), device-side greedy.
+#pragma once
+
+#include <cstdint>
+#include <cstring>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/m40llm.h"
+#include "decode_batch.hpp"
+#include "kv_compression.hpp"
+#include "kv_selection.hpp"
+#include "sampling.hpp"
+
+namespace m40host {
+
+struct ModelConfig {
+    uint32_t n_layers, d_model, q_heads, kv_heads, head_dim, ffn, vocab;
+    float rms_eps, rope_base, rope_scale;
+    uint32_t rope_layout;         // 0 adjacent (Llama), 1 NeoX (Qwen): src/infer/types.rs:34-40
+    uint32_t has_qkv_bias;
+    uint32_t norm_weight_dtype;   // 0 f16, 1 f32
+    uint32_t max_seq_len, max_sequences;
+};
+
+struct LayerWeights {   // device pointers; f16 GGUF layout [N cols][K]
+    const void *wq, *wk, *wv, *wo, *wgate, *wup, *wdown;
+    const void *bq, *bk, *bv;         // f32, or all null
+    const void *attn_norm, *ffn_norm;
+};
+
+#define M40H_TRY(expr)                                                                    \
+    do {                                                                                  \
+        const int rc__ = (expr);                                                          \
+        if (rc__ != 0) throw std::runtime_error(std::string(#expr) + " -> " + std::to_string(rc__)); \
+    } while (0)
+
+class DeviceBuf {
+public:
+    DeviceBuf() = default;
+    DeviceBuf(M40llmCudaContext* ctx, size_t bytes) : ctx_(ctx), bytes_(bytes) {
+        if (m40llm_device_malloc(ctx, bytes ? bytes : 4, &p_) != 0) throw std::runtime_error("device_malloc failed");
+    }
+    DeviceBuf(DeviceBuf&& o) noexcept : ctx_(o.ctx_), p_(o.p_), bytes_(o.bytes_) { o.p_ = nullptr; }
+    DeviceBuf& operator=(DeviceBuf&& o) noexcept {
+        reset();
+        ctx_ = o.ctx_; p_ = o.p_; bytes_ = o.bytes_; o.p_ = nullptr;
+        return *this;
+    }
+    DeviceBuf(const DeviceBuf&) = delete;
+    DeviceBuf& operator=(const DeviceBuf&) = delete;
+    ~DeviceBuf() { reset(); }
+    void reset() { if (p_) m40llm_device_free(ctx_, p_); p_ = nullptr; }
+    void* ptr() const { return p_; }
+    float* f32(size_t off = 0) const { return static_cast<float*>(p_) + off; }
+    size_t bytes() const { return bytes_; }
+
+private:
+    M40llmCudaContext* ctx_ = nullptr;
+    void* p_ = nullptr;
+    size_t bytes_ = 0;
+};
+
+// Named f32 scratch buffers sized by row count (src/infer/workspace.rs:60-126).
+struct ForwardWorkspace {
+    uint32_t rows = 0;
+    DeviceBuf xn, q, k, v, ctx_out, y_attn, x1, x1n, gate, up, hid, y_mlp, scratch_a, scratch_b, norm_hidden, logits;
+    DeviceBuf argmax_idx, argmax_gap, positions;
+    void ensure(M40llmCudaContext* c, const ModelConfig& m, uint32_t want_rows) {
+        if (want_rows <= rows) return;
+        const size_t D = m.d_model, KV = (size_t)m.kv_heads * m.head_dim, F = m.ffn, R = want_rows;
+        xn = DeviceBuf(c, R * D * 4); q = DeviceBuf(c, R * D * 4); k = DeviceBuf(c, R * KV * 4); v = DeviceBuf(c, R * KV * 4);
+        ctx_out = DeviceBuf(c, R * D * 4); y_attn = DeviceBuf(c, R * D * 4); x1 = DeviceBuf(c, R * D * 4);
+        x1n = DeviceBuf(c, R * D * 4); gate = DeviceBuf(c, R * F * 4); up = DeviceBuf(c, R * F * 4);
+        hid = DeviceBuf(c, R * F * 4); y_mlp = DeviceBuf(c, R * D * 4); scratch_a = DeviceBuf(c, R * D * 4);
+        scratch_b = DeviceBuf(c, R * D * 4); norm_hidden = DeviceBuf(c, R * D * 4);
+        logits = DeviceBuf(c, R * (size_t)m.vocab * 4);
+        argmax_idx = DeviceBuf(c, R * 4); argmax_gap = DeviceBuf(c, R * 4); positions = DeviceBuf(c, R * 4 * 2);
+        rows = want_rows;
+    }
+};
+
+class DecodeModel {
+public:
+    DecodeModel(M40llmCudaContext* ctx, const ModelConfig& cfg, const LayerWeights* layers, const void* out_norm,
+                const void* lm_head, const void* tok_emb, const KvCompressionConfig& kvcfg)
+        : ctx_(ctx), cfg_(cfg), layers_(layers, layers + cfg.n_layers), out_norm_(out_norm), lm_head_(lm_head),
+          tok_emb_(tok_emb), kvcfg_(kvcfg) {
+        if (cfg.d_model != cfg.q_heads * cfg.head_dim)
+            throw std::invalid_argument("d_model != query heads * head_dim");     // forward.rs:288-295
+        if (cfg.q_heads == 0 || cfg.kv_heads == 0 || cfg.q_heads % cfg.kv_heads != 0)
+            throw std::invalid_argument("query heads must be a multiple of kv heads");
+        const std::string err = kvcfg.validate_runtime_support(cfg.max_seq_len, cfg.head_dim);
+        if (!err.empty()) throw std::invalid_argument(err);
+        const uint32_t slots = cfg.max_sequences * cfg.n_layers;   // one slot per (sequence, layer)
+        if (kvcfg.uses_compressed_exact_old_backing()) {
+            kv_ = m40llm_kvcache_create_compressed(ctx, cfg.max_seq_len, slots, cfg.kv_heads, cfg.head_dim,
+                                                   kvcfg.recent_window, kvcfg.block_size, kvcfg.top_blocks,
+                                                   kvcfg.representatives, (uint32_t)kvcfg.representative_policy,
+                                                   (uint32_t)kvcfg.effective_exact_old_backing());
+        } else {
+            kv_ = m40llm_kvcache_create(ctx, cfg.max_seq_len, slots, cfg.kv_heads, cfg.head_dim);
+        }
+        if (!kv_) throw std::runtime_error("KV cache allocation failed");
+        ws_.ensure(ctx, cfg, 1);
+    }
+    ~DecodeModel() {
+        if (kv_) m40llm_kvcache_destroy(kv_);
+    }
+    DecodeModel(const DecodeModel&) = delete;
+    DecodeModel& operator=(const DecodeModel&) = delete;
+
+    const ModelConfig& config() const { return cfg_; }
+    M40llmKVCache* kv() const { return kv_; }
+    M40llmCudaContext* ctx() const { return ctx_; }
+    uint32_t mode() const { return mode_; }
+    void set_mode(uint32_t m) { mode_ = m; }
+    uint32_t kv_slot(uint32_t seq, uint32_t layer) const {
+        if (seq >= cfg_.max_sequences) throw std::out_of_range("sequence id out of range");   // kv.rs:92-107
+        return seq * cfg_.n_layers + layer;
+    }
+
+    // ---- single sequence ---------------------------------------------------------------------
+    // token embedding row (f16) -> f32 activation (embeddings.rs:64-79)
+    void embed(uint32_t token_id, float* d_x) {
+        if (token_id >= cfg_.vocab) throw std::out_of_range("token id out of range");
+        const char* row = static_cast<const char*>(tok_emb_) + (size_t)token_id * cfg_.d_model * 2;
+        M40H_TRY(m40llm_f16_to_f32(ctx_, row, d_x, cfg_.d_model));
+    }
+
+    // One decoder layer for the token at position seq_len-1, reference call order.
+    void layer_reference(uint32_t layer, uint32_t seq, uint32_t seq_len, const float* d_x, float* d_out) {
+        const LayerWeights& w = layers_[layer];
+        const uint32_t D = cfg_.d_model, KV = cfg_.kv_heads * cfg_.head_dim, F = cfg_.ffn;
+        const uint32_t slot = kv_slot(seq, layer), pos = seq_len - 1;
+        const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
+        // 1. attention norm (decode stream)
+        M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, d_x, w.attn_norm, ws_.xn.ptr(), 1, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
+        // 2. QKV projections (prefill stream, blocking)
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.xn.ptr(), w.wq, ws_.q.ptr(), 1, (int)D, (int)D));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.xn.ptr(), w.wk, ws_.k.ptr(), 1, (int)KV, (int)D));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.xn.ptr(), w.wv, ws_.v.ptr(), 1, (int)KV, (int)D));
+        // 3. optional biases: residual_add per row (forward.rs:124-163)
+        if (cfg_.has_qkv_bias) {
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, ws_.q.ptr(), w.bq, ws_.q.ptr(), D));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, ws_.k.ptr(), w.bk, ws_.k.ptr(), KV));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, ws_.v.ptr(), w.bv, ws_.v.ptr(), KV));
+        }
+        // 4. RoPE on Q, 5. fused RoPE-K + f16 append at `pos`
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+        M40H_TRY(m40llm_rope_f32_inplace_layout_async(ctx_, ws_.q.ptr(), 1, cfg_.q_heads, cfg_.head_dim, pos, cfg_.rope_base,
+                                                      cfg_.rope_scale, cfg_.rope_layout));
+        M40H_TRY(m40llm_kvcache_append_token_f32_rope_k_at_layout_async(ctx_, kv_, slot, ws_.k.ptr(), ws_.v.ptr(), pos, pos,
+                                                                        cfg_.rope_base, cfg_.rope_scale, cfg_.rope_layout));
+        // 6. attention, dispatched on the KV-compression mode
+        run_attention(layer, slot, seq_len, ws_.q.f32(), ws_.ctx_out.f32());
+        // 7. output projection, 8. residual
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.ctx_out.ptr(), w.wo, ws_.y_attn.ptr(), 1, (int)D, (int)D));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+        M40H_TRY(m40llm_residual_add_f32_async(ctx_, d_x, ws_.y_attn.ptr(), ws_.x1.ptr(), D));
+        // 9. FFN norm, 10. gate/up, 11. SwiGLU, 12. down, 13. residual
+        M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, ws_.x1.ptr(), w.ffn_norm, ws_.x1n.ptr(), 1, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.x1n.ptr(), w.wgate, ws_.gate.ptr(), 1, (int)F, (int)D));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.x1n.ptr(), w.wup, ws_.up.ptr(), 1, (int)F, (int)D));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+        M40H_TRY(m40llm_swiglu_f32_async(ctx_, ws_.gate.ptr(), ws_.up.ptr(), ws_.hid.ptr(), F));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.hid.ptr(), w.wdown, ws_.y_mlp.ptr(), 1, (int)D, (int)F));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+        M40H_TRY(m40llm_residual_add_f32_async(ctx_, ws_.x1.ptr(), ws_.y_mlp.ptr(), d_out, D));
+    }
+
+    // All layers for one token; returns the device pointer that holds the final hidden state.
+    const float* forward_token(uint32_t seq, uint32_t pos, uint32_t token_id) {
+        if (pos >= cfg_.max_seq_len) throw std::out_of_range("position beyond max_seq_len");
+        ws_.ensure(ctx_, cfg_, 1);
+        float* a = ws_.scratch_a.f32();
+        float* b = ws_.scratch_b.f32();
+        embed(token_id, a);
+        for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
+            kv_selection::set_attention_context(l, pos);
+            layer_reference(l, seq, pos + 1, a, b);
+            std::swap(a, b);
+        }
+        return a;
+    }
+
+    // output norm -> lm_head GEMV -> sync -> D2H (logits.rs:57-116)
+    void logits_from_hidden(const float* d_hidden, float* host_logits) {
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, M40LLM_STREAM_PREFILL, M40LLM_STREAM_DECODE));
+        M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, d_hidden, out_norm_, ws_.norm_hidden.ptr(), 1, cfg_.d_model,
+                                                    cfg_.rms_eps, cfg_.norm_weight_dtype));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, M40LLM_STREAM_PREFILL, M40LLM_STREAM_DECODE));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.norm_hidden.ptr(), lm_head_, ws_.logits.ptr(), 1, (int)cfg_.vocab,
+                                              (int)cfg_.d_model));
+        M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_PREFILL));
+        M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits, ws_.logits.ptr(), (size_t)cfg_.vocab * 4));
+    }
+
+    // Greedy decode of one sequence: prompt tokens from start_pos, then n_gen sampled tokens
+    // (Sampler with top_k = 1).  ids_out holds n_prompt + n_gen ids.
+    void decode_greedy(uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t n_gen, uint32_t start_pos,
+                       uint32_t* ids_out, float* gaps_out) {
+        Sampler sampler = greedy_sampler(42);
+        std::vector<float> logits(cfg_.vocab);
+        uint32_t pos = start_pos;
+        const float* hidden = nullptr;
+        for (uint32_t i = 0; i < n_prompt; ++i) {
+            ids_out[i] = prompt[i];
+            hidden = forward_token(seq, pos++, prompt[i]);
+        }
+        for (uint32_t g = 0; g < n_gen; ++g) {
+            if (!hidden) throw std::invalid_argument("decode_greedy needs at least one prompt token");
+            logits_from_hidden(hidden, logits.data());
+            const uint32_t next = (uint32_t)sampler.sample(logits.data(), logits.size());
+            if (gaps_out) gaps_out[g] = top2_gap(logits);
+            ids_out[n_prompt + g] = next;
+            if (g + 1 < n_gen) hidden = forward_token(seq, pos++, next);
+        }
+    }
+
+    // ---- row-batched variable-length decode (forward.rs:1729-2140) ----------------------------
+    // One step for `rows` sequences: token_ids[r] is the input token of sequence seq_ids[r] whose
+    // cache currently holds kv_lens[r] tokens; afterwards each holds kv_lens[r] + 1.
+    // d_hidden_out receives [rows][d_model].
+    const float* forward_batched(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* token_ids, uint32_t rows) {
+        if (rows == 0) throw std::invalid_argument("empty batch");
+        if (kvcfg_.is_enabled()) throw std::invalid_argument("batched decode requires the dense KV cache");
+        ws_.ensure(ctx_, cfg_, rows);
+        const uint32_t D = cfg_.d_model, KV = cfg_.kv_heads * cfg_.head_dim, F = cfg_.ffn;
+        const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
+        float* a = ws_.scratch_a.f32();
+        float* b = ws_.scratch_b.f32();
+        for (uint32_t r = 0; r < rows; ++r) {
+            if (kv_lens[r] + 1 > cfg_.max_seq_len) throw std::out_of_range("sequence would exceed max_seq_len");
+            embed(token_ids[r], a + (size_t)r * D);
+        }
+        for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
+            const LayerWeights& w = layers_[l];
+            // plan for this layer: slot ids and lengths after the append
+            std::vector<DecodeRequestState> reqs;
+            for (uint32_t r = 0; r < rows; ++r)
+                reqs.push_back(DecodeRequestState::active(r, kv_slot(seq_ids[r], l), kv_lens[r] + 1));
+            DeviceDecodeBatchPlan plan(ctx_, DecodeBatchPlan::from_requests(reqs));
+            M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, a, w.attn_norm, ws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.xn.ptr(), w.wq, ws_.q.ptr(), (int)rows, (int)D, (int)D));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.xn.ptr(), w.wk, ws_.k.ptr(), (int)rows, (int)KV, (int)D));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.xn.ptr(), w.wv, ws_.v.ptr(), (int)rows, (int)KV, (int)D));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            for (uint32_t r = 0; r < rows; ++r) {
+                float* qr = ws_.q.f32((size_t)r * D);
+                float* kr = ws_.k.f32((size_t)r * KV);
+                float* vr = ws_.v.f32((size_t)r * KV);
+                if (cfg_.has_qkv_bias) {
+                    M40H_TRY(m40llm_residual_add_f32_async(ctx_, qr, w.bq, qr, D));
+                    M40H_TRY(m40llm_residual_add_f32_async(ctx_, kr, w.bk, kr, KV));
+                    M40H_TRY(m40llm_residual_add_f32_async(ctx_, vr, w.bv, vr, KV));
+                }
+                const uint32_t pos = kv_lens[r];
+                M40H_TRY(m40llm_rope_f32_inplace_layout_async(ctx_, qr, 1, cfg_.q_heads, cfg_.head_dim, pos, cfg_.rope_base,
+                                                              cfg_.rope_scale, cfg_.rope_layout));
+                M40H_TRY(m40llm_kvcache_append_token_f32_rope_k_at_layout_async(ctx_, kv_, kv_slot(seq_ids[r], l), kr, vr, pos, pos,
+                                                                                cfg_.rope_base, cfg_.rope_scale, cfg_.rope_layout));
+            }
+            M40H_TRY(plan.dispatch_attention_async(kv_, ws_.q.ptr(), cfg_.q_heads, ws_.ctx_out.ptr()));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.ctx_out.ptr(), w.wo, ws_.y_attn.ptr(), (int)rows, (int)D, (int)D));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, a, ws_.y_attn.ptr(), ws_.x1.ptr(), (size_t)rows * D));
+            M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, ws_.x1.ptr(), w.ffn_norm, ws_.x1n.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.x1n.ptr(), w.wgate, ws_.gate.ptr(), (int)rows, (int)F, (int)D));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.x1n.ptr(), w.wup, ws_.up.ptr(), (int)rows, (int)F, (int)D));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_swiglu_f32_async(ctx_, ws_.gate.ptr(), ws_.up.ptr(), ws_.hid.ptr(), (size_t)rows * F));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.hid.ptr(), w.wdown, ws_.y_mlp.ptr(), (int)rows, (int)D, (int)F));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, ws_.x1.ptr(), ws_.y_mlp.ptr(), b, (size_t)rows * D));
+            M40H_TRY(m40llm_stream_synchronize(ctx_, DEC));   // the plan's device arrays are freed at scope end
+            std::swap(a, b);
+        }
+        return a;
+    }
+
+    // logits for `rows` hidden rows -> host [rows][vocab]
+    void logits_from_hidden_rows(const float* d_hidden, uint32_t rows, float* host_logits) {
+        const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, d_hidden, out_norm_, ws_.norm_hidden.ptr(), rows, cfg_.d_model,
+                                                    cfg_.rms_eps, cfg_.norm_weight_dtype));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, ws_.norm_hidden.ptr(), lm_head_, ws_.logits.ptr(), (int)rows,
+                                              (int)cfg_.vocab, (int)cfg_.d_model));
+        M40H_TRY(m40llm_stream_synchronize(ctx_, PRE));
+        M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits, ws_.logits.ptr(), (size_t)rows * cfg_.vocab * 4));
+    }
+
+    // `steps` greedy steps for a batch of sequences whose caches already hold kv_lens[r] tokens;
+    // first_tokens[r] is the input of step 0.  ids_out: [rows][steps], gaps_out (optional) likewise.
+    void decode_batch_greedy(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens,
+                             uint32_t rows, uint32_t steps, uint32_t* ids_out, float* gaps_out) {
+        std::vector<uint32_t> lens(kv_lens, kv_lens + rows), toks(first_tokens, first_tokens + rows);
+        std::vector<float> logits((size_t)rows * cfg_.vocab);
+        std::vector<Sampler> samplers(rows, greedy_sampler(42));
+        for (uint32_t s = 0; s < steps; ++s) {
+            const float* hidden = forward_batched(seq_ids, lens.data(), toks.data(), rows);
+            logits_from_hidden_rows(hidden, rows, logits.data());
+            for (uint32_t r = 0; r < rows; ++r) {
+                const float* lr = logits.data() + (size_t)r * cfg_.vocab;
+                const uint32_t next = (uint32_t)samplers[r].sample(lr, cfg_.vocab);
+                ids_out[(size_t)r * steps + s] = next;
+                if (gaps_out) gaps_out[(size_t)r * steps + s] = top2_gap(lr, cfg_.vocab);
+                toks[r] = next;
+                lens[r] += 1;
+            }
+        }
+    }
+
+    static float top2_gap(const float* l, size_t n) {
+        float a = -INFINITY, b = -INFINITY;
+        for (size_t i = 0; i < n; ++i) {
+            if (l[i] > a) { b = a; a = l[i]; }
+            else if (l[i] > b) b = l[i];
+        }
+        return a - b;
+    }
+    static float top2_gap(const std::vector<float>& l) { return top2_gap(l.data(), l.size()); }
+
+    ForwardWorkspace& workspace() { return ws_; }
+    const std::vector<LayerWeights>& layers() const { return layers_; }
+    const void* out_norm() const { return out_norm_; }
+    const void* lm_head() const { return lm_head_; }
+    const void* tok_emb() const { return tok_emb_; }
+    const KvCompressionConfig& kv_config() const { return kvcfg_; }
+
+private:
+    // Attention dispatch on the KV-compression mode (src/infer/kv.rs:433-765).
+    void run_attention(uint32_t layer, uint32_t slot, uint32_t seq_len, const float* d_q, float* d_out) {
+        (void)layer;
+        if (kvcfg_.mode == KvCompressMode::Off) {
+            M40H_TRY(m40llm_attention_last_token_f32_gqa_async(ctx_, kv_, slot, d_q, cfg_.q_heads, seq_len, d_out));
+            return;
+        }
+        if (kvcfg_.mode == KvCompressMode::BlockSelectExact &&
+            kvcfg_.effective_exact_old_backing() == KvExactOldBacking::Fp16KQ4V &&
+            kvcfg_.effective_exact_old_attention() == KvExactOldAttention::Fp16KQ4VDirect) {
+            if (kv_selection::enabled() && seq_len > kvcfg_.recent_window) {
+                // telemetry twin: q-head 0 only, host-side re-scoring (kv.rs:523-539)
+                uint32_t blocks[2048], start[2048], end[2048], count = 0, total = 0;
+                float scores[2048];
+                if (m40llm_kvcache_debug_select_old_blocks(ctx_, kv_, slot, d_q, cfg_.q_heads, seq_len, kvcfg_.recent_window,
+                                                           kvcfg_.block_size, kvcfg_.top_blocks, blocks, scores, start, end,
+                                                           &count, 2048, &total) == 0) {
+                    std::vector<KvSelectedBlock> sel;
+                    for (uint32_t i = 0; i < count; ++i) sel.push_back({i, blocks[i], scores[i], start[i], end[i]});
+                    kv_selection::record_scored_timed(std::move(sel), total, kvcfg_.top_blocks, std::nullopt);
+                }
+            }
+            M40H_TRY(m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async(
+                ctx_, kv_, slot, d_q, cfg_.q_heads, seq_len, kvcfg_.recent_window, kvcfg_.block_size, kvcfg_.top_blocks, d_out));
+            return;
+        }
+        throw std::invalid_argument("KV compression mode not built: only off and block-select-exact/fp16-k-q4-v-direct");
+    }
+
+    M40llmCudaContext* ctx_;
+    ModelConfig cfg_;
+    std::vector<LayerWeights> layers_;
+    const void* out_norm_;
+    const void* lm_head_;
+    const void* tok_emb_;
+    KvCompressionConfig kvcfg_;
+    M40llmKVCache* kv_ = nullptr;
+    ForwardWorkspace ws_;
+    uint32_t mode_ = 0;
+};
+
+}  // namespace m40host
