@@ -1,0 +1,155 @@
+#!/usr/bin/env python3
+"""Benchmark of the decode-step hot path on one MI355X.
+
+A step is one decoded token: embedding row -> all decoder layers (RMSNorm, QKV/O/FFN GEMVs over f16 weights,
+RoPE, f32->f16 KV append, last-token GQA attention over the f16 KV cache) -> output norm -> lm_head GEMV ->
+greedy sample.  Workload at N=1: the TinyLlama-1.1B-shaped random-init model of BASELINE.json configs[1]
+(22 layers, hidden 2048, 32/4 heads, head_dim 64, FFN 5632, vocab 32000, f16 weights N(0,0.02)), 32 random prompt
+ids, then greedy decode at batch 1.  Weights and KV cache are resident in HBM before the timed region.
+
+Prints ONE JSON line (see README / DESIGN.md for the field meanings).
+"""
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+
+
+def algorithmic_bytes_per_token(cfg):
+    """Minimum HBM traffic of one decoded token at batch 1: every layer weight and the lm_head once (f16)."""
+    D, F, V, L = cfg["d_model"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
+    KV = cfg["kv_heads"] * cfg["head_dim"]
+    per_layer = (D * D * 2 + 2 * KV * D + 3 * F * D) * 2
+    return L * per_layer + V * D * 2
+
+
+def measure_dominant_kernel(pkg, ctx, dm, cfg, reps):
+    """Average launch duration of the kernel that moves most of the bytes of a token: the FFN gate/up GEMV
+    (f32 activations x f16 GGUF weights, N=ffn, K=hidden), timed with HIP events on the library's decode stream.
+    Launches cycle through the layers' own weight matrices so that no launch finds its weights in cache."""
+    D, F, L = cfg["d_model"], cfg["ffn"], cfg["n_layers"]
+    x = ctx.to_device(np.random.default_rng(1).standard_normal(D).astype(np.float32))
+    y = ctx.alloc(F * 4)
+    mats = []
+    for l in range(L):
+        mats.append(dm.layers[l].wgate); mats.append(dm.layers[l].wup)
+    lib = ctx.lib
+    for i in range(len(mats)):      # warm-up: code objects, clocks
+        pkg.check(lib.m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx.h, x.ptr, mats[i], y.ptr, 1, F, D, 1), "gemv")
+    ctx.sync(1)
+    e0, e1 = ctx.event(), ctx.event()
+    ctx.record(e0, 1)
+    n = 0
+    for r in range(reps):
+        for mptr in mats:
+            lib.m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx.h, x.ptr, mptr, y.ptr, 1, F, D, 1)
+            n += 1
+    ctx.record(e1, 1)
+    ms = ctx.elapsed_ms(e0, e1)
+    ctx.event_destroy(e0); ctx.event_destroy(e1)
+    avg_us = ms * 1e3 / n
+    bytes_per_launch = F * D * 2 + D * 4 + F * 4      # weights + activations in + out
+    return dict(kernel="gemv_f32xf16_gguf_kernel", shape=f"M=1 N={F} K={D}", launches=n, avg_us=avg_us,
+                bytes=bytes_per_launch)
+
+
+def cpu_baseline(cfg, W, steps, threads):
+    """The CPU oracle (a scalar port of the reference's semantics) timed on this host: `steps` greedy decode
+    tokens from an empty KV cache.  At this size a token is bound by the 2.07 GB of weights, not by context."""
+    from oracle import pyoracle as orc
+    orc.set_threads(threads)
+    om = orc.Model(dict(cfg, qkv_bias=bool(cfg.get("qkv_bias"))), W)
+    om.alloc_kv(steps + 4, 1)
+    t0 = time.perf_counter()
+    om.decode_greedy(0, [1], steps)          # 1 prompt token + (steps-1) further forwards + `steps` lm_head passes
+    dt = time.perf_counter() - t0
+    return dict(value=steps / dt, unit="tok/s", cores=threads, kind="port",
+                sample=f"{steps} greedy decode tokens of the same model from an empty KV cache, oracle/oracle.c "
+                       f"(gcc -O2, {threads} thread{'s' if threads > 1 else ''})")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--mode", type=int, default=int(os.environ.get("M40_BENCH_MODE", "-1")),
+                    help="-1 best available, 0 reference call sequence, 1 fused, 2 fused + graph")
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count (debug only; invalidates the metric)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-steps", type=int, default=8)
+    ap.add_argument("--kernel-reps", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU form (each box has one MI355X); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    pkg = importlib.import_module("m40-llm_amd")
+    syn = importlib.import_module("m40-llm_amd.synthetic")
+
+    cfg = dict(syn.TINYLLAMA_1B)
+    if args.layers:
+        cfg["n_layers"] = args.layers
+    n_prompt = 32
+    max_seq = n_prompt + args.warmup + args.steps + 8
+    t_setup = time.perf_counter()
+    W = syn.make_weights(cfg, seed=0)
+    ctx = pkg.Context(0)
+    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=max_seq, max_sequences=1)
+    mode = args.mode
+    if mode < 0:
+        mode = 2 if hasattr(ctx.lib, "m40llm_ext_decode_layer_fused_async") else 0
+    dm.set_mode(mode)
+    prompt = np.random.default_rng(0).integers(0, cfg["vocab"], size=n_prompt).astype(np.uint32)
+    setup_s = time.perf_counter() - t_setup
+
+    torch.cuda.synchronize()
+    ids, elapsed_ms = dm.decode_timed(0, prompt, args.warmup, args.steps)     # timed region brackets itself with full syncs
+    torch.cuda.synchronize()
+    tok_s = args.steps / (elapsed_ms / 1e3)
+    ms_per_step = elapsed_ms / args.steps
+
+    dom = measure_dominant_kernel(pkg, ctx, dm, cfg, args.kernel_reps)
+    achieved = dom["bytes"] / (dom["avg_us"] * 1e-6) / 1e9
+    token_bytes = algorithmic_bytes_per_token(cfg)
+    out = {
+        "metric": "decode tok/s at B=1 and B=8; attn+GEMV HBM GB/s as % of MI355X peak",
+        "value": tok_s, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "TinyLlama-1.1B-shaped random-init dense decode (BASELINE configs[1]): 22 layers, hidden 2048, "
+                               "32 q / 4 kv heads, head_dim 64, FFN 5632, vocab 32000, f16 weights N(0,0.02), 32 random prompt "
+                               "ids, greedy decode, batch 1",
+                   "batch": 1, "prompt_tokens": n_prompt, "layers": cfg["n_layers"],
+                   "host_path": ["reference call sequence", "fused", "fused + graph"][mode],
+                   "whole_step_hbm_gbs": token_bytes / (ms_per_step * 1e-3) / 1e9,
+                   "whole_step_hbm_frac": token_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                   "algorithmic_bytes_per_token": token_bytes, "setup_s": round(setup_s, 1),
+                   "first_generated_ids": [int(i) for i in ids[n_prompt:n_prompt + 8]]},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom["kernel"], "shape": dom["shape"],
+                     "avg_launch_us": dom["avg_us"], "launches_timed": dom["launches"],
+                     "algorithmic_bytes_per_launch": dom["bytes"]},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, W, args.cpu_steps, 1)
+    dm.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -140,6 +140,14 @@ int m40host_model_forward_token(M40HostModel* model, uint32_t sequence_id, uint3
                                 float* hidden_host, float* logits_host);
 int m40host_model_decode_greedy(M40HostModel* model, uint32_t sequence_id, const uint32_t* prompt, uint32_t n_prompt,
                                 uint32_t n_gen, uint32_t start_pos, uint32_t* ids_out, float* gaps_out);
+/* prompt (untimed) + `warmup` untimed greedy steps + `steps` greedy steps timed on the host clock between two
+ * stream synchronisations; ids_out holds n_prompt + warmup + steps ids; elapsed_ms covers the timed steps only */
+int m40host_model_decode_timed(M40HostModel* model, uint32_t sequence_id, const uint32_t* prompt, uint32_t n_prompt,
+                               uint32_t warmup, uint32_t steps, uint32_t* ids_out, double* elapsed_ms);
+/* same for a batch of sequences whose caches are pre-filled to kv_lens; ids_out [rows][warmup+steps] */
+int m40host_model_decode_batch_timed(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
+                                     const uint32_t* first_tokens, uint32_t rows, uint32_t warmup, uint32_t steps,
+                                     uint32_t* ids_out, double* elapsed_ms);
 /* one batched step: hidden_host [rows][d_model] and logits_host [rows][vocab] may be NULL */
 int m40host_model_forward_batched(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
                                   const uint32_t* token_ids, uint32_t rows, float* hidden_host, float* logits_host);

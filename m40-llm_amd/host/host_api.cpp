@@ -341,6 +341,20 @@ int m40host_model_decode_greedy(M40HostModel* m, uint32_t seq, const uint32_t* p
                                 uint32_t start_pos, uint32_t* ids_out, float* gaps_out) {
     return guarded([&]() -> int { m->m->decode_greedy(seq, prompt, n_prompt, n_gen, start_pos, ids_out, gaps_out); return 0; }, -100);
 }
+int m40host_model_decode_timed(M40HostModel* m, uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t warmup,
+                               uint32_t steps, uint32_t* ids_out, double* elapsed_ms) {
+    return guarded([&]() -> int { m->m->decode_timed(seq, prompt, n_prompt, warmup, steps, ids_out, elapsed_ms); return 0; }, -100);
+}
+int m40host_model_decode_batch_timed(M40HostModel* m, const uint32_t* seq_ids, const uint32_t* kv_lens,
+                                     const uint32_t* first_tokens, uint32_t rows, uint32_t warmup, uint32_t steps,
+                                     uint32_t* ids_out, double* elapsed_ms) {
+    return guarded(
+        [&]() -> int {
+            m->m->decode_batch_timed(seq_ids, kv_lens, first_tokens, rows, warmup, steps, ids_out, elapsed_ms);
+            return 0;
+        },
+        -100);
+}
 int m40host_model_forward_batched(M40HostModel* m, const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* tokens,
                                   uint32_t rows, float* hidden_host, float* logits_host) {
     return guarded(

@@ -18,6 +18,8 @@
 //   mode 1 "fused": single decode stream, fused entry points (m40llm_ext_*), device-side greedy.
 #pragma once
 
+#include <chrono>
+#include <cmath>
 #include <cstdint>
 #include <cstring>
 #include <optional>
@@ -339,6 +341,64 @@ public:
                 lens[r] += 1;
             }
         }
+    }
+
+    // Greedy decode with a timed region: prompt and `warmup` steps untimed, then `steps` steps between two full
+    // synchronisations of both streams.
+    void decode_timed(uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t warmup, uint32_t steps,
+                      uint32_t* ids_out, double* elapsed_ms) {
+        if (n_prompt == 0) throw std::invalid_argument("decode_timed needs a prompt");
+        std::vector<float> logits(cfg_.vocab);
+        Sampler sampler = greedy_sampler(42);
+        uint32_t pos = 0;
+        const float* hidden = nullptr;
+        for (uint32_t i = 0; i < n_prompt; ++i) {
+            ids_out[i] = prompt[i];
+            hidden = forward_token(seq, pos++, prompt[i]);
+        }
+        auto step = [&](uint32_t out_index) {
+            logits_from_hidden(hidden, logits.data());
+            const uint32_t next = (uint32_t)sampler.sample(logits.data(), logits.size());
+            ids_out[out_index] = next;
+            hidden = forward_token(seq, pos++, next);
+        };
+        for (uint32_t w = 0; w < warmup; ++w) step(n_prompt + w);
+        sync_all();
+        const auto t0 = std::chrono::steady_clock::now();
+        for (uint32_t s = 0; s < steps; ++s) step(n_prompt + warmup + s);
+        sync_all();
+        const auto t1 = std::chrono::steady_clock::now();
+        if (elapsed_ms) *elapsed_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    }
+
+    void decode_batch_timed(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens, uint32_t rows,
+                            uint32_t warmup, uint32_t steps, uint32_t* ids_out, double* elapsed_ms) {
+        std::vector<uint32_t> lens(kv_lens, kv_lens + rows), toks(first_tokens, first_tokens + rows);
+        std::vector<float> logits((size_t)rows * cfg_.vocab);
+        std::vector<Sampler> samplers(rows, greedy_sampler(42));
+        const uint32_t total = warmup + steps;
+        auto step = [&](uint32_t s) {
+            const float* hidden = forward_batched(seq_ids, lens.data(), toks.data(), rows);
+            logits_from_hidden_rows(hidden, rows, logits.data());
+            for (uint32_t r = 0; r < rows; ++r) {
+                const uint32_t next = (uint32_t)samplers[r].sample(logits.data() + (size_t)r * cfg_.vocab, cfg_.vocab);
+                ids_out[(size_t)r * total + s] = next;
+                toks[r] = next;
+                lens[r] += 1;
+            }
+        };
+        for (uint32_t w = 0; w < warmup; ++w) step(w);
+        sync_all();
+        const auto t0 = std::chrono::steady_clock::now();
+        for (uint32_t s = 0; s < steps; ++s) step(warmup + s);
+        sync_all();
+        const auto t1 = std::chrono::steady_clock::now();
+        if (elapsed_ms) *elapsed_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+    }
+
+    void sync_all() {
+        M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_PREFILL));
+        M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
     }
 
     static float top2_gap(const float* l, size_t n) {

@@ -170,6 +170,25 @@ class DeviceModel:
                  "m40host_model_decode_batch_greedy")
         return ids, gaps
 
+    def decode_timed(self, seq, prompt, warmup, steps):
+        prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+        ids = np.zeros(len(prompt) + warmup + steps, dtype=np.uint32)
+        ms = C.c_double()
+        self._ok(self.H.m40host_model_decode_timed(self.h, seq, prompt.ctypes.data_as(C.c_void_p), len(prompt), warmup, steps,
+                                                   ids.ctypes.data_as(C.c_void_p), C.byref(ms)), "m40host_model_decode_timed")
+        return ids, ms.value
+
+    def decode_batch_timed(self, seq_ids, kv_lens, first_tokens, warmup, steps):
+        s = np.ascontiguousarray(seq_ids, dtype=np.uint32); l = np.ascontiguousarray(kv_lens, dtype=np.uint32)
+        t = np.ascontiguousarray(first_tokens, dtype=np.uint32)
+        ids = np.zeros((len(s), warmup + steps), dtype=np.uint32)
+        ms = C.c_double()
+        self._ok(self.H.m40host_model_decode_batch_timed(self.h, s.ctypes.data_as(C.c_void_p), l.ctypes.data_as(C.c_void_p),
+                                                         t.ctypes.data_as(C.c_void_p), len(s), warmup, steps,
+                                                         ids.ctypes.data_as(C.c_void_p), C.byref(ms)),
+                 "m40host_model_decode_batch_timed")
+        return ids, ms.value
+
     def fill_kv(self, seq, layer, k16, v16):
         """Pre-fill one (sequence, layer) slot from f16 rows [L, kv_heads, head_dim] (already rotated K)."""
         slot = self.H.m40host_model_kv_slot(self.h, seq, layer)
