@@ -112,7 +112,7 @@ def main():
     dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=max_seq, max_sequences=1)
     mode = args.mode
     if mode < 0:
-        mode = 2 if hasattr(ctx.lib, "m40llm_ext_decode_layer_fused_async") else 0
+        mode = 2
     dm.set_mode(mode)
     prompt = np.random.default_rng(0).integers(0, cfg["vocab"], size=n_prompt).astype(np.uint32)
     setup_s = time.perf_counter() - t_setup

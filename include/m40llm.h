@@ -293,6 +293,45 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
  * writes the top-1 minus top-2 gap to out_gap_dev (may be NULL).  Decode stream. */
 int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t rows,
                                 size_t n, uint32_t* out_idx_dev, float* out_gap_dev);
+/* Fused batch-1 decode-step entry points (decode stream, asynchronous).  They compute exactly what the
+ * reference's per-op call sequence computes (src/infer/forward.rs:304-662), several steps per launch:
+ *   steps 1-5: RMSNorm -> Q/K/V projections (+bias) -> RoPE(Q) -> d_q_out; RoPE(K) and V -> f16 append at the
+ *              position (taken from position_dev when that is not NULL); dense caches only. */
+int m40llm_ext_fused_norm_qkv_rope_append_async(
+    M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id, const void* d_x_f32, const void* d_norm_w,
+    uint32_t norm_weight_dtype, float eps, const void* d_wq_f16, const void* d_wk_f16, const void* d_wv_f16,
+    const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32, uint32_t d_model, uint32_t q_heads,
+    uint32_t position, const uint32_t* position_dev, float freq_base, float freq_scale, uint32_t rope_layout, void* d_q_out_f32);
+/*   steps 7-8 / 12-13: out = residual + W . a (residual may be NULL or alias out) */
+int m40llm_ext_gemv_residual_f32xf16_async(M40llmCudaContext* ctx, const void* d_a_f32, const void* d_w_f16,
+                                           const void* d_residual_f32, void* d_out_f32, int N, int K);
+/*   steps 9-11: hid = silu(Wgate . xn) * (Wup . xn), xn = RMSNorm(x) * w */
+int m40llm_ext_fused_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                               uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
+                                               const void* d_wup_f16, void* d_hid_f32, int ffn, int d_model);
+/*   output norm + lm_head (src/infer/logits.rs:57-116 without the copy to the host) */
+/*   With d_block_top2 (3 planes of top2_capacity 4-byte entries: largest, second largest, first index of the
+ *   largest, one entry per workgroup) the kernel also leaves per-workgroup top-2 candidates for
+ *   m40llm_ext_greedy_step_async; *out_n_blocks (host) receives the number of entries. */
+int m40llm_ext_fused_norm_gemv_f32xf16_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                             uint32_t norm_weight_dtype, float eps, const void* d_w_f16,
+                                             void* d_out_f32, int N, int K, void* d_block_top2,
+                                             uint32_t top2_capacity, uint32_t* out_n_blocks);
+/* attention with the length taken from the device: seq_len = *position_dev + 1 <= max_len_hint */
+int m40llm_ext_attention_last_token_f32_gqa_position_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                               uint32_t seq_id, const void* q_dev_f32,
+                                                               uint32_t q_heads, const uint32_t* position_dev,
+                                                               uint32_t max_len_hint, void* out_dev_f32);
+/* embedding row of the token id stored at token_dev (f16 table [vocab][d_model]) -> f32 */
+int m40llm_ext_embed_token_dev_async(M40llmCudaContext* ctx, const void* d_table_f16, const uint32_t* token_dev,
+                                     uint32_t vocab, uint32_t d_model, void* d_out_f32);
+/* device-side greedy step over logits[n] (scanned directly, or through the per-workgroup candidates in
+ * d_block_top2): state_dev = {position, step, token, capacity, ids[capacity], gaps[capacity] (f32 bits)}; stores
+ * the first index of the maximum and the top-1/top-2 gap at [step], sets token, increments step and position.
+ * With d_table_f16 (f16 [n][d_model]) the embedding row of the picked token is written to d_x_out_f32. */
+int m40llm_ext_greedy_step_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t n,
+                                 const void* d_block_top2, uint32_t top2_capacity, uint32_t n_blocks,
+                                 uint32_t* state_dev, const void* d_table_f16, uint32_t d_model, void* d_x_out_f32);
 const char* m40llm_ext_build_info(void);
 
 /* ---- present but unavailable (return -1, as cuda/stub.c does) ---------------------- */

@@ -4,7 +4,7 @@
  * The reference's host side is Rust (src/decode.rs, src/decode_batch.rs, src/kv_compression.rs,
  * src/kv_selection.rs, src/sampling.rs and the decode part of src/infer/forward.rs); no Rust
  * toolchain exists in this build environment, so the same modules are written in C++
- * (m40-llm_amd/host/*.hpp) and exposed here so that tests and bindings in any language can drive
+ * (the headers under m40-llm_amd/host) and exposed here so that tests and bindings in any language can drive
  * them.  Every function that can fail returns a negative value and leaves a message for
  * m40host_last_error().
  */

@@ -29,6 +29,7 @@ struct AttnParams {
     uint32_t max_seq_len, kv_heads, q_heads, window;
     uint32_t chunk, nchunks;
     uint32_t subgroups;           // q-head subgroups per kv head
+    uint32_t len_bias;            // added to a device-side length (position -> length)
 };
 
 // HD in {64, 128}; G = q heads handled per workgroup (<= 8)
@@ -44,7 +45,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
 
     const uint32_t b = blockIdx.z;
     const uint32_t seq_id = p.seq_ids_dev ? p.seq_ids_dev[b] : p.seq_id;
-    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] : p.seq_len;
+    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t cbeg = t0 + blockIdx.y * p.chunk;
@@ -76,21 +77,24 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
         q[h][4] = q1.x; q[h][5] = q1.y; q[h][6] = q1.z; q[h][7] = q1.w;
     }
 
-    const uint32_t per_wave = p.chunk / kWaves;           // chunk is a multiple of kWaves*TPW
-    const uint32_t wbeg = cbeg + wave * per_wave;
+    // Token rows of the chunk are dealt to the waves in groups of TPW, round robin, so that every wave
+    // works on real tokens whatever the length: group gi = it * kWaves + wave covers rows gi*TPW .. +TPW-1.
+    const uint32_t n_tok = cend - cbeg;
+    const uint32_t n_groups = (n_tok + TPW - 1) / TPW;
 
     // ---- pass A: scores ---------------------------------------------------------------
     float lmax[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) lmax[h] = -INFINITY;
-    for (uint32_t it = 0; it < per_wave; it += TPW) {
-        const uint32_t t = wbeg + it + tg;
-        const bool valid = t < cend;
+#pragma unroll 2
+    for (uint32_t gi = wave; gi < n_groups; gi += kWaves) {
+        const uint32_t tl = gi * TPW + tg;
+        const uint32_t t = cbeg + tl;
+        const bool valid = tl < n_tok;
         uint4 kw = make_uint4(0, 0, 0, 0);
         if (valid) kw = *reinterpret_cast<const uint4*>(Kb + (size_t)t * row_stride);
         float kf[8];
         m40_unpack8(kw, kf);
-        const uint32_t tl = wave * per_wave + it + tg;
 #pragma unroll
         for (int h = 0; h < G; ++h) {
             float d = 0.0f;
@@ -99,7 +103,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
             d = LPT == 8 ? m40_sum8(d) : m40_sum16(d);
             const float s = valid ? d * inv_sqrt : -INFINITY;
             lmax[h] = fmaxf(lmax[h], s);
-            if (c == 0) sc[h * p.chunk + tl] = s;
+            if (c == 0 && valid) sc[h * p.chunk + tl] = s;
         }
     }
 #pragma unroll
@@ -121,11 +125,10 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
     float lsum[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) lsum[h] = 0.0f;
-    for (uint32_t tl = tid; tl < p.chunk; tl += kAttnThreads) {
+    for (uint32_t tl = tid; tl < n_tok; tl += kAttnThreads) {
 #pragma unroll
         for (int h = 0; h < G; ++h) {
-            const float s = sc[h * p.chunk + tl];
-            const float e = s == -INFINITY ? 0.0f : expf(s - mh[h]);
+            const float e = expf(sc[h * p.chunk + tl] - mh[h]);
             sc[h * p.chunk + tl] = e;
             lsum[h] += e;
         }
@@ -143,13 +146,13 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
     for (int h = 0; h < G; ++h)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[h][j] = 0.0f;
-    for (uint32_t it = 0; it < per_wave; it += TPW) {
-        const uint32_t t = wbeg + it + tg;
-        if (t < cend) {
-            const uint4 vw = *reinterpret_cast<const uint4*>(Vb + (size_t)t * row_stride);
+#pragma unroll 2
+    for (uint32_t gi = wave; gi < n_groups; gi += kWaves) {
+        const uint32_t tl = gi * TPW + tg;
+        if (tl < n_tok) {
+            const uint4 vw = *reinterpret_cast<const uint4*>(Vb + (size_t)(cbeg + tl) * row_stride);
             float vf[8];
             m40_unpack8(vw, vf);
-            const uint32_t tl = wave * per_wave + it + tg;
 #pragma unroll
             for (int h = 0; h < G; ++h) {
                 const float pw = sc[h * p.chunk + tl];
@@ -204,7 +207,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
 template <int HD>
 __global__ __launch_bounds__(HD) void attn_combine_kernel(AttnParams p) {
     const uint32_t qh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
-    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] : p.seq_len;
+    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t n = (len - t0 + p.chunk - 1) / p.chunk;
@@ -229,7 +232,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p, uint32_t
     const uint32_t d = blockIdx.x * 64 + threadIdx.x;
     if (d >= head_dim) return;
     const uint32_t seq_id = p.seq_ids_dev ? p.seq_ids_dev[b] : p.seq_id;
-    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] : p.seq_len;
+    const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t kvh = qh / (p.q_heads / p.kv_heads);
@@ -265,8 +268,11 @@ int launch_partial(hipStream_t stream, const AttnParams& p, uint32_t batch) {
 }
 
 template <int HD>
-int launch_hd(hipStream_t stream, AttnParams& p, uint32_t batch, uint32_t group) {
+int launch_hd(hipStream_t stream, AttnParams& p, uint32_t batch, uint32_t group, uint32_t span) {
     int G = group >= 8 ? 8 : (group >= 4 ? 4 : (group >= 2 ? 2 : 1));
+    // Short rows are latency-bound, not bandwidth-bound: spread the q heads over more workgroups
+    // (K/V of a short row stay in L2, so re-reading them per head pair costs nothing).
+    if (span <= 1024 && (uint64_t)batch * p.kv_heads * p.nchunks < 64) G = G > 2 ? 2 : G;
     if (group % G != 0) {
         // uneven group sizes (3, 5, 6, 7...) run with the largest subgroup that fits
         G = group >= 8 ? 8 : (group > 4 ? 8 : (group > 2 ? 4 : 2));
@@ -295,6 +301,7 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
     p.seq_id = a.seq_id; p.seq_len = a.seq_len;
     p.max_seq_len = a.max_seq_len; p.kv_heads = a.kv_heads; p.q_heads = a.q_heads; p.window = a.window;
     p.subgroups = 1;
+    p.len_bias = a.len_bias;
     (void)hipGetLastError();
     const uint32_t group = a.q_heads / a.kv_heads;
     uint32_t span = a.max_len_hint;
@@ -304,9 +311,13 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
     if ((a.head_dim == 64 || a.head_dim == 128) && m40_aligned16(a.Q) && m40_aligned16(a.K) && m40_aligned16(a.V)) {
         // chunk: small when there is little work so that more CUs take part; the per-row
         // partial buffer bounds the chunk count.
+        // Up to 512 tokens a single chunk per kv head finishes in a few microseconds and needs no
+        // merge launch; longer rows are split until the grid covers the CUs about twice.
         const uint64_t rows = (uint64_t)a.batch * a.kv_heads;
         uint32_t chunk = 512;
-        while (chunk > 64 && rows * ((span + chunk - 1) / chunk) < 2u * (uint32_t)ctx->num_cus) chunk >>= 1;
+        if (span > 512) {
+            while (chunk > 64 && rows * ((span + chunk - 1) / chunk) < 2u * (uint32_t)ctx->num_cus) chunk >>= 1;
+        }
         M40StreamScratch& sc = ctx->scratch[stream_kind];
         for (;;) {
             p.chunk = chunk;
@@ -317,8 +328,8 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
             chunk <<= 1;
         }
         p.ws = static_cast<float*>(sc.attn_partial);
-        if (a.head_dim == 64) launch_hd<64>(stream, p, a.batch, group);
-        else launch_hd<128>(stream, p, a.batch, group);
+        if (a.head_dim == 64) launch_hd<64>(stream, p, a.batch, group, span);
+        else launch_hd<128>(stream, p, a.batch, group, span);
     } else {
         p.chunk = span; p.nchunks = 1;
         dim3 grid((a.head_dim + 63) / 64, a.q_heads, a.batch);
@@ -408,6 +419,24 @@ int m40llm_attention_last_token_f32_gqa_seq_len_dev_async(M40llmCudaContext* ctx
     a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = 0;
     a.seq_lens_dev = seq_len_dev;            // row 0 of a one-row batch
     a.max_len_hint = kv->max_seq_len;        // the length is unknown on the host: size for the maximum
+    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+}
+
+// Extension: the sequence length is (*position_dev + 1); max_len_hint bounds it and sizes the grid.
+int m40llm_ext_attention_last_token_f32_gqa_position_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                               uint32_t seq_id, const void* q_dev_f32,
+                                                               uint32_t q_heads, const uint32_t* position_dev,
+                                                               uint32_t max_len_hint, void* out_dev_f32) {
+    if (!ctx || !kv || !q_dev_f32 || !position_dev || !out_dev_f32) return -1;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (max_len_hint == 0 || max_len_hint > kv->max_seq_len) return -3;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -6;
+    if (!kv->d_k || !kv->d_v) return -4;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = 0;
+    a.seq_lens_dev = position_dev; a.len_bias = 1; a.max_len_hint = max_len_hint;
     return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
 }
 

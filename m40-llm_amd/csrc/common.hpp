@@ -107,6 +107,7 @@ struct M40AttnArgs {
     const uint32_t* seq_lens_dev;   // also used alone for the seq_len_dev variant (batch==1)
     uint32_t max_len_hint;          // upper bound of any row's length (sizes the grid)
     uint32_t window;                // 0 = whole sequence, else only the last `window` tokens
+    uint32_t len_bias;              // added to lengths read from seq_lens_dev
 };
 int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
                                const M40AttnArgs& a);
@@ -125,8 +126,12 @@ typedef float m40_float4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float m40_h2f(uint16_t bits) {
     return static_cast<float>(__builtin_bit_cast(_Float16, bits));
 }
-// round-to-nearest-even f32 -> f16 (v_cvt_f16_f32 in the default rounding mode)
+// round-to-nearest-even f32 -> f16 (v_cvt_f16_f32 in the default rounding mode).  The empty asm pins the
+// f32 value first: without it the compiler folds a preceding multiply(-add) and the conversion into one
+// mixed-precision FMA that rounds once, to f16, where the reference rounds to f32 and then to f16 (the two
+// differ whenever the f32 result sits exactly between two f16 values).
 __device__ __forceinline__ uint16_t m40_f2h(float x) {
+    asm volatile("" : "+v"(x));
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(x));
 }
 
@@ -202,9 +207,12 @@ __device__ __forceinline__ void m40_rope_pair(uint32_t head, uint32_t off, uint3
         *i1 = *i0 + 1u;
     }
 }
-__device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off, uint32_t head_dim,
-                                                float base, float scale, float x0, float x1,
-                                                float* y0, float* y1) {
+// cos/sin of the rotation angle of pair `off` at `position`.  Deliberately not inlined: every kernel
+// that rotates (standalone RoPE, the rotating KV appends, the fused QKV kernel) must produce the same
+// bits for the same input, and the compiler's choices inside the inlined trigonometric code were seen
+// to differ by an ulp between call sites.
+__device__ __noinline__ static float2 m40_rope_cos_sin(uint32_t position, uint32_t off, uint32_t head_dim, float base,
+                                                       float scale) {
     const float pos = static_cast<float>(position) * scale;
     // The per-pair frequency is evaluated in double and rounded once: theta multiplies it by
     // the position, so a one-ulp difference in a float powf would grow to ~position * 2^-23
@@ -213,10 +221,15 @@ __device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off,
     const float exponent = -2.0f * static_cast<float>(off) / static_cast<float>(head_dim);
     const float inv_freq = static_cast<float>(pow(static_cast<double>(base), static_cast<double>(exponent)));
     const float theta = pos * inv_freq;
-    const float c = cosf(theta);
-    const float s = sinf(theta);
-    *y0 = x0 * c - x1 * s;
-    *y1 = x0 * s + x1 * c;
+    return make_float2(cosf(theta), sinf(theta));
+}
+__device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off, uint32_t head_dim,
+                                                float base, float scale, float x0, float x1,
+                                                float* y0, float* y1) {
+    const float2 cs = m40_rope_cos_sin(position, off, head_dim, base, scale);
+    // explicit fused multiply-adds: the same rounding in every kernel that inlines this rotation
+    *y0 = fmaf(x0, cs.x, -(x1 * cs.y));
+    *y1 = fmaf(x0, cs.y, x1 * cs.x);
 }
 
 // q4 V pair, two's-complement nibbles, even dim in the low nibble

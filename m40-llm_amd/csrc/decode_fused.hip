@@ -1,0 +1,426 @@
+// Fused batch-1 decode-step kernels for gfx950 (no counterpart in the reference, which issues one
+// launch per primitive op).  Each kernel streams f16 GGUF-layout weights exactly once with 128-bit
+// loads, keeps the activation vector in LDS, and folds the neighbouring elementwise ops into the
+// GEMV prologue / epilogue:
+//
+//   norm_qkv_rope_append : RMSNorm(x) -> Q,K,V projections (+bias) -> RoPE(Q) -> q_out,
+//                          RoPE(K) -> f16 K append, f16 V append                      (steps 1-5)
+//   gemv_residual        : out = residual + W . a                                     (steps 7-8, 12-13)
+//   norm_gate_up_swiglu  : RMSNorm(x) -> gate, up projections -> silu(gate) * up      (steps 9-11)
+//   norm_gemv            : RMSNorm(x) -> W . xn                                       (output norm + lm_head)
+//   embed_token_dev / greedy_step : device-side token feedback so consecutive tokens need no host round trip
+//
+// The arithmetic of every output element follows the unfused kernels operation for operation
+// (same reduction order for the norm, same lane->k mapping and FMA chain for the dot products, the
+// shared RoPE rotation), so this path and the reference call sequence produce identical bits.
+// Step numbers refer to the reference's per-layer call order, src/infer/forward.rs:304-662.
+#include "common.hpp"
+#include "gemv_core.hpp"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWavesPerBlock = 4;
+
+// x -> LDS as normalised activations: a[k] = x[k] * scale * w[k], scale = 1/sqrt(sum(x^2)/K + eps).
+// Reduction order identical to rms_norm_kernel (elementwise.hip).
+__device__ __forceinline__ void stage_normed(const float* __restrict__ x, const void* __restrict__ w,
+                                             uint32_t w_dtype, float eps, int K, float* __restrict__ a_lds,
+                                             float* __restrict__ wave_sums) {
+    const int tid = threadIdx.x;
+    float ss = 0.0f;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    for (int i = tid; i < K / 4; i += kThreads) {
+        const float4 v = x4[i];
+        ss = fmaf(v.x, v.x, ss);
+        ss = fmaf(v.y, v.y, ss);
+        ss = fmaf(v.z, v.z, ss);
+        ss = fmaf(v.w, v.w, ss);
+    }
+    ss = m40_sum64(ss);
+    if ((tid & 63) == 0) wave_sums[tid >> 6] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kWavesPerBlock; ++i) total += wave_sums[i];
+    const float scale = 1.0f / sqrtf(total / static_cast<float>(K) + eps);
+    const uint16_t* w16 = reinterpret_cast<const uint16_t*>(w);
+    const float* w32 = reinterpret_cast<const float*>(w);
+    for (int i = tid; i < K; i += kThreads) {
+        const float wv = w_dtype == 0u ? m40_h2f(w16[i]) : w32[i];
+        a_lds[i] = x[i] * scale * wv;
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ void stage_plain(const float* __restrict__ x, int K, float* __restrict__ a_lds) {
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    float4* a4 = reinterpret_cast<float4*>(a_lds);
+    for (int i = threadIdx.x; i < K / 4; i += kThreads) a4[i] = x4[i];
+    __syncthreads();
+}
+
+struct QkvArgs {
+    const float* x;
+    const void* norm_w;
+    const uint16_t *wq, *wk, *wv;
+    const float *bq, *bk, *bv;
+    float* q_out;
+    uint16_t* k_cache;   // base of this slot: [max_seq_len][kvh][hd]
+    uint16_t* v_cache;
+    uint32_t* seq_map_entry;
+    const uint32_t* position_dev;
+    uint32_t position, max_seq_len;
+    uint32_t d_model, q_heads, kv_heads, head_dim, rope_layout, norm_dtype;
+    float eps, rope_base, rope_scale;
+};
+
+// One wave per rotation pair (two output columns).  Pair space: Q pairs, then K pairs, then V pairs.
+__global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs p) {
+    extern __shared__ float a_lds[];
+    __shared__ float wave_sums[kWavesPerBlock];
+    const int K = (int)p.d_model;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t half = p.head_dim / 2u;
+    const uint32_t q_pairs = p.q_heads * half, kv_pairs = p.kv_heads * half;
+    uint32_t pair = blockIdx.x * kWavesPerBlock + wave;
+    const bool live = pair < q_pairs + 2u * kv_pairs;
+    if (!live) pair = 0;
+    int which;       // 0 Q, 1 K, 2 V
+    uint32_t local;
+    if (pair < q_pairs) { which = 0; local = pair; }
+    else if (pair < q_pairs + kv_pairs) { which = 1; local = pair - q_pairs; }
+    else { which = 2; local = pair - q_pairs - kv_pairs; }
+    const uint32_t head = local / half, off = local % half;
+    size_t i0, i1;
+    m40_rope_pair(head, off, p.head_dim, which == 2 ? M40LLM_ROPE_LAYOUT_ADJACENT : p.rope_layout, &i0, &i1);
+    const uint16_t* W = which == 0 ? p.wq : (which == 1 ? p.wk : p.wv);
+    const float* bias = which == 0 ? p.bq : (which == 1 ? p.bk : p.bv);
+    const uint4* bp[2] = {reinterpret_cast<const uint4*>(W + i0 * (size_t)K),
+                          reinterpret_cast<const uint4*>(W + i1 * (size_t)K)};
+    // weights are requested first; the norm prologue runs while they are in flight
+    GemvRegs<2> regs;
+    gemv_prefetch<2>(bp, 0, K >> 3, lane, regs);
+    stage_normed(p.x, p.norm_w, p.norm_dtype, p.eps, K, a_lds, wave_sums);
+    float d[2];
+    gemv_accumulate<2>(bp, a_lds, 0, K >> 3, lane, regs, d);
+    gemv_finish<2, 1>(d, nullptr, wave, lane);
+    if (!live || lane != 0) return;
+    const uint32_t position = p.position_dev ? *p.position_dev : p.position;
+    if (position >= p.max_seq_len) return;
+    float y0 = d[0], y1 = d[1];
+    if (bias) { y0 = y0 + bias[i0]; y1 = y1 + bias[i1]; }
+    if (which != 2) m40_rope_rotate(position, off, p.head_dim, p.rope_base, p.rope_scale, y0, y1, &y0, &y1);
+    if (which == 0) {
+        p.q_out[i0] = y0;
+        p.q_out[i1] = y1;
+    } else {
+        uint16_t* dst = (which == 1 ? p.k_cache : p.v_cache) + (size_t)position * p.kv_heads * p.head_dim;
+        dst[i0] = m40_f2h(y0);
+        dst[i1] = m40_f2h(y1);
+        if (which == 1 && local == 0) *p.seq_map_entry = position + 1u;
+    }
+}
+
+// out[n] = residual[n] + W[n] . a      (residual may alias out)
+template <int COLS, int KSPLIT>
+__global__ __launch_bounds__(kThreads) void gemv_residual_kernel(const float* __restrict__ a,
+                                                                 const uint16_t* __restrict__ W,
+                                                                 const float* residual, float* out, int N, int K) {
+    __shared__ float red[4 * COLS];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int col0 = KSPLIT == 1 ? (blockIdx.x * kWavesPerBlock + wave) * COLS : blockIdx.x * COLS;
+    if (col0 >= N) return;
+    const uint4* bp[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) bp[c] = reinterpret_cast<const uint4*>(W + (size_t)(col0 + c < N ? col0 + c : N - 1) * K);
+    int c_begin, c_end;
+    gemv_range<KSPLIT>(K, wave, &c_begin, &c_end);
+    GemvRegs<COLS> regs;
+    gemv_prefetch<COLS>(bp, c_begin, c_end, lane, regs);
+    float d[COLS];
+    gemv_accumulate<COLS>(bp, a, c_begin, c_end, lane, regs, d);
+    gemv_finish<COLS, KSPLIT>(d, red, wave, lane);
+    if (lane == 0 && (KSPLIT == 1 || wave == 0)) {
+#pragma unroll
+        for (int c = 0; c < COLS; ++c)
+            if (col0 + c < N) out[col0 + c] = residual ? residual[col0 + c] + d[c] : d[c];
+    }
+}
+
+// hid[j] = silu(Wg[j] . xn) * (Wu[j] . xn),  xn = RMSNorm(x) * w
+__global__ __launch_bounds__(kThreads) void norm_gate_up_swiglu_kernel(const float* __restrict__ x,
+                                                                       const void* __restrict__ norm_w,
+                                                                       uint32_t norm_dtype, float eps,
+                                                                       const uint16_t* __restrict__ Wg,
+                                                                       const uint16_t* __restrict__ Wu,
+                                                                       float* __restrict__ hid, int F, int K) {
+    extern __shared__ float a_lds[];
+    __shared__ float wave_sums[kWavesPerBlock];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    int j = blockIdx.x * kWavesPerBlock + wave;
+    const bool live = j < F;
+    if (!live) j = F - 1;
+    const uint4* bp[2] = {reinterpret_cast<const uint4*>(Wg + (size_t)j * K),
+                          reinterpret_cast<const uint4*>(Wu + (size_t)j * K)};
+    GemvRegs<2> regs;
+    gemv_prefetch<2>(bp, 0, K >> 3, lane, regs);
+    stage_normed(x, norm_w, norm_dtype, eps, K, a_lds, wave_sums);
+    float d[2];
+    gemv_accumulate<2>(bp, a_lds, 0, K >> 3, lane, regs, d);
+    gemv_finish<2, 1>(d, nullptr, wave, lane);
+    if (live && lane == 0) {
+        const float g = d[0];
+        const float silu = g / (1.0f + expf(-g));
+        hid[j] = silu * d[1];
+    }
+}
+
+// logits = W . RMSNorm(x); optionally the workgroup's top-2 (largest, second, first index of largest) goes
+// to blk_top (a | b | idx planes of `top_cap` entries) for the device-side greedy pick.
+template <int COLS>
+__global__ __launch_bounds__(kThreads) void norm_gemv_kernel(const float* __restrict__ x,
+                                                             const void* __restrict__ norm_w, uint32_t norm_dtype,
+                                                             float eps, const uint16_t* __restrict__ W,
+                                                             float* __restrict__ out, int N, int K,
+                                                             float* __restrict__ blk_top, uint32_t top_cap) {
+    extern __shared__ float a_lds[];
+    __shared__ float wave_sums[kWavesPerBlock];
+    __shared__ float top_a[kWavesPerBlock], top_b[kWavesPerBlock];
+    __shared__ uint32_t top_i[kWavesPerBlock];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int col0 = (blockIdx.x * kWavesPerBlock + wave) * COLS;
+    const bool live = col0 < N;
+    const uint4* bp[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        const int col = (live && col0 + c < N) ? col0 + c : N - 1;
+        bp[c] = reinterpret_cast<const uint4*>(W + (size_t)col * K);
+    }
+    GemvRegs<COLS> regs;
+    gemv_prefetch<COLS>(bp, 0, K >> 3, lane, regs);
+    stage_normed(x, norm_w, norm_dtype, eps, K, a_lds, wave_sums);
+    float d[COLS];
+    gemv_accumulate<COLS>(bp, a_lds, 0, K >> 3, lane, regs, d);
+    gemv_finish<COLS, 1>(d, nullptr, wave, lane);
+    if (lane == 0) {
+        float a = -INFINITY, b = -INFINITY;
+        uint32_t ia = 0xffffffffu;
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            if (live && col0 + c < N) {
+                out[col0 + c] = d[c];
+                if (d[c] > a) { b = a; a = d[c]; ia = (uint32_t)(col0 + c); }
+                else if (d[c] > b) b = d[c];
+            }
+        }
+        top_a[wave] = a; top_b[wave] = b; top_i[wave] = ia;
+    }
+    if (blk_top == nullptr) return;
+    __syncthreads();
+    if (threadIdx.x == 0 && blockIdx.x < top_cap) {
+        float a = top_a[0], b = top_b[0];
+        uint32_t ia = top_i[0];
+        for (int w = 1; w < kWavesPerBlock; ++w) {     // ascending columns: ties keep the lower index
+            const float oa = top_a[w], ob = top_b[w];
+            if (oa > a) { b = fmaxf(a, ob); a = oa; ia = top_i[w]; }
+            else b = fmaxf(b, oa);
+        }
+        blk_top[blockIdx.x] = a;
+        blk_top[top_cap + blockIdx.x] = b;
+        reinterpret_cast<uint32_t*>(blk_top)[2 * (size_t)top_cap + blockIdx.x] = ia;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void embed_token_dev_kernel(const uint16_t* __restrict__ table,
+                                                                   const uint32_t* __restrict__ token_dev,
+                                                                   uint32_t vocab, uint32_t d_model,
+                                                                   float* __restrict__ out) {
+    uint32_t tok = *token_dev;
+    if (tok >= vocab) tok = vocab - 1;
+    const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+    if (i < d_model) out[i] = m40_h2f(table[(size_t)tok * d_model + i]);
+}
+
+// Device-side greedy bookkeeping.  state: [0] position, [1] step, [2] current token,
+// [3] capacity, then ids[capacity], then gaps[capacity] (f32 bits).  Candidates come either from the
+// per-workgroup top-2 planes written by norm_gemv_kernel (n_blocks entries) or from a scan of the logits.
+// With a table, the embedding row of the picked token is converted to f32 into x_out as well.
+__global__ __launch_bounds__(1024) void greedy_step_kernel(const float* __restrict__ logits, uint32_t n,
+                                                           const float* __restrict__ blk_top, uint32_t top_cap,
+                                                           uint32_t n_blocks, uint32_t* __restrict__ state,
+                                                           const uint16_t* __restrict__ table, uint32_t d_model,
+                                                           float* __restrict__ x_out) {
+    __shared__ float sa[16], sb[16];
+    __shared__ uint32_t si[16];
+    __shared__ uint32_t s_tok;
+    float a = -INFINITY, b = -INFINITY;
+    uint32_t ia = 0xffffffffu;
+    auto offer = [&](float oa, float ob, uint32_t oi) {
+        if (oa > a || (oa == a && oi < ia)) { b = fmaxf(a, ob); a = oa; ia = oi; }
+        else b = fmaxf(b, oa);
+    };
+    if (blk_top) {
+        const uint32_t* idx = reinterpret_cast<const uint32_t*>(blk_top) + 2 * (size_t)top_cap;
+        for (uint32_t i = threadIdx.x; i < n_blocks; i += blockDim.x) offer(blk_top[i], blk_top[top_cap + i], idx[i]);
+    } else {
+        for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) offer(logits[i], -INFINITY, i);
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float oa = __shfl_xor(a, o, 64), ob = __shfl_xor(b, o, 64);
+        const uint32_t oi = __shfl_xor(ia, o, 64);
+        offer(oa, ob, oi);
+    }
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0u) { sa[wave] = a; sb[wave] = b; si[wave] = ia; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < blockDim.x / 64u; ++w) offer(sa[w], sb[w], si[w]);
+        uint32_t tok = ia == 0xffffffffu ? 0u : ia;
+        if (tok >= n) tok = n - 1;
+        const uint32_t step = state[1], cap = state[3];
+        if (step < cap) {
+            state[4 + step] = tok;
+            state[4 + cap + step] = __float_as_uint(a - b);
+        }
+        state[2] = tok;
+        state[1] = step + 1u;
+        state[0] = state[0] + 1u;
+        s_tok = tok;
+    }
+    if (table == nullptr) return;
+    __syncthreads();
+    const uint32_t tok = s_tok;
+    for (uint32_t i = threadIdx.x; i < d_model; i += blockDim.x) x_out[i] = m40_h2f(table[(size_t)tok * d_model + i]);
+}
+
+bool fast_ok(const void* a, const void* b, int K) { return K % 8 == 0 && m40_aligned16(a) && m40_aligned16(b); }
+
+}  // namespace
+
+extern "C" {
+
+int m40llm_ext_fused_norm_qkv_rope_append_async(
+    M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id, const void* d_x_f32, const void* d_norm_w,
+    uint32_t norm_weight_dtype, float eps, const void* d_wq_f16, const void* d_wk_f16, const void* d_wv_f16,
+    const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32, uint32_t d_model, uint32_t q_heads,
+    uint32_t position, const uint32_t* position_dev, float freq_base, float freq_scale, uint32_t rope_layout, void* d_q_out_f32) {
+    if (!ctx || !kv || !d_x_f32 || !d_norm_w || !d_wq_f16 || !d_wk_f16 || !d_wv_f16 || !d_q_out_f32) return -1;
+    if (kv->compressed || !kv->d_k || !kv->d_v) return -2;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (norm_weight_dtype > 1) return -4;
+    if (kv->head_dim == 0 || kv->head_dim % 2 != 0 || kv->num_heads == 0 || q_heads == 0) return -3;
+    if (!position_dev && position >= kv->max_seq_len) return -5;
+    if (d_model == 0) return -3;
+    const uint32_t D = d_model;
+    if (!fast_ok(d_x_f32, d_wq_f16, (int)D) || !m40_aligned16(d_wk_f16) || !m40_aligned16(d_wv_f16) ||
+        (size_t)D * 4 > 60 * 1024)
+        return -6;
+    QkvArgs p{};
+    p.x = static_cast<const float*>(d_x_f32);
+    p.norm_w = d_norm_w;
+    p.wq = static_cast<const uint16_t*>(d_wq_f16);
+    p.wk = static_cast<const uint16_t*>(d_wk_f16);
+    p.wv = static_cast<const uint16_t*>(d_wv_f16);
+    p.bq = static_cast<const float*>(d_bq_f32);
+    p.bk = static_cast<const float*>(d_bk_f32);
+    p.bv = static_cast<const float*>(d_bv_f32);
+    p.q_out = static_cast<float*>(d_q_out_f32);
+    const size_t ept = (size_t)kv->num_heads * kv->head_dim;
+    p.k_cache = kv->d_k + (size_t)seq_id * kv->max_seq_len * ept;
+    p.v_cache = kv->d_v + (size_t)seq_id * kv->max_seq_len * ept;
+    p.seq_map_entry = kv->d_seq_map + seq_id;
+    p.position_dev = position_dev;
+    p.position = position;
+    p.max_seq_len = kv->max_seq_len;
+    p.d_model = D; p.q_heads = q_heads; p.kv_heads = kv->num_heads; p.head_dim = kv->head_dim;
+    p.rope_layout = rope_layout; p.norm_dtype = norm_weight_dtype;
+    p.eps = eps; p.rope_base = freq_base; p.rope_scale = freq_scale;
+    const uint32_t pairs = (q_heads + 2u * kv->num_heads) * (kv->head_dim / 2u);
+    (void)hipGetLastError();
+    norm_qkv_rope_append_kernel<<<(pairs + kWavesPerBlock - 1) / kWavesPerBlock, kThreads, (size_t)D * 4, ctx->decode_stream>>>(p);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_gemv_residual_f32xf16_async(M40llmCudaContext* ctx, const void* d_a_f32, const void* d_w_f16,
+                                           const void* d_residual_f32, void* d_out_f32, int N, int K) {
+    if (!ctx || !d_a_f32 || !d_w_f16 || !d_out_f32) return -1;
+    if (N <= 0 || K <= 0) return -2;
+    if (!fast_ok(d_a_f32, d_w_f16, K)) return -6;
+    (void)hipGetLastError();
+    const float* a = static_cast<const float*>(d_a_f32);
+    const uint16_t* W = static_cast<const uint16_t*>(d_w_f16);
+    const float* r = static_cast<const float*>(d_residual_f32);
+    float* o = static_cast<float*>(d_out_f32);
+    const GemvShape g = gemv_pick_shape(N, K);
+    if (g.ksplit == 4) gemv_residual_kernel<1, 4><<<g.blocks, kThreads, 0, ctx->decode_stream>>>(a, W, r, o, N, K);
+    else if (g.cols == 4) gemv_residual_kernel<4, 1><<<g.blocks, kThreads, 0, ctx->decode_stream>>>(a, W, r, o, N, K);
+    else if (g.cols == 2) gemv_residual_kernel<2, 1><<<g.blocks, kThreads, 0, ctx->decode_stream>>>(a, W, r, o, N, K);
+    else gemv_residual_kernel<1, 1><<<g.blocks, kThreads, 0, ctx->decode_stream>>>(a, W, r, o, N, K);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_fused_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                               uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
+                                               const void* d_wup_f16, void* d_hid_f32, int ffn, int d_model) {
+    if (!ctx || !d_x_f32 || !d_norm_w || !d_wgate_f16 || !d_wup_f16 || !d_hid_f32) return -1;
+    if (ffn <= 0 || d_model <= 0) return -2;
+    if (norm_weight_dtype > 1) return -4;
+    if (!fast_ok(d_x_f32, d_wgate_f16, d_model) || !m40_aligned16(d_wup_f16) || (size_t)d_model * 4 > 60 * 1024) return -6;
+    (void)hipGetLastError();
+    norm_gate_up_swiglu_kernel<<<(ffn + 3) / 4, kThreads, (size_t)d_model * 4, ctx->decode_stream>>>(
+        static_cast<const float*>(d_x_f32), d_norm_w, norm_weight_dtype, eps, static_cast<const uint16_t*>(d_wgate_f16),
+        static_cast<const uint16_t*>(d_wup_f16), static_cast<float*>(d_hid_f32), ffn, d_model);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_fused_norm_gemv_f32xf16_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                             uint32_t norm_weight_dtype, float eps, const void* d_w_f16,
+                                             void* d_out_f32, int N, int K, void* d_block_top2,
+                                             uint32_t top2_capacity, uint32_t* out_n_blocks) {
+    if (!ctx || !d_x_f32 || !d_norm_w || !d_w_f16 || !d_out_f32) return -1;
+    if (N <= 0 || K <= 0) return -2;
+    if (norm_weight_dtype > 1) return -4;
+    if (!fast_ok(d_x_f32, d_w_f16, K) || (size_t)K * 4 > 60 * 1024) return -6;
+    (void)hipGetLastError();
+    const float* x = static_cast<const float*>(d_x_f32);
+    const uint16_t* W = static_cast<const uint16_t*>(d_w_f16);
+    float* o = static_cast<float*>(d_out_f32);
+    float* top = static_cast<float*>(d_block_top2);
+    const size_t lds = (size_t)K * 4;
+    const int cols = N >= 16384 ? 4 : (N >= 6144 ? 2 : 1);
+    const int blocks = (N + 4 * cols - 1) / (4 * cols);
+    if (top && (uint32_t)blocks > top2_capacity) return -5;
+    if (out_n_blocks) *out_n_blocks = (uint32_t)blocks;
+    if (cols == 4) norm_gemv_kernel<4><<<blocks, kThreads, lds, ctx->decode_stream>>>(x, d_norm_w, norm_weight_dtype, eps, W, o, N, K, top, top2_capacity);
+    else if (cols == 2) norm_gemv_kernel<2><<<blocks, kThreads, lds, ctx->decode_stream>>>(x, d_norm_w, norm_weight_dtype, eps, W, o, N, K, top, top2_capacity);
+    else norm_gemv_kernel<1><<<blocks, kThreads, lds, ctx->decode_stream>>>(x, d_norm_w, norm_weight_dtype, eps, W, o, N, K, top, top2_capacity);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_embed_token_dev_async(M40llmCudaContext* ctx, const void* d_table_f16, const uint32_t* token_dev,
+                                     uint32_t vocab, uint32_t d_model, void* d_out_f32) {
+    if (!ctx || !d_table_f16 || !token_dev || !d_out_f32) return -1;
+    if (vocab == 0 || d_model == 0) return -2;
+    (void)hipGetLastError();
+    embed_token_dev_kernel<<<(d_model + kThreads - 1) / kThreads, kThreads, 0, ctx->decode_stream>>>(
+        static_cast<const uint16_t*>(d_table_f16), token_dev, vocab, d_model, static_cast<float*>(d_out_f32));
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_greedy_step_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t n,
+                                 const void* d_block_top2, uint32_t top2_capacity, uint32_t n_blocks,
+                                 uint32_t* state_dev, const void* d_table_f16, uint32_t d_model, void* d_x_out_f32) {
+    if (!ctx || !state_dev || (!d_logits_f32 && !d_block_top2)) return -1;
+    if (n == 0) return -2;
+    if (d_block_top2 && (n_blocks == 0 || n_blocks > top2_capacity)) return -2;
+    if (d_table_f16 && (!d_x_out_f32 || d_model == 0)) return -1;
+    (void)hipGetLastError();
+    greedy_step_kernel<<<1, 1024, 0, ctx->decode_stream>>>(
+        static_cast<const float*>(d_logits_f32), n, static_cast<const float*>(d_block_top2), top2_capacity, n_blocks,
+        state_dev, static_cast<const uint16_t*>(d_table_f16), d_model, static_cast<float*>(d_x_out_f32));
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+}  // extern "C"

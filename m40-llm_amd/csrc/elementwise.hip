@@ -27,10 +27,10 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const float* __restr
         const float4* x4 = reinterpret_cast<const float4*>(x);
         for (uint32_t i = tid; i < dim / 4u; i += kThreads) {
             const float4 v = x4[i];
-            ss += v.x * v.x;
-            ss += v.y * v.y;
-            ss += v.z * v.z;
-            ss += v.w * v.w;
+            ss = fmaf(v.x, v.x, ss);
+            ss = fmaf(v.y, v.y, ss);
+            ss = fmaf(v.z, v.z, ss);
+            ss = fmaf(v.w, v.w, ss);
         }
     } else {
         for (uint32_t i = tid; i < dim; i += kThreads) ss += x[i] * x[i];

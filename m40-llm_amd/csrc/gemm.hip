@@ -1,8 +1,9 @@
 // GEMV / skinny GEMM family for gfx950: C[M,N] f32 = A[M,K] x B, f32 accumulation.
 //
-//   M == 1      : wave-per-column GEMV.  64 lanes stride the K dimension with 128-bit loads of
-//                 the f16 weights (GGUF layout: K contiguous per output column), f32 FMA per
-//                 lane, one DPP/shuffle butterfly per column.  HBM-bound; bytes = 2*N*K.
+//   M == 1      : wave-per-column GEMV (gemv_core.hpp).  64 lanes stride the K dimension with 128-bit
+//                 loads of the f16 weights (GGUF layout: K contiguous per output column), f32 FMA
+//                 per lane, one DPP/shuffle butterfly per column; few columns x long K splits K over
+//                 the four waves of a workgroup.  HBM-bound; bytes = 2*N*K.
 //   2 <= M <= 16: MFMA (v_mfma_f32_16x16x32_f16).  The f32 activations are split exactly into
 //                 f16 hi + f16 lo parts (after a per-row power-of-two scale), the f16 weights go
 //                 from HBM to the B operand registers without passing LDS: lane (n, g) loads the
@@ -13,50 +14,38 @@
 // Reference semantics: gemm_f32xf16_gguf_f32_kernel cuda/kernels.cu:5037-5052 and the entry
 // points :5068-5302 (which run on the prefill stream and block until done).
 #include "common.hpp"
+#include "gemv_core.hpp"
 
 namespace {
 
 // ---------------------------------------------------------------------------------------
 // M == 1
 // ---------------------------------------------------------------------------------------
-template <int COLS>
+template <int COLS, int KSPLIT>
 __global__ __launch_bounds__(256) void gemv_f32xf16_gguf_kernel(const float* __restrict__ A,
                                                                 const uint16_t* __restrict__ B,
                                                                 float* __restrict__ C, int N, int K) {
+    __shared__ float red[4 * COLS];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int col0 = (blockIdx.x * 4 + wave) * COLS;
-    if (col0 >= N) return;
-    const int nchunks = K >> 3;  // 8 halves = 16 bytes per chunk
+    const int col0 = KSPLIT == 1 ? (blockIdx.x * 4 + wave) * COLS : blockIdx.x * COLS;
+    if (col0 >= N) return;   // uniform per wave (KSPLIT 1) or per workgroup (KSPLIT 4)
     const uint4* bp[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         const int col = col0 + c < N ? col0 + c : N - 1;
         bp[c] = reinterpret_cast<const uint4*>(B + (size_t)col * K);
     }
-    const float4* a4 = reinterpret_cast<const float4*>(A);
+    int c_begin, c_end;
+    gemv_range<KSPLIT>(K, wave, &c_begin, &c_end);
+    GemvRegs<COLS> regs;
+    gemv_prefetch<COLS>(bp, c_begin, c_end, lane, regs);
     float acc[COLS];
+    gemv_accumulate<COLS>(bp, A, c_begin, c_end, lane, regs, acc);
+    gemv_finish<COLS, KSPLIT>(acc, red, wave, lane);
+    if (lane == 0 && (KSPLIT == 1 || wave == 0)) {
 #pragma unroll
-    for (int c = 0; c < COLS; ++c) acc[c] = 0.0f;
-
-#pragma unroll 2
-    for (int kc = lane; kc < nchunks; kc += 64) {
-        const float4 a0 = a4[2 * kc], a1 = a4[2 * kc + 1];
-        const float av[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
-        uint4 w[COLS];
-#pragma unroll
-        for (int c = 0; c < COLS; ++c) w[c] = m40_load_stream(bp[c] + kc);
-#pragma unroll
-        for (int c = 0; c < COLS; ++c) {
-            float f[8];
-            m40_unpack8(w[c], f);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) acc[c] = fmaf(av[j], f[j], acc[c]);
-        }
-    }
-#pragma unroll
-    for (int c = 0; c < COLS; ++c) {
-        const float s = m40_sum64(acc[c]);
-        if (lane == 0 && col0 + c < N) C[col0 + c] = s;
+        for (int c = 0; c < COLS; ++c)
+            if (col0 + c < N) C[col0 + c] = acc[c];
     }
 }
 
@@ -309,15 +298,11 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
     (void)hipGetLastError();
     const bool fast = (K % 8 == 0) && m40_aligned16(A) && m40_aligned16(B);
     if (fast && M == 1) {
-        // columns per wave: keep >= ~2048 waves, give each lane several loads in flight
-        const long long waves1 = N;
-        if (waves1 >= 16384) {
-            gemv_f32xf16_gguf_kernel<4><<<(N + 15) / 16, 256, 0, stream>>>(A, B, C, N, K);
-        } else if (waves1 >= 6144) {
-            gemv_f32xf16_gguf_kernel<2><<<(N + 7) / 8, 256, 0, stream>>>(A, B, C, N, K);
-        } else {
-            gemv_f32xf16_gguf_kernel<1><<<(N + 3) / 4, 256, 0, stream>>>(A, B, C, N, K);
-        }
+        const GemvShape g = gemv_pick_shape(N, K);
+        if (g.ksplit == 4) gemv_f32xf16_gguf_kernel<1, 4><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
+        else if (g.cols == 4) gemv_f32xf16_gguf_kernel<4, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
+        else if (g.cols == 2) gemv_f32xf16_gguf_kernel<2, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
+        else gemv_f32xf16_gguf_kernel<1, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
     } else if (fast && K % 64 == 0 && (size_t)K * 64 <= ctx->scratch[stream_kind].gemm_pack_bytes - 256) {
         M40StreamScratch& sc = ctx->scratch[stream_kind];
         const int KT = K >> 6;

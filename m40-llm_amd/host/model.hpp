@@ -126,6 +126,7 @@ public:
         ws_.ensure(ctx, cfg, 1);
     }
     ~DecodeModel() {
+        drop_graph();
         if (kv_) m40llm_kvcache_destroy(kv_);
     }
     DecodeModel(const DecodeModel&) = delete;
@@ -195,19 +196,163 @@ public:
         M40H_TRY(m40llm_residual_add_f32_async(ctx_, ws_.x1.ptr(), ws_.y_mlp.ptr(), d_out, D));
     }
 
+    // One decoder layer, fused entry points, decode stream only.  The position comes from the host
+    // (position_dev == nullptr) or from device memory (graph replay).
+    void layer_fused(uint32_t layer, uint32_t seq, uint32_t pos, const uint32_t* position_dev, uint32_t max_len_hint,
+                     const float* d_x, float* d_out) {
+        const LayerWeights& w = layers_[layer];
+        const uint32_t D = cfg_.d_model, F = cfg_.ffn;
+        const uint32_t slot = kv_slot(seq, layer);
+        M40H_TRY(m40llm_ext_fused_norm_qkv_rope_append_async(ctx_, kv_, slot, d_x, w.attn_norm, cfg_.norm_weight_dtype,
+                                                             cfg_.rms_eps, w.wq, w.wk, w.wv, w.bq, w.bk, w.bv, cfg_.d_model,
+                                                             cfg_.q_heads, pos, position_dev, cfg_.rope_base, cfg_.rope_scale,
+                                                             cfg_.rope_layout, ws_.q.ptr()));
+        if (position_dev) {
+            M40H_TRY(m40llm_ext_attention_last_token_f32_gqa_position_dev_async(ctx_, kv_, slot, ws_.q.ptr(), cfg_.q_heads,
+                                                                                position_dev, max_len_hint, ws_.ctx_out.ptr()));
+        } else {
+            M40H_TRY(m40llm_attention_last_token_f32_gqa_async(ctx_, kv_, slot, ws_.q.ptr(), cfg_.q_heads, pos + 1,
+                                                               ws_.ctx_out.ptr()));
+        }
+        M40H_TRY(m40llm_ext_gemv_residual_f32xf16_async(ctx_, ws_.ctx_out.ptr(), w.wo, d_x, ws_.x1.ptr(), (int)D, (int)D));
+        M40H_TRY(m40llm_ext_fused_norm_gate_up_swiglu_async(ctx_, ws_.x1.ptr(), w.ffn_norm, cfg_.norm_weight_dtype, cfg_.rms_eps,
+                                                            w.wgate, w.wup, ws_.hid.ptr(), (int)F, (int)D));
+        M40H_TRY(m40llm_ext_gemv_residual_f32xf16_async(ctx_, ws_.hid.ptr(), w.wdown, ws_.x1.ptr(), d_out, (int)D, (int)F));
+    }
+
+    bool fused_available() const { return !kvcfg_.is_enabled(); }
+
     // All layers for one token; returns the device pointer that holds the final hidden state.
     const float* forward_token(uint32_t seq, uint32_t pos, uint32_t token_id) {
         if (pos >= cfg_.max_seq_len) throw std::out_of_range("position beyond max_seq_len");
         ws_.ensure(ctx_, cfg_, 1);
         float* a = ws_.scratch_a.f32();
         float* b = ws_.scratch_b.f32();
+        const bool fused = mode_ >= 1 && fused_available();
+        // the embedding is written on the prefill stream: decode-stream work of the previous token that still
+        // reads or writes the ping-pong buffers must be ordered before it
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, M40LLM_STREAM_PREFILL, M40LLM_STREAM_DECODE));
         embed(token_id, a);
         for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
             kv_selection::set_attention_context(l, pos);
-            layer_reference(l, seq, pos + 1, a, b);
+            if (fused) layer_fused(l, seq, pos, nullptr, 0, a, b);
+            else layer_reference(l, seq, pos + 1, a, b);
             std::swap(a, b);
         }
         return a;
+    }
+
+    // ---- device-driven greedy loop (modes 1 and 2) ---------------------------------------------
+    // state = {position of the last processed token, step, token, capacity, ids[cap], gaps[cap]}
+    static constexpr float kGreedyTieGuard = 1e-6f;
+    void ensure_state(uint32_t capacity) {
+        if (capacity <= state_cap_) return;
+        state_ = DeviceBuf(ctx_, (size_t)(4 + 2 * capacity) * 4);
+        state_cap_ = capacity;
+        drop_graph();
+    }
+    void drop_graph() {
+        if (graph_) m40llm_cuda_graph_destroy(graph_);
+        graph_ = nullptr;
+    }
+    uint32_t* state_dev() const { return static_cast<uint32_t*>(state_.ptr()); }
+
+    // lm_head on `hidden` -> device greedy pick -> embedding of the picked token -> all layers at
+    // the device-side position; leaves the new hidden state in `hidden` (ping-pong safe).
+    void enqueue_generation_step(uint32_t seq, float* hidden, float* other, uint32_t max_len_hint) {
+        if (!top2_.ptr()) top2_ = DeviceBuf(ctx_, (size_t)3 * kTop2Capacity * 4);
+        uint32_t n_blocks = 0;
+        M40H_TRY(m40llm_ext_fused_norm_gemv_f32xf16_async(ctx_, hidden, out_norm_, cfg_.norm_weight_dtype, cfg_.rms_eps, lm_head_,
+                                                          ws_.logits.ptr(), (int)cfg_.vocab, (int)cfg_.d_model, top2_.ptr(),
+                                                          kTop2Capacity, &n_blocks));
+        // greedy pick from the per-workgroup candidates + embedding row of the picked token into `hidden`
+        M40H_TRY(m40llm_ext_greedy_step_async(ctx_, ws_.logits.ptr(), cfg_.vocab, top2_.ptr(), kTop2Capacity, n_blocks,
+                                              state_dev(), tok_emb_, cfg_.d_model, hidden));
+        float* a = hidden;
+        float* b = other;
+        for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
+            layer_fused(l, seq, 0, state_dev(), max_len_hint, a, b);
+            std::swap(a, b);
+        }
+        if (a != hidden)   // odd layer count: bring the result back so every step starts from `hidden`
+            M40H_TRY(m40llm_memcpy_d2d_async(ctx_, hidden, a, (size_t)cfg_.d_model * 4, M40LLM_STREAM_DECODE));
+    }
+
+    uint32_t len_hint_for(uint32_t last_pos_inclusive) const {
+        uint32_t h = ((last_pos_inclusive + 1 + 511u) / 512u) * 512u;
+        return h > cfg_.max_seq_len ? cfg_.max_seq_len : h;
+    }
+
+    // Runs `steps` generation steps starting after `n_done` steps already taken; positions advance on the device.
+    void run_generation_steps(uint32_t seq, float* hidden, float* other, uint32_t first_new_pos, uint32_t steps) {
+        uint32_t done = 0;
+        while (done < steps) {
+            const uint32_t pos = first_new_pos + done;
+            const uint32_t hint = len_hint_for(pos);
+            // steps that share this attention grid size
+            uint32_t n = steps - done;
+            if (hint < cfg_.max_seq_len && pos + n > hint) n = hint - pos;
+            if (mode_ >= 2) {
+                if (!graph_ || graph_seq_ != seq || graph_hint_ != hint || graph_hidden_ != hidden) {
+                    drop_graph();
+                    M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
+                    M40H_TRY(m40llm_cuda_graph_begin_capture(ctx_, M40LLM_STREAM_DECODE));
+                    try {
+                        enqueue_generation_step(seq, hidden, other, hint);
+                    } catch (...) {
+                        m40llm_cuda_graph_cancel_capture(ctx_, M40LLM_STREAM_DECODE);
+                        throw;
+                    }
+                    M40H_TRY(m40llm_cuda_graph_end_capture(ctx_, M40LLM_STREAM_DECODE, &graph_));
+                    graph_seq_ = seq; graph_hint_ = hint; graph_hidden_ = hidden;
+                }
+                for (uint32_t i = 0; i < n; ++i) M40H_TRY(m40llm_cuda_graph_launch(ctx_, graph_, M40LLM_STREAM_DECODE));
+            } else {
+                for (uint32_t i = 0; i < n; ++i) enqueue_generation_step(seq, hidden, other, hint);
+            }
+            done += n;
+        }
+    }
+
+    // Greedy decode on the device path.  Returns false when a top-1/top-2 logit gap fell under the tie guard
+    // (the host sampler's tie rule could then differ from a plain argmax): the caller redoes the decode on the
+    // host-sampled path.
+    bool decode_greedy_device(uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t warmup, uint32_t steps,
+                              uint32_t start_pos, uint32_t* ids_out, float* gaps_out, double* elapsed_ms) {
+        if (n_prompt == 0) throw std::invalid_argument("decode needs at least one prompt token");
+        const uint32_t total = warmup + steps;
+        if (start_pos + n_prompt + total > cfg_.max_seq_len) throw std::out_of_range("decode would exceed max_seq_len");
+        ws_.ensure(ctx_, cfg_, 1);
+        ensure_state(total);
+        uint32_t pos = start_pos;
+        const float* h = nullptr;
+        for (uint32_t i = 0; i < n_prompt; ++i) {
+            ids_out[i] = prompt[i];
+            h = forward_token(seq, pos++, prompt[i]);
+        }
+        float* hidden = const_cast<float*>(h);
+        float* other = hidden == ws_.scratch_a.f32() ? ws_.scratch_b.f32() : ws_.scratch_a.f32();
+        std::vector<uint32_t> st(4 + 2 * (size_t)state_cap_, 0);
+        st[0] = pos - 1; st[1] = 0; st[2] = prompt[n_prompt - 1]; st[3] = state_cap_;
+        M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, state_.ptr(), st.data(), st.size() * 4));
+        if (warmup) run_generation_steps(seq, hidden, other, pos, warmup);
+        sync_all();
+        const auto t0 = std::chrono::steady_clock::now();
+        run_generation_steps(seq, hidden, other, pos + warmup, steps);
+        sync_all();
+        const auto t1 = std::chrono::steady_clock::now();
+        if (elapsed_ms) *elapsed_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+        M40H_TRY(m40llm_memcpy_d2h(ctx_, st.data(), state_.ptr(), st.size() * 4));
+        bool ok = true;
+        for (uint32_t g = 0; g < total; ++g) {
+            ids_out[n_prompt + g] = st[4 + g];
+            float gap;
+            std::memcpy(&gap, &st[4 + state_cap_ + g], 4);
+            if (gaps_out) gaps_out[g] = gap;
+            if (!(gap >= kGreedyTieGuard)) ok = false;
+        }
+        return ok;
     }
 
     // output norm -> lm_head GEMV -> sync -> D2H (logits.rs:57-116)
@@ -226,6 +371,10 @@ public:
     // (Sampler with top_k = 1).  ids_out holds n_prompt + n_gen ids.
     void decode_greedy(uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t n_gen, uint32_t start_pos,
                        uint32_t* ids_out, float* gaps_out) {
+        if (mode_ >= 1 && fused_available() && n_gen > 0) {
+            // The device loop also runs the layers for the last sampled token (its KV entry is written); ids are the same.
+            if (decode_greedy_device(seq, prompt, n_prompt, 0, n_gen, start_pos, ids_out, gaps_out, nullptr)) return;
+        }
         Sampler sampler = greedy_sampler(42);
         std::vector<float> logits(cfg_.vocab);
         uint32_t pos = start_pos;
@@ -256,6 +405,8 @@ public:
         const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
         float* a = ws_.scratch_a.f32();
         float* b = ws_.scratch_b.f32();
+        // decode-stream work of the previous step must not overlap the embedding writes (prefill stream)
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
         for (uint32_t r = 0; r < rows; ++r) {
             if (kv_lens[r] + 1 > cfg_.max_seq_len) throw std::out_of_range("sequence would exceed max_seq_len");
             embed(token_ids[r], a + (size_t)r * D);
@@ -348,6 +499,10 @@ public:
     void decode_timed(uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t warmup, uint32_t steps,
                       uint32_t* ids_out, double* elapsed_ms) {
         if (n_prompt == 0) throw std::invalid_argument("decode_timed needs a prompt");
+        if (mode_ >= 1 && fused_available()) {
+            if (decode_greedy_device(seq, prompt, n_prompt, warmup, steps, 0, ids_out, nullptr, elapsed_ms)) return;
+            throw std::runtime_error("near-tie in a greedy pick on the device path; rerun in mode 0");
+        }
         std::vector<float> logits(cfg_.vocab);
         Sampler sampler = greedy_sampler(42);
         uint32_t pos = 0;
@@ -458,6 +613,13 @@ private:
     M40llmKVCache* kv_ = nullptr;
     ForwardWorkspace ws_;
     uint32_t mode_ = 0;
+    DeviceBuf state_;
+    DeviceBuf top2_;
+    static constexpr uint32_t kTop2Capacity = 1u << 16;
+    uint32_t state_cap_ = 0;
+    M40llmCudaGraphExec* graph_ = nullptr;
+    uint32_t graph_seq_ = 0, graph_hint_ = 0;
+    float* graph_hidden_ = nullptr;
 };
 
 }  // namespace m40host
