@@ -34,34 +34,47 @@ def algorithmic_bytes_per_token(cfg):
     return L * per_layer + V * D * 2
 
 
-def measure_dominant_kernel(pkg, ctx, dm, cfg, reps):
-    """Average launch duration of the kernel that moves most of the bytes of a token: the FFN gate/up GEMV
-    (f32 activations x f16 GGUF weights, N=ffn, K=hidden), timed with HIP events on the library's decode stream.
-    Launches cycle through the layers' own weight matrices so that no launch finds its weights in cache."""
+def measure_dominant_kernel(pkg, ctx, dm, cfg, reps, mode):
+    """Average launch duration of the kernel that moves most of the bytes of a token, timed with HIP events on
+    the library's decode stream.  Fused modes: RMSNorm + FFN gate/up GEMV + SwiGLU in one launch (two f16 GGUF
+    matrices of N=ffn, K=hidden).  Reference call sequence: the gate (or up) GEMV alone.  Launches cycle through
+    the layers' own weight matrices so that no launch finds its weights in a cache."""
     D, F, L = cfg["d_model"], cfg["ffn"], cfg["n_layers"]
     x = ctx.to_device(np.random.default_rng(1).standard_normal(D).astype(np.float32))
     y = ctx.alloc(F * 4)
-    mats = []
-    for l in range(L):
-        mats.append(dm.layers[l].wgate); mats.append(dm.layers[l].wup)
     lib = ctx.lib
-    for i in range(len(mats)):      # warm-up: code objects, clocks
-        pkg.check(lib.m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx.h, x.ptr, mats[i], y.ptr, 1, F, D, 1), "gemv")
+    if mode >= 1:
+        def launch(l):
+            ly = dm.layers[l]
+            return lib.m40llm_ext_fused_norm_gate_up_swiglu_async(ctx.h, x.ptr, ly.ffn_norm, 1, cfg["rms_eps"], ly.wgate,
+                                                                  ly.wup, y.ptr, F, D)
+        n_variants = L
+        name, shape = "norm_gate_up_swiglu_kernel", f"M=1 N=2x{F} K={D}"
+        bytes_per_launch = 2 * F * D * 2 + 2 * D * 4 + F * 4      # two matrices + x + norm weights in, hidden out
+    else:
+        mats = []
+        for l in range(L):
+            mats.append(dm.layers[l].wgate); mats.append(dm.layers[l].wup)
+
+        def launch(i):
+            return lib.m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx.h, x.ptr, mats[i], y.ptr, 1, F, D, 1)
+        n_variants = len(mats)
+        name, shape = "gemv_f32xf16_gguf_kernel", f"M=1 N={F} K={D}"
+        bytes_per_launch = F * D * 2 + D * 4 + F * 4              # weights + activations in + out
+    for i in range(n_variants):      # warm-up: code objects, clocks
+        pkg.check(launch(i), name)
     ctx.sync(1)
     e0, e1 = ctx.event(), ctx.event()
     ctx.record(e0, 1)
     n = 0
     for r in range(reps):
-        for mptr in mats:
-            lib.m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx.h, x.ptr, mptr, y.ptr, 1, F, D, 1)
+        for i in range(n_variants):
+            launch(i)
             n += 1
     ctx.record(e1, 1)
     ms = ctx.elapsed_ms(e0, e1)
     ctx.event_destroy(e0); ctx.event_destroy(e1)
-    avg_us = ms * 1e3 / n
-    bytes_per_launch = F * D * 2 + D * 4 + F * 4      # weights + activations in + out
-    return dict(kernel="gemv_f32xf16_gguf_kernel", shape=f"M=1 N={F} K={D}", launches=n, avg_us=avg_us,
-                bytes=bytes_per_launch)
+    return dict(kernel=name, shape=shape, launches=n, avg_us=ms * 1e3 / n, bytes=bytes_per_launch)
 
 
 def cpu_baseline(cfg, W, steps, threads):
@@ -123,7 +136,7 @@ def main():
     tok_s = args.steps / (elapsed_ms / 1e3)
     ms_per_step = elapsed_ms / args.steps
 
-    dom = measure_dominant_kernel(pkg, ctx, dm, cfg, args.kernel_reps)
+    dom = measure_dominant_kernel(pkg, ctx, dm, cfg, args.kernel_reps, mode)
     achieved = dom["bytes"] / (dom["avg_us"] * 1e-6) / 1e9
     token_bytes = algorithmic_bytes_per_token(cfg)
     out = {

@@ -223,13 +223,15 @@ __device__ __noinline__ static float2 m40_rope_cos_sin(uint32_t position, uint32
     const float theta = pos * inv_freq;
     return make_float2(cosf(theta), sinf(theta));
 }
-__device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off, uint32_t head_dim,
-                                                float base, float scale, float x0, float x1,
-                                                float* y0, float* y1) {
-    const float2 cs = m40_rope_cos_sin(position, off, head_dim, base, scale);
+__device__ __forceinline__ void m40_rope_apply(float2 cs, float x0, float x1, float* y0, float* y1) {
     // explicit fused multiply-adds: the same rounding in every kernel that inlines this rotation
     *y0 = fmaf(x0, cs.x, -(x1 * cs.y));
     *y1 = fmaf(x0, cs.y, x1 * cs.x);
+}
+__device__ __forceinline__ void m40_rope_rotate(uint32_t position, uint32_t off, uint32_t head_dim,
+                                                float base, float scale, float x0, float x1,
+                                                float* y0, float* y1) {
+    m40_rope_apply(m40_rope_cos_sin(position, off, head_dim, base, scale), x0, x1, y0, y1);
 }
 
 // q4 V pair, two's-complement nibbles, even dim in the low nibble

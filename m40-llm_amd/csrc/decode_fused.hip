@@ -101,16 +101,19 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
     // weights are requested first; the norm prologue runs while they are in flight
     GemvRegs<2> regs;
     gemv_prefetch<2>(bp, 0, K >> 3, lane, regs);
+    // the rotation angle does not depend on the data: evaluated while the weights are in flight
+    const uint32_t position = p.position_dev ? *p.position_dev : p.position;
+    float2 cs = make_float2(1.0f, 0.0f);
+    if (which != 2) cs = m40_rope_cos_sin(position, off, p.head_dim, p.rope_base, p.rope_scale);
     stage_normed(p.x, p.norm_w, p.norm_dtype, p.eps, K, a_lds, wave_sums);
     float d[2];
     gemv_accumulate<2>(bp, a_lds, 0, K >> 3, lane, regs, d);
     gemv_finish<2, 1>(d, nullptr, wave, lane);
     if (!live || lane != 0) return;
-    const uint32_t position = p.position_dev ? *p.position_dev : p.position;
     if (position >= p.max_seq_len) return;
     float y0 = d[0], y1 = d[1];
     if (bias) { y0 = y0 + bias[i0]; y1 = y1 + bias[i1]; }
-    if (which != 2) m40_rope_rotate(position, off, p.head_dim, p.rope_base, p.rope_scale, y0, y1, &y0, &y1);
+    if (which != 2) m40_rope_apply(cs, y0, y1, &y0, &y1);
     if (which == 0) {
         p.q_out[i0] = y0;
         p.q_out[i1] = y1;

@@ -1,0 +1,204 @@
+"""Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
+
+    python m40-llm_amd/kernel_bench.py [--only attn,gemv,gemm8,q80,bsel] [--json out.jsonl]
+
+Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
+events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
+distinct buffers that no launch finds its operands in a cache left warm by the previous one (a decode
+step never re-reads a weight or a KV row within a token).  "GB/s" is algorithmic bytes (the minimum
+traffic of the operation) divided by the average launch time; "frac" is that over 8 TB/s.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+m40 = importlib.import_module("m40-llm_amd")
+
+PEAK_GBS = 8000.0
+
+
+class Bench:
+    def __init__(self):
+        self.ctx = m40.Context(0)
+        self.lib = self.ctx.lib
+        self.h = self.ctx.h
+        self.rows = []
+        self.e0, self.e1 = self.ctx.event(), self.ctx.event()
+
+    def call(self, name, *args):
+        rc = getattr(self.lib, name)(self.h, *args)
+        if rc != 0:
+            raise m40.M40Error(name, rc)
+
+    def time(self, name, shape, algo_bytes, launch, n_variants, stream=1, reps=None, warm=None):
+        """launch(i) enqueues one launch on variant i; returns microseconds per launch."""
+        reps = reps or max(2 * n_variants, 64)
+        warm = warm or max(n_variants, 8)
+        for i in range(warm):
+            launch(i % n_variants)
+        self.ctx.sync(0); self.ctx.sync(1)
+        self.ctx.record(self.e0, stream)
+        for i in range(reps):
+            launch(i % n_variants)
+        self.ctx.record(self.e1, stream)
+        ms = self.ctx.elapsed_ms(self.e0, self.e1)
+        us = ms * 1e3 / reps
+        gbs = algo_bytes / us / 1e3
+        row = dict(kernel=name, shape=shape, us_per_launch=round(us, 3), algorithmic_bytes=int(algo_bytes),
+                   gbs=round(gbs, 1), frac=round(gbs / PEAK_GBS, 4), launches=reps, buffers=n_variants)
+        self.rows.append(row)
+        print(f"{name:34s} {shape:44s} {us:9.2f} us {gbs:8.1f} GB/s  frac {gbs / PEAK_GBS:6.3f}", flush=True)
+        return us
+
+
+def f16(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32).astype(np.float16).view(np.uint16))
+
+
+def n_rot(nbytes, budget=3 << 30, cap=64):
+    return int(max(2, min(cap, budget // max(nbytes, 1))))
+
+
+def bench_attention(b: Bench):
+    rng = np.random.default_rng(0)
+    # dense last-token GQA attention: config 1 shape, and the same heads at longer contexts
+    for qh, kvh, hd, L in ((32, 4, 64, 128), (32, 4, 64, 512), (32, 4, 64, 4096), (16, 2, 128, 4096), (32, 8, 128, 32768)):
+        kv_bytes = L * kvh * hd * 2 * 2
+        nseq = n_rot(kv_bytes, budget=2 << 30, cap=32)
+        kv = m40.KVCache(b.ctx, L, nseq, kvh, hd)
+        k = f16(rng.standard_normal((L, kvh, hd))); v = f16(rng.standard_normal((L, kvh, hd)))
+        dk, dv = b.ctx.to_device(k), b.ctx.to_device(v)
+        for s in range(nseq):
+            b.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, s, dk.ptr, dv.ptr, L)
+        q = b.ctx.to_device(rng.standard_normal(qh * hd).astype(np.float32))
+        out = b.ctx.alloc(qh * hd * 4)
+        algo = kv_bytes + 2 * qh * hd * 4
+        b.time("attention_last_token_gqa", f"qh{qh} kvh{kvh} hd{hd} L{L}", algo,
+               lambda i: b.call("m40llm_attention_last_token_f32_gqa_async", kv.h, i, q.ptr, qh, L, out.ptr), nseq)
+        kv.destroy()
+    # row-batched variable-length attention: config 3 shape
+    qh, kvh, hd, B, maxL = 16, 2, 128, 8, 4160
+    lens = rng.integers(256, 4097, size=B).astype(np.uint32)
+    nset = 4
+    kv = m40.KVCache(b.ctx, maxL, B * nset, kvh, hd)
+    k = f16(rng.standard_normal((maxL, kvh, hd))); dk = b.ctx.to_device(k)
+    for s in range(B * nset):
+        b.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, s, dk.ptr, dk.ptr, int(lens[s % B]))
+    q = b.ctx.to_device(rng.standard_normal((B, qh * hd)).astype(np.float32))
+    out = b.ctx.alloc(B * qh * hd * 4)
+    dl = b.ctx.to_device(lens)
+    ids = [b.ctx.to_device((np.arange(B) + B * i).astype(np.uint32)) for i in range(nset)]
+    algo = int(lens.sum()) * kvh * hd * 2 * 2 + 2 * B * qh * hd * 4
+    b.time("attention_gqa_batched", f"B8 qh16 kvh2 hd128 lens U[256,4096] sum {int(lens.sum())}", algo,
+           lambda i: b.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, ids[i].ptr, dl.ptr, B, q.ptr, qh,
+                            out.ptr), nset)
+    kv.destroy()
+
+
+def bench_gemv(b: Bench, M: int):
+    rng = np.random.default_rng(1)
+    shapes = [(2048, 2048), (256, 2048), (5632, 2048), (2048, 5632), (32000, 2048)] if M == 1 else \
+             [(2048, 2048), (256, 2048), (11008, 2048), (2048, 11008), (151936, 2048)]
+    for N, K in shapes:
+        wbytes = N * K * 2
+        nb = n_rot(wbytes, budget=3 << 30, cap=48)
+        w = f16(rng.standard_normal((N, K)) * 0.02)
+        bufs = [b.ctx.to_device(w) for _ in range(nb)]
+        a = b.ctx.to_device(rng.standard_normal((M, K)).astype(np.float32))
+        c = b.ctx.alloc(M * N * 4)
+        algo = wbytes + M * K * 4 + M * N * 4
+        b.time(f"gemm_f32xf16_gguf M={M}", f"N={N} K={K}", algo,
+               lambda i: b.call("m40llm_ext_gemm_f32xf16_gguf_f32_async", a.ptr, bufs[i].ptr, c.ptr, M, N, K, 1), nb)
+        for x in bufs:
+            x.free()
+
+
+def bench_q80(b: Bench):
+    rng = np.random.default_rng(2)
+    d_model, ffn = 4096, 14336
+
+    def q80(n, k):
+        blocks = n * k // 32
+        raw = np.zeros((blocks, 34), dtype=np.uint8)
+        raw[:, :2] = rng.uniform(0.001, 0.01, blocks).astype(np.float16).view(np.uint8).reshape(blocks, 2)
+        raw[:, 2:] = rng.integers(-127, 128, size=(blocks, 32)).astype(np.int8).view(np.uint8)
+        return raw
+    gate, up, down = q80(ffn, d_model), q80(ffn, d_model), q80(d_model, ffn)
+    nset = 6
+    sets = [(b.ctx.to_device(gate), b.ctx.to_device(up), b.ctx.to_device(down)) for _ in range(nset)]
+    wbytes = gate.nbytes + up.nbytes + down.nbytes
+    for M in (1, 4, 16):
+        x = b.ctx.to_device(rng.standard_normal((M, d_model)).astype(np.float32))
+        scratch = b.ctx.alloc(2 * M * ffn * 4)
+        out = b.ctx.alloc(M * d_model * 4)
+        algo = wbytes + M * (d_model * 4 * 2)
+        b.time("ffn_swiglu_q80", f"M={M} d_model 4096 ffn 14336", algo,
+               lambda i: b.call("m40llm_ext_ffn_swiglu_q80_f32_async", x.ptr, sets[i][0].ptr, sets[i][1].ptr, sets[i][2].ptr,
+                                scratch.ptr, out.ptr, M, d_model, ffn), nset)
+    a = b.ctx.to_device(rng.standard_normal((1, d_model)).astype(np.float32))
+    c = b.ctx.alloc(ffn * 4)
+    b.time("gemm_f32xq80_gguf M=1", "N=14336 K=4096", gate.nbytes,
+           lambda i: b.call("m40llm_ext_gemm_f32xq80_gguf_f32", a.ptr, sets[i][0].ptr, c.ptr, 1, ffn, d_model), nset, stream=0)
+
+
+def bench_block_select(b: Bench):
+    rng = np.random.default_rng(3)
+    qh, kvh, hd, L, bs, top, W = 32, 8, 128, 32768, 64, 64, 512
+    nseq = 4
+    kv = m40.KVCache(b.ctx, L, nseq, kvh, hd, compressed=dict(recent_window=W, block_size=bs, top_blocks=top))
+    for s in range(nseq):
+        k = f16(rng.standard_normal((L, kvh, hd))); v = f16(rng.standard_normal((L, kvh, hd)))
+        dk, dv = b.ctx.to_device(k), b.ctx.to_device(v)
+        b.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, s, dk.ptr, dv.ptr, L)
+        dk.free(); dv.free()
+    q = b.ctx.to_device(rng.standard_normal(qh * hd).astype(np.float32))
+    out = b.ctx.alloc(qh * hd * 4)
+    old = L - W
+    score = old * kvh * hd * 2
+    attend = qh * (top * bs * hd * 2 + W * hd * 2 + top * bs * (hd // 2 + 4) + W * hd * 2)
+    algo = score + attend
+    name = "m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async"
+    b.time("block_select fp16-K/q4-V, B=1", f"qh32 kvh8 hd128 L32768 bs64 top64 W512", algo,
+           lambda i: b.call(name, kv.h, i, q.ptr, qh, L, W, bs, top, out.ptr), nseq)
+
+    def four(i):
+        for s in range(nseq):
+            b.call(name, kv.h, s, q.ptr, qh, L, W, bs, top, out.ptr)
+    b.time("block_select fp16-K/q4-V, B=4", "4 slots per step", 4 * algo, four, 1, reps=16, warm=2)
+    kv.destroy()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--only", default="attn,gemv,gemm8,q80,bsel")
+    ap.add_argument("--json", default=None)
+    args = ap.parse_args()
+    which = set(args.only.split(","))
+    b = Bench()
+    print(b.lib.m40llm_ext_build_info().decode() if hasattr(b.lib, "m40llm_ext_build_info") else "")
+    if "attn" in which:
+        bench_attention(b)
+    if "gemv" in which:
+        bench_gemv(b, 1)
+    if "gemm8" in which:
+        bench_gemv(b, 8)
+    if "q80" in which:
+        bench_q80(b)
+    if "bsel" in which:
+        bench_block_select(b)
+    if args.json:
+        with open(args.json, "w") as f:
+            for r in b.rows:
+                f.write(json.dumps(r) + "\n")
+
+
+if __name__ == "__main__":
+    main()
