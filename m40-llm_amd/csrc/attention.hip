@@ -1,11 +1,12 @@
 // Last-token GQA attention over the dense f16 KV cache for gfx950 (single sequence, device
 // length, recent-window and variable-length batched forms share one kernel).
 //
-// Work split: grid = (kv_head x q-head subgroup, token chunk, batch row).  A workgroup streams its
-// chunk of K and V exactly once with 128-bit loads and serves every q head of the GQA group
-// from it, so K/V traffic is 1/group of a per-q-head kernel.  Per chunk it produces the
-// softmax partial (max, sum, weighted V); a small second kernel merges chunks in ascending
-// order.  With a single chunk the first kernel writes the final output itself.
+// Work split: grid = (kv_head x q-head subgroup, token chunk, batch row).  A workgroup of eight waves
+// owns a chunk of 8 * TPW * S token rows (TPW = rows per 64-lane load: 8 at head_dim 64, 4 at 128).
+// Every lane issues all of its S K-row and S V-row 128-bit loads before any arithmetic, so a chunk
+// costs one memory round trip; the rows serve all G q heads of the subgroup.  Scores stay in
+// registers.  With one chunk the kernel writes the output; otherwise it writes the softmax partial
+// (max, sum, weighted V) and a second kernel merges the chunks in ascending order.
 //
 // Reference semantics: three-pass softmax per q head, kv head = qh / (q_heads / kv_heads),
 // scale literals for head_dim 64 / 128: cuda/kernels.cu:1367-1655, entry points :3837-4023,
@@ -14,7 +15,7 @@
 
 namespace {
 
-constexpr int kAttnThreads = 256;
+constexpr int kAttnThreads = 512;
 constexpr int kWaves = kAttnThreads / 64;
 
 struct AttnParams {
@@ -32,16 +33,14 @@ struct AttnParams {
     uint32_t len_bias;            // added to a device-side length (position -> length)
 };
 
-// HD in {64, 128}; G = q heads handled per workgroup (<= 8)
-template <int HD, int G>
-__global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p) {
+// HD in {64, 128}; G = q heads per workgroup (<= 4); S = token rows per lane group
+template <int HD, int G, int S>
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_partial_kernel(AttnParams p) {
     constexpr int LPT = HD / 8;      // lanes per token row
-    constexpr int TPW = 64 / LPT;    // token rows per wave step
-    extern __shared__ float lds[];
-    float* sc = lds;                              // [G][chunk]
-    float* red = sc + (size_t)G * p.chunk;        // [kWaves][G][HD]
-    float* wmax = red + (size_t)kWaves * G * HD;  // [kWaves][G]
-    float* wsum = wmax + kWaves * G;              // [kWaves][G]
+    constexpr int TPW = 64 / LPT;    // token rows per wave load
+    __shared__ float red[kWaves][G][HD];
+    __shared__ float wmax[kWaves][G];
+    __shared__ float wsum[kWaves][G];
 
     const uint32_t b = blockIdx.z;
     const uint32_t seq_id = p.seq_ids_dev ? p.seq_ids_dev[b] : p.seq_id;
@@ -61,11 +60,25 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int c = lane % LPT, tg = lane / LPT;
     const size_t row_stride = (size_t)p.kv_heads * HD;
-    const uint16_t* Kb = p.K + ((size_t)seq_id * p.max_seq_len) * row_stride + (size_t)kvh * HD + 8 * c;
-    const uint16_t* Vb = p.V + ((size_t)seq_id * p.max_seq_len) * row_stride + (size_t)kvh * HD + 8 * c;
+    const size_t base = ((size_t)seq_id * p.max_seq_len) * row_stride + (size_t)kvh * HD + 8 * c;
+    const uint16_t* Kb = p.K + base;
+    const uint16_t* Vb = p.V + base;
     const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
 
-    // q slice of this lane for every head of the subgroup
+    // every load of this lane, issued before anything waits on memory
+    uint4 kw[S], vw[S];
+    bool valid[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const uint32_t t = cbeg + (uint32_t)((s * kWaves + wave) * TPW + tg);
+        valid[s] = t < cend;
+        kw[s] = make_uint4(0, 0, 0, 0);
+        vw[s] = make_uint4(0, 0, 0, 0);
+        if (valid[s]) {
+            kw[s] = *reinterpret_cast<const uint4*>(Kb + (size_t)t * row_stride);
+            vw[s] = *reinterpret_cast<const uint4*>(Vb + (size_t)t * row_stride);
+        }
+    }
     float q[G][8];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
@@ -77,93 +90,64 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
         q[h][4] = q1.x; q[h][5] = q1.y; q[h][6] = q1.z; q[h][7] = q1.w;
     }
 
-    // Token rows of the chunk are dealt to the waves in groups of TPW, round robin, so that every wave
-    // works on real tokens whatever the length: group gi = it * kWaves + wave covers rows gi*TPW .. +TPW-1.
-    const uint32_t n_tok = cend - cbeg;
-    const uint32_t n_groups = (n_tok + TPW - 1) / TPW;
-
-    // ---- pass A: scores ---------------------------------------------------------------
+    // ---- scores (every lane of a row group ends up with the row's score) -----------------------
+    float sc[S][G];
     float lmax[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) lmax[h] = -INFINITY;
-#pragma unroll 2
-    for (uint32_t gi = wave; gi < n_groups; gi += kWaves) {
-        const uint32_t tl = gi * TPW + tg;
-        const uint32_t t = cbeg + tl;
-        const bool valid = tl < n_tok;
-        uint4 kw = make_uint4(0, 0, 0, 0);
-        if (valid) kw = *reinterpret_cast<const uint4*>(Kb + (size_t)t * row_stride);
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
         float kf[8];
-        m40_unpack8(kw, kf);
+        m40_unpack8(kw[s], kf);
 #pragma unroll
         for (int h = 0; h < G; ++h) {
             float d = 0.0f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) d = fmaf(q[h][j], kf[j], d);
             d = LPT == 8 ? m40_sum8(d) : m40_sum16(d);
-            const float s = valid ? d * inv_sqrt : -INFINITY;
-            lmax[h] = fmaxf(lmax[h], s);
-            if (c == 0 && valid) sc[h * p.chunk + tl] = s;
+            sc[s][h] = valid[s] ? d * inv_sqrt : -INFINITY;
+            lmax[h] = fmaxf(lmax[h], sc[s][h]);
         }
     }
 #pragma unroll
     for (int h = 0; h < G; ++h) {
         const float m = m40_max64(lmax[h]);
-        if (lane == 0) wmax[wave * G + h] = m;
+        if (lane == 0) wmax[wave][h] = m;
     }
     __syncthreads();
     float mh[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-        float m = wmax[h];
+        float m = wmax[0][h];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, wmax[w * G + h]);
+        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, wmax[w][h]);
         mh[h] = m;
     }
 
-    // ---- pass B0: p = exp(s - max), row sums ---------------------------------------------
+    // ---- exp, row sums, weighted V -----------------------------------------------------------
     float lsum[G];
-#pragma unroll
-    for (int h = 0; h < G; ++h) lsum[h] = 0.0f;
-    for (uint32_t tl = tid; tl < n_tok; tl += kAttnThreads) {
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-            const float e = expf(sc[h * p.chunk + tl] - mh[h]);
-            sc[h * p.chunk + tl] = e;
-            lsum[h] += e;
-        }
-    }
-#pragma unroll
-    for (int h = 0; h < G; ++h) {
-        const float s = m40_sum64(lsum[h]);
-        if (lane == 0) wsum[wave * G + h] = s;
-    }
-    __syncthreads();
-
-    // ---- pass B: weighted V -----------------------------------------------------------------
     float acc[G][8];
 #pragma unroll
-    for (int h = 0; h < G; ++h)
+    for (int h = 0; h < G; ++h) {
+        lsum[h] = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[h][j] = 0.0f;
-#pragma unroll 2
-    for (uint32_t gi = wave; gi < n_groups; gi += kWaves) {
-        const uint32_t tl = gi * TPW + tg;
-        if (tl < n_tok) {
-            const uint4 vw = *reinterpret_cast<const uint4*>(Vb + (size_t)(cbeg + tl) * row_stride);
-            float vf[8];
-            m40_unpack8(vw, vf);
+    }
 #pragma unroll
-            for (int h = 0; h < G; ++h) {
-                const float pw = sc[h * p.chunk + tl];
+    for (int s = 0; s < S; ++s) {
+        float vf[8];
+        m40_unpack8(vw[s], vf);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc[h][j] = fmaf(pw, vf[j], acc[h][j]);
-            }
+        for (int h = 0; h < G; ++h) {
+            const float e = valid[s] ? expf(sc[s][h] - mh[h]) : 0.0f;
+            if (c == 0) lsum[h] += e;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[h][j] = fmaf(e, vf[j], acc[h][j]);
         }
     }
     // join the TPW token rows of the wave (lanes with equal c), then the waves
 #pragma unroll
-    for (int h = 0; h < G; ++h)
+    for (int h = 0; h < G; ++h) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             float v = acc[h][j];
@@ -171,11 +155,14 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
             for (int o = LPT; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
             acc[h][j] = v;
         }
+        const float ssum = m40_sum64(lsum[h]);
+        if (lane == 0) wsum[wave][h] = ssum;
+    }
     if (tg == 0) {
 #pragma unroll
         for (int h = 0; h < G; ++h)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) red[((size_t)wave * G + h) * HD + 8 * c + j] = acc[h][j];
+            for (int j = 0; j < 8; ++j) red[wave][h][8 * c + j] = acc[h][j];
     }
     __syncthreads();
 
@@ -185,8 +172,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
         float v = 0.0f, l = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            v += red[((size_t)w * G + h) * HD + d];
-            l += wsum[w * G + h];
+            v += red[w][h][d];
+            l += wsum[w][h];
         }
         const uint32_t qh = qh0 + h;
         if (final_out) {
@@ -203,26 +190,49 @@ __global__ __launch_bounds__(kAttnThreads) void attn_partial_kernel(AttnParams p
     }
 }
 
-// Merge chunk partials in ascending chunk order: grid (q_heads, batch), HD threads.
+// Merge chunk partials: grid (q_heads, batch), 256 threads = 256/HD chunk lanes x HD dims.  Each chunk lane
+// folds chunks lane, lane + n_lanes, ... with a running maximum; the chunk lanes are then folded in order.
 template <int HD>
-__global__ __launch_bounds__(HD) void attn_combine_kernel(AttnParams p) {
-    const uint32_t qh = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+__global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
+    constexpr int NCG = 256 / HD;
+    __shared__ float s_m[NCG], s_den[NCG];
+    __shared__ float s_num[NCG][HD];
+    const uint32_t qh = blockIdx.x, b = blockIdx.y;
+    const uint32_t d = threadIdx.x % HD, cg = threadIdx.x / HD;
     const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t n = (len - t0 + p.chunk - 1) / p.chunk;
     const float* w = p.ws + (((size_t)b * p.q_heads + qh) * p.nchunks) * (HD + 2);
-    float M = -INFINITY;
-    for (uint32_t c = 0; c < n; ++c) M = fmaxf(M, w[(size_t)c * (HD + 2)]);
-    float num = 0.0f, den = 0.0f;
-    for (uint32_t c = 0; c < n; ++c) {
-        const float* wc = w + (size_t)c * (HD + 2);
-        const float f = expf(wc[0] - M);
-        num = fmaf(wc[2 + d], f, num);
-        den = fmaf(wc[1], f, den);
+    float m = -INFINITY, num = 0.0f, den = 0.0f;
+#pragma unroll 4
+    for (uint32_t ch = cg; ch < n; ch += NCG) {
+        const float* wc = w + (size_t)ch * (HD + 2);
+        const float mc = wc[0], lc = wc[1], vc = wc[2 + d];
+        const float nm = fmaxf(m, mc);
+        const float fa = m == -INFINITY ? 0.0f : expf(m - nm);
+        const float fb = mc == -INFINITY ? 0.0f : expf(mc - nm);
+        num = fmaf(num, fa, vc * fb);
+        den = fmaf(den, fa, lc * fb);
+        m = nm;
     }
-    den = den > 0.0f ? den : 1.0f;
-    p.Out[((size_t)b * p.q_heads + qh) * HD + d] = num / den;
+    s_num[cg][d] = num;
+    if (d == 0) { s_m[cg] = m; s_den[cg] = den; }
+    __syncthreads();
+    if (cg == 0) {
+#pragma unroll
+        for (int g = 1; g < NCG; ++g) {
+            const float mc = s_m[g];
+            const float nm = fmaxf(m, mc);
+            const float fa = m == -INFINITY ? 0.0f : expf(m - nm);
+            const float fb = mc == -INFINITY ? 0.0f : expf(mc - nm);
+            num = fmaf(num, fa, s_num[g][d] * fb);
+            den = fmaf(den, fa, s_den[g] * fb);
+            m = nm;
+        }
+        den = den > 0.0f ? den : 1.0f;
+        p.Out[((size_t)b * p.q_heads + qh) * HD + d] = num / den;
+    }
 }
 
 // Any head_dim: one thread per output element, the reference's three passes verbatim
@@ -259,34 +269,65 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p, uint32_t
     p.Out[((size_t)b * p.q_heads + qh) * head_dim + d] = acc / den;
 }
 
-template <int HD, int G>
-int launch_partial(hipStream_t stream, const AttnParams& p, uint32_t batch) {
-    const size_t lds = ((size_t)G * p.chunk + (size_t)kWaves * G * HD + 2 * kWaves * G) * sizeof(float);
+template <int HD, int G, int S>
+void launch_partial(hipStream_t stream, const AttnParams& p, uint32_t batch) {
     dim3 grid(p.kv_heads * p.subgroups, p.nchunks, batch);
-    attn_partial_kernel<HD, G><<<grid, kAttnThreads, lds, stream>>>(p);
-    return 0;
+    attn_partial_kernel<HD, G, S><<<grid, kAttnThreads, 0, stream>>>(p);
 }
 
+template <int HD, int G>
+void launch_g(hipStream_t stream, const AttnParams& p, uint32_t batch, int S) {
+    switch (S) {
+        case 8: launch_partial<HD, G, 8>(stream, p, batch); break;
+        case 4: launch_partial<HD, G, 4>(stream, p, batch); break;
+        case 2: launch_partial<HD, G, 2>(stream, p, batch); break;
+        default: launch_partial<HD, G, 1>(stream, p, batch); break;
+    }
+}
+
+// Chooses rows per lane group (S), q heads per workgroup (G) and the chunking for a span of `span` tokens.
 template <int HD>
-int launch_hd(hipStream_t stream, AttnParams& p, uint32_t batch, uint32_t group, uint32_t span) {
-    int G = group >= 8 ? 8 : (group >= 4 ? 4 : (group >= 2 ? 2 : 1));
+int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, AttnParams& p, uint32_t batch,
+              uint32_t group, uint32_t span) {
+    constexpr uint32_t kRowsPerStep = kWaves * (64 / (HD / 8));   // token rows one workgroup covers per S
+    int G = group >= 4 ? 4 : (group >= 2 ? 2 : 1);
+    const uint64_t rows = (uint64_t)batch * p.kv_heads;
     // Short rows are latency-bound, not bandwidth-bound: spread the q heads over more workgroups
     // (K/V of a short row stay in L2, so re-reading them per head pair costs nothing).
-    if (span <= 1024 && (uint64_t)batch * p.kv_heads * p.nchunks < 64) G = G > 2 ? 2 : G;
-    if (group % G != 0) {
-        // uneven group sizes (3, 5, 6, 7...) run with the largest subgroup that fits
-        G = group >= 8 ? 8 : (group > 4 ? 8 : (group > 2 ? 4 : 2));
-    }
+    if (span <= 1024 && rows * ((group + G - 1) / G) < 64 && G > 2) G = 2;
     p.subgroups = (group + G - 1) / G;
+    int S = 8;
+    if (span <= kRowsPerStep * 8) {
+        // one chunk, no merge launch: the smallest S that covers the span
+        S = 1;
+        while ((uint32_t)S * kRowsPerStep < span) S <<= 1;
+    } else {
+        // split until the grid covers the CUs about twice
+        while (S > 2 && rows * p.subgroups * ((span + kRowsPerStep * S - 1) / (kRowsPerStep * S)) < 2u * (uint32_t)ctx->num_cus)
+            S >>= 1;
+    }
+    p.chunk = kRowsPerStep * (uint32_t)S;
+    p.nchunks = (span + p.chunk - 1) / p.chunk;
+    M40StreamScratch& sc = ctx->scratch[stream_kind];
+    if (p.nchunks > 1) {
+        const size_t need = (size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float);
+        if (need > sc.attn_partial_bytes) {
+            if (S == 8) return -7;
+            S = 8;
+            p.chunk = kRowsPerStep * 8u;
+            p.nchunks = (span + p.chunk - 1) / p.chunk;
+            if ((size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float) > sc.attn_partial_bytes) return -7;
+        }
+    }
+    p.ws = static_cast<float*>(sc.attn_partial);
     switch (G) {
-        case 8: launch_partial<HD, 8>(stream, p, batch); break;
-        case 4: launch_partial<HD, 4>(stream, p, batch); break;
-        case 2: launch_partial<HD, 2>(stream, p, batch); break;
-        default: launch_partial<HD, 1>(stream, p, batch); break;
+        case 4: launch_g<HD, 4>(stream, p, batch, S); break;
+        case 2: launch_g<HD, 2>(stream, p, batch, S); break;
+        default: launch_g<HD, 1>(stream, p, batch, S); break;
     }
     if (p.nchunks > 1) {
         dim3 grid(p.q_heads, batch);
-        attn_combine_kernel<HD><<<grid, HD, 0, stream>>>(p);
+        attn_combine_kernel<HD><<<grid, 256, 0, stream>>>(p);
     }
     return 0;
 }
@@ -309,27 +350,9 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
     if (span == 0) span = 1;
 
     if ((a.head_dim == 64 || a.head_dim == 128) && m40_aligned16(a.Q) && m40_aligned16(a.K) && m40_aligned16(a.V)) {
-        // chunk: small when there is little work so that more CUs take part; the per-row
-        // partial buffer bounds the chunk count.
-        // Up to 512 tokens a single chunk per kv head finishes in a few microseconds and needs no
-        // merge launch; longer rows are split until the grid covers the CUs about twice.
-        const uint64_t rows = (uint64_t)a.batch * a.kv_heads;
-        uint32_t chunk = 512;
-        if (span > 512) {
-            while (chunk > 64 && rows * ((span + chunk - 1) / chunk) < 2u * (uint32_t)ctx->num_cus) chunk >>= 1;
-        }
-        M40StreamScratch& sc = ctx->scratch[stream_kind];
-        for (;;) {
-            p.chunk = chunk;
-            p.nchunks = (span + chunk - 1) / chunk;
-            const size_t need = (size_t)a.batch * a.q_heads * p.nchunks * (a.head_dim + 2) * sizeof(float);
-            if (p.nchunks == 1 || need <= sc.attn_partial_bytes) break;
-            if (chunk >= 1024) return -7;   // LDS holds G x chunk scores
-            chunk <<= 1;
-        }
-        p.ws = static_cast<float*>(sc.attn_partial);
-        if (a.head_dim == 64) launch_hd<64>(stream, p, a.batch, group, span);
-        else launch_hd<128>(stream, p, a.batch, group, span);
+        const int rc = a.head_dim == 64 ? launch_hd<64>(ctx, stream, stream_kind, p, a.batch, group, span)
+                                        : launch_hd<128>(ctx, stream, stream_kind, p, a.batch, group, span);
+        if (rc != 0) return rc;
     } else {
         p.chunk = span; p.nchunks = 1;
         dim3 grid((a.head_dim + 63) / 64, a.q_heads, a.batch);
