@@ -93,6 +93,11 @@ M40_HD static inline bool m40_aligned16(const void* p) { return (reinterpret_cas
 // GEMM family (gemm.hip)
 int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
                                  const float* A, const uint16_t* B, float* C, int M, int N, int K);
+// skinny MFMA GEMM (skinny_mfma.hip): fmt 0 = f16 GGUF weights, 1 = q8_0 blocks.  `up` != null multiplies
+// silu(A) by it while packing; W1/C1 give an optional second matrix of the same shape.
+bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
+int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
+                      const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);
 // attention over an explicit dense range (attention.hip)
 struct M40AttnArgs {
     const uint16_t* K;       // base of the cache (sequence 0)

@@ -303,6 +303,8 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
         else if (g.cols == 4) gemv_f32xf16_gguf_kernel<4, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else if (g.cols == 2) gemv_f32xf16_gguf_kernel<2, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else gemv_f32xf16_gguf_kernel<1, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
+    } else if (fast && m40_skinny_supported(ctx, stream_kind, M, N, K, 0)) {
+        return m40_launch_skinny(ctx, stream, stream_kind, 0, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     } else if (fast && K % 64 == 0 && (size_t)K * 64 <= ctx->scratch[stream_kind].gemm_pack_bytes - 256) {
         M40StreamScratch& sc = ctx->scratch[stream_kind];
         const int KT = K >> 6;
@@ -334,7 +336,10 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
-static int launch_q80(hipStream_t stream, const float* A, const uint8_t* B, float* C, int M, int N, int K) {
+static int launch_q80(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint8_t* B,
+                      float* C, int M, int N, int K) {
+    if (m40_aligned16(B) && m40_skinny_supported(ctx, stream_kind, M, N, K, 1))
+        return m40_launch_skinny(ctx, stream, stream_kind, 1, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     (void)hipGetLastError();
     for (int r0 = 0; r0 < M; r0 += 4) {
         const int m = M - r0;
@@ -410,7 +415,7 @@ int m40llm_ext_gemm_f32xq80_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32
                                      void* d_C_f32, int M, int N, int K) {
     if (!ctx || !d_A_f32 || !d_B_q80 || !d_C_f32) return -1;
     if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return -2;
-    int rc = launch_q80(ctx->prefill_stream, static_cast<const float*>(d_A_f32),
+    int rc = launch_q80(ctx, ctx->prefill_stream, 0, static_cast<const float*>(d_A_f32),
                         static_cast<const uint8_t*>(d_B_q80), static_cast<float*>(d_C_f32), M, N, K);
     if (rc != 0) return rc;
     return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
@@ -425,14 +430,24 @@ int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_
     float* gate = static_cast<float*>(d_scratch_f32);
     float* up = gate + (size_t)M * ffn;
     const float* x = static_cast<const float*>(d_x_f32);
-    int rc = launch_q80(ctx->decode_stream, x, static_cast<const uint8_t*>(d_w_gate_q80), gate, M, ffn, d_model);
+    const uint8_t* wg = static_cast<const uint8_t*>(d_w_gate_q80);
+    const uint8_t* wu = static_cast<const uint8_t*>(d_w_up_q80);
+    const uint8_t* wd = static_cast<const uint8_t*>(d_w_down_q80);
+    float* out = static_cast<float*>(d_out_f32);
+    if (m40_aligned16(wg) && m40_aligned16(wu) && m40_aligned16(wd) && m40_skinny_supported(ctx, 1, M, ffn, d_model, 1) &&
+        m40_skinny_supported(ctx, 1, M, d_model, ffn, 1)) {
+        // gate and up in one launch; SwiGLU is applied while the hidden row is packed for the down projection
+        int rc = m40_launch_skinny(ctx, ctx->decode_stream, 1, 1, x, nullptr, wg, gate, wu, up, M, ffn, d_model);
+        if (rc != 0) return rc;
+        return m40_launch_skinny(ctx, ctx->decode_stream, 1, 1, gate, up, wd, out, nullptr, nullptr, M, d_model, ffn);
+    }
+    int rc = launch_q80(ctx, ctx->decode_stream, 1, x, wg, gate, M, ffn, d_model);
     if (rc != 0) return rc;
-    rc = launch_q80(ctx->decode_stream, x, static_cast<const uint8_t*>(d_w_up_q80), up, M, ffn, d_model);
+    rc = launch_q80(ctx, ctx->decode_stream, 1, x, wu, up, M, ffn, d_model);
     if (rc != 0) return rc;
     rc = m40llm_swiglu_f32_async(ctx, gate, up, gate, (size_t)M * ffn);
     if (rc != 0) return -3;
-    return launch_q80(ctx->decode_stream, gate, static_cast<const uint8_t*>(d_w_down_q80),
-                      static_cast<float*>(d_out_f32), M, d_model, ffn);
+    return launch_q80(ctx, ctx->decode_stream, 1, gate, wd, out, M, d_model, ffn);
 }
 
 }  // extern "C"

@@ -283,6 +283,30 @@ def test_q80_gemm_and_ffn_vs_oracle(dev, orc, M):
     close(out.download(np.float32, (M, d_model)), want, 1e-3, 1e-4 * max(np.abs(want).max(), 1.0))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 1000, 768), (8, 4096, 2048), (9, 520, 1280), (16, 2048, 4096),
+                                   (20, 333, 256), (2, 64, 96)])
+def test_q80_gemm_shapes_vs_oracle(dev, orc, M, N, K):
+    """MFMA path (K % 256 == 0; column tails, split K, more than 16 rows) and the simple path (K = 96)."""
+    rng = np.random.default_rng(M * 7919 + N + K)
+    d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
+    qs = rng.integers(-127, 128, size=(N, K // 32, 32)).astype(np.int8)
+    qs[0, 0, :] = -127; qs[N - 1, -1, :] = 127; qs[N // 2, 0, ::2] = 0          # extremes of the int8 -> f16 step
+    W = np.ascontiguousarray(np.stack([_q80_pack(d[i], qs[i]) for i in range(N)]))
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    if M > 1:
+        A[1] *= 1e-3
+    if M > 2:
+        A[2] *= 3e4
+    dA, dW, dC = dev.up(A), dev.up(W), dev.zeros(M * N * 4)
+    dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dA.ptr, dW.ptr, dC.ptr, M, N, K)
+    got = dC.download(np.float32, (M, N))
+    want = orc.gemm("f32xq80_gguf", A, W, M, N, K)
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    close(got / scale, want / scale)
+    f64 = A.astype(np.float64) @ (d.astype(np.float64)[:, :, None] * qs.astype(np.float64)).reshape(N, K).T
+    close(got / scale, f64 / scale, 1e-4, 1e-5)
+
+
 # ------------------------------------------------------------------ dense attention
 def _attention_case(dev, orc, qh, kvh, hd, L, k, v, q, max_seq=None, seq=0, batch=1):
     max_seq = max_seq or L
