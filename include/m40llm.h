@@ -332,6 +332,41 @@ int m40llm_ext_embed_token_dev_async(M40llmCudaContext* ctx, const void* d_table
 int m40llm_ext_greedy_step_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t n,
                                  const void* d_block_top2, uint32_t top2_capacity, uint32_t n_blocks,
                                  uint32_t* state_dev, const void* d_table_f16, uint32_t d_model, void* d_x_out_f32);
+/* Fused row-batched decode step (1 <= rows <= 16, decode stream, asynchronous; dense caches, f16 weights, K a
+ * multiple of 256).  They compute what the reference's row-batched sequence computes (src/infer/forward.rs:1729-2140),
+ * several steps per call, on the MFMA skinny GEMM.  seq_lens_dev[row] is the number of tokens the row's cache holds
+ * before the step (= the position of the new token); ids and lengths are read on the device only.
+ *   RMSNorm -> Q/K/V projections (+bias) -> RoPE at each row's position -> q; K, V -> f16 cache rows */
+int m40llm_ext_batched_norm_qkv_rope_append_async(
+    M40llmCudaContext* ctx, M40llmKVCache* kv, const uint32_t* seq_ids_dev, const uint32_t* seq_lens_dev, uint32_t rows,
+    const void* d_x_f32, const void* d_norm_w, uint32_t norm_weight_dtype, float eps, const void* d_wq_f16,
+    const void* d_wk_f16, const void* d_wv_f16, const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32,
+    uint32_t d_model, uint32_t q_heads, float freq_base, float freq_scale, uint32_t rope_layout, void* d_q_out_f32);
+/*   attention of every row over seq_lens_dev[row] + len_bias tokens (no host-side validation: rows with an id or
+ *   length out of range are skipped); max_len_hint >= every row's length */
+int m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                                   const uint32_t* seq_ids_dev,
+                                                                   const uint32_t* seq_lens_dev, uint32_t len_bias,
+                                                                   uint32_t batch_size, uint32_t max_len_hint,
+                                                                   const void* q_dev_f32, uint32_t q_heads,
+                                                                   void* out_dev_f32);
+/*   out[rows][N] = residual + a[rows][K] . W^T (residual may be NULL or alias out) */
+int m40llm_ext_batched_gemm_residual_f32xf16_async(M40llmCudaContext* ctx, const void* d_a_f32, const void* d_w_f16,
+                                                   const void* d_residual_f32, void* d_out_f32, uint32_t rows, int N, int K);
+/*   hid[rows][ffn] = silu(gate(xn)) * up(xn), xn = RMSNorm(x) * w */
+int m40llm_ext_batched_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                                 uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
+                                                 const void* d_wup_f16, void* d_hid_f32, uint32_t rows, int ffn, int d_model);
+/*   out[rows][N] = (RMSNorm(x) * w) . W^T  (output norm + lm_head) */
+int m40llm_ext_batched_norm_gemm_f32xf16_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                               uint32_t norm_weight_dtype, float eps, const void* d_w_f16, void* d_out_f32,
+                                               uint32_t rows, int N, int K);
+/*   per row: first index of the maximum of logits[row][n] and the top-1/top-2 gap -> ids_dev/gaps_dev[row][step of the
+ *   row] (row stride = capacity); seq_lens_dev[row] += 1; embedding row of the pick -> d_x_out_f32[row].
+ *   state_dev = {unused, capacity, step of row 0, step of row 1, ...} */
+int m40llm_ext_batched_greedy_step_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t rows, uint32_t n,
+                                         uint32_t* state_dev, uint32_t* seq_lens_dev, uint32_t* ids_dev, float* gaps_dev,
+                                         const void* d_table_f16, uint32_t d_model, void* d_x_out_f32);
 const char* m40llm_ext_build_info(void);
 
 /* ---- present but unavailable (return -1, as cuda/stub.c does) ---------------------- */

@@ -31,6 +31,7 @@ struct AttnParams {
     uint32_t chunk, nchunks;
     uint32_t subgroups;           // q-head subgroups per kv head
     uint32_t len_bias;            // added to a device-side length (position -> length)
+    uint32_t max_batch;           // device-side sequence ids at or above this are skipped (0 = not checked)
 };
 
 // HD in {64, 128}; G = q heads per workgroup (<= 4); S = token rows per lane group
@@ -46,6 +47,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_partial_kernel(AttnParam
     const uint32_t seq_id = p.seq_ids_dev ? p.seq_ids_dev[b] : p.seq_id;
     const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
+    if (p.max_batch != 0 && seq_id >= p.max_batch) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t cbeg = t0 + blockIdx.y * p.chunk;
     if (cbeg >= len) return;
@@ -201,6 +203,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     const uint32_t d = threadIdx.x % HD, cg = threadIdx.x / HD;
     const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
+    if (p.max_batch != 0 && p.seq_ids_dev && p.seq_ids_dev[b] >= p.max_batch) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t n = (len - t0 + p.chunk - 1) / p.chunk;
     const float* w = p.ws + (((size_t)b * p.q_heads + qh) * p.nchunks) * (HD + 2);
@@ -343,6 +346,7 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
     p.max_seq_len = a.max_seq_len; p.kv_heads = a.kv_heads; p.q_heads = a.q_heads; p.window = a.window;
     p.subgroups = 1;
     p.len_bias = a.len_bias;
+    p.max_batch = a.max_batch;
     (void)hipGetLastError();
     const uint32_t group = a.q_heads / a.kv_heads;
     uint32_t span = a.max_len_hint;
@@ -503,6 +507,29 @@ static int batched_impl(M40llmCudaContext* ctx, const M40llmKVCache* kv, const u
     if (rc != 0) return -4;
     if (synchronize && hipStreamSynchronize(ctx->decode_stream) != hipSuccess) return -5;
     return 0;
+}
+
+// Row-batched attention whose ids / lengths stay on the device: nothing is copied back for validation; rows whose
+// id or length (+ len_bias) is out of range are skipped by the kernel.  max_len_hint bounds every row's length.
+int m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                                   const uint32_t* seq_ids_dev,
+                                                                   const uint32_t* seq_lens_dev, uint32_t len_bias,
+                                                                   uint32_t batch_size, uint32_t max_len_hint,
+                                                                   const void* q_dev_f32, uint32_t q_heads,
+                                                                   void* out_dev_f32) {
+    if (!ctx || !kv || !seq_ids_dev || !seq_lens_dev || !q_dev_f32 || !out_dev_f32) return -1;
+    if (batch_size == 0) return -2;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -3;
+    if (kv->head_dim != 64 && kv->head_dim != 128) return -6;
+    if (!kv->d_k || !kv->d_v) return -6;
+    if (max_len_hint == 0 || max_len_hint > kv->max_seq_len) return -8;
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = batch_size;
+    a.seq_ids_dev = seq_ids_dev; a.seq_lens_dev = seq_lens_dev; a.len_bias = len_bias; a.max_len_hint = max_len_hint;
+    a.max_batch = kv->max_batch_size;
+    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a) == 0 ? 0 : -4;
 }
 
 int m40llm_attention_last_token_f32_gqa_batched(M40llmCudaContext* ctx, const M40llmKVCache* kv,

@@ -113,6 +113,7 @@ struct M40AttnArgs {
     uint32_t max_len_hint;          // upper bound of any row's length (sizes the grid)
     uint32_t window;                // 0 = whole sequence, else only the last `window` tokens
     uint32_t len_bias;              // added to lengths read from seq_lens_dev
+    uint32_t max_batch;             // 0, or the bound that device-side sequence ids are checked against
 };
 int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
                                const M40AttnArgs& a);

@@ -29,21 +29,42 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 // Fragment i (k = 32 i .. 32 i + 31) is 64 x 16 bytes: entry g*16 + row holds the eight halves k = 32 i + 8 g + 0..7
 // of that row.  STACKED (M <= 8): rows 0-7 hold hi, rows 8-15 lo.  Otherwise two fragment sets: hi, then lo at
 // +K/32*64 entries.  With `up`, the packed value is silu(A) * up (the SwiGLU of an FFN) instead of A.
+// With `norm_w`, the packed value is the RMS-normalised row: A * rsqrt(mean(A^2) + eps) * norm_w.
 __global__ __launch_bounds__(256) void pack_a_blocked_kernel(const float* __restrict__ A, const float* __restrict__ up,
+                                                             const void* __restrict__ norm_w, uint32_t norm_dtype, float eps,
                                                              int M, int K, int stacked, uint4* __restrict__ P,
                                                              float* __restrict__ row_scale) {
     __shared__ float wave_max[4];
+    __shared__ float wave_sq[4];
     const int row = blockIdx.x;  // 0..7 (stacked) or 0..15
     const int tid = threadIdx.x;
+    // grid.y slices the fragments; every slice recomputes the row maximum (the row sits in L2)
     const bool live = row < M;
+    float rms = 1.0f;
+    if (live && norm_w) {
+        float sq = 0.0f;
+#pragma unroll 4
+        for (int k = tid; k < K; k += 256) {
+            const float a = A[(size_t)row * K + k];
+            sq = fmaf(a, a, sq);
+        }
+        sq = m40_sum64(sq);
+        if ((tid & 63) == 0) wave_sq[tid >> 6] = sq;
+        __syncthreads();
+        rms = rsqrtf((wave_sq[0] + wave_sq[1] + wave_sq[2] + wave_sq[3]) / (float)K + eps);
+    }
+    const uint16_t* nw16 = static_cast<const uint16_t*>(norm_w);
+    const float* nw32 = static_cast<const float*>(norm_w);
     auto value = [&](int k) -> float {
         const float a = A[(size_t)row * K + k];
+        if (norm_w) return a * rms * (norm_dtype == 0u ? m40_h2f(nw16[k]) : nw32[k]);
         if (!up) return a;
         return a / (1.0f + expf(-a)) * up[(size_t)row * K + k];
     };
     float inv_scale = 1.0f, scale = 1.0f;
     if (live) {
         float mx = 0.0f;
+#pragma unroll 4
         for (int k = tid; k < K; k += 256) mx = fmaxf(mx, fabsf(value(k)));
         mx = m40_max64(mx);
         if ((tid & 63) == 0) wave_max[tid >> 6] = mx;
@@ -58,10 +79,12 @@ __global__ __launch_bounds__(256) void pack_a_blocked_kernel(const float* __rest
             inv_scale = ldexpf(1.0f, -e);
         }
     }
-    if (tid == 0) row_scale[row] = scale;
+    if (tid == 0 && blockIdx.y == 0) row_scale[row] = scale;
     const int frags = K >> 5;
     uint4* P_lo = P + (size_t)frags * 64;
-    for (int f = tid; f < frags * 4; f += 256) {
+    const int f_begin = (int)(((long long)blockIdx.y * frags * 4) / gridDim.y);
+    const int f_end = (int)(((long long)(blockIdx.y + 1) * frags * 4) / gridDim.y);
+    for (int f = f_begin + tid; f < f_end; f += 256) {
         const int g = f & 3, i = f >> 2;
         const int k0 = 32 * i + 8 * g;
         uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
@@ -97,10 +120,13 @@ __device__ __forceinline__ uint32_t q8_pair_to_f16(uint32_t spread) {
 struct SkinnyArgs {
     const uint4* P;            // packed activations
     const float* row_scale;
-    const void* W[2];          // up to two weight matrices of the same shape (grid.z)
-    float* C[2];               // their outputs [M][N]
-    float* partial;            // [grid.z][S][16][N] when S > 1
-    int M, N, K, S;
+    const void* W[3];          // up to three weight matrices with the same K (Q/K/V, gate/up)
+    float* C[3];               // direct outputs [M][N z] (S == 1 and no epilogue kernel)
+    int N[3];
+    int tile_begin[4];         // first 16-column tile of each matrix in the launch-wide tile list
+    size_t part_off[3];        // float offset of matrix z in `partial`; layout there [S][16][N z]
+    float* partial;
+    int nmat, M, K, S, direct;
 };
 
 // FMT 0: f16 weights, 1: q8_0 weights.
@@ -113,33 +139,35 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int j = lane & 15, g = lane >> 4;
-    const int ntiles = (p.N + 15) >> 4;
-    int ntile = blockIdx.x * kWavesPerGroup + wave;
-    const bool tile_live = ntile < ntiles;
-    if (!tile_live) ntile = ntiles - 1;
-    const int n0 = ntile * 16;
+    const int ntiles = p.tile_begin[p.nmat];
+    int gtile = blockIdx.x * kWavesPerGroup + wave;
+    const bool tile_live = gtile < ntiles;
+    if (!tile_live) gtile = ntiles - 1;
+    const int z = (p.nmat > 2 && gtile >= p.tile_begin[2]) ? 2 : ((p.nmat > 1 && gtile >= p.tile_begin[1]) ? 1 : 0);
+    const int N = p.N[z];
+    const int n0 = (gtile - p.tile_begin[z]) * 16;
     const int KT = p.K / kTileK;
     const int kt0 = (int)(((long long)blockIdx.y * KT) / p.S), kt1 = (int)(((long long)(blockIdx.y + 1) * KT) / p.S);
     const int frags_total = p.K >> 5;
     const uint4* P_lo = p.P + (size_t)frags_total * 64;
 
     // ---- weight addressing
-    const int col = n0 + j < p.N ? n0 + j : p.N - 1;
+    const int col = n0 + j < N ? n0 + j : N - 1;
     const uint16_t* w16 = nullptr;
     const uint8_t* q_src[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     int q_dst[5] = {0, 0, 0, 0, 0};
     uint8_t* my_b = b_lds + (FMT == 1 ? wave * kQ8TileBytes : 0);
     if (FMT == 0) {
-        w16 = static_cast<const uint16_t*>(p.W[blockIdx.z]) + (size_t)col * p.K + 8 * g;
+        w16 = static_cast<const uint16_t*>(p.W[z]) + (size_t)col * p.K + 8 * g;
     } else {
         const size_t col_stride = (size_t)(p.K >> 5) * 34;
-        const uint8_t* base = static_cast<const uint8_t*>(p.W[blockIdx.z]);
+        const uint8_t* base = static_cast<const uint8_t*>(p.W[z]);
 #pragma unroll
         for (int i = 0; i < 5; ++i) {
             const int q = i * 64 + lane;          // 16-byte piece of the 16 x 272-byte tile
             if (q < 272) {
                 const int c = q / 17, piece = q % 17;
-                const int cc = n0 + c < p.N ? n0 + c : p.N - 1;
+                const int cc = n0 + c < N ? n0 + c : N - 1;
                 q_src[i] = base + (size_t)cc * col_stride + 16 * piece;
                 q_dst[i] = c * 272 + 16 * piece;
             }
@@ -220,36 +248,231 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], 32, 64);  // hi rows + lo rows
     }
-    if (!tile_live || n0 + j >= p.N) return;
+    if (!tile_live || n0 + j >= N) return;
     if (STACKED && g >= 2) return;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
-        if (p.S == 1) {
-            if (row < p.M) p.C[blockIdx.z][(size_t)row * p.N + n0 + j] = acc[r] * p.row_scale[row];
+        if (p.direct) {
+            if (row < p.M) p.C[z][(size_t)row * N + n0 + j] = acc[r] * p.row_scale[row];
         } else {
-            p.partial[(((size_t)blockIdx.z * p.S + blockIdx.y) * 16 + row) * p.N + n0 + j] = acc[r];
+            p.partial[p.part_off[z] + ((size_t)blockIdx.y * 16 + row) * N + n0 + j] = acc[r];
         }
     }
 }
 
-// C[row][n] = row_scale[row] * sum over slices (ascending) of partial[z][slice][row][n]
-__global__ __launch_bounds__(256) void skinny_reduce_kernel(SkinnyArgs p, int rows) {
+// scaled sum over the K slices (ascending) of one output element
+__device__ __forceinline__ float skinny_sum(const SkinnyArgs& p, int z, int row, int n) {
+    const float* src = p.partial + p.part_off[z] + (size_t)row * p.N[z] + n;
+    const size_t slice_stride = (size_t)16 * p.N[z];
+    float part[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) part[s] = s < p.S ? src[(size_t)s * slice_stride] : 0.0f;
+    float v = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) v += part[s];
+    return v * p.row_scale[row];
+}
+
+// Epilogue over the slice partials; grid (ceil(N/256), rows, matrices).
+//   mode 0: out z[row][n] = sum (+ bias[n]) (+ residual[row][n])        (residual may alias out)
+//   mode 1: out 0[row][n] = silu(sum of matrix 0) * (sum of matrix 1)   (SwiGLU of gate and up)
+struct EpilogueArgs {
+    SkinnyArgs g;
+    float* out[3];
+    const float* bias;
+    const float* residual;
+    int mode;
+};
+__global__ __launch_bounds__(256) void skinny_epilogue_kernel(EpilogueArgs e) {
+    const int z = blockIdx.z, row = blockIdx.y;
     const int n = blockIdx.x * 256 + threadIdx.x;
-    if (n >= p.N) return;
-    const int z = blockIdx.z;
-    for (int row = blockIdx.y; row < rows; row += gridDim.y) {
-        float v = 0.0f;
-        for (int s = 0; s < p.S; ++s) v += p.partial[(((size_t)z * p.S + s) * 16 + row) * p.N + n];
-        p.C[z][(size_t)row * p.N + n] = v * p.row_scale[row];
+    if (n >= e.g.N[z]) return;
+    if (e.mode == 1) {
+        const float gate = skinny_sum(e.g, 0, row, n), up = skinny_sum(e.g, 1, row, n);
+        e.out[0][(size_t)row * e.g.N[0] + n] = gate / (1.0f + expf(-gate)) * up;
+        return;
+    }
+    float v = skinny_sum(e.g, z, row, n);
+    if (e.bias) v = v + e.bias[n];
+    if (e.residual) v = e.residual[(size_t)row * e.g.N[z] + n] + v;
+    e.out[z][(size_t)row * e.g.N[z] + n] = v;
+}
+
+// Q/K/V epilogue of a batched decode step: bias, RoPE at each row's position, q to its buffer, K and V (f16) into
+// the cache row of (sequence ids[row], position lens[row]).  One thread per rotation pair; pair space = Q pairs,
+// K pairs, V pairs (V pairs are adjacent elements, not rotated).
+struct QkvEpilogueArgs {
+    SkinnyArgs g;
+    const float* bq; const float* bk; const float* bv;
+    float* q_out;                 // [rows][q_heads * head_dim]
+    uint16_t* k_cache; uint16_t* v_cache; uint32_t* seq_map;
+    const uint32_t* ids_dev; const uint32_t* lens_dev;
+    uint32_t max_seq_len, max_batch, q_heads, kv_heads, head_dim, rope_layout;
+    float rope_base, rope_scale;
+};
+__global__ __launch_bounds__(256) void skinny_qkv_epilogue_kernel(QkvEpilogueArgs e) {
+    const uint32_t row = blockIdx.y;
+    const uint32_t half = e.head_dim / 2u;
+    const uint32_t q_pairs = e.q_heads * half, kv_pairs = e.kv_heads * half;
+    const uint32_t pair = blockIdx.x * 256u + threadIdx.x;
+    if (pair >= q_pairs + 2u * kv_pairs) return;
+    int which;
+    uint32_t local;
+    if (pair < q_pairs) { which = 0; local = pair; }
+    else if (pair < q_pairs + kv_pairs) { which = 1; local = pair - q_pairs; }
+    else { which = 2; local = pair - q_pairs - kv_pairs; }
+    const uint32_t head = local / half, off = local % half;
+    size_t i0, i1;
+    m40_rope_pair(head, off, e.head_dim, which == 2 ? M40LLM_ROPE_LAYOUT_ADJACENT : e.rope_layout, &i0, &i1);
+    const float* bias = which == 0 ? e.bq : (which == 1 ? e.bk : e.bv);
+    float y0 = skinny_sum(e.g, which, (int)row, (int)i0), y1 = skinny_sum(e.g, which, (int)row, (int)i1);
+    if (bias) { y0 = y0 + bias[i0]; y1 = y1 + bias[i1]; }
+    const uint32_t position = e.lens_dev[row];
+    const uint32_t seq = e.ids_dev[row];
+    if (position >= e.max_seq_len || seq >= e.max_batch) return;
+    if (which != 2) m40_rope_rotate(position, off, e.head_dim, e.rope_base, e.rope_scale, y0, y1, &y0, &y1);
+    if (which == 0) {
+        float* q = e.q_out + (size_t)row * e.q_heads * e.head_dim;
+        q[i0] = y0;
+        q[i1] = y1;
+    } else {
+        const size_t ept = (size_t)e.kv_heads * e.head_dim;
+        uint16_t* dst = (which == 1 ? e.k_cache : e.v_cache) + ((size_t)seq * e.max_seq_len + position) * ept;
+        dst[i0] = m40_f2h(y0);
+        dst[i1] = m40_f2h(y1);
+        if (which == 1 && local == 0) e.seq_map[seq] = position + 1u;
     }
 }
 
-int pick_slices(int ntiles, int KT, int nmat, int num_cus) {
-    const long long groups = (long long)((ntiles + kWavesPerGroup - 1) / kWavesPerGroup) * nmat;
+// Batched greedy step: one workgroup per row.  First index of the row maximum of logits[rows][n] and the
+// top-1/top-2 gap go to ids[row][step] / gaps[row][step]; lens[row] += 1; the embedding row of the pick becomes the
+// row's next input.  state = {unused, capacity, step of row 0, step of row 1, ...}.
+struct GreedyBatchArgs {
+    const float* logits; uint32_t n;
+    uint32_t* state;              // [1] capacity, [2 + row] step of the row
+    uint32_t* lens; uint32_t* ids; float* gaps;
+    const uint16_t* table; uint32_t d_model; float* x_out;
+};
+__global__ __launch_bounds__(1024) void greedy_batch_kernel(GreedyBatchArgs a) {
+    __shared__ float sa[16], sb[16];
+    __shared__ uint32_t si[16];
+    __shared__ uint32_t s_tok;
+    const uint32_t row = blockIdx.x;
+    const float* lg = a.logits + (size_t)row * a.n;
+    float va = -INFINITY, vb = -INFINITY;
+    uint32_t ia = 0xffffffffu;
+    auto offer = [&](float oa, float ob, uint32_t oi) {
+        if (oa > va || (oa == va && oi < ia)) { vb = fmaxf(va, ob); va = oa; ia = oi; }
+        else vb = fmaxf(vb, oa);
+    };
+#pragma unroll 4
+    for (uint32_t i = threadIdx.x; i < a.n; i += 1024u) offer(lg[i], -INFINITY, i);
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float oa = __shfl_xor(va, o, 64), ob = __shfl_xor(vb, o, 64);
+        const uint32_t oi = __shfl_xor(ia, o, 64);
+        offer(oa, ob, oi);
+    }
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0u) { sa[wave] = va; sb[wave] = vb; si[wave] = ia; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < 16u; ++w) offer(sa[w], sb[w], si[w]);
+        uint32_t tok = ia == 0xffffffffu ? 0u : ia;
+        if (tok >= a.n) tok = a.n - 1;
+        const uint32_t step = a.state[2 + row], cap = a.state[1];
+        if (step < cap) {
+            a.ids[(size_t)row * cap + step] = tok;
+            a.gaps[(size_t)row * cap + step] = va - vb;
+        }
+        a.state[2 + row] = step + 1u;
+        a.lens[row] = a.lens[row] + 1u;
+        s_tok = tok;
+    }
+    __syncthreads();
+    const uint32_t tok = s_tok;
+    for (uint32_t i = threadIdx.x; i < a.d_model; i += 1024u)
+        a.x_out[(size_t)row * a.d_model + i] = m40_h2f(a.table[(size_t)tok * a.d_model + i]);
+}
+
+int pick_slices(int ntiles, int KT, int num_cus) {
+    const long long groups = (ntiles + kWavesPerGroup - 1) / kWavesPerGroup;
     int s = 1;
     while (s < 16 && groups * s < 2LL * num_cus && KT / (s * 2) >= 1) s *= 2;
     return s > KT ? KT : s;
+}
+
+struct PackSpec {
+    const float* A;
+    const float* up;          // SwiGLU partner, or null
+    const void* norm_w;       // RMSNorm weights, or null
+    uint32_t norm_dtype;
+    float eps;
+};
+
+// Packs `m` (<= 16) rows and launches the MFMA kernel over nmat matrices.  Returns the filled args (for an
+// epilogue kernel) through *out; direct != 0 writes scaled results to C when the K range is not split.
+int launch_core(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const PackSpec& pk, int m, int K,
+                int nmat, const void* const* W, const int* N, float* const* C, bool want_direct, SkinnyArgs* out) {
+    M40StreamScratch& sc = ctx->scratch[stream_kind];
+    float* row_scale = static_cast<float*>(sc.gemm_pack);
+    uint4* P = reinterpret_cast<uint4*>(static_cast<char*>(sc.gemm_pack) + 256);
+    SkinnyArgs a{};
+    a.P = P; a.row_scale = row_scale; a.partial = static_cast<float*>(sc.attn_partial);
+    a.nmat = nmat; a.M = m; a.K = K;
+    int tiles = 0;
+    size_t n_total = 0;
+    for (int z = 0; z < nmat; ++z) {
+        a.W[z] = W[z]; a.N[z] = N[z]; a.C[z] = C ? C[z] : nullptr;
+        a.tile_begin[z] = tiles;
+        tiles += (N[z] + 15) >> 4;
+        n_total += (size_t)N[z];
+    }
+    a.tile_begin[nmat] = tiles;
+    const int KT = K / kTileK;
+    int S = pick_slices(tiles, KT, ctx->num_cus);
+    while (S > 1 && (size_t)S * 16 * n_total * sizeof(float) > sc.attn_partial_bytes) S >>= 1;
+    if ((size_t)S * 16 * n_total * sizeof(float) > sc.attn_partial_bytes && !(want_direct && S == 1)) return -2;
+    a.S = S;
+    a.direct = (want_direct && S == 1) ? 1 : 0;
+    size_t off = 0;
+    for (int z = 0; z < nmat; ++z) {
+        a.part_off[z] = off;
+        off += (size_t)S * 16 * N[z];
+    }
+    const bool stacked = m <= 8;
+    const int pack_slices = K >= 8192 ? 8 : (K >= 2048 ? 4 : 1);
+    pack_a_blocked_kernel<<<dim3(stacked ? 8 : 16, pack_slices), 256, 0, stream>>>(pk.A, pk.up, pk.norm_w, pk.norm_dtype, pk.eps, m,
+                                                                                   K, stacked ? 1 : 0, P, row_scale);
+    dim3 grid((tiles + kWavesPerGroup - 1) / kWavesPerGroup, S);
+    if (fmt == 0) {
+        if (stacked) skinny_mfma_kernel<0, true><<<grid, kThreads, 0, stream>>>(a);
+        else skinny_mfma_kernel<0, false><<<grid, kThreads, 0, stream>>>(a);
+    } else {
+        if (stacked) skinny_mfma_kernel<1, true><<<grid, kThreads, 0, stream>>>(a);
+        else skinny_mfma_kernel<1, false><<<grid, kThreads, 0, stream>>>(a);
+    }
+    *out = a;
+    return 0;
+}
+
+void launch_plain_epilogue(hipStream_t stream, const SkinnyArgs& a, int nmat, float* const* out, const float* bias,
+                           const float* residual, int mode) {
+    EpilogueArgs e{};
+    e.g = a;
+    int nmax = 0;
+    for (int z = 0; z < nmat; ++z) {
+        e.out[z] = out[z];
+        nmax = a.N[z] > nmax ? a.N[z] : nmax;
+    }
+    e.bias = bias; e.residual = residual; e.mode = mode;
+    dim3 grid((nmax + 255) / 256, a.M, mode == 1 ? 1 : nmat);
+    skinny_epilogue_kernel<<<grid, 256, 0, stream>>>(e);
+}
+
+bool rows_ok(const M40llmCudaContext* ctx, int rows, int K) {
+    return rows >= 1 && rows <= 16 && K > 0 && K % kTileK == 0 && (size_t)K * 64 + 256 <= ctx->scratch[1].gemm_pack_bytes;
 }
 
 }  // namespace
@@ -267,38 +490,124 @@ int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t strea
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return -2;
     if (!m40_skinny_supported(ctx, stream_kind, M, N, K, fmt)) return -2;
-    M40StreamScratch& sc = ctx->scratch[stream_kind];
-    float* row_scale = static_cast<float*>(sc.gemm_pack);
-    uint4* P = reinterpret_cast<uint4*>(static_cast<char*>(sc.gemm_pack) + 256);
     const int nmat = W1 ? 2 : 1;
-    const int ntiles = (N + 15) >> 4;
-    const int KT = K / kTileK;
-    int S = pick_slices(ntiles, KT, nmat, ctx->num_cus);
-    while (S > 1 && (size_t)nmat * S * 16 * N * sizeof(float) > sc.attn_partial_bytes) S >>= 1;
     (void)hipGetLastError();
     for (int r0 = 0; r0 < M; r0 += 16) {
         const int m = M - r0 < 16 ? M - r0 : 16;
-        const bool stacked = m <= 8;
-        pack_a_blocked_kernel<<<stacked ? 8 : 16, 256, 0, stream>>>(A + (size_t)r0 * K, up ? up + (size_t)r0 * K : nullptr,
-                                                                    m, K, stacked ? 1 : 0, P, row_scale);
+        PackSpec pk{A + (size_t)r0 * K, up ? up + (size_t)r0 * K : nullptr, nullptr, 0, 0.0f};
+        const void* W[2] = {W0, W1};
+        const int Ns[2] = {N, N};
+        float* C[2] = {C0 + (size_t)r0 * N, C1 ? C1 + (size_t)r0 * N : nullptr};
         SkinnyArgs a{};
-        a.P = P; a.row_scale = row_scale;
-        a.W[0] = W0; a.W[1] = W1;
-        a.C[0] = C0 + (size_t)r0 * N; a.C[1] = C1 ? C1 + (size_t)r0 * N : nullptr;
-        a.partial = static_cast<float*>(sc.attn_partial);
-        a.M = m; a.N = N; a.K = K; a.S = S;
-        dim3 grid((ntiles + kWavesPerGroup - 1) / kWavesPerGroup, S, nmat);
-        if (fmt == 0) {
-            if (stacked) skinny_mfma_kernel<0, true><<<grid, kThreads, 0, stream>>>(a);
-            else skinny_mfma_kernel<0, false><<<grid, kThreads, 0, stream>>>(a);
-        } else {
-            if (stacked) skinny_mfma_kernel<1, true><<<grid, kThreads, 0, stream>>>(a);
-            else skinny_mfma_kernel<1, false><<<grid, kThreads, 0, stream>>>(a);
-        }
-        if (S > 1) {
-            dim3 rgrid((N + 255) / 256, m < 4 ? m : 4, nmat);
-            skinny_reduce_kernel<<<rgrid, 256, 0, stream>>>(a, m);
-        }
+        const int rc = launch_core(ctx, stream, stream_kind, fmt, pk, m, K, nmat, W, Ns, C, true, &a);
+        if (rc != 0) return rc;
+        if (!a.direct) launch_plain_epilogue(stream, a, nmat, C, nullptr, nullptr, 0);
     }
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
+
+// ---- batched decode step entry points (rows <= 16, decode stream) -------------------------------------------
+extern "C" {
+
+int m40llm_ext_batched_norm_qkv_rope_append_async(
+    M40llmCudaContext* ctx, M40llmKVCache* kv, const uint32_t* seq_ids_dev, const uint32_t* seq_lens_dev, uint32_t rows,
+    const void* d_x_f32, const void* d_norm_w, uint32_t norm_weight_dtype, float eps, const void* d_wq_f16,
+    const void* d_wk_f16, const void* d_wv_f16, const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32,
+    uint32_t d_model, uint32_t q_heads, float freq_base, float freq_scale, uint32_t rope_layout, void* d_q_out_f32) {
+    if (!ctx || !kv || !seq_ids_dev || !seq_lens_dev || !d_x_f32 || !d_norm_w || !d_wq_f16 || !d_wk_f16 || !d_wv_f16 ||
+        !d_q_out_f32)
+        return -1;
+    if (kv->compressed || !kv->d_k || !kv->d_v) return -2;
+    if (norm_weight_dtype > 1) return -4;
+    if (kv->head_dim == 0 || kv->head_dim % 2 != 0 || kv->num_heads == 0 || q_heads == 0) return -3;
+    if (!rows_ok(ctx, (int)rows, (int)d_model)) return -6;
+    if (!m40_aligned16(d_wq_f16) || !m40_aligned16(d_wk_f16) || !m40_aligned16(d_wv_f16)) return -6;
+    (void)hipGetLastError();
+    const int QN = (int)(q_heads * kv->head_dim), KN = (int)(kv->num_heads * kv->head_dim);
+    PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
+    const void* W[3] = {d_wq_f16, d_wk_f16, d_wv_f16};
+    const int Ns[3] = {QN, KN, KN};
+    SkinnyArgs a{};
+    int rc = launch_core(ctx, ctx->decode_stream, 1, 0, pk, (int)rows, (int)d_model, 3, W, Ns, nullptr, false, &a);
+    if (rc != 0) return -6;
+    QkvEpilogueArgs e{};
+    e.g = a;
+    e.bq = static_cast<const float*>(d_bq_f32); e.bk = static_cast<const float*>(d_bk_f32);
+    e.bv = static_cast<const float*>(d_bv_f32);
+    e.q_out = static_cast<float*>(d_q_out_f32);
+    e.k_cache = kv->d_k; e.v_cache = kv->d_v; e.seq_map = kv->d_seq_map;
+    e.ids_dev = seq_ids_dev; e.lens_dev = seq_lens_dev;
+    e.max_seq_len = kv->max_seq_len; e.max_batch = kv->max_batch_size; e.q_heads = q_heads; e.kv_heads = kv->num_heads;
+    e.head_dim = kv->head_dim; e.rope_layout = rope_layout; e.rope_base = freq_base; e.rope_scale = freq_scale;
+    const uint32_t pairs = (q_heads + 2u * kv->num_heads) * (kv->head_dim / 2u);
+    skinny_qkv_epilogue_kernel<<<dim3((pairs + 255u) / 256u, rows), 256, 0, ctx->decode_stream>>>(e);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_batched_gemm_residual_f32xf16_async(M40llmCudaContext* ctx, const void* d_a_f32, const void* d_w_f16,
+                                                   const void* d_residual_f32, void* d_out_f32, uint32_t rows, int N, int K) {
+    if (!ctx || !d_a_f32 || !d_w_f16 || !d_out_f32) return -1;
+    if (N <= 0 || K <= 0) return -2;
+    if (!rows_ok(ctx, (int)rows, K) || !m40_aligned16(d_w_f16)) return -6;
+    (void)hipGetLastError();
+    PackSpec pk{static_cast<const float*>(d_a_f32), nullptr, nullptr, 0, 0.0f};
+    const void* W[1] = {d_w_f16};
+    const int Ns[1] = {N};
+    float* out[1] = {static_cast<float*>(d_out_f32)};
+    SkinnyArgs a{};
+    if (launch_core(ctx, ctx->decode_stream, 1, 0, pk, (int)rows, K, 1, W, Ns, nullptr, false, &a) != 0) return -6;
+    launch_plain_epilogue(ctx->decode_stream, a, 1, out, nullptr, static_cast<const float*>(d_residual_f32), 0);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_batched_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                                 uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
+                                                 const void* d_wup_f16, void* d_hid_f32, uint32_t rows, int ffn, int d_model) {
+    if (!ctx || !d_x_f32 || !d_norm_w || !d_wgate_f16 || !d_wup_f16 || !d_hid_f32) return -1;
+    if (ffn <= 0 || d_model <= 0) return -2;
+    if (norm_weight_dtype > 1) return -4;
+    if (!rows_ok(ctx, (int)rows, d_model) || !m40_aligned16(d_wgate_f16) || !m40_aligned16(d_wup_f16)) return -6;
+    (void)hipGetLastError();
+    PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
+    const void* W[2] = {d_wgate_f16, d_wup_f16};
+    const int Ns[2] = {ffn, ffn};
+    float* out[2] = {static_cast<float*>(d_hid_f32), nullptr};
+    SkinnyArgs a{};
+    if (launch_core(ctx, ctx->decode_stream, 1, 0, pk, (int)rows, d_model, 2, W, Ns, nullptr, false, &a) != 0) return -6;
+    launch_plain_epilogue(ctx->decode_stream, a, 2, out, nullptr, nullptr, 1);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_batched_norm_gemm_f32xf16_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                               uint32_t norm_weight_dtype, float eps, const void* d_w_f16, void* d_out_f32,
+                                               uint32_t rows, int N, int K) {
+    if (!ctx || !d_x_f32 || !d_norm_w || !d_w_f16 || !d_out_f32) return -1;
+    if (N <= 0 || K <= 0) return -2;
+    if (norm_weight_dtype > 1) return -4;
+    if (!rows_ok(ctx, (int)rows, K) || !m40_aligned16(d_w_f16)) return -6;
+    (void)hipGetLastError();
+    PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
+    const void* W[1] = {d_w_f16};
+    const int Ns[1] = {N};
+    float* out[1] = {static_cast<float*>(d_out_f32)};
+    SkinnyArgs a{};
+    if (launch_core(ctx, ctx->decode_stream, 1, 0, pk, (int)rows, K, 1, W, Ns, out, true, &a) != 0) return -6;
+    if (!a.direct) launch_plain_epilogue(ctx->decode_stream, a, 1, out, nullptr, nullptr, 0);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+int m40llm_ext_batched_greedy_step_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t rows, uint32_t n,
+                                         uint32_t* state_dev, uint32_t* seq_lens_dev, uint32_t* ids_dev, float* gaps_dev,
+                                         const void* d_table_f16, uint32_t d_model, void* d_x_out_f32) {
+    if (!ctx || !d_logits_f32 || !state_dev || !seq_lens_dev || !ids_dev || !gaps_dev || !d_table_f16 || !d_x_out_f32) return -1;
+    if (rows == 0 || n == 0 || d_model == 0) return -2;
+    (void)hipGetLastError();
+    GreedyBatchArgs a{};
+    a.logits = static_cast<const float*>(d_logits_f32); a.n = n; a.state = state_dev; a.lens = seq_lens_dev;
+    a.ids = ids_dev; a.gaps = gaps_dev; a.table = static_cast<const uint16_t*>(d_table_f16); a.d_model = d_model;
+    a.x_out = static_cast<float*>(d_x_out_f32);
+    greedy_batch_kernel<<<rows, 1024, 0, ctx->decode_stream>>>(a);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+}  // extern "C"

@@ -127,6 +127,7 @@ public:
     }
     ~DecodeModel() {
         drop_graph();
+        drop_batch_graph();
         if (kv_) m40llm_kvcache_destroy(kv_);
     }
     DecodeModel(const DecodeModel&) = delete;
@@ -473,10 +474,131 @@ public:
         M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits, ws_.logits.ptr(), (size_t)rows * cfg_.vocab * 4));
     }
 
+    // ---- device-driven row-batched greedy loop (modes 1 and 2; rows <= 16, dense cache) -------------------------
+    // Per step: every layer as five fused calls on the decode stream, output norm + lm_head, then the greedy pick,
+    // the length increment and the next embedding on the device.  Nothing is read back until the end.
+    bool batched_fused_available(uint32_t rows) const {
+        return !kvcfg_.is_enabled() && rows >= 1 && rows <= 16 && cfg_.d_model % 256 == 0 && cfg_.ffn % 256 == 0;
+    }
+    void batched_layer_fused(uint32_t l, const uint32_t* slots_dev, const uint32_t* lens_dev, uint32_t rows, uint32_t hint,
+                             const float* d_x, float* d_out) {
+        const LayerWeights& w = layers_[l];
+        const uint32_t D = cfg_.d_model, F = cfg_.ffn;
+        M40H_TRY(m40llm_ext_batched_norm_qkv_rope_append_async(ctx_, kv_, slots_dev, lens_dev, rows, d_x, w.attn_norm,
+                                                               cfg_.norm_weight_dtype, cfg_.rms_eps, w.wq, w.wk, w.wv, w.bq, w.bk,
+                                                               w.bv, D, cfg_.q_heads, cfg_.rope_base, cfg_.rope_scale,
+                                                               cfg_.rope_layout, ws_.q.ptr()));
+        M40H_TRY(m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async(ctx_, kv_, slots_dev, lens_dev, 1, rows, hint,
+                                                                                ws_.q.ptr(), cfg_.q_heads, ws_.ctx_out.ptr()));
+        M40H_TRY(m40llm_ext_batched_gemm_residual_f32xf16_async(ctx_, ws_.ctx_out.ptr(), w.wo, d_x, ws_.x1.ptr(), rows, (int)D, (int)D));
+        M40H_TRY(m40llm_ext_batched_norm_gate_up_swiglu_async(ctx_, ws_.x1.ptr(), w.ffn_norm, cfg_.norm_weight_dtype, cfg_.rms_eps,
+                                                              w.wgate, w.wup, ws_.hid.ptr(), rows, (int)F, (int)D));
+        M40H_TRY(m40llm_ext_batched_gemm_residual_f32xf16_async(ctx_, ws_.hid.ptr(), w.wdown, ws_.x1.ptr(), d_out, rows, (int)D, (int)F));
+    }
+    void enqueue_batched_step(uint32_t rows, uint32_t hint, float* hidden, float* other) {
+        const uint32_t* slots = static_cast<const uint32_t*>(bslots_.ptr());
+        uint32_t* lens = static_cast<uint32_t*>(blens_.ptr());
+        float* a = hidden;
+        float* b = other;
+        for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
+            batched_layer_fused(l, slots + (size_t)l * rows, lens, rows, hint, a, b);
+            std::swap(a, b);
+        }
+        M40H_TRY(m40llm_ext_batched_norm_gemm_f32xf16_async(ctx_, a, out_norm_, cfg_.norm_weight_dtype, cfg_.rms_eps, lm_head_,
+                                                            ws_.logits.ptr(), rows, (int)cfg_.vocab, (int)cfg_.d_model));
+        M40H_TRY(m40llm_ext_batched_greedy_step_async(ctx_, ws_.logits.ptr(), rows, cfg_.vocab,
+                                                      static_cast<uint32_t*>(bstate_.ptr()), lens,
+                                                      static_cast<uint32_t*>(bids_.ptr()), static_cast<float*>(bgaps_.ptr()),
+                                                      tok_emb_, cfg_.d_model, hidden));
+    }
+    // Returns false when a pick was a near-tie (the caller then repeats the decode on the host-sampled path).
+    bool decode_batch_device(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens, uint32_t rows,
+                             uint32_t warmup, uint32_t steps, uint32_t* ids_out, float* gaps_out, double* elapsed_ms) {
+        const uint32_t total = warmup + steps;
+        uint32_t max_len = 0;
+        for (uint32_t r = 0; r < rows; ++r) {
+            if (kv_lens[r] + total > cfg_.max_seq_len) throw std::out_of_range("sequence would exceed max_seq_len");
+            if (seq_ids[r] >= cfg_.max_sequences) throw std::out_of_range("sequence id out of range");
+            max_len = kv_lens[r] > max_len ? kv_lens[r] : max_len;
+        }
+        ws_.ensure(ctx_, cfg_, rows);
+        // device state: slot ids per layer, lengths, per-row step counters, picks and gaps
+        std::vector<uint32_t> slots((size_t)cfg_.n_layers * rows);
+        for (uint32_t l = 0; l < cfg_.n_layers; ++l)
+            for (uint32_t r = 0; r < rows; ++r) slots[(size_t)l * rows + r] = kv_slot(seq_ids[r], l);
+        std::vector<uint32_t> state(2 + rows, 0);
+        state[1] = total;
+        sync_all();
+        drop_batch_graph();
+        bslots_ = DeviceBuf(ctx_, slots.size() * 4); blens_ = DeviceBuf(ctx_, (size_t)rows * 4);
+        bstate_ = DeviceBuf(ctx_, state.size() * 4);
+        bids_ = DeviceBuf(ctx_, (size_t)rows * total * 4); bgaps_ = DeviceBuf(ctx_, (size_t)rows * total * 4);
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, bslots_.ptr(), slots.data(), slots.size() * 4));
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, blens_.ptr(), kv_lens, (size_t)rows * 4));
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, bstate_.ptr(), state.data(), state.size() * 4));
+        float* hidden = ws_.scratch_a.f32();
+        float* other = ws_.scratch_b.f32();
+        for (uint32_t r = 0; r < rows; ++r) embed(first_tokens[r], hidden + (size_t)r * cfg_.d_model);
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, M40LLM_STREAM_DECODE, M40LLM_STREAM_PREFILL));
+        auto run = [&](uint32_t first_step, uint32_t n_steps) {
+            uint32_t done = 0;
+            while (done < n_steps) {
+                const uint32_t longest = max_len + first_step + done;       // tokens held by the longest row before the step
+                const uint32_t hint = len_hint_for(longest);                // >= longest + 1
+                uint32_t n = n_steps - done;
+                if (hint < cfg_.max_seq_len && longest + n > hint) n = hint - longest;
+                if (mode_ >= 2) {
+                    if (!bgraph_ || bgraph_rows_ != rows || bgraph_hint_ != hint) {
+                        drop_batch_graph();
+                        M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
+                        M40H_TRY(m40llm_cuda_graph_begin_capture(ctx_, M40LLM_STREAM_DECODE));
+                        try {
+                            enqueue_batched_step(rows, hint, hidden, other);
+                        } catch (...) {
+                            m40llm_cuda_graph_cancel_capture(ctx_, M40LLM_STREAM_DECODE);
+                            throw;
+                        }
+                        M40H_TRY(m40llm_cuda_graph_end_capture(ctx_, M40LLM_STREAM_DECODE, &bgraph_));
+                        bgraph_rows_ = rows; bgraph_hint_ = hint;
+                    }
+                    for (uint32_t i = 0; i < n; ++i) M40H_TRY(m40llm_cuda_graph_launch(ctx_, bgraph_, M40LLM_STREAM_DECODE));
+                } else {
+                    for (uint32_t i = 0; i < n; ++i) enqueue_batched_step(rows, hint, hidden, other);
+                }
+                done += n;
+            }
+        };
+        if (warmup) run(0, warmup);
+        sync_all();
+        const auto t0 = std::chrono::steady_clock::now();
+        run(warmup, steps);
+        sync_all();
+        const auto t1 = std::chrono::steady_clock::now();
+        if (elapsed_ms) *elapsed_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
+        std::vector<float> gaps((size_t)rows * total);
+        M40H_TRY(m40llm_memcpy_d2h(ctx_, ids_out, bids_.ptr(), (size_t)rows * total * 4));
+        M40H_TRY(m40llm_memcpy_d2h(ctx_, gaps.data(), bgaps_.ptr(), gaps.size() * 4));
+        drop_batch_graph();       // the graph holds pointers into the per-call state buffers
+        bool ok = true;
+        for (size_t i = 0; i < gaps.size(); ++i) {
+            if (gaps_out) gaps_out[i] = gaps[i];
+            if (!(gaps[i] >= kGreedyTieGuard)) ok = false;
+        }
+        return ok;
+    }
+    void drop_batch_graph() {
+        if (bgraph_) m40llm_cuda_graph_destroy(bgraph_);
+        bgraph_ = nullptr;
+    }
+
     // `steps` greedy steps for a batch of sequences whose caches already hold kv_lens[r] tokens;
     // first_tokens[r] is the input of step 0.  ids_out: [rows][steps], gaps_out (optional) likewise.
     void decode_batch_greedy(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens,
                              uint32_t rows, uint32_t steps, uint32_t* ids_out, float* gaps_out) {
+        if (mode_ >= 1 && batched_fused_available(rows)) {
+            if (decode_batch_device(seq_ids, kv_lens, first_tokens, rows, 0, steps, ids_out, gaps_out, nullptr)) return;
+            // near-tie somewhere: redo on the host-sampled path (same cache rows are rewritten)
+        }
         std::vector<uint32_t> lens(kv_lens, kv_lens + rows), toks(first_tokens, first_tokens + rows);
         std::vector<float> logits((size_t)rows * cfg_.vocab);
         std::vector<Sampler> samplers(rows, greedy_sampler(42));
@@ -528,6 +650,10 @@ public:
 
     void decode_batch_timed(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens, uint32_t rows,
                             uint32_t warmup, uint32_t steps, uint32_t* ids_out, double* elapsed_ms) {
+        if (mode_ >= 1 && batched_fused_available(rows)) {
+            if (decode_batch_device(seq_ids, kv_lens, first_tokens, rows, warmup, steps, ids_out, nullptr, elapsed_ms)) return;
+            throw std::runtime_error("near-tie in a greedy pick on the device path; rerun in mode 0");
+        }
         std::vector<uint32_t> lens(kv_lens, kv_lens + rows), toks(first_tokens, first_tokens + rows);
         std::vector<float> logits((size_t)rows * cfg_.vocab);
         std::vector<Sampler> samplers(rows, greedy_sampler(42));
@@ -617,6 +743,9 @@ private:
     DeviceBuf top2_;
     static constexpr uint32_t kTop2Capacity = 1u << 16;
     uint32_t state_cap_ = 0;
+    DeviceBuf bslots_, blens_, bstate_, bids_, bgaps_;
+    M40llmCudaGraphExec* bgraph_ = nullptr;
+    uint32_t bgraph_rows_ = 0, bgraph_hint_ = 0;
     M40llmCudaGraphExec* graph_ = nullptr;
     uint32_t graph_seq_ = 0, graph_hint_ = 0;
     float* graph_hidden_ = nullptr;

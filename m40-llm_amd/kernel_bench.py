@@ -176,9 +176,47 @@ def bench_block_select(b: Bench):
     kv.destroy()
 
 
+def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
+    """BASELINE config 3: Qwen2.5-3B-shaped random-init model, 8 sequences with contexts ~U[256, 4096], row-batched
+    greedy decode through the host layer.  Four distinct random layers are repeated over the 36 (own device copy
+    each); the embedding table is the lm_head matrix."""
+    syn = importlib.import_module("m40-llm_amd.synthetic")
+    cfg = dict(syn.QWEN25_3B)
+    B = 8
+    rng = np.random.default_rng(0)
+    lens = rng.integers(256, 4097, size=B).astype(np.uint32)
+    max_seq = 4096 + warmup + steps + 8
+    W = syn.make_weights(cfg, seed=0, unique_layers=4, tie_embeddings=True)
+    dm = syn.DeviceModel(b.ctx, cfg, W, max_seq_len=max_seq, max_sequences=B)
+    dm.set_mode(mode)
+    k16 = f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"])))
+    v16 = f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"])))
+    dk, dv = b.ctx.to_device(k16), b.ctx.to_device(v16)
+    for s in range(B):
+        for l in range(cfg["n_layers"]):
+            slot = dm.H.m40host_model_kv_slot(dm.h, s, l)
+            b.call("m40llm_ext_kvcache_bulk_fill_f16", dm.kv_handle(), slot, dk.ptr, dv.ptr, int(lens[s]))
+    first = rng.integers(0, cfg["vocab"], size=B).astype(np.uint32)
+    ids, ms = dm.decode_batch_timed(np.arange(B), lens, first, warmup, steps)
+    D, F, V, L = cfg["d_model"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
+    KV = cfg["kv_heads"] * cfg["head_dim"]
+    wbytes = L * 2 * (D * (D + 2 * KV) + D * D + 3 * D * F) + 2 * V * D
+    kvbytes = int(lens.sum() + B * (warmup + steps / 2)) * L * KV * 2 * 2
+    us = ms * 1e3 / steps
+    gbs = (wbytes + kvbytes) / us / 1e3
+    tok_s = B * steps / (ms / 1e3)
+    row = dict(kernel=f"decode step Qwen2.5-3B shape B=8 mode {mode}", shape=f"36 layers, lens sum {int(lens.sum())}", us_per_launch=round(us, 1),
+               algorithmic_bytes=int(wbytes + kvbytes), gbs=round(gbs, 1), frac=round(gbs / PEAK_GBS, 4), tok_s=round(tok_s, 1),
+               launches=steps, buffers=1)
+    b.rows.append(row)
+    print(f"{row['kernel']:34s} {row['shape']:44s} {us:9.1f} us {gbs:8.1f} GB/s  frac {gbs / PEAK_GBS:6.3f}  {tok_s:8.1f} tok/s aggregate",
+          flush=True)
+    dm.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="attn,gemv,gemm8,q80,bsel")
+    ap.add_argument("--only", default="attn,gemv,gemm8,q80,bsel,decode8")
     ap.add_argument("--json", default=None)
     args = ap.parse_args()
     which = set(args.only.split(","))
@@ -194,6 +232,8 @@ def main():
         bench_q80(b)
     if "bsel" in which:
         bench_block_select(b)
+    if "decode8" in which:
+        bench_decode_batch(b)
     if args.json:
         with open(args.json, "w") as f:
             for r in b.rows:

@@ -15,8 +15,11 @@ QWEN25_3B = dict(n_layers=36, d_model=2048, q_heads=16, kv_heads=2, head_dim=128
                  rms_eps=1e-6, rope_base=1e6, rope_scale=1.0, rope_layout=1, qkv_bias=True)
 
 
-def make_weights(cfg: dict, seed: int = 0, std: float = 0.02, emb_std: float | None = None) -> dict:
-    """f16 weights ~ N(0, std), norm weights 1.0 (f32), Q/K/V biases ~ N(0, std) when cfg['qkv_bias']."""
+def make_weights(cfg: dict, seed: int = 0, std: float = 0.02, emb_std: float | None = None,
+                 unique_layers: int | None = None, tie_embeddings: bool = False) -> dict:
+    """f16 weights ~ N(0, std), norm weights 1.0 (f32), Q/K/V biases ~ N(0, std) when cfg['qkv_bias'].
+    unique_layers: draw only that many distinct layers and repeat them cyclically (throughput runs only: every
+    layer still gets its own device copy, so nothing is served from a cache that a real model would miss)."""
     L, D, F, V = cfg["n_layers"], cfg["d_model"], cfg["ffn"], cfg["vocab"]
     KV = cfg["kv_heads"] * cfg["head_dim"]
     ss = np.random.SeedSequence(seed)
@@ -37,7 +40,11 @@ def make_weights(cfg: dict, seed: int = 0, std: float = 0.02, emb_std: float | N
     W = dict(wq=[], wk=[], wv=[], wo=[], wgate=[], wup=[], wdown=[], attn_norm=[], ffn_norm=[])
     if cfg.get("qkv_bias"):
         W.update(bq=[], bk=[], bv=[])
-    for _ in range(L):
+    for l in range(L):
+        if unique_layers and l >= unique_layers:
+            for name in W:
+                W[name].append(W[name][l % unique_layers])
+            continue
         W["wq"].append(w(D, D)); W["wk"].append(w(KV, D)); W["wv"].append(w(KV, D)); W["wo"].append(w(D, D))
         W["wgate"].append(w(F, D)); W["wup"].append(w(F, D)); W["wdown"].append(w(D, F))
         W["attn_norm"].append(np.ones(D, dtype=np.float32)); W["ffn_norm"].append(np.ones(D, dtype=np.float32))
@@ -45,7 +52,7 @@ def make_weights(cfg: dict, seed: int = 0, std: float = 0.02, emb_std: float | N
             W["bq"].append(b(D)); W["bk"].append(b(KV)); W["bv"].append(b(KV))
     W["out_norm"] = np.ones(D, dtype=np.float32)
     W["lm_head"] = w(V, D)
-    W["tok_emb"] = w(V, D, emb_std if emb_std is not None else std)
+    W["tok_emb"] = W["lm_head"] if tie_embeddings else w(V, D, emb_std if emb_std is not None else std)
     return W
 
 

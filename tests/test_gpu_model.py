@@ -148,29 +148,70 @@ def test_tinyllama_shape_reduced_depth_greedy_ids(ctx, orc):
 
 def test_qwen_shape_reduced_depth_batched_greedy_ids(ctx, orc):
     """BASELINE config 3 shape (hidden 2048, 16/2 heads, hd 128, FFN 11008, vocab 151936, biases, NeoX RoPE theta 1e6)
-    with 2 layers: batch 8, context lengths U[256,4096], pre-filled N(0,1) KV, 4 greedy steps, ids exact."""
+    with 2 layers: batch 8, context lengths U[256,4096], pre-filled N(0,1) KV, 4 greedy steps, ids exact - on the
+    reference's row-batched call sequence (mode 0) and on the fused MFMA path replayed from a graph (mode 2)."""
     cfg = dict(syn.QWEN25_3B); cfg["n_layers"] = 2
     W = syn.make_weights(cfg, seed=0)
     B, S, steps = 8, 4096 + 8, 4
     rng = np.random.default_rng(0)
     lens = rng.integers(256, 4097, size=B).astype(np.uint32)
-    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=B)
     om = _oracle_model(orc, cfg, W, S, B)
     Ko, Vo = om.kv_views()
+    fills = []
     for s in range(B):
         for l in range(cfg["n_layers"]):
             k16 = rng.standard_normal((int(lens[s]), cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32).astype(np.float16).view(np.uint16)
             v16 = rng.standard_normal((int(lens[s]), cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32).astype(np.float16).view(np.uint16)
-            dm.fill_kv(s, l, k16, v16)
+            fills.append((s, l, k16, v16))
             Ko[s * cfg["n_layers"] + l, :lens[s]] = k16; Vo[s * cfg["n_layers"] + l, :lens[s]] = v16
     toks = rng.integers(0, cfg["vocab"], size=B).astype(np.uint32)
-    ids, gaps = dm.decode_batch_greedy(np.arange(B), lens, toks, steps)
     orc.set_threads(16)
-    for s in range(B):
-        want, wg = om.decode_greedy(s, [toks[s]], steps, start_pos=int(lens[s]))
-        assert np.array_equal(ids[s], want[1:]), (s, ids[s], want[1:], gaps[s], wg)
-    print(f"[qwen-2L B=8] min top-2 logit gap over {B * steps} decisions: {gaps.min():.3e}")
-    dm.close()
+    want = [om.decode_greedy(s, [toks[s]], steps, start_pos=int(lens[s])) for s in range(B)]
+    for mode in (0, 2):
+        dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=B)
+        dm.set_mode(mode)
+        for s, l, k16, v16 in fills:
+            dm.fill_kv(s, l, k16, v16)
+        ids, gaps = dm.decode_batch_greedy(np.arange(B), lens, toks, steps)
+        for s in range(B):
+            assert np.array_equal(ids[s], want[s][0][1:]), (mode, s, ids[s], want[s][0][1:], gaps[s], want[s][1])
+        print(f"[qwen-2L B=8 mode {mode}] min top-2 logit gap over {B * steps} decisions: {gaps.min():.3e}")
+        dm.close()
+
+
+@pytest.mark.parametrize("rows", [1, 4, 11])
+def test_batched_fused_path_matches_oracle(ctx, orc, rows):
+    """Fused row-batched step (modes 1 and 2; stacked MFMA rows up to 8, two fragment sets above): greedy ids equal to
+    the oracle's per-sequence decode and to the reference call sequence, across a 512-token length bucket boundary."""
+    cfg = _toy_cfg(1, True, 128); cfg["ffn"] = 512
+    W = syn.make_weights(cfg, seed=7, std=0.08, emb_std=1.0)
+    S, steps = 560, 8
+    rng = np.random.default_rng(rows)
+    lens = rng.integers(1, 40, size=rows).astype(np.uint32)
+    lens[0] = 507                                   # crosses 512 during the run
+    KVH, HD, L = cfg["kv_heads"], cfg["head_dim"], cfg["n_layers"]
+    om = _oracle_model(orc, cfg, W, S, rows)
+    Ko, Vo = om.kv_views()
+    fills = []
+    for s in range(rows):
+        for l in range(L):
+            k16 = rng.standard_normal((int(lens[s]), KVH, HD)).astype(np.float16).view(np.uint16)
+            v16 = rng.standard_normal((int(lens[s]), KVH, HD)).astype(np.float16).view(np.uint16)
+            fills.append((s, l, k16, v16))
+            Ko[s * L + l, :lens[s]] = k16; Vo[s * L + l, :lens[s]] = v16
+    toks = rng.integers(0, cfg["vocab"], size=rows).astype(np.uint32)
+    seqs = np.arange(rows)[::-1].copy()             # rows address the sequences in reverse order
+    want = {int(s): om.decode_greedy(int(s), [toks[r]], steps, start_pos=int(lens[s]))[0][1:] for r, s in enumerate(seqs)}
+    for mode in (0, 1, 2):
+        dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=rows)
+        dm.set_mode(mode)
+        for s, l, k16, v16 in fills:
+            dm.fill_kv(s, l, k16, v16)
+        ids, gaps = dm.decode_batch_greedy(seqs, lens[seqs], toks, steps)
+        for r, s in enumerate(seqs):
+            assert np.array_equal(ids[r], want[int(s)]), (mode, r, ids[r], want[int(s)], gaps[r])
+        assert (gaps > 0).all()
+        dm.close()
 
 
 @pytest.mark.parametrize("layout,bias,hd", [(0, False, 64), (1, True, 128)])
