@@ -11,28 +11,13 @@
 // Reference semantics: three-pass softmax per q head, kv head = qh / (q_heads / kv_heads),
 // scale literals for head_dim 64 / 128: cuda/kernels.cu:1367-1655, entry points :3837-4023,
 // batched :1740-1823 and :4694-4832.
-#include "common.hpp"
+#include "attention_params.hpp"
 
 namespace {
 
 constexpr int kAttnThreads = 512;
 constexpr int kWaves = kAttnThreads / 64;
 
-struct AttnParams {
-    const uint16_t* K;
-    const uint16_t* V;
-    const float* Q;
-    float* Out;
-    float* ws;                    // partials: [batch][q_heads][nchunks][hd + 2]
-    const uint32_t* seq_ids_dev;  // may be null
-    const uint32_t* seq_lens_dev; // may be null
-    uint32_t seq_id, seq_len;
-    uint32_t max_seq_len, kv_heads, q_heads, window;
-    uint32_t chunk, nchunks;
-    uint32_t subgroups;           // q-head subgroups per kv head
-    uint32_t len_bias;            // added to a device-side length (position -> length)
-    uint32_t max_batch;           // device-side sequence ids at or above this are skipped (0 = not checked)
-};
 
 // HD in {64, 128}; G = q heads per workgroup (<= 4); S = token rows per lane group
 template <int HD, int G, int S>
@@ -293,6 +278,29 @@ template <int HD>
 int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, AttnParams& p, uint32_t batch,
               uint32_t group, uint32_t span) {
     constexpr uint32_t kRowsPerStep = kWaves * (64 / (HD / 8));   // token rows one workgroup covers per S
+    M40StreamScratch& scr = ctx->scratch[stream_kind];
+    if (span > 512) {
+        // long rows: matrix-core kernel, chunks of a multiple of 128 tokens sized so the grid covers the CUs about twice
+        p.subgroups = (group + 7) / 8;
+        const uint64_t groups = (uint64_t)batch * p.kv_heads * p.subgroups;
+        uint64_t chunk = ((uint64_t)span * groups + 2ull * ctx->num_cus - 1) / (2ull * ctx->num_cus);
+        chunk = ((chunk + 127) / 128) * 128;
+        if (chunk < 128) chunk = 128;
+        if (chunk > 2048) chunk = 2048;
+        for (;;) {
+            p.chunk = (uint32_t)chunk;
+            p.nchunks = (span + p.chunk - 1) / p.chunk;
+            if (p.nchunks == 1 || (size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float) <= scr.attn_partial_bytes) break;
+            chunk *= 2;
+        }
+        p.ws = static_cast<float*>(scr.attn_partial);
+        m40_launch_attn_mfma(stream, p, HD, batch);
+        if (p.nchunks > 1) {
+            dim3 grid(p.q_heads, batch);
+            attn_combine_kernel<HD><<<grid, 256, 0, stream>>>(p);
+        }
+        return 0;
+    }
     int G = group >= 4 ? 4 : (group >= 2 ? 2 : 1);
     const uint64_t rows = (uint64_t)batch * p.kv_heads;
     // Short rows are latency-bound, not bandwidth-bound: spread the q heads over more workgroups

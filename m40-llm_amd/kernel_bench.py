@@ -218,6 +218,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--only", default="attn,gemv,gemm8,q80,bsel,decode8")
     ap.add_argument("--json", default=None)
+    ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
     which = set(args.only.split(","))
     b = Bench()
@@ -233,7 +234,7 @@ def main():
     if "bsel" in which:
         bench_block_select(b)
     if "decode8" in which:
-        bench_decode_batch(b)
+        bench_decode_batch(b, mode=args.decode_mode)
     if args.json:
         with open(args.json, "w") as f:
             for r in b.rows:
