@@ -338,7 +338,7 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
 
 static int launch_q80(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint8_t* B,
                       float* C, int M, int N, int K) {
-    if (m40_aligned16(B) && m40_skinny_supported(ctx, stream_kind, M, N, K, 1))
+    if (m40_aligned16(B) && m40_aligned16(A) && m40_skinny_supported(ctx, stream_kind, M, N, K, 1))
         return m40_launch_skinny(ctx, stream, stream_kind, 1, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     (void)hipGetLastError();
     for (int r0 = 0; r0 < M; r0 += 4) {
@@ -434,7 +434,8 @@ int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_
     const uint8_t* wu = static_cast<const uint8_t*>(d_w_up_q80);
     const uint8_t* wd = static_cast<const uint8_t*>(d_w_down_q80);
     float* out = static_cast<float*>(d_out_f32);
-    if (m40_aligned16(wg) && m40_aligned16(wu) && m40_aligned16(wd) && m40_skinny_supported(ctx, 1, M, ffn, d_model, 1) &&
+    if (m40_aligned16(wg) && m40_aligned16(wu) && m40_aligned16(wd) && m40_aligned16(x) && m40_aligned16(gate) &&
+        m40_skinny_supported(ctx, 1, M, ffn, d_model, 1) &&
         m40_skinny_supported(ctx, 1, M, d_model, ffn, 1)) {
         // gate and up in one launch; SwiGLU is applied while the hidden row is packed for the down projection
         int rc = m40_launch_skinny(ctx, ctx->decode_stream, 1, 1, x, nullptr, wg, gate, wu, up, M, ffn, d_model);

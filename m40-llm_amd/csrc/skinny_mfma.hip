@@ -25,86 +25,6 @@ constexpr int kQ8TileBytes = 16 * 272;            // 16 columns x 8 blocks x 34 
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-// ---- activation packing -----------------------------------------------------------------------------------
-// Fragment i (k = 32 i .. 32 i + 31) is 64 x 16 bytes: entry g*16 + row holds the eight halves k = 32 i + 8 g + 0..7
-// of that row.  STACKED (M <= 8): rows 0-7 hold hi, rows 8-15 lo.  Otherwise two fragment sets: hi, then lo at
-// +K/32*64 entries.  With `up`, the packed value is silu(A) * up (the SwiGLU of an FFN) instead of A.
-// With `norm_w`, the packed value is the RMS-normalised row: A * rsqrt(mean(A^2) + eps) * norm_w.
-__global__ __launch_bounds__(256) void pack_a_blocked_kernel(const float* __restrict__ A, const float* __restrict__ up,
-                                                             const void* __restrict__ norm_w, uint32_t norm_dtype, float eps,
-                                                             int M, int K, int stacked, uint4* __restrict__ P,
-                                                             float* __restrict__ row_scale) {
-    __shared__ float wave_max[4];
-    __shared__ float wave_sq[4];
-    const int row = blockIdx.x;  // 0..7 (stacked) or 0..15
-    const int tid = threadIdx.x;
-    // grid.y slices the fragments; every slice recomputes the row maximum (the row sits in L2)
-    const bool live = row < M;
-    float rms = 1.0f;
-    if (live && norm_w) {
-        float sq = 0.0f;
-#pragma unroll 4
-        for (int k = tid; k < K; k += 256) {
-            const float a = A[(size_t)row * K + k];
-            sq = fmaf(a, a, sq);
-        }
-        sq = m40_sum64(sq);
-        if ((tid & 63) == 0) wave_sq[tid >> 6] = sq;
-        __syncthreads();
-        rms = rsqrtf((wave_sq[0] + wave_sq[1] + wave_sq[2] + wave_sq[3]) / (float)K + eps);
-    }
-    const uint16_t* nw16 = static_cast<const uint16_t*>(norm_w);
-    const float* nw32 = static_cast<const float*>(norm_w);
-    auto value = [&](int k) -> float {
-        const float a = A[(size_t)row * K + k];
-        if (norm_w) return a * rms * (norm_dtype == 0u ? m40_h2f(nw16[k]) : nw32[k]);
-        if (!up) return a;
-        return a / (1.0f + expf(-a)) * up[(size_t)row * K + k];
-    };
-    float inv_scale = 1.0f, scale = 1.0f;
-    if (live) {
-        float mx = 0.0f;
-#pragma unroll 4
-        for (int k = tid; k < K; k += 256) mx = fmaxf(mx, fabsf(value(k)));
-        mx = m40_max64(mx);
-        if ((tid & 63) == 0) wave_max[tid >> 6] = mx;
-        __syncthreads();
-        mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-        if (mx > 0.0f && mx < INFINITY) {
-            int e;
-            (void)frexpf(mx, &e);         // mx = f * 2^e, f in [0.5, 1)
-            e -= 11;                      // scaled max in [2^10, 2^11)
-            e = e < -100 ? -100 : (e > 100 ? 100 : e);
-            scale = ldexpf(1.0f, e);
-            inv_scale = ldexpf(1.0f, -e);
-        }
-    }
-    if (tid == 0 && blockIdx.y == 0) row_scale[row] = scale;
-    const int frags = K >> 5;
-    uint4* P_lo = P + (size_t)frags * 64;
-    const int f_begin = (int)(((long long)blockIdx.y * frags * 4) / gridDim.y);
-    const int f_end = (int)(((long long)(blockIdx.y + 1) * frags * 4) / gridDim.y);
-    for (int f = f_begin + tid; f < f_end; f += 256) {
-        const int g = f & 3, i = f >> 2;
-        const int k0 = 32 * i + 8 * g;
-        uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
-        if (live) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float a = value(k0 + j) * inv_scale;
-                const _Float16 h = static_cast<_Float16>(a);
-                const _Float16 l = static_cast<_Float16>(a - static_cast<float>(h));
-                hi[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (j & 1));
-                lo[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, l) << (16 * (j & 1));
-            }
-        }
-        const size_t base = (size_t)i * 64 + (size_t)g * 16;
-        P[base + row] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-        if (stacked) P[base + row + 8] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        else P_lo[base + row] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-    }
-}
-
 __device__ __forceinline__ m40_float4 mfma16x16x32(const uint4& a, const uint4& b, m40_float4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(m40_half8, a),
                                                   __builtin_bit_cast(m40_half8, b), c, 0, 0, 0);
@@ -118,8 +38,11 @@ __device__ __forceinline__ uint32_t q8_pair_to_f16(uint32_t spread) {
 }
 
 struct SkinnyArgs {
-    const uint4* P;            // packed activations
-    const float* row_scale;
+    const float* A;            // activations [M][K], f32
+    const float* up;           // not null: the operand is silu(A) * up (SwiGLU of an FFN)
+    const void* norm_w;        // not null: the operand is A * rsqrt(mean(A^2) + eps) * norm_w (RMSNorm)
+    uint32_t norm_dtype;       // 0 f16, 1 f32
+    float eps;
     const void* W[3];          // up to three weight matrices with the same K (Q/K/V, gate/up)
     float* C[3];               // direct outputs [M][N z] (S == 1 and no epilogue kernel)
     int N[3];
@@ -148,8 +71,7 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
     const int n0 = (gtile - p.tile_begin[z]) * 16;
     const int KT = p.K / kTileK;
     const int kt0 = (int)(((long long)blockIdx.y * KT) / p.S), kt1 = (int)(((long long)(blockIdx.y + 1) * KT) / p.S);
-    const int frags_total = p.K >> 5;
-    const uint4* P_lo = p.P + (size_t)frags_total * 64;
+    __shared__ float scale_s[16];      // factor that undoes each row's power-of-two scaling (this K slice)
 
     // ---- weight addressing
     const int col = n0 + j < N ? n0 + j : N - 1;
@@ -174,12 +96,34 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
         }
     }
 
-    uint4 ra[kASets];          // this thread's share of the activation fragments of a step
+    // ---- activation addressing: 32 threads per row, thread (arow, acol) owns k = 256 kt + 8 acol .. +7 of a step,
+    // which is entry (MFMA i = acol / 4, group acol % 4) of the step's fragments
+    constexpr int kARows = STACKED ? 8 : 16;
+    const int arow = tid >> 5, acol = tid & 31;
+    const bool a_thread = arow < kARows;
+    const bool a_live = a_thread && arow < p.M;
+    const float* a_ptr = p.A + (size_t)(a_live ? arow : 0) * p.K + 8 * acol;
+    const float* u_ptr = p.up ? p.up + (size_t)(a_live ? arow : 0) * p.K + 8 * acol : nullptr;
+    const uint16_t* nw16 = static_cast<const uint16_t*>(p.norm_w);
+    const float* nw32 = static_cast<const float*>(p.norm_w);
+    auto load8 = [&](const float* src, float (&v)[8]) {
+        const float4 x0 = *reinterpret_cast<const float4*>(src);
+        const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
+        v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+    };
+    auto load_norm8 = [&](int k, float (&v)[8]) {
+        if (p.norm_dtype == 0u) m40_unpack8(*reinterpret_cast<const uint4*>(nw16 + k), v);
+        else load8(nw32 + k, v);
+    };
+
+    float fa[8], fb[8];        // this thread's activations of a step (and their SwiGLU partner or norm weights)
     uint4 rb[8];               // f16: the eight 16-byte weight loads of a step; q8_0: five tile pieces
     auto issue_loads = [&](int kt) {
-        const size_t f0 = (size_t)kt * 8 * 64;
-        ra[0] = p.P[f0 + tid];
-        if (!STACKED) ra[1] = P_lo[f0 + tid];
+        if (a_thread) {
+            load8(a_ptr + (size_t)kt * kTileK, fa);
+            if (u_ptr) load8(u_ptr + (size_t)kt * kTileK, fb);
+            else if (p.norm_w) load_norm8(kt * kTileK + 8 * acol, fb);
+        }
         if (FMT == 0) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
@@ -192,11 +136,76 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
     };
 
     m40_float4 acc = {0.f, 0.f, 0.f, 0.f};
-    if (kt0 < kt1) issue_loads(kt0);
+    if (kt0 < kt1) issue_loads(kt0);           // weights of the first step are in flight during the prologue
+
+    // ---- per-row statistics: RMS over the whole row (RMSNorm), largest operand of this K slice -> power-of-two scale
+    float rms = 1.0f, inv_scale = 1.0f;
+    if (a_thread) {
+        if (p.norm_w && a_live) {
+            float sq = 0.0f;
+            for (int k = 0; k < p.K; k += kTileK) {
+                float v[8];
+                load8(a_ptr + k, v);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sq = fmaf(v[e], v[e], sq);
+            }
+#pragma unroll
+            for (int o = 1; o < 32; o <<= 1) sq += __shfl_xor(sq, o, 64);
+            rms = rsqrtf(sq / (float)p.K + p.eps);
+        }
+        float mx = 0.0f;
+        if (a_live) {
+            for (int kt = kt0; kt < kt1; ++kt) {
+                float v[8], w[8];
+                load8(a_ptr + (size_t)kt * kTileK, v);
+                if (u_ptr) load8(u_ptr + (size_t)kt * kTileK, w);
+                else if (p.norm_w) load_norm8(kt * kTileK + 8 * acol, w);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float x = v[e];
+                    if (u_ptr) x = x / (1.0f + expf(-x)) * w[e];
+                    else if (p.norm_w) x = x * rms * w[e];
+                    mx = fmaxf(mx, fabsf(x));
+                }
+            }
+        }
+#pragma unroll
+        for (int o = 1; o < 32; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        float scale = 1.0f;
+        if (mx > 0.0f && mx < INFINITY) {
+            int e;
+            (void)frexpf(mx, &e);         // mx = f * 2^e, f in [0.5, 1)
+            e -= 11;                      // scaled maximum in [2^10, 2^11)
+            e = e < -100 ? -100 : (e > 100 ? 100 : e);
+            scale = ldexpf(1.0f, e);
+            inv_scale = ldexpf(1.0f, -e);
+        }
+        if (acol == 0) scale_s[arow] = scale;
+    }
+
     for (int kt = kt0; kt < kt1; ++kt) {
         const int buf = kABufs == 2 ? ((kt - kt0) & 1) : 0;
-        a_lds[buf][0][tid] = ra[0];
-        if (!STACKED) a_lds[buf][1][tid] = ra[1];
+        if (a_thread) {
+            // f32 -> f16 hi + f16 lo of the scaled operand, straight into the step's fragment entries
+            uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+            if (a_live) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float x = fa[e];
+                    if (u_ptr) x = x / (1.0f + expf(-x)) * fb[e];
+                    else if (p.norm_w) x = x * rms * fb[e];
+                    x *= inv_scale;
+                    const _Float16 h = static_cast<_Float16>(x);
+                    const _Float16 l = static_cast<_Float16>(x - static_cast<float>(h));
+                    hi[e >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (e & 1));
+                    lo[e >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, l) << (16 * (e & 1));
+                }
+            }
+            const int entry = (acol >> 2) * 64 + (acol & 3) * 16 + arow;
+            a_lds[buf][0][entry] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            if (STACKED) a_lds[buf][0][entry + 8] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            else a_lds[buf][kASets - 1][entry] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        }
         uint4 wb[8];
         if (FMT == 0) {
 #pragma unroll
@@ -254,14 +263,14 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
         if (p.direct) {
-            if (row < p.M) p.C[z][(size_t)row * N + n0 + j] = acc[r] * p.row_scale[row];
+            if (row < p.M) p.C[z][(size_t)row * N + n0 + j] = acc[r] * scale_s[row];
         } else {
-            p.partial[p.part_off[z] + ((size_t)blockIdx.y * 16 + row) * N + n0 + j] = acc[r];
+            p.partial[p.part_off[z] + ((size_t)blockIdx.y * 16 + row) * N + n0 + j] = acc[r] * scale_s[row];
         }
     }
 }
 
-// scaled sum over the K slices (ascending) of one output element
+// sum over the K slices (ascending) of one output element
 __device__ __forceinline__ float skinny_sum(const SkinnyArgs& p, int z, int row, int n) {
     const float* src = p.partial + p.part_off[z] + (size_t)row * p.N[z] + n;
     const size_t slice_stride = (size_t)16 * p.N[z];
@@ -271,7 +280,7 @@ __device__ __forceinline__ float skinny_sum(const SkinnyArgs& p, int z, int row,
     float v = 0.0f;
 #pragma unroll
     for (int s = 0; s < 16; ++s) v += part[s];
-    return v * p.row_scale[row];
+    return v;
 }
 
 // Epilogue over the slice partials; grid (ceil(N/256), rows, matrices).
@@ -411,15 +420,15 @@ struct PackSpec {
     float eps;
 };
 
-// Packs `m` (<= 16) rows and launches the MFMA kernel over nmat matrices.  Returns the filled args (for an
+// Launches the MFMA kernel for `m` (<= 16) rows over nmat matrices.  Returns the filled args (for an
 // epilogue kernel) through *out; direct != 0 writes scaled results to C when the K range is not split.
 int launch_core(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const PackSpec& pk, int m, int K,
                 int nmat, const void* const* W, const int* N, float* const* C, bool want_direct, SkinnyArgs* out) {
     M40StreamScratch& sc = ctx->scratch[stream_kind];
-    float* row_scale = static_cast<float*>(sc.gemm_pack);
-    uint4* P = reinterpret_cast<uint4*>(static_cast<char*>(sc.gemm_pack) + 256);
+    if (!m40_aligned16(pk.A) || (pk.up && !m40_aligned16(pk.up)) || (pk.norm_w && !m40_aligned16(pk.norm_w))) return -2;
     SkinnyArgs a{};
-    a.P = P; a.row_scale = row_scale; a.partial = static_cast<float*>(sc.attn_partial);
+    a.A = pk.A; a.up = pk.up; a.norm_w = pk.norm_w; a.norm_dtype = pk.norm_dtype; a.eps = pk.eps;
+    a.partial = static_cast<float*>(sc.attn_partial);
     a.nmat = nmat; a.M = m; a.K = K;
     int tiles = 0;
     size_t n_total = 0;
@@ -442,9 +451,6 @@ int launch_core(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind
         off += (size_t)S * 16 * N[z];
     }
     const bool stacked = m <= 8;
-    const int pack_slices = K >= 8192 ? 8 : (K >= 2048 ? 4 : 1);
-    pack_a_blocked_kernel<<<dim3(stacked ? 8 : 16, pack_slices), 256, 0, stream>>>(pk.A, pk.up, pk.norm_w, pk.norm_dtype, pk.eps, m,
-                                                                                   K, stacked ? 1 : 0, P, row_scale);
     dim3 grid((tiles + kWavesPerGroup - 1) / kWavesPerGroup, S);
     if (fmt == 0) {
         if (stacked) skinny_mfma_kernel<0, true><<<grid, kThreads, 0, stream>>>(a);
@@ -472,7 +478,8 @@ void launch_plain_epilogue(hipStream_t stream, const SkinnyArgs& a, int nmat, fl
 }
 
 bool rows_ok(const M40llmCudaContext* ctx, int rows, int K) {
-    return rows >= 1 && rows <= 16 && K > 0 && K % kTileK == 0 && (size_t)K * 64 + 256 <= ctx->scratch[1].gemm_pack_bytes;
+    (void)ctx;
+    return rows >= 1 && rows <= 16 && K > 0 && K % kTileK == 0;
 }
 
 }  // namespace
@@ -481,8 +488,8 @@ bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, in
     (void)M;
     if (K % kTileK != 0 || N <= 0) return false;
     if (fmt != 0 && fmt != 1) return false;
-    const M40StreamScratch& sc = ctx->scratch[stream_kind];
-    return (size_t)K * 64 + 256 <= sc.gemm_pack_bytes;
+    (void)ctx; (void)stream_kind;
+    return true;
 }
 
 // up != nullptr: the activations are silu(A) * up.  W1/C1 may be null (one matrix).

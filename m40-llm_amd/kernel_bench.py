@@ -100,6 +100,10 @@ def bench_attention(b: Bench):
     b.time("attention_gqa_batched", f"B8 qh16 kvh2 hd128 lens U[256,4096] sum {int(lens.sum())}", algo,
            lambda i: b.call("m40llm_attention_last_token_f32_gqa_batched_async", kv.h, ids[i].ptr, dl.ptr, B, q.ptr, qh,
                             out.ptr), nset)
+    lens_m1 = b.ctx.to_device((lens - 1).astype(np.uint32))
+    b.time("attention_gqa_batched (lens on device)", f"B8 qh16 kvh2 hd128 lens U[256,4096] sum {int(lens.sum())}", algo,
+           lambda i: b.call("m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async", kv.h, ids[i].ptr, lens_m1.ptr, 1, B,
+                            4096, q.ptr, qh, out.ptr), nset)
     kv.destroy()
 
 
