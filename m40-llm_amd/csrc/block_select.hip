@@ -94,170 +94,209 @@ __global__ __launch_bounds__(256) void bs_score_kernel(BsParams p) {
 }
 
 // ---- 2. top-k selection per q head -----------------------------------------------------------
+// Rank by counting: block b is at rank #{o : score[o] > score[b] or (== and o < b)}, which is the order the
+// reference's strict-'>' insertion produces (cuda/kernels.cu:2980-3022).  Grid (q head, 128 candidates); eight lanes
+// share the count of one candidate.  The workgroup that owns the last block also writes the list length, the
+// attended-token count and the unused tail of the list.
 __global__ __launch_bounds__(1024) void bs_select_kernel(BsParams p) {
     extern __shared__ float s_sc[];  // [nblk]
+    __shared__ uint32_t s_valid[16];
+    __shared__ uint32_t s_last_rank;
     const uint32_t qh = blockIdx.x;
     const float* sc = p.scores + (size_t)qh * p.nblk;
-    for (uint32_t b = threadIdx.x; b < p.nblk; b += blockDim.x) s_sc[b] = sc[b];
-    for (uint32_t i = threadIdx.x; i < 64; i += blockDim.x) {
-        p.sel[qh * 64 + i] = 0xffffffffu;
-        p.sel_scores[qh * 64 + i] = -1e30f;
+    uint32_t valid = 0;
+    for (uint32_t b = threadIdx.x; b < p.nblk; b += 1024u) {
+        const float v = sc[b];
+        s_sc[b] = v;
+        valid += (v > -1e30f) ? 1u : 0u;       // NaN and anything <= -1e30 never enter the list
     }
-    __shared__ uint32_t s_count, s_tok;
-    if (threadIdx.x == 0) { s_count = 0; s_tok = 0; }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) valid += __shfl_xor(valid, o, 64);
+    if ((threadIdx.x & 63u) == 0u) s_valid[threadIdx.x >> 6] = valid;
+    if (threadIdx.x == 0) s_last_rank = 0xffffffffu;
     __syncthreads();
-    for (uint32_t b = threadIdx.x; b < p.nblk; b += blockDim.x) {
-        const float s = s_sc[b];
-        if (!(s > -1e30f)) continue;       // NaN and anything <= -1e30 never enter the list
-        uint32_t rank = 0;
-        for (uint32_t o = 0; o < p.nblk; ++o) {
+    const uint32_t b = blockIdx.y * 128u + (threadIdx.x >> 3), part = threadIdx.x & 7u;
+    uint32_t rank = 0;
+    float s = 0.0f;
+    const bool cand = b < p.nblk;
+    if (cand) {
+        s = s_sc[b];
+        const uint32_t o_begin = (uint32_t)(((uint64_t)part * p.nblk) / 8u), o_end = (uint32_t)(((uint64_t)(part + 1u) * p.nblk) / 8u);
+        for (uint32_t o = o_begin; o < o_end; ++o) {
             const float so = s_sc[o];
             rank += (so > s || (so == s && o < b)) ? 1u : 0u;
         }
-        if (rank < p.top_n) {
-            p.sel[qh * 64 + rank] = b;
-            p.sel_scores[qh * 64 + rank] = s;
-            const uint32_t start = b * p.block_size;
-            const uint32_t end = start + p.block_size < p.old_len ? start + p.block_size : p.old_len;
-            atomicAdd(&s_count, 1u);
-            atomicAdd(&s_tok, end - start);
+    }
+    rank += __shfl_xor(rank, 1, 64);
+    rank += __shfl_xor(rank, 2, 64);
+    rank += __shfl_xor(rank, 4, 64);
+    const bool listed = cand && part == 0u && (s > -1e30f) && rank < p.top_n;
+    if (listed) {
+        p.sel[qh * 64 + rank] = b;
+        p.sel_scores[qh * 64 + rank] = s;
+    }
+    if (cand && part == 0u && b + 1u == p.nblk) s_last_rank = listed ? rank : 0xffffffffu;
+    __syncthreads();
+    if (blockIdx.y == gridDim.y - 1u) {
+        uint32_t total_valid = 0;
+        for (int w = 0; w < 16; ++w) total_valid += s_valid[w];
+        const uint32_t count = total_valid < p.top_n ? total_valid : p.top_n;
+        for (uint32_t i = count + threadIdx.x; i < 64u; i += 1024u) {
+            p.sel[qh * 64 + i] = 0xffffffffu;
+            p.sel_scores[qh * 64 + i] = -1e30f;
+        }
+        if (threadIdx.x == 0) {
+            uint32_t tokens = count * p.block_size;
+            if (s_last_rank != 0xffffffffu) tokens -= p.nblk * p.block_size - p.old_len;   // the last block may be partial
+            p.counts[qh] = count;
+            p.ntok[qh] = tokens + (p.seq_len - p.old_len);
         }
     }
-    __syncthreads();
+}
+
+// no old blocks: empty lists, every q head attends the recent tokens only
+__global__ void bs_empty_selection_kernel(BsParams p) {
+    const uint32_t qh = blockIdx.x;
+    for (uint32_t i = threadIdx.x; i < 64u; i += blockDim.x) {
+        p.sel[qh * 64 + i] = 0xffffffffu;
+        p.sel_scores[qh * 64 + i] = -1e30f;
+    }
     if (threadIdx.x == 0) {
-        p.counts[qh] = s_count;
-        p.ntok[qh] = s_tok + (p.seq_len - p.old_len);
+        p.counts[qh] = 0;
+        p.ntok[qh] = p.seq_len - p.old_len;
     }
 }
 
 // ---- 3. attention over the token list ---------------------------------------------------------
+// Grid (q head, chunk of 128 list positions).  Eight waves; every lane issues the K and V loads of all of its token
+// rows before any arithmetic (one memory round trip per workgroup), scores stay in registers.
+constexpr int kBsChunk = 128;
 template <int HD>
-__global__ __launch_bounds__(256) void bs_attend_kernel(BsParams p) {
-    constexpr int LPT = HD / 8, TPW = 64 / LPT, kWaves = 4;
-    extern __shared__ float lds[];
-    float* sc = lds;                                                   // [chunk]
-    uint32_t* tok = reinterpret_cast<uint32_t*>(sc + p.chunk);         // [chunk]
-    float* red = reinterpret_cast<float*>(tok + p.chunk);              // [kWaves][HD]
-    float* wred = red + kWaves * HD;                                   // [2*kWaves]
+__global__ __launch_bounds__(512) void bs_attend_kernel(BsParams p) {
+    constexpr int LPT = HD / 8, TPW = 64 / LPT, kWaves = 8;
+    constexpr int S = kBsChunk / (kWaves * TPW);
     __shared__ uint32_t pre[65];
+    __shared__ float red[kWaves][HD];
+    __shared__ float wmax[kWaves], wsum[kWaves];
 
     const uint32_t qh = blockIdx.x;
     const uint32_t n = p.ntok[qh];
-    const uint32_t cbeg = blockIdx.y * p.chunk;
+    const uint32_t cbeg = blockIdx.y * kBsChunk;
     if (cbeg >= n) return;
-    const uint32_t cend = cbeg + p.chunk < n ? cbeg + p.chunk : n;
+    const uint32_t cend = cbeg + kBsChunk < n ? cbeg + kBsChunk : n;
     const uint32_t count = p.counts[qh];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 
-    // list position -> token id.  pre[r] = first list position of the r-th selected block.
-    if (tid == 0) {
-        uint32_t acc = 0;
-        for (uint32_t r = 0; r < count; ++r) {
-            pre[r] = acc;
-            const uint32_t b = p.sel[qh * 64 + r];
+    // pre[r] = first list position of the r-th selected block (exclusive prefix of the block lengths)
+    if (wave == 0) {
+        uint32_t len = 0;
+        if ((uint32_t)lane < count) {
+            const uint32_t b = p.sel[qh * 64 + lane];
             const uint32_t start = b * p.block_size;
             const uint32_t end = start + p.block_size < p.old_len ? start + p.block_size : p.old_len;
-            acc += end - start;
+            len = end - start;
         }
-        pre[count] = acc;
+        uint32_t incl = len;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
+        }
+        pre[lane] = incl - len;
+        if (lane == 63) pre[64] = incl;
     }
     __syncthreads();
-    const uint32_t old_tokens = pre[count];
-    for (uint32_t i = tid; i < p.chunk; i += 256) {
-        const uint32_t pos = cbeg + i;
-        uint32_t t = 0xffffffffu;
-        if (pos < cend) {
-            if (pos >= old_tokens) {
-                t = p.old_len + (pos - old_tokens);
-            } else {
-                uint32_t r = 0;
-                while (r + 1 < count && pre[r + 1] <= pos) ++r;
-                t = p.sel[qh * 64 + r] * p.block_size + (pos - pre[r]);
-            }
-        }
-        tok[i] = t;
-    }
-    __syncthreads();
+    const uint32_t old_tokens = pre[64];
 
     const uint32_t kvh = qh / (p.q_heads / p.kv_heads);
     const int c = lane % LPT, tg = lane / LPT;
     const size_t row_stride = (size_t)p.kv_heads * HD;
     const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
-    float q[8];
-    {
-        const float* qp = p.Q + (size_t)qh * HD + 8 * c;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) q[j] = qp[j];
-    }
-    const uint32_t per_wave = p.chunk / kWaves;
 
-    // pass A: scores
-    float lmax = -INFINITY;
-    for (uint32_t it = 0; it < per_wave; it += TPW) {
-        const uint32_t tl = wave * per_wave + it + tg;
-        const uint32_t t = tok[tl];
-        const bool valid = t != 0xffffffffu;
-        uint4 kw = make_uint4(0, 0, 0, 0);
-        if (valid) {
+    uint4 kw[S], vw[S];
+    bool valid[S], quant[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const uint32_t pos = cbeg + (uint32_t)((s * kWaves + wave) * TPW + tg);
+        valid[s] = pos < cend;
+        quant[s] = false;
+        kw[s] = make_uint4(0, 0, 0, 0);
+        vw[s] = make_uint4(0, 0, 0, 0);
+        if (valid[s]) {
+            uint32_t t;
+            if (pos >= old_tokens) {
+                t = p.old_len + (pos - old_tokens);
+            } else {
+                uint32_t lo = 0, hi = count;          // largest r with pre[r] <= pos
+                while (hi - lo > 1u) {
+                    const uint32_t mid = (lo + hi) >> 1;
+                    if (pre[mid] <= pos) lo = mid; else hi = mid;
+                }
+                t = p.sel[qh * 64 + lo] * p.block_size + (pos - pre[lo]);
+            }
             const uint16_t* kp;
             if (t < p.old_len) kp = p.old_k + (size_t)t * row_stride;
             else kp = p.new_k + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
-            kw = *reinterpret_cast<const uint4*>(kp + (size_t)kvh * HD + 8 * c);
+            kw[s] = *reinterpret_cast<const uint4*>(kp + (size_t)kvh * HD + 8 * c);
+            if (p.compressed && t < p.old_len) {
+                quant[s] = true;
+                vw[s].x = *reinterpret_cast<const uint32_t*>(p.q4_v + ((size_t)t * p.kv_heads + kvh) * (HD / 2) + 4 * c);
+                vw[s].y = __float_as_uint(p.q4_scale[(size_t)t * p.kv_heads + kvh]);
+            } else {
+                const uint16_t* vp = p.dense_v + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
+                vw[s] = *reinterpret_cast<const uint4*>(vp + (size_t)kvh * HD + 8 * c);
+            }
         }
+    }
+    float q[8];
+    {
+        const float4 q0 = *reinterpret_cast<const float4*>(p.Q + (size_t)qh * HD + 8 * c);
+        const float4 q1 = *reinterpret_cast<const float4*>(p.Q + (size_t)qh * HD + 8 * c + 4);
+        q[0] = q0.x; q[1] = q0.y; q[2] = q0.z; q[3] = q0.w; q[4] = q1.x; q[5] = q1.y; q[6] = q1.z; q[7] = q1.w;
+    }
+    float sc[S];
+    float lmax = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
         float kf[8];
-        m40_unpack8(kw, kf);
+        m40_unpack8(kw[s], kf);
         float d = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) d = fmaf(q[j], kf[j], d);
         d = LPT == 8 ? m40_sum8(d) : m40_sum16(d);
-        const float s = valid ? d * inv_sqrt : -INFINITY;
-        lmax = fmaxf(lmax, s);
-        if (c == 0) sc[tl] = s;
+        sc[s] = valid[s] ? d * inv_sqrt : -INFINITY;
+        lmax = fmaxf(lmax, sc[s]);
     }
     lmax = m40_max64(lmax);
-    if (lane == 0) wred[wave] = lmax;
+    if (lane == 0) wmax[wave] = lmax;
     __syncthreads();
-    const float m = fmaxf(fmaxf(wred[0], wred[1]), fmaxf(wred[2], wred[3]));
+    float m = wmax[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) m = fmaxf(m, wmax[w]);
 
-    // pass B0: exp and row sum
     float lsum = 0.0f;
-    for (uint32_t tl = tid; tl < p.chunk; tl += 256) {
-        const float s = sc[tl];
-        const float e = s == -INFINITY ? 0.0f : expf(s - m);
-        sc[tl] = e;
-        lsum += e;
-    }
-    lsum = m40_sum64(lsum);
-    if (lane == 0) wred[kWaves + wave] = lsum;
-    __syncthreads();
-
-    // pass B: weighted V
     float acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
-    for (uint32_t it = 0; it < per_wave; it += TPW) {
-        const uint32_t tl = wave * per_wave + it + tg;
-        const uint32_t t = tok[tl];
-        if (t == 0xffffffffu) continue;
-        const float pw = sc[tl];
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const float e = valid[s] ? expf(sc[s] - m) : 0.0f;
+        if (c == 0) lsum += e;
         float vf[8];
-        if (p.compressed && t < p.old_len) {
-            const uint32_t packed = *reinterpret_cast<const uint32_t*>(
-                p.q4_v + ((size_t)t * p.kv_heads + kvh) * (HD / 2) + 4 * c);
-            const float scale = p.q4_scale[(size_t)t * p.kv_heads + kvh];
+        if (quant[s]) {
+            const uint32_t packed = vw[s].x;
+            const float scale = __uint_as_float(vw[s].y);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int nib = (int)((packed >> (4 * j)) & 0xfu);
                 const int sv = nib >= 8 ? nib - 16 : nib;
-                vf[j] = m40_h2f(m40_f2h((float)sv * scale));
+                vf[j] = m40_h2f(m40_f2h((float)sv * scale));       // the reference rounds the product through f16
             }
         } else {
-            const uint16_t* vp = p.dense_v + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
-            const uint4 vw = *reinterpret_cast<const uint4*>(vp + (size_t)kvh * HD + 8 * c);
-            m40_unpack8(vw, vf);
+            m40_unpack8(vw[s], vf);
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] = fmaf(pw, vf[j], acc[j]);
+        for (int j = 0; j < 8; ++j) acc[j] = fmaf(e, vf[j], acc[j]);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -266,17 +305,19 @@ __global__ __launch_bounds__(256) void bs_attend_kernel(BsParams p) {
         for (int o = LPT; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
         acc[j] = v;
     }
+    lsum = m40_sum64(lsum);
+    if (lane == 0) wsum[wave] = lsum;
     if (tg == 0) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) red[wave * HD + 8 * c + j] = acc[j];
+        for (int j = 0; j < 8; ++j) red[wave][8 * c + j] = acc[j];
     }
     __syncthreads();
     if (tid < HD) {
         float v = 0.0f, l = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) {
-            v += red[w * HD + tid];
-            l += wred[kWaves + w];
+            v += red[w][tid];
+            l += wsum[w];
         }
         if (p.nchunks == 1) {
             p.Out[(size_t)qh * HD + tid] = v / (l > 0.0f ? l : 1.0f);
@@ -288,22 +329,44 @@ __global__ __launch_bounds__(256) void bs_attend_kernel(BsParams p) {
     }
 }
 
+// Merge the chunk partials of one q head: 1024 threads = 1024/HD chunk lanes x HD dims, each lane folds chunks
+// lane, lane + n_lanes, ... with a running maximum; the lanes are then folded in order.
 template <int HD>
-__global__ __launch_bounds__(HD) void bs_combine_kernel(BsParams p) {
-    const uint32_t qh = blockIdx.x, d = threadIdx.x;
-    const uint32_t n = (p.ntok[qh] + p.chunk - 1) / p.chunk;
+__global__ __launch_bounds__(1024) void bs_combine_kernel(BsParams p) {
+    constexpr int NCG = 1024 / HD;
+    __shared__ float s_m[NCG], s_den[NCG];
+    __shared__ float s_num[NCG][HD];
+    const uint32_t qh = blockIdx.x, d = threadIdx.x % HD, cg = threadIdx.x / HD;
+    const uint32_t n = (p.ntok[qh] + kBsChunk - 1) / kBsChunk;
     if (n == 0) return;
     const float* w = p.partial + (size_t)qh * p.nchunks * (HD + 2);
-    float M = -INFINITY;
-    for (uint32_t c = 0; c < n; ++c) M = fmaxf(M, w[(size_t)c * (HD + 2)]);
-    float num = 0.0f, den = 0.0f;
-    for (uint32_t c = 0; c < n; ++c) {
-        const float* wc = w + (size_t)c * (HD + 2);
-        const float f = expf(wc[0] - M);
-        num = fmaf(wc[2 + d], f, num);
-        den = fmaf(wc[1], f, den);
+    float m = -INFINITY, num = 0.0f, den = 0.0f;
+    for (uint32_t ch = cg; ch < n; ch += NCG) {
+        const float* wc = w + (size_t)ch * (HD + 2);
+        const float mc = wc[0], lc = wc[1], vc = wc[2 + d];
+        const float nm = fmaxf(m, mc);
+        const float fa = m == -INFINITY ? 0.0f : expf(m - nm);
+        const float fb = mc == -INFINITY ? 0.0f : expf(mc - nm);
+        num = fmaf(num, fa, vc * fb);
+        den = fmaf(den, fa, lc * fb);
+        m = nm;
     }
-    p.Out[(size_t)qh * HD + d] = num / (den > 0.0f ? den : 1.0f);
+    s_num[cg][d] = num;
+    if (d == 0) { s_m[cg] = m; s_den[cg] = den; }
+    __syncthreads();
+    if (cg == 0) {
+#pragma unroll
+        for (int g = 1; g < NCG; ++g) {
+            const float mc = s_m[g];
+            const float nm = fmaxf(m, mc);
+            const float fa = m == -INFINITY ? 0.0f : expf(m - nm);
+            const float fb = mc == -INFINITY ? 0.0f : expf(mc - nm);
+            num = fmaf(num, fa, s_num[g][d] * fb);
+            den = fmaf(den, fa, s_den[g] * fb);
+            m = nm;
+        }
+        p.Out[(size_t)qh * HD + d] = num / (den > 0.0f ? den : 1.0f);
+    }
 }
 
 uint32_t policy_from_env() {
@@ -358,9 +421,7 @@ int prepare(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, co
     p->sel_scores = reinterpret_cast<float*>(p->sel + (size_t)q_heads * 64);
     p->counts = reinterpret_cast<uint32_t*>(p->sel_scores + (size_t)q_heads * 64);
     p->ntok = p->counts + q_heads;
-    uint32_t chunk = 128;
-    while (chunk < 1024 && (size_t)q_heads * ((capacity + chunk - 1) / chunk) * (hd + 2) * 4 > sc.attn_partial_bytes)
-        chunk <<= 1;
+    const uint32_t chunk = kBsChunk;
     p->chunk = chunk;
     p->nchunks = (capacity + chunk - 1) / chunk;
     if ((size_t)q_heads * p->nchunks * (hd + 2) * 4 > sc.attn_partial_bytes) return -7;
@@ -379,12 +440,12 @@ int launch_all(hipStream_t s, const BsParams& p, bool selection_only) {
         else if (group >= 2) bs_score_kernel<HD, 2><<<grid, 256, 0, s>>>(p);
         else bs_score_kernel<HD, 1><<<grid, 256, 0, s>>>(p);
     }
-    bs_select_kernel<<<p.q_heads, 1024, (size_t)(p.nblk ? p.nblk : 1) * 4, s>>>(p);
+    if (p.nblk > 0) bs_select_kernel<<<dim3(p.q_heads, (p.nblk + 127) / 128), 1024, (size_t)p.nblk * 4, s>>>(p);
+    else bs_empty_selection_kernel<<<p.q_heads, 64, 0, s>>>(p);
     if (!selection_only) {
-        const size_t lds = ((size_t)2 * p.chunk + 4 * HD + 8) * sizeof(float);
         dim3 grid(p.q_heads, p.nchunks);
-        bs_attend_kernel<HD><<<grid, 256, lds, s>>>(p);
-        if (p.nchunks > 1) bs_combine_kernel<HD><<<p.q_heads, HD, 0, s>>>(p);
+        bs_attend_kernel<HD><<<grid, 512, 0, s>>>(p);
+        if (p.nchunks > 1) bs_combine_kernel<HD><<<p.q_heads, 1024, 0, s>>>(p);
     }
     return hipGetLastError() == hipSuccess ? 0 : -8;
 }
