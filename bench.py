@@ -77,6 +77,18 @@ def measure_dominant_kernel(pkg, ctx, dm, cfg, reps, mode):
     return dict(kernel=name, shape=shape, launches=n, avg_us=ms * 1e3 / n, bytes=bytes_per_launch)
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
+    each scaled by the same counter's reading for a copy of known size); None when no summary covers the kernel."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "decode_b1_tinyllama_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+        return rec.get(kernel, {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
 def cpu_baseline(cfg, W, steps, threads):
     """The CPU oracle (a scalar port of the reference's semantics) timed on this host: `steps` greedy decode
     tokens from an empty KV cache.  At this size a token is bound by the 2.07 GB of weights, not by context."""
@@ -103,6 +115,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--kernel-reps", type=int, default=10)
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run one 256 MiB device-to-device copy through the library (calibrates rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings against a transfer of known size)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU form (each box has one MI355X); run with --gpus 1",
@@ -136,6 +151,13 @@ def main():
     tok_s = args.steps / (elapsed_ms / 1e3)
     ms_per_step = elapsed_ms / args.steps
 
+    if args.traffic_probe:
+        n = 256 << 20
+        src, dst = ctx.alloc(n), ctx.alloc(n)
+        for _ in range(3):
+            pkg.check(ctx.lib.m40llm_memcpy_d2d_async(ctx.h, dst.ptr, src.ptr, n, 1), "m40llm_memcpy_d2d_async")
+        ctx.sync(1)
+        src.free(); dst.free()
     dom = measure_dominant_kernel(pkg, ctx, dm, cfg, args.kernel_reps, mode)
     achieved = dom["bytes"] / (dom["avg_us"] * 1e-6) / 1e9
     token_bytes = algorithmic_bytes_per_token(cfg)
@@ -154,7 +176,8 @@ def main():
                    "algorithmic_bytes_per_token": token_bytes, "setup_s": round(setup_s, 1),
                    "first_generated_ids": [int(i) for i in ids[n_prompt:n_prompt + 8]]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "kernel": dom["kernel"], "shape": dom["shape"],
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(dom["kernel"]), "kernel": dom["kernel"],
+                     "shape": dom["shape"],
                      "avg_launch_us": dom["avg_us"], "launches_timed": dom["launches"],
                      "algorithmic_bytes_per_launch": dom["bytes"]},
     }
