@@ -54,10 +54,10 @@ struct SkinnyArgs {
 
 // FMT 0: f16 weights, 1: q8_0 weights.
 template <int FMT, bool STACKED>
-__global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
+__global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) {
     constexpr int kASets = STACKED ? 1 : 2;
-    constexpr int kABufs = STACKED ? 2 : 1;                             // LDS budget: two sets are single-buffered
-    __shared__ uint4 a_lds[kABufs][kASets][8 * 64];                     // activation fragments of a step
+    __shared__ __attribute__((aligned(16))) uint2 a_lds[2][kASets][8 * 64 * 2];                    // activation fragments of a step, two buffers
+    __shared__ float tscale_s[2][16];                                   // factor that undoes each row's scaling of the step
     __shared__ __attribute__((aligned(16))) uint8_t b_lds[FMT == 1 ? kWavesPerGroup * kQ8TileBytes : 16];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -71,7 +71,6 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
     const int n0 = (gtile - p.tile_begin[z]) * 16;
     const int KT = p.K / kTileK;
     const int kt0 = (int)(((long long)blockIdx.y * KT) / p.S), kt1 = (int)(((long long)(blockIdx.y + 1) * KT) / p.S);
-    __shared__ float scale_s[16];      // factor that undoes each row's power-of-two scaling (this K slice)
 
     // ---- weight addressing
     const int col = n0 + j < N ? n0 + j : N - 1;
@@ -96,34 +95,51 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
         }
     }
 
-    // ---- activation addressing: 32 threads per row, thread (arow, acol) owns k = 256 kt + 8 acol .. +7 of a step,
-    // which is entry (MFMA i = acol / 4, group acol % 4) of the step's fragments
-    constexpr int kARows = STACKED ? 8 : 16;
-    const int arow = tid >> 5, acol = tid & 31;
-    const bool a_thread = arow < kARows;
-    const bool a_live = a_thread && arow < p.M;
-    const float* a_ptr = p.A + (size_t)(a_live ? arow : 0) * p.K + 8 * acol;
-    const float* u_ptr = p.up ? p.up + (size_t)(a_live ? arow : 0) * p.K + 8 * acol : nullptr;
+    // ---- activation addressing: thread (arow, acol) owns EPT consecutive k of row arow in every step:
+    // k = 256 kt + EPT acol .. ; eight consecutive k form entry (MFMA i = k / 32, group (k / 8) % 4) of the fragments.
+    // Up to eight rows: a whole wave per row (4 elements per lane); above: 32 lanes per row (8 elements per lane).
+    constexpr int EPT = STACKED ? 4 : 8;
+    constexpr int TPR = kTileK / EPT;
+    const int arow = tid / TPR, acol = tid % TPR;
+    const bool a_live = arow < p.M;
+    const float* a_ptr = p.A + (size_t)(a_live ? arow : 0) * p.K + EPT * acol;
+    const float* u_ptr = p.up ? p.up + (size_t)(a_live ? arow : 0) * p.K + EPT * acol : nullptr;
     const uint16_t* nw16 = static_cast<const uint16_t*>(p.norm_w);
     const float* nw32 = static_cast<const float*>(p.norm_w);
-    auto load8 = [&](const float* src, float (&v)[8]) {
-        const float4 x0 = *reinterpret_cast<const float4*>(src);
-        const float4 x1 = *reinterpret_cast<const float4*>(src + 4);
-        v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
+    auto load_f32 = [&](const float* src, float (&v)[EPT]) {
+#pragma unroll
+        for (int e = 0; e < EPT; e += 4) {
+            const float4 x = *reinterpret_cast<const float4*>(src + e);
+            v[e] = x.x; v[e + 1] = x.y; v[e + 2] = x.z; v[e + 3] = x.w;
+        }
     };
-    auto load_norm8 = [&](int k, float (&v)[8]) {
-        if (p.norm_dtype == 0u) m40_unpack8(*reinterpret_cast<const uint4*>(nw16 + k), v);
-        else load8(nw32 + k, v);
+    auto load_norm = [&](int k, float (&v)[EPT]) {
+        if (p.norm_dtype == 0u) {
+#pragma unroll
+            for (int e = 0; e < EPT; e += 4) {
+                const uint2 w = *reinterpret_cast<const uint2*>(nw16 + k + e);
+                v[e] = m40_h2f((uint16_t)(w.x & 0xffffu)); v[e + 1] = m40_h2f((uint16_t)(w.x >> 16));
+                v[e + 2] = m40_h2f((uint16_t)(w.y & 0xffffu)); v[e + 3] = m40_h2f((uint16_t)(w.y >> 16));
+            }
+        } else {
+            load_f32(nw32 + k, v);
+        }
+    };
+    auto row_reduce_max = [&](float x) -> float {
+        if (STACKED) return m40_max64(x);
+#pragma unroll
+        for (int o = 1; o < 32; o <<= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+        return x;
     };
 
-    float fa[8], fb[8];        // this thread's activations of a step (and their SwiGLU partner or norm weights)
+    float fa[EPT], fb[EPT];    // this thread's activations of a step (and their SwiGLU partner or norm weights)
     uint4 rb[8];               // f16: the eight 16-byte weight loads of a step; q8_0: five tile pieces
-    auto issue_loads = [&](int kt) {
-        if (a_thread) {
-            load8(a_ptr + (size_t)kt * kTileK, fa);
-            if (u_ptr) load8(u_ptr + (size_t)kt * kTileK, fb);
-            else if (p.norm_w) load_norm8(kt * kTileK + 8 * acol, fb);
-        }
+    auto issue_a = [&](int kt) {
+        load_f32(a_ptr + (size_t)kt * kTileK, fa);
+        if (u_ptr) load_f32(u_ptr + (size_t)kt * kTileK, fb);
+        else if (p.norm_w) load_norm(kt * kTileK + EPT * acol, fb);
+    };
+    auto issue_w = [&](int kt) {
         if (FMT == 0) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
@@ -136,76 +152,84 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
     };
 
     m40_float4 acc = {0.f, 0.f, 0.f, 0.f};
-    if (kt0 < kt1) issue_loads(kt0);           // weights of the first step are in flight during the prologue
+    issue_w(kt0);              // weights of the first step are in flight during the prologue
+    issue_a(kt0);
 
-    // ---- per-row statistics: RMS over the whole row (RMSNorm), largest operand of this K slice -> power-of-two scale
-    float rms = 1.0f, inv_scale = 1.0f;
-    if (a_thread) {
-        if (p.norm_w && a_live) {
-            float sq = 0.0f;
-            for (int k = 0; k < p.K; k += kTileK) {
-                float v[8];
-                load8(a_ptr + k, v);
+    // RMS over the whole row (RMSNorm operand only)
+    float rms = 1.0f;
+    if (p.norm_w && a_live) {
+        float sq = 0.0f;
+        for (int k = 0; k < p.K; k += kTileK) {
+            float v[EPT];
+            load_f32(a_ptr + k, v);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) sq = fmaf(v[e], v[e], sq);
-            }
+            for (int e = 0; e < EPT; ++e) sq = fmaf(v[e], v[e], sq);
+        }
+        if (STACKED) {
+            sq = m40_sum64(sq);
+        } else {
 #pragma unroll
             for (int o = 1; o < 32; o <<= 1) sq += __shfl_xor(sq, o, 64);
-            rms = rsqrtf(sq / (float)p.K + p.eps);
         }
-        float mx = 0.0f;
-        if (a_live) {
-            for (int kt = kt0; kt < kt1; ++kt) {
-                float v[8], w[8];
-                load8(a_ptr + (size_t)kt * kTileK, v);
-                if (u_ptr) load8(u_ptr + (size_t)kt * kTileK, w);
-                else if (p.norm_w) load_norm8(kt * kTileK + 8 * acol, w);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float x = v[e];
-                    if (u_ptr) x = x / (1.0f + expf(-x)) * w[e];
-                    else if (p.norm_w) x = x * rms * w[e];
-                    mx = fmaxf(mx, fabsf(x));
-                }
-            }
-        }
-#pragma unroll
-        for (int o = 1; o < 32; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        float scale = 1.0f;
-        if (mx > 0.0f && mx < INFINITY) {
-            int e;
-            (void)frexpf(mx, &e);         // mx = f * 2^e, f in [0.5, 1)
-            e -= 11;                      // scaled maximum in [2^10, 2^11)
-            e = e < -100 ? -100 : (e > 100 ? 100 : e);
-            scale = ldexpf(1.0f, e);
-            inv_scale = ldexpf(1.0f, -e);
-        }
-        if (acol == 0) scale_s[arow] = scale;
+        rms = rsqrtf(sq / (float)p.K + p.eps);
     }
 
-    for (int kt = kt0; kt < kt1; ++kt) {
-        const int buf = kABufs == 2 ? ((kt - kt0) & 1) : 0;
-        if (a_thread) {
-            // f32 -> f16 hi + f16 lo of the scaled operand, straight into the step's fragment entries
-            uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
-            if (a_live) {
+    // f32 -> f16 hi + f16 lo of the operand held in fa/fb, scaled by a power of two taken from the largest value of
+    // the row within this step, straight into the fragment entries of buffer `buf`
+    auto convert = [&](int buf) {
+        float x[EPT];
+        float mx = 0.0f;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float x = fa[e];
-                    if (u_ptr) x = x / (1.0f + expf(-x)) * fb[e];
-                    else if (p.norm_w) x = x * rms * fb[e];
-                    x *= inv_scale;
-                    const _Float16 h = static_cast<_Float16>(x);
-                    const _Float16 l = static_cast<_Float16>(x - static_cast<float>(h));
-                    hi[e >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (e & 1));
-                    lo[e >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, l) << (16 * (e & 1));
-                }
-            }
-            const int entry = (acol >> 2) * 64 + (acol & 3) * 16 + arow;
-            a_lds[buf][0][entry] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-            if (STACKED) a_lds[buf][0][entry + 8] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-            else a_lds[buf][kASets - 1][entry] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        for (int e = 0; e < EPT; ++e) {
+            float v = a_live ? fa[e] : 0.0f;
+            if (u_ptr) v = v / (1.0f + expf(-v)) * fb[e];
+            else if (p.norm_w) v = v * rms * fb[e];
+            if (!a_live) v = 0.0f;
+            x[e] = v;
+            mx = fmaxf(mx, fabsf(v));
         }
+        mx = row_reduce_max(mx);
+        float scale = 1.0f, inv_scale = 1.0f;
+        if (mx > 0.0f && mx < INFINITY) {
+            int ex;
+            (void)frexpf(mx, &ex);        // mx = f * 2^ex, f in [0.5, 1)
+            ex -= 11;                     // scaled maximum in [2^10, 2^11)
+            ex = ex < -100 ? -100 : (ex > 100 ? 100 : ex);
+            scale = ldexpf(1.0f, ex);
+            inv_scale = ldexpf(1.0f, -ex);
+        }
+        uint32_t hi[EPT / 2], lo[EPT / 2];
+#pragma unroll
+        for (int e = 0; e < EPT; e += 2) {
+            uint32_t h2 = 0, l2 = 0;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const float v = x[e + q] * inv_scale;
+                const _Float16 h = static_cast<_Float16>(v);
+                const _Float16 l = static_cast<_Float16>(v - static_cast<float>(h));
+                h2 |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * q);
+                l2 |= (uint32_t)__builtin_bit_cast(uint16_t, l) << (16 * q);
+            }
+            hi[e / 2] = h2; lo[e / 2] = l2;
+        }
+        const int k0 = EPT * acol;                                   // first k of this thread within the step
+        const int entry = (k0 >> 5) * 64 + ((k0 >> 3) & 3) * 16 + arow;
+#pragma unroll
+        for (int e = 0; e < EPT / 4; ++e) {
+            const int sub = ((k0 >> 2) & 1) + e;                     // which half of the 8-half entry
+            a_lds[buf][0][entry * 2 + sub] = make_uint2(hi[2 * e], hi[2 * e + 1]);
+            if (STACKED) a_lds[buf][0][(entry + 8) * 2 + sub] = make_uint2(lo[2 * e], lo[2 * e + 1]);
+            else a_lds[buf][kASets - 1][entry * 2 + sub] = make_uint2(lo[2 * e], lo[2 * e + 1]);
+        }
+        if (acol == 0) {
+            tscale_s[buf][arow] = scale;
+            if (STACKED) tscale_s[buf][arow + 8] = scale;
+        }
+    };
+    convert(0);
+
+    for (int kt = kt0; kt < kt1; ++kt) {
+        const int buf = (kt - kt0) & 1;
         uint4 wb[8];
         if (FMT == 0) {
 #pragma unroll
@@ -215,14 +239,21 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
             for (int i = 0; i < 5; ++i)
                 if (q_src[i]) *reinterpret_cast<uint4*>(my_b + q_dst[i]) = rb[i];
         }
-        __syncthreads();
-        if (kt + 1 < kt1) issue_loads(kt + 1);
+        __syncthreads();       // fragments of this step are complete; nobody still reads the other buffer
+        const bool more = kt + 1 < kt1;
+        if (more) {
+            issue_w(kt + 1);
+            issue_a(kt + 1);
+        }
+        m40_float4 tacc = {0.f, 0.f, 0.f, 0.f};
+        const uint4* a_hi_frag = reinterpret_cast<const uint4*>(a_lds[buf][0]);
+        const uint4* a_lo_frag = reinterpret_cast<const uint4*>(a_lds[buf][kASets - 1]);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint4 a_hi = a_lds[buf][0][i * 64 + lane];
+            const uint4 a_hi = a_hi_frag[i * 64 + lane];
             if (FMT == 0) {
-                acc = mfma16x16x32(a_hi, wb[i], acc);
-                if (!STACKED) acc = mfma16x16x32(a_lds[buf][1][i * 64 + lane], wb[i], acc);
+                tacc = mfma16x16x32(a_hi, wb[i], tacc);
+                if (!STACKED) tacc = mfma16x16x32(a_lo_frag[i * 64 + lane], wb[i], tacc);
             } else {
                 const uint8_t* blk = my_b + j * 272 + 34 * i;
                 const float d = m40_h2f(*reinterpret_cast<const uint16_t*>(blk));
@@ -245,12 +276,14 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
                 const uint4 bq = make_uint4(q8_pair_to_f16(s0), q8_pair_to_f16(s1), q8_pair_to_f16(s2), q8_pair_to_f16(s3));
                 const m40_float4 zero = {0.f, 0.f, 0.f, 0.f};
                 m40_float4 dblk = mfma16x16x32(a_hi, bq, zero);
-                if (!STACKED) dblk = mfma16x16x32(a_lds[buf][1][i * 64 + lane], bq, dblk);
+                if (!STACKED) dblk = mfma16x16x32(a_lo_frag[i * 64 + lane], bq, dblk);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[r] = fmaf(d, dblk[r], acc[r]);
+                for (int r = 0; r < 4; ++r) tacc[r] = fmaf(d, dblk[r], tacc[r]);
             }
         }
-        if (kABufs == 1) __syncthreads();   // the single buffer is rewritten by the next step
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] = fmaf(tscale_s[buf][4 * g + r], tacc[r], acc[r]);
+        if (more) convert(buf ^ 1);      // next step's fragments, while the other waves finish this one
     }
     // lane (j, g) holds rows 4g + r of column j
     if (STACKED) {
@@ -263,9 +296,9 @@ __global__ __launch_bounds__(kThreads) void skinny_mfma_kernel(SkinnyArgs p) {
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
         if (p.direct) {
-            if (row < p.M) p.C[z][(size_t)row * N + n0 + j] = acc[r] * scale_s[row];
+            if (row < p.M) p.C[z][(size_t)row * N + n0 + j] = acc[r];
         } else {
-            p.partial[p.part_off[z] + ((size_t)blockIdx.y * 16 + row) * N + n0 + j] = acc[r] * scale_s[row];
+            p.partial[p.part_off[z] + ((size_t)blockIdx.y * 16 + row) * N + n0 + j] = acc[r];
         }
     }
 }
