@@ -21,7 +21,9 @@ namespace {
 constexpr int kTileK = 256;                       // k per step
 constexpr int kWavesPerGroup = 8;                 // 16-column tiles per workgroup
 constexpr int kThreads = kWavesPerGroup * 64;
-constexpr int kQ8TileBytes = 16 * 272;            // 16 columns x 8 blocks x 34 bytes
+constexpr int kQ8ColStride = 276;                 // LDS bytes per column of a staged tile: 272 + 4, an odd number of
+                                                  // dwords, so that the 16 columns start in different banks
+constexpr int kQ8TileBytes = 16 * kQ8ColStride;   // 16 columns x (8 blocks x 34 bytes + pad)
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
                 const int c = q / 17, piece = q % 17;
                 const int cc = n0 + c < N ? n0 + c : N - 1;
                 q_src[i] = base + (size_t)cc * col_stride + 16 * piece;
-                q_dst[i] = c * 272 + 16 * piece;
+                q_dst[i] = c * kQ8ColStride + 16 * piece;
             }
         }
     }
@@ -237,7 +239,10 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
         } else {
 #pragma unroll
             for (int i = 0; i < 5; ++i)
-                if (q_src[i]) *reinterpret_cast<uint4*>(my_b + q_dst[i]) = rb[i];
+                if (q_src[i]) {
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(my_b + q_dst[i]);      // 4-byte aligned only
+                    dst[0] = rb[i].x; dst[1] = rb[i].y; dst[2] = rb[i].z; dst[3] = rb[i].w;
+                }
         }
         __syncthreads();       // fragments of this step are complete; nobody still reads the other buffer
         const bool more = kt + 1 < kt1;
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
                 tacc = mfma16x16x32(a_hi, wb[i], tacc);
                 if (!STACKED) tacc = mfma16x16x32(a_lo_frag[i * 64 + lane], wb[i], tacc);
             } else {
-                const uint8_t* blk = my_b + j * 272 + 34 * i;
+                const uint8_t* blk = my_b + j * kQ8ColStride + 34 * i;
                 const float d = m40_h2f(*reinterpret_cast<const uint16_t*>(blk));
                 uint32_t s0, s1, s2, s3;   // byte pairs (0,1) (2,3) (4,5) (6,7) of the lane's eight quants, spread to 16-bit lanes
                 if (i & 1) {               // quants 4-byte aligned

@@ -181,3 +181,124 @@ def test_lm_head_top2_and_greedy_step(dev, orc, V, K):
     assert dev.lib.m40llm_ext_fused_norm_gemv_f32xf16_async(dev.h, dx.ptr, dnw.ptr, 1, 1e-5, dW.ptr, logits.ptr, V, K,
                                                             top2.ptr, 0, None) == -5
     assert dev.lib.m40llm_ext_greedy_step_async(dev.h, None, V, None, 0, 0, dst.ptr, None, 0, None) == -1
+
+
+# ------------------------------------------------------------------ row-batched fused entry points
+def _rows_case(rng, rows, K):
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    if rows > 1:
+        x[1] *= 1e-3            # rows of very different magnitude (per-row, per-step scaling of the f16 split)
+    if rows > 2:
+        x[2] *= 3e3
+    return x
+
+
+@pytest.mark.parametrize("rows", [1, 8, 13])
+def test_batched_gemm_residual_and_norm_gate_up_vs_oracle(dev, orc, rows):
+    rng = np.random.default_rng(rows)
+    D, F = 512, 768
+    x = _rows_case(rng, rows, D)
+    nw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    wg = f16bits(rng.standard_normal((F, D)) * 0.05); wu = f16bits(rng.standard_normal((F, D)) * 0.05)
+    wd = f16bits(rng.standard_normal((D, F)) * 0.05)
+    dx, dnw, dwg, dwu, dwd = dev.up(x), dev.up(nw), dev.up(wg), dev.up(wu), dev.up(wd)
+    hid = dev.zeros(rows * F * 4)
+    dev.call("m40llm_ext_batched_norm_gate_up_swiglu_async", dx.ptr, dnw.ptr, 1, 1e-5, dwg.ptr, dwu.ptr, hid.ptr, rows, F, D)
+    out = dev.zeros(rows * D * 4)
+    dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", hid.ptr, dwd.ptr, dx.ptr, out.ptr, rows, D, F)
+    dev.sync()
+    xn = orc.rms_norm(x, 1e-5, nw, 1)
+    want_h = orc.swiglu(orc.gemm("f32xf16_gguf", xn, wg, rows, F, D), orc.gemm("f32xf16_gguf", xn, wu, rows, F, D))
+    got_h = hid.download(np.float32, (rows, F))
+    sc = np.abs(want_h).max(axis=1, keepdims=True)
+    close(got_h / sc, want_h / sc)
+    want = x + orc.gemm("f32xf16_gguf", want_h, wd, rows, D, F)
+    got = out.download(np.float32, (rows, D))
+    sc = np.abs(want).max(axis=1, keepdims=True)
+    close(got / sc, want / sc)
+    # argument checks: more than 16 rows, K not a multiple of 256
+    dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", hid.ptr, dwd.ptr, dx.ptr, out.ptr, 17, D, F, expect=-6)
+    dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", hid.ptr, dwd.ptr, dx.ptr, out.ptr, rows, D, F - 64, expect=-6)
+
+
+@pytest.mark.parametrize("qh,kvh,hd,layout,bias,rows", [(8, 2, 64, 0, False, 5), (4, 2, 128, 1, True, 8), (4, 1, 128, 1, True, 12)])
+def test_batched_norm_qkv_rope_append_vs_oracle(dev, orc, qh, kvh, hd, layout, bias, rows):
+    rng = np.random.default_rng(qh + rows)
+    D = qh * hd
+    x = _rows_case(rng, rows, D)
+    nw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    wq = f16bits(rng.standard_normal((qh * hd, D)) * 0.05)
+    wk = f16bits(rng.standard_normal((kvh * hd, D)) * 0.05)
+    wv = f16bits(rng.standard_normal((kvh * hd, D)) * 0.05)
+    bq = (rng.standard_normal(qh * hd) * 0.1).astype(np.float32)
+    bk = (rng.standard_normal(kvh * hd) * 0.1).astype(np.float32)
+    bv = (rng.standard_normal(kvh * hd) * 0.1).astype(np.float32)
+    nseq, S = 16, 64
+    kv = m40.KVCache(dev.ctx, S, nseq, kvh, hd)
+    ids = rng.permutation(nseq)[:rows].astype(np.uint32)
+    lens = rng.integers(0, S, size=rows).astype(np.uint32)
+    dx, dnw, dwq, dwk, dwv = dev.up(x), dev.up(nw), dev.up(wq), dev.up(wk), dev.up(wv)
+    dbq, dbk, dbv = dev.up(bq), dev.up(bk), dev.up(bv)
+    dids, dlens = dev.up(ids), dev.up(lens)
+    dq = dev.zeros(rows * qh * hd * 4)
+    base = 1e6 if layout else 1e4
+    dev.call("m40llm_ext_batched_norm_qkv_rope_append_async", kv.h, dids.ptr, dlens.ptr, rows, dx.ptr, dnw.ptr, 1, 1e-6,
+             dwq.ptr, dwk.ptr, dwv.ptr, dbq.ptr if bias else None, dbk.ptr if bias else None, dbv.ptr if bias else None,
+             D, qh, base, 1.0, layout, dq.ptr)
+    dev.sync()
+    got_q = dq.download(np.float32, (rows, qh * hd))
+    xn = orc.rms_norm(x, 1e-6, nw, 1)
+    q = orc.gemm("f32xf16_gguf", xn, wq, rows, qh * hd, D) + (bq if bias else 0)
+    k = orc.gemm("f32xf16_gguf", xn, wk, rows, kvh * hd, D) + (bk if bias else 0)
+    v = orc.gemm("f32xf16_gguf", xn, wv, rows, kvh * hd, D) + (bv if bias else 0)
+    for r in range(rows):
+        pos, seq = int(lens[r]), int(ids[r])
+        want_q = orc.rope(q[r:r + 1].astype(np.float32), qh, hd, pos, base, 1.0, layout)[0]
+        want_k = orc.rope(k[r:r + 1].astype(np.float32), kvh, hd, pos, base, 1.0, layout)[0]
+        sq = np.abs(want_q).max()
+        close(got_q[r] / sq, want_q / sq)
+        gk, gv = kv.read_token(seq, pos)
+        sk = np.abs(want_k).max()
+        close(gk.view(np.float16).astype(np.float32) / sk, want_k / sk, 2e-3, 1e-3)       # f16 storage
+        sv = np.abs(v[r]).max()
+        close(gv.view(np.float16).astype(np.float32) / sv, v[r] / sv, 2e-3, 1e-3)
+    kv.destroy()
+
+
+def test_batched_greedy_step_and_lm_head(dev, orc):
+    rng = np.random.default_rng(3)
+    rows, V, D = 6, 5000, 256
+    x = _rows_case(rng, rows, D)
+    nw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    W = f16bits(rng.standard_normal((V, D)) * 0.05)
+    table = f16bits(rng.standard_normal((V, D)))
+    dx, dnw, dW, dT = dev.up(x), dev.up(nw), dev.up(W), dev.up(table)
+    logits = dev.zeros(rows * V * 4)
+    dev.call("m40llm_ext_batched_norm_gemm_f32xf16_async", dx.ptr, dnw.ptr, 1, 1e-5, dW.ptr, logits.ptr, rows, V, D)
+    dev.sync()
+    lg = logits.download(np.float32, (rows, V))
+    want = orc.gemm("f32xf16_gguf", orc.rms_norm(x, 1e-5, nw, 1), W, rows, V, D)
+    sc = np.abs(want).max(axis=1, keepdims=True)
+    close(lg / sc, want / sc)
+    lg[4, 100] = lg[4, 4000] = lg[4].max() + 1.0            # exact tie: the lower index wins, gap 0
+    logits.upload(lg)
+    cap = 3
+    state = np.zeros(2 + rows, dtype=np.uint32); state[1] = cap; state[2:] = 1
+    lens = np.arange(10, 10 + rows, dtype=np.uint32)
+    dstate, dlens = dev.up(state), dev.up(lens)
+    dids, dgaps = dev.zeros(rows * cap * 4), dev.zeros(rows * cap * 4)
+    xout = dev.zeros(rows * D * 4)
+    dev.call("m40llm_ext_batched_greedy_step_async", logits.ptr, rows, V, dstate.ptr, dlens.ptr, dids.ptr, dgaps.ptr, dT.ptr, D,
+             xout.ptr)
+    dev.sync()
+    ids = dids.download(np.uint32, (rows, cap)); gaps = dgaps.download(np.float32, (rows, cap))
+    xo = xout.download(np.float32, (rows, D))
+    assert np.array_equal(dlens.download(np.uint32, (rows,)), lens + 1)
+    assert np.array_equal(dstate.download(np.uint32, state.shape)[2:], np.full(rows, 2))
+    for r in range(rows):
+        tok = orc.sample_greedy(lg[r])
+        assert ids[r, 1] == tok == int(np.argmax(lg[r]))
+        srt = np.sort(lg[r])
+        assert gaps[r, 1] == srt[-1] - srt[-2]
+        assert np.array_equal(xo[r], table[tok].view(np.float16).astype(np.float32))
+    assert ids[4, 1] == 100 and gaps[4, 1] == 0.0
