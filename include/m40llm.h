@@ -279,6 +279,14 @@ int m40llm_ext_block_select_read_selection(M40llmCudaContext* ctx, const M40llmK
                                            uint32_t block_size, uint32_t top_blocks,
                                            uint32_t* out_blocks_host, uint32_t* out_counts_host,
                                            float* out_scores_host);
+/* The fp16-K / q4-V block-select attention of up to 8 different sequences (slots) in one set of launches, so that
+ * independent slots overlap on the device.  seq_ids_host / seq_lens_host are host arrays of n_slots entries;
+ * q_dev_f32 and out_dev_f32 hold n_slots rows of q_heads * head_dim floats.  Same results and error codes as
+ * n_slots calls of m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async. */
+int m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async(
+    M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t n_slots, const uint32_t* seq_ids_host,
+    const uint32_t* seq_lens_host, const void* q_dev_f32, uint32_t q_heads, uint32_t recent_window, uint32_t block_size,
+    uint32_t top_blocks, void* out_dev_f32);
 /* Fill positions [0, seq_len) of one sequence from f16 K/V rows [seq_len][kv_heads][head_dim]
  * on the device, leaving the cache exactly as seq_len ordered appends of those (already
  * rotated) rows would: dense caches get the rows, compressed caches get old-K copies,

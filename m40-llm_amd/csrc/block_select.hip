@@ -42,9 +42,16 @@ struct BsParams {
     uint32_t old_len, nblk, chunk, nchunks, compressed;
 };
 
+constexpr int kBsMaxSlots = 8;
+// Several independent slots (sequences) per launch: blockIdx.z picks the slot.
+struct BsMulti {
+    BsParams slot[kBsMaxSlots];
+};
+
 // ---- 1. block scores ------------------------------------------------------------------------
 template <int HD, int G>
-__global__ __launch_bounds__(256) void bs_score_kernel(BsParams p) {
+__global__ __launch_bounds__(256) void bs_score_kernel(BsMulti multi) {
+    const BsParams& p = multi.slot[blockIdx.z];
     constexpr int C = HD / 8;   // 16-byte chunks per K row
     constexpr int R = 64 / C;   // rows per wave step
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -98,11 +105,28 @@ __global__ __launch_bounds__(256) void bs_score_kernel(BsParams p) {
 // reference's strict-'>' insertion produces (cuda/kernels.cu:2980-3022).  Grid (q head, 128 candidates); eight lanes
 // share the count of one candidate.  The workgroup that owns the last block also writes the list length, the
 // attended-token count and the unused tail of the list.
-__global__ __launch_bounds__(1024) void bs_select_kernel(BsParams p) {
+__global__ __launch_bounds__(1024) void bs_select_kernel(BsMulti multi) {
+    const BsParams& p = multi.slot[blockIdx.z];
     extern __shared__ float s_sc[];  // [nblk]
     __shared__ uint32_t s_valid[16];
     __shared__ uint32_t s_last_rank;
     const uint32_t qh = blockIdx.x;
+    if (p.nblk == 0) {
+        // no old blocks: empty list, the q head attends the recent tokens only
+        if (blockIdx.y == 0) {
+            for (uint32_t i = threadIdx.x; i < 64u; i += 1024u) {
+                p.sel[qh * 64 + i] = 0xffffffffu;
+                p.sel_scores[qh * 64 + i] = -1e30f;
+            }
+            if (threadIdx.x == 0) {
+                p.counts[qh] = 0;
+                p.ntok[qh] = p.seq_len - p.old_len;
+            }
+        }
+        return;
+    }
+    const uint32_t parts = (p.nblk + 127u) / 128u;
+    if (blockIdx.y >= parts) return;
     const float* sc = p.scores + (size_t)qh * p.nblk;
     uint32_t valid = 0;
     for (uint32_t b = threadIdx.x; b < p.nblk; b += 1024u) {
@@ -137,7 +161,7 @@ __global__ __launch_bounds__(1024) void bs_select_kernel(BsParams p) {
     }
     if (cand && part == 0u && b + 1u == p.nblk) s_last_rank = listed ? rank : 0xffffffffu;
     __syncthreads();
-    if (blockIdx.y == gridDim.y - 1u) {
+    if (blockIdx.y == parts - 1u) {
         uint32_t total_valid = 0;
         for (int w = 0; w < 16; ++w) total_valid += s_valid[w];
         const uint32_t count = total_valid < p.top_n ? total_valid : p.top_n;
@@ -154,25 +178,13 @@ __global__ __launch_bounds__(1024) void bs_select_kernel(BsParams p) {
     }
 }
 
-// no old blocks: empty lists, every q head attends the recent tokens only
-__global__ void bs_empty_selection_kernel(BsParams p) {
-    const uint32_t qh = blockIdx.x;
-    for (uint32_t i = threadIdx.x; i < 64u; i += blockDim.x) {
-        p.sel[qh * 64 + i] = 0xffffffffu;
-        p.sel_scores[qh * 64 + i] = -1e30f;
-    }
-    if (threadIdx.x == 0) {
-        p.counts[qh] = 0;
-        p.ntok[qh] = p.seq_len - p.old_len;
-    }
-}
-
 // ---- 3. attention over the token list ---------------------------------------------------------
 // Grid (q head, chunk of 128 list positions).  Eight waves; every lane issues the K and V loads of all of its token
 // rows before any arithmetic (one memory round trip per workgroup), scores stay in registers.
 constexpr int kBsChunk = 128;
 template <int HD>
-__global__ __launch_bounds__(512) void bs_attend_kernel(BsParams p) {
+__global__ __launch_bounds__(512) void bs_attend_kernel(BsMulti multi) {
+    const BsParams& p = multi.slot[blockIdx.z];
     constexpr int LPT = HD / 8, TPW = 64 / LPT, kWaves = 8;
     constexpr int S = kBsChunk / (kWaves * TPW);
     __shared__ uint32_t pre[65];
@@ -332,7 +344,9 @@ __global__ __launch_bounds__(512) void bs_attend_kernel(BsParams p) {
 // Merge the chunk partials of one q head: 1024 threads = 1024/HD chunk lanes x HD dims, each lane folds chunks
 // lane, lane + n_lanes, ... with a running maximum; the lanes are then folded in order.
 template <int HD>
-__global__ __launch_bounds__(1024) void bs_combine_kernel(BsParams p) {
+__global__ __launch_bounds__(1024) void bs_combine_kernel(BsMulti multi) {
+    const BsParams& p = multi.slot[blockIdx.z];
+    if (p.nchunks <= 1) return;      // the attend kernel wrote the output itself
     constexpr int NCG = 1024 / HD;
     __shared__ float s_m[NCG], s_den[NCG];
     __shared__ float s_num[NCG][HD];
@@ -383,7 +397,9 @@ uint32_t order_from_env() {
 
 // Fills the parameter block and checks scratch capacity.  Returns 0 or a negative code.
 int prepare(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q, uint32_t q_heads,
-            uint32_t seq_len, uint32_t W, uint32_t bs, uint32_t top, void* out, bool compressed, BsParams* p) {
+            uint32_t seq_len, uint32_t W, uint32_t bs, uint32_t top, void* out, bool compressed, BsParams* p,
+            size_t* select_used = nullptr, size_t* partial_used = nullptr) {
+    const size_t select_off = select_used ? *select_used : 0, partial_off = partial_used ? *partial_used : 0;
     std::memset(p, 0, sizeof(*p));
     const uint32_t hd = kv->head_dim, kvh = kv->num_heads;
     const size_t ept = (size_t)kvh * hd;
@@ -414,8 +430,9 @@ int prepare(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, co
     // select scratch: scores | sel | sel_scores | counts | ntok
     const size_t scores_bytes = ((size_t)q_heads * (nblk ? nblk : 1) * 4 + 255) & ~(size_t)255;
     const size_t fixed = (size_t)q_heads * (64 * 4 + 64 * 4 + 4 + 4) + 1024;
-    if (scores_bytes + fixed > sc.select_bytes) return -7;
-    char* base = static_cast<char*>(sc.select);
+    const size_t select_need = (scores_bytes + fixed + 255) & ~(size_t)255;
+    if (select_off + select_need > sc.select_bytes) return -7;
+    char* base = static_cast<char*>(sc.select) + select_off;
     p->scores = reinterpret_cast<float*>(base);
     p->sel = reinterpret_cast<uint32_t*>(base + scores_bytes);
     p->sel_scores = reinterpret_cast<float*>(p->sel + (size_t)q_heads * 64);
@@ -424,30 +441,45 @@ int prepare(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, co
     const uint32_t chunk = kBsChunk;
     p->chunk = chunk;
     p->nchunks = (capacity + chunk - 1) / chunk;
-    if ((size_t)q_heads * p->nchunks * (hd + 2) * 4 > sc.attn_partial_bytes) return -7;
-    p->partial = static_cast<float*>(sc.attn_partial);
+    const size_t partial_need = (((size_t)q_heads * p->nchunks * (hd + 2) * 4) + 255) & ~(size_t)255;
+    if (partial_off + partial_need > sc.attn_partial_bytes) return -7;
+    p->partial = reinterpret_cast<float*>(static_cast<char*>(sc.attn_partial) + partial_off);
+    if (select_used) *select_used = select_off + select_need;
+    if (partial_used) *partial_used = partial_off + partial_need;
     if ((size_t)nblk * 4 > 60 * 1024) return -7;  // block scores of one q head live in LDS
     return 0;
 }
 
 template <int HD>
-int launch_all(hipStream_t s, const BsParams& p, bool selection_only) {
+int launch_multi(hipStream_t s, const BsMulti& m, uint32_t n, bool selection_only) {
     (void)hipGetLastError();
-    const uint32_t group = p.q_heads / p.kv_heads;
-    if (p.nblk > 0) {
-        dim3 grid((p.nblk + 3) / 4, p.kv_heads);
-        if (group >= 4) bs_score_kernel<HD, 4><<<grid, 256, 0, s>>>(p);
-        else if (group >= 2) bs_score_kernel<HD, 2><<<grid, 256, 0, s>>>(p);
-        else bs_score_kernel<HD, 1><<<grid, 256, 0, s>>>(p);
+    const BsParams& p0 = m.slot[0];
+    const uint32_t group = p0.q_heads / p0.kv_heads;
+    uint32_t max_nblk = 0, max_chunks = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        max_nblk = m.slot[i].nblk > max_nblk ? m.slot[i].nblk : max_nblk;
+        max_chunks = m.slot[i].nchunks > max_chunks ? m.slot[i].nchunks : max_chunks;
     }
-    if (p.nblk > 0) bs_select_kernel<<<dim3(p.q_heads, (p.nblk + 127) / 128), 1024, (size_t)p.nblk * 4, s>>>(p);
-    else bs_empty_selection_kernel<<<p.q_heads, 64, 0, s>>>(p);
+    if (max_nblk > 0) {
+        dim3 grid((max_nblk + 3) / 4, p0.kv_heads, n);
+        if (group >= 4) bs_score_kernel<HD, 4><<<grid, 256, 0, s>>>(m);
+        else if (group >= 2) bs_score_kernel<HD, 2><<<grid, 256, 0, s>>>(m);
+        else bs_score_kernel<HD, 1><<<grid, 256, 0, s>>>(m);
+    }
+    bs_select_kernel<<<dim3(p0.q_heads, max_nblk ? (max_nblk + 127) / 128 : 1, n), 1024, (size_t)(max_nblk ? max_nblk : 1) * 4, s>>>(m);
     if (!selection_only) {
-        dim3 grid(p.q_heads, p.nchunks);
-        bs_attend_kernel<HD><<<grid, 512, 0, s>>>(p);
-        if (p.nchunks > 1) bs_combine_kernel<HD><<<p.q_heads, 1024, 0, s>>>(p);
+        bs_attend_kernel<HD><<<dim3(p0.q_heads, max_chunks, n), 512, 0, s>>>(m);
+        if (max_chunks > 1) bs_combine_kernel<HD><<<dim3(p0.q_heads, 1, n), 1024, 0, s>>>(m);
     }
     return hipGetLastError() == hipSuccess ? 0 : -8;
+}
+
+template <int HD>
+int launch_all(hipStream_t s, const BsParams& p, bool selection_only) {
+    BsMulti m;
+    std::memset(&m, 0, sizeof(m));
+    m.slot[0] = p;
+    return launch_multi<HD>(s, m, 1, selection_only);
 }
 
 int common_checks(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, const void* q, uint32_t q_heads,
@@ -502,6 +534,33 @@ int m40llm_attention_last_token_f32_gqa_block_select_exact_async(
     if (rc != 0) return rc;
     return kv->head_dim == 64 ? launch_all<64>(ctx->decode_stream, p, false)
                               : launch_all<128>(ctx->decode_stream, p, false);
+}
+
+int m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async(
+    M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t n_slots, const uint32_t* seq_ids_host,
+    const uint32_t* seq_lens_host, const void* q_dev_f32, uint32_t q_heads, uint32_t recent_window, uint32_t block_size,
+    uint32_t top_blocks, void* out_dev_f32) {
+    if (!seq_ids_host || !seq_lens_host) return -1;
+    if (n_slots == 0 || n_slots > (uint32_t)kBsMaxSlots) return -2;
+    if (!kv) return -1;
+    const size_t row = (size_t)q_heads * kv->head_dim;
+    BsMulti m;
+    std::memset(&m, 0, sizeof(m));
+    size_t select_used = 0, partial_used = 0;
+    for (uint32_t i = 0; i < n_slots; ++i) {
+        const float* q = static_cast<const float*>(q_dev_f32) + i * row;
+        float* out = static_cast<float*>(out_dev_f32) + i * row;
+        int rc = common_checks(ctx, kv, seq_ids_host[i], q_dev_f32 ? q : nullptr, q_heads, seq_lens_host[i], recent_window,
+                               block_size, top_blocks, out_dev_f32 ? out : nullptr, true);
+        if (rc != 0) return rc;
+        for (uint32_t k = 0; k < i; ++k)
+            if (seq_ids_host[k] == seq_ids_host[i]) return -2;      // a slot at most once per call
+        rc = prepare(ctx, kv, seq_ids_host[i], q, q_heads, seq_lens_host[i], recent_window, block_size, top_blocks, out, true,
+                     &m.slot[i], &select_used, &partial_used);
+        if (rc != 0) return rc;
+    }
+    return kv->head_dim == 64 ? launch_multi<64>(ctx->decode_stream, m, n_slots, false)
+                              : launch_multi<128>(ctx->decode_stream, m, n_slots, false);
 }
 
 int m40llm_ext_block_select_read_selection(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,

@@ -176,7 +176,15 @@ def bench_block_select(b: Bench):
     def four(i):
         for s in range(nseq):
             b.call(name, kv.h, s, q.ptr, qh, L, W, bs, top, out.ptr)
-    b.time("block_select fp16-K/q4-V, B=4", "4 slots per step", 4 * algo, four, 1, reps=16, warm=2)
+    b.time("block_select fp16-K/q4-V, B=4", "4 slots per step, one call per slot", 4 * algo, four, 1, reps=16, warm=2)
+    q4 = b.ctx.to_device(rng.standard_normal((nseq, qh * hd)).astype(np.float32))
+    out4 = b.ctx.alloc(nseq * qh * hd * 4)
+    ids_h = np.arange(nseq, dtype=np.uint32); lens_h = np.full(nseq, L, dtype=np.uint32)
+    import ctypes as C
+    b.time("block_select fp16-K/q4-V, B=4", "4 slots per step, multi-slot call", 4 * algo,
+           lambda i: b.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, nseq,
+                            ids_h.ctypes.data_as(C.c_void_p), lens_h.ctypes.data_as(C.c_void_p), q4.ptr, qh, W, bs, top, out4.ptr),
+           1, reps=16, warm=2)
     kv.destroy()
 
 

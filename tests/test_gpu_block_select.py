@@ -1,4 +1,6 @@
 """fp16-K / q4-V compressed cache and block-select attention: HIP path vs the CPU oracle (through the C-ABI)."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -255,3 +257,38 @@ def test_debug_select_old_blocks_host_twin(dev, orc):
     assert rc == 0 and n == len(wb) == 3 and total[0] == wtot == 10
     assert np.array_equal(blocks[:n], wb) and np.array_equal(scores[:n], ws)
     assert np.array_equal(start[:n], wst) and np.array_equal(end[:n], wen)
+
+
+def test_multi_slot_call_equals_per_slot_calls(dev, orc):
+    """Several sequences in one set of launches: same bits as one call per sequence (different lengths, one sequence
+    still without old blocks)."""
+    rng = np.random.default_rng(21)
+    qh, kvh, hd, W, bs, top, S = 8, 2, 128, 16, 8, 5, 200
+    nseq = 4
+    lens = np.array([200, 9, 77, 130], dtype=np.uint32)
+    kv = m40.KVCache(dev.ctx, S, nseq, kvh, hd, compressed=dict(recent_window=W, block_size=bs, top_blocks=top))
+    for s in range(nseq):
+        k16 = f16bits(rng.standard_normal((int(lens[s]), kvh, hd))); v16 = f16bits(rng.standard_normal((int(lens[s]), kvh, hd)))
+        dk, dv = dev.up(k16), dev.up(v16)
+        dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, s, dk.ptr, dv.ptr, int(lens[s]))
+    q = rng.standard_normal((nseq, qh * hd)).astype(np.float32)
+    dq = dev.up(q)
+    single = dev.zeros(q.nbytes); multi = dev.zeros(q.nbytes)
+    name = "m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async"
+    order = np.array([2, 0, 3, 1], dtype=np.uint32)          # slots in arbitrary order
+    for i, s in enumerate(order):
+        dev.call(name, kv.h, int(s), dq.ptr + i * qh * hd * 4, qh, int(lens[s]), W, bs, top, single.ptr + i * qh * hd * 4)
+    ids = order.copy(); ls = lens[order].copy()
+    dev.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, nseq, ids.ctypes.data_as(C.c_void_p),
+             ls.ctypes.data_as(C.c_void_p), dq.ptr, qh, W, bs, top, multi.ptr)
+    dev.sync()
+    a = single.download(np.float32, q.shape); b = multi.download(np.float32, q.shape)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.isfinite(a).all() and np.abs(a).max() > 0
+    # the same slot twice, too many slots
+    ids2 = np.array([1, 1], dtype=np.uint32)
+    dev.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, 2, ids2.ctypes.data_as(C.c_void_p),
+             ls.ctypes.data_as(C.c_void_p), dq.ptr, qh, W, bs, top, multi.ptr, expect=-2)
+    dev.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, 9, ids.ctypes.data_as(C.c_void_p),
+             ls.ctypes.data_as(C.c_void_p), dq.ptr, qh, W, bs, top, multi.ptr, expect=-2)
+    kv.destroy()
