@@ -7,7 +7,9 @@ greedy sample.  Workload at N=1: the TinyLlama-1.1B-shaped random-init model of 
 (22 layers, hidden 2048, 32/4 heads, head_dim 64, FFN 5632, vocab 32000, f16 weights N(0,0.02)), 32 random prompt
 ids, then greedy decode at batch 1.  Weights and KV cache are resident in HBM before the timed region.
 
-Prints ONE JSON line (see README / DESIGN.md for the field meanings).
+Prints ONE JSON line: value = decoded tokens per second (whole job); roofline = the dominant kernel's algorithmic
+bytes per launch over its event-timed launch duration against 8 TB/s, plus its measured HBM traffic; cpu_baseline =
+the CPU oracle timed on this host on a short sample of the same workload.
 """
 import argparse
 import ctypes as C
