@@ -259,6 +259,9 @@ int m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direc
  * the semantics of m40llm_gemm_f32xf16_gguf_f32.  Blocking, prefill stream. */
 int m40llm_ext_gemm_f32xq80_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_q80,
                                      void* d_C_f32, int M, int N, int K);
+/* The same product, asynchronous on the stream stream_kind names (0 prefill, 1 decode). */
+int m40llm_ext_gemm_f32xq80_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_q80,
+                                           void* d_C_f32, int M, int N, int K, uint32_t stream_kind);
 /* out[M,d_model] = down(swiglu(gate(x), up(x))) with q8_0 matrices; d_scratch_f32 holds
  * 2*M*ffn floats.  Decode stream, asynchronous. */
 int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_f32,

@@ -279,6 +279,208 @@ __global__ __launch_bounds__(256) void gemm_f32xq80_kernel(const float* __restri
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// q8_0 GEMV for one or two activation rows.  The activations never change between columns, so every
+// lane keeps the 32-value slice of the one block position it owns in registers for the whole launch
+// and streams only weights: kw waves (a team) split the blocks of a column into contiguous parts of an
+// even number of blocks, and a team walks over several columns with the blocks of the next columns
+// already in flight.  A block is 34 bytes at 2-byte alignment; with an even block count per column the
+// block's offset modulo 4 is twice its parity, which equals the lane's parity, so each lane reads nine
+// dwords from the dword-aligned address below its block and shifts by a per-lane constant.  The two
+// bytes read beyond an even block belong to the odd block that always follows it in the column; the
+// two bytes read before an odd block belong to the even block in front of it.  Quants go int8 -> f32
+// exactly; per block the partial sum of a*q is formed first and scaled by d once, as in the kernel
+// above.
+// ---------------------------------------------------------------------------------------
+constexpr int kQ80GemvThreads = 512;
+constexpr int kQ80GemvWaves = kQ80GemvThreads / 64;
+constexpr int kQ80GemvMaxCols = 32;   // columns per team of waves
+constexpr int kQ80GemvDepth = 4;      // columns in flight per wave
+constexpr int kQ80GemvChunk = 128;    // blocks of activations staged through LDS at a time (two float4 per thread)
+constexpr int kQ80GemvMaxChunks = 64 * kQ80GemvWaves / kQ80GemvChunk;
+static_assert(kQ80GemvChunk * 8 == 2 * kQ80GemvThreads, "two float4 per thread and chunk");
+
+struct Q80GemvArgs {
+    const float* A;        // [M][K]
+    const float* up;       // not null: the activations are silu(A) * up
+    const uint8_t* W[2];   // columns [0, N0) come from W[0] into C[0], [N0, N) from W[1] into C[1]
+    float* C[2];
+    int N0, N, K;
+    int kw;                // waves per column: 1, 2, 4 or 8
+    int per;               // blocks per wave (even, at most 64)
+};
+
+typedef uint32_t q80_u32x4 __attribute__((ext_vector_type(4), aligned(4)));   // dword-aligned 16-byte load
+
+__device__ __forceinline__ float q80_byte(uint32_t w, int n) {
+    return static_cast<float>(static_cast<int8_t>(w >> (8 * n)));
+}
+
+template <int ROWS>
+__global__ __launch_bounds__(kQ80GemvThreads) void q80_gemv_kernel(Q80GemvArgs p) {
+    __shared__ float part_s[kQ80GemvWaves][kQ80GemvMaxCols][ROWS];
+    __shared__ float act_s[ROWS][kQ80GemvChunk * 33];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int kw = p.kw, tpw = kQ80GemvWaves / kw;
+    const int kpart = wave & (kw - 1), team_local = wave / kw;
+    const int team = blockIdx.x * tpw + team_local, nteams = gridDim.x * tpw;
+    const int nblk = p.K >> 5;
+    const unsigned sh = (lane & 1) * 2;
+    const int blk_own = kpart * p.per + lane;
+    const bool have = lane < p.per && blk_own < nblk;
+    // Lanes without a block read a block of their own parity with zero activations, and columns beyond
+    // the last one re-read the last one: the loop below has no branch around a load, so the loads of
+    // the next columns stay in flight while one column is summed.
+    const int blk = have ? blk_own : (lane & 1);
+    const size_t col_bytes = (size_t)nblk * 34;
+    const size_t blk_off = (size_t)blk * 34 - sh;
+
+    uint32_t w[kQ80GemvDepth][9];
+    auto fetch = [&](uint32_t* dst, int col) {
+        col = min(col, p.N - 1);
+        const int m = col >= p.N0;
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(p.W[m] + (size_t)(col - (m ? p.N0 : 0)) * col_bytes + blk_off);
+        const q80_u32x4 lo = *reinterpret_cast<const q80_u32x4*>(src);
+        const q80_u32x4 hi = *reinterpret_cast<const q80_u32x4*>(src + 4);
+        dst[0] = lo.x; dst[1] = lo.y; dst[2] = lo.z; dst[3] = lo.w;
+        dst[4] = hi.x; dst[5] = hi.y; dst[6] = hi.z; dst[7] = hi.w;
+        dst[8] = src[8];
+    };
+#pragma unroll
+    for (int d = 0; d < kQ80GemvDepth; ++d) fetch(w[d], team + d * nteams);
+
+    // Activations: the workgroup reads each row once, coalesced (SwiGLU applied here when asked for), and
+    // passes it through LDS in chunks of 128 blocks, from which every lane picks the slice of its block.
+    // Rows of a block sit 33 floats apart so that the per-lane reads spread over the banks.
+    float a[ROWS][32];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+        for (int q = 0; q < 32; ++q) a[r][q] = 0.0f;
+    {
+        const int nchunks = (nblk + kQ80GemvChunk - 1) / kQ80GemvChunk;
+        float4 g[ROWS][kQ80GemvMaxChunks][2];
+#pragma unroll
+        for (int c = 0; c < kQ80GemvMaxChunks; ++c) {
+            if (c >= nchunks) break;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int e = (c * kQ80GemvChunk * 8 + h * kQ80GemvThreads + threadIdx.x) * 4;
+                    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                    if (e < p.K) {
+                        v = *reinterpret_cast<const float4*>(p.A + (size_t)r * p.K + e);
+                        if (p.up) {
+                            const float4 u = *reinterpret_cast<const float4*>(p.up + (size_t)r * p.K + e);
+                            v.x = v.x / (1.0f + expf(-v.x)) * u.x;
+                            v.y = v.y / (1.0f + expf(-v.y)) * u.y;
+                            v.z = v.z / (1.0f + expf(-v.z)) * u.z;
+                            v.w = v.w / (1.0f + expf(-v.w)) * u.w;
+                        }
+                    }
+                    g[r][c][h] = v;
+                }
+        }
+#pragma unroll
+        for (int c = 0; c < kQ80GemvMaxChunks; ++c) {
+            if (c >= nchunks) break;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int e = h * kQ80GemvThreads + threadIdx.x;     // float4 index inside the chunk
+                    float* dst = &act_s[r][(e >> 3) * 33 + (e & 7) * 4];
+                    dst[0] = g[r][c][h].x; dst[1] = g[r][c][h].y; dst[2] = g[r][c][h].z; dst[3] = g[r][c][h].w;
+                }
+            __syncthreads();
+            if (have && blk_own / kQ80GemvChunk == c) {
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r)
+#pragma unroll
+                    for (int q = 0; q < 32; ++q) a[r][q] = act_s[r][(blk_own % kQ80GemvChunk) * 33 + q];
+            }
+            __syncthreads();
+        }
+    }
+
+    int ncols = 0;
+    const int team_cols = team < p.N ? (p.N - team + nteams - 1) / nteams : 0;
+    for (int i0 = 0; i0 < team_cols; i0 += kQ80GemvDepth) {
+#pragma unroll
+        for (int d = 0; d < kQ80GemvDepth; ++d) {
+            const int col = team + (i0 + d) * nteams;
+            float acc[ROWS];
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) acc[r] = 0.0f;
+            uint32_t x[9];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = __builtin_amdgcn_alignbyte(w[d][i + 1], w[d][i], sh);
+            x[8] = __builtin_amdgcn_alignbyte(0u, w[d][8], sh);
+            fetch(w[d], col + kQ80GemvDepth * nteams);
+            const float dscale = m40_h2f(static_cast<uint16_t>(x[0] & 0xffffu));
+#pragma unroll
+            for (int q = 0; q < 32; ++q) {
+                const float f = q80_byte(x[(q + 2) >> 2], (q + 2) & 3);
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) acc[r] = fmaf(a[r][q], f, acc[r]);
+            }
+            const int m = col >= p.N0;
+            const int c = col - (m ? p.N0 : 0), nm = m ? p.N - p.N0 : p.N0;
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const float s = m40_sum64(acc[r] * dscale);
+                if (lane == 0 && col < p.N) {
+                    if (kw == 1) p.C[m][(size_t)r * nm + c] = s;
+                    else part_s[wave][i0 + d][r] = s;
+                }
+            }
+        }
+    }
+    (void)ncols;
+    if (kw == 1) return;
+    __syncthreads();
+    // One thread per (team, column, row) adds the K-parts in a fixed order.
+    for (int t = threadIdx.x; t < tpw * kQ80GemvMaxCols * ROWS; t += kQ80GemvThreads) {
+        const int r = t % ROWS, i = (t / ROWS) % kQ80GemvMaxCols, tl = t / (ROWS * kQ80GemvMaxCols);
+        const int col = blockIdx.x * tpw + tl + i * nteams;
+        if (col >= p.N) continue;
+        float s = 0.0f;
+        for (int k = 0; k < kw; ++k) s += part_s[tl * kw + k][i][r];
+        const int m = col >= p.N0;
+        const int c = col - (m ? p.N0 : 0), nm = m ? p.N - p.N0 : p.N0;
+        p.C[m][(size_t)r * nm + c] = s;
+    }
+}
+
+bool q80_gemv_supported(int M, int N, int K) {
+    // beyond two rows the f32 multiply-adds outweigh the weight stream and the matrix-core kernel is faster
+    return M >= 1 && M <= 2 && N >= 1 && K % 64 == 0 && K <= 64 * 32 * kQ80GemvWaves;
+}
+
+// W1/C1 may be null (one matrix of N columns); otherwise both matrices have N columns.
+int launch_q80_gemv(hipStream_t stream, const float* A, const float* up, const uint8_t* W0, float* C0,
+                    const uint8_t* W1, float* C1, int M, int N, int K) {
+    Q80GemvArgs p;
+    p.A = A; p.up = up;
+    p.W[0] = W0; p.C[0] = C0; p.W[1] = W1; p.C[1] = C1;
+    p.N0 = N; p.N = W1 ? 2 * N : N; p.K = K;
+    const int nblk = K / 32;
+    p.kw = 1;
+    while (p.kw * 64 < nblk) p.kw *= 2;
+    p.per = (nblk + p.kw - 1) / p.kw;
+    p.per += p.per & 1;
+    const int tpw = kQ80GemvWaves / p.kw;
+    const int cols_target = 16;   // columns per team: amortises the activation staging; measured best of 4..32
+    int nteams = (p.N + cols_target - 1) / cols_target;
+    int blocks = (nteams + tpw - 1) / tpw;
+    if (blocks < 1) blocks = 1;
+    if ((p.N + blocks * tpw - 1) / (blocks * tpw) > kQ80GemvMaxCols) return -2;
+    if (M == 1) q80_gemv_kernel<1><<<blocks, kQ80GemvThreads, 0, stream>>>(p);
+    else q80_gemv_kernel<2><<<blocks, kQ80GemvThreads, 0, stream>>>(p);
+    return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
 int pick_mfma_shape(int ntiles, int KT, int* T, int* S) {
     // Aim for a few thousand waves in flight and >= 512 workgroups where N allows it.
     int s = 1;
@@ -338,6 +540,8 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
 
 static int launch_q80(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint8_t* B,
                       float* C, int M, int N, int K) {
+    if (m40_aligned16(B) && m40_aligned16(A) && q80_gemv_supported(M, N, K))
+        return launch_q80_gemv(stream, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     if (m40_aligned16(B) && m40_aligned16(A) && m40_skinny_supported(ctx, stream_kind, M, N, K, 1))
         return m40_launch_skinny(ctx, stream, stream_kind, 1, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     (void)hipGetLastError();
@@ -421,6 +625,16 @@ int m40llm_ext_gemm_f32xq80_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32
     return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
 }
 
+int m40llm_ext_gemm_f32xq80_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_q80,
+                                           void* d_C_f32, int M, int N, int K, uint32_t stream_kind) {
+    if (!ctx || !d_A_f32 || !d_B_q80 || !d_C_f32) return -1;
+    if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0) return -2;
+    hipStream_t stream = m40_select_stream(ctx, stream_kind);
+    if (!stream) return -4;
+    return launch_q80(ctx, stream, stream_kind, static_cast<const float*>(d_A_f32),
+                      static_cast<const uint8_t*>(d_B_q80), static_cast<float*>(d_C_f32), M, N, K);
+}
+
 int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_w_gate_q80,
                                         const void* d_w_up_q80, const void* d_w_down_q80,
                                         void* d_scratch_f32, void* d_out_f32, int M, int d_model, int ffn) {
@@ -434,7 +648,16 @@ int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_
     const uint8_t* wu = static_cast<const uint8_t*>(d_w_up_q80);
     const uint8_t* wd = static_cast<const uint8_t*>(d_w_down_q80);
     float* out = static_cast<float*>(d_out_f32);
-    if (m40_aligned16(wg) && m40_aligned16(wu) && m40_aligned16(wd) && m40_aligned16(x) && m40_aligned16(gate) &&
+    const bool aligned = m40_aligned16(wg) && m40_aligned16(wu) && m40_aligned16(wd) && m40_aligned16(x) &&
+                         m40_aligned16(gate) && m40_aligned16(up);
+    if (aligned && q80_gemv_supported(M, ffn, d_model) && q80_gemv_supported(M, d_model, ffn)) {
+        // gate and up in one launch; SwiGLU is applied while each lane loads its slices for the down projection
+        (void)hipGetLastError();
+        int rc = launch_q80_gemv(ctx->decode_stream, x, nullptr, wg, gate, wu, up, M, ffn, d_model);
+        if (rc != 0) return rc;
+        return launch_q80_gemv(ctx->decode_stream, gate, up, wd, out, nullptr, nullptr, M, d_model, ffn);
+    }
+    if (aligned &&
         m40_skinny_supported(ctx, 1, M, ffn, d_model, 1) &&
         m40_skinny_supported(ctx, 1, M, d_model, ffn, 1)) {
         // gate and up in one launch; SwiGLU is applied while the hidden row is packed for the down projection

@@ -139,7 +139,7 @@ def bench_q80(b: Bench):
     nset = 6
     sets = [(b.ctx.to_device(gate), b.ctx.to_device(up), b.ctx.to_device(down)) for _ in range(nset)]
     wbytes = gate.nbytes + up.nbytes + down.nbytes
-    for M in (1, 4, 16):
+    for M in (1, 2, 4, 16):
         x = b.ctx.to_device(rng.standard_normal((M, d_model)).astype(np.float32))
         scratch = b.ctx.alloc(2 * M * ffn * 4)
         out = b.ctx.alloc(M * d_model * 4)
@@ -147,10 +147,14 @@ def bench_q80(b: Bench):
         b.time("ffn_swiglu_q80", f"M={M} d_model 4096 ffn 14336", algo,
                lambda i: b.call("m40llm_ext_ffn_swiglu_q80_f32_async", x.ptr, sets[i][0].ptr, sets[i][1].ptr, sets[i][2].ptr,
                                 scratch.ptr, out.ptr, M, d_model, ffn), nset)
-    a = b.ctx.to_device(rng.standard_normal((1, d_model)).astype(np.float32))
-    c = b.ctx.alloc(ffn * 4)
-    b.time("gemm_f32xq80_gguf M=1", "N=14336 K=4096", gate.nbytes,
-           lambda i: b.call("m40llm_ext_gemm_f32xq80_gguf_f32", a.ptr, sets[i][0].ptr, c.ptr, 1, ffn, d_model), nset, stream=0)
+    for M in (1, 2, 4, 16):
+        a = b.ctx.to_device(rng.standard_normal((M, d_model)).astype(np.float32))
+        c = b.ctx.alloc(M * ffn * 4)
+        b.time(f"gemm_f32xq80_gguf M={M}", "N=14336 K=4096", gate.nbytes,
+               lambda i: b.call("m40llm_ext_gemm_f32xq80_gguf_f32_async", a.ptr, sets[i][0].ptr, c.ptr, M, ffn, d_model, 1), nset)
+        a2 = b.ctx.to_device(rng.standard_normal((M, ffn)).astype(np.float32))
+        b.time(f"gemm_f32xq80_gguf M={M}", "N=4096 K=14336", down.nbytes,
+               lambda i: b.call("m40llm_ext_gemm_f32xq80_gguf_f32_async", a2.ptr, sets[i][2].ptr, c.ptr, M, d_model, ffn, 1), nset)
 
 
 def bench_block_select(b: Bench):

@@ -261,7 +261,7 @@ def test_gemm_rowmajor_vs_oracle(dev, orc):
     close(dC.download(np.float32, (M, N)), orc.gemm("f16xf16_rowmajor", A16, B, M, N, K), 1e-4, 1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 16])
 def test_q80_gemm_and_ffn_vs_oracle(dev, orc, M):
     rng = np.random.default_rng(11 + M)
     d_model, ffn = 256, 512
@@ -284,9 +284,11 @@ def test_q80_gemm_and_ffn_vs_oracle(dev, orc, M):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 1000, 768), (8, 4096, 2048), (9, 520, 1280), (16, 2048, 4096),
-                                   (20, 333, 256), (2, 64, 96)])
+                                   (20, 333, 256), (2, 64, 96), (1, 1000, 4096), (2, 777, 8192), (1, 513, 14336),
+                                   (2, 260, 11008), (1, 40, 16384), (2, 3, 64)])
 def test_q80_gemm_shapes_vs_oracle(dev, orc, M, N, K):
-    """MFMA path (K % 256 == 0; column tails, split K, more than 16 rows) and the simple path (K = 96)."""
+    """MFMA path (3 rows and more, K % 256 == 0; column tails, split K, more than 16 rows), the register-resident
+    GEMV of one and two rows (K % 64 == 0, one, two and four K-parts per column) and the simple path (K = 96)."""
     rng = np.random.default_rng(M * 7919 + N + K)
     d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
     qs = rng.integers(-127, 128, size=(N, K // 32, 32)).astype(np.int8)
