@@ -2,24 +2,28 @@
 // per pass and W either f16 (GGUF order, K contiguous per output column) or q8_0 (34-byte blocks along K).
 //
 // The activations are split once per call into f16 hi + f16 lo fragments with a per-row power-of-two scale
-// (pack kernel below); the product runs on v_mfma_f32_16x16x32_f16 with f32 accumulation.  One MFMA covers
+// (inside the kernel, step by step); the product runs on v_mfma_f32_16x16x32_f16 with f32 accumulation.  One MFMA covers
 // 32 consecutive k, which is exactly one q8_0 block, so the block scale multiplies the MFMA result.
 //
-// A workgroup is eight waves = eight 16-column tiles that walk the same range of K in steps of 256.  The
-// activation fragments of a step (8 KB, or 16 KB above eight rows) are loaded once per workgroup into LDS and
-// shared by the eight waves; weights are read once, straight from their GGUF bytes:
+// A workgroup is four waves = four 16-column tiles that walk the same range of K in steps of 256.  The
+// activation fragments of a step (8 KB, or 16 KB above eight rows) are converted once per workgroup into LDS
+// and shared by the four waves; weights are read once, straight from their GGUF bytes:
 //   f16  : lane (column j, group g) loads its 16 bytes of k = 32 i + 8 g .. +7 per MFMA;
 //   q8_0 : the 16 columns x 272 bytes of a step are copied with full 16-byte loads into a wave-private LDS
 //          tile; each lane then reads the 8 quants of its (column, block, group) and turns them into f16 with
 //          the 1024 + (q xor 0x80) construction (exact).
-// Loads of step t+1 are in flight while step t is multiplied.  K is split over grid.y; slices write partial
-// sums that a second kernel adds in slice order, so results never depend on timing.
+// Weight loads run two steps ahead of the step being multiplied and activation loads one step ahead, in a
+// fixed issue order with no load under a branch, so that each wait names exactly the loads it needs and the
+// younger ones stay in flight.  K is split over grid.y; slices write partial sums that a second kernel adds in
+// slice order, so results never depend on timing.
 #include "common.hpp"
+
+#include <type_traits>
 
 namespace {
 
 constexpr int kTileK = 256;                       // k per step
-constexpr int kWavesPerGroup = 8;                 // 16-column tiles per workgroup
+constexpr int kWavesPerGroup = 4;                 // 16-column tiles per workgroup
 constexpr int kThreads = kWavesPerGroup * 64;
 constexpr int kQ8ColStride = 276;                 // LDS bytes per column of a staged tile: 272 + 4, an odd number of
                                                   // dwords, so that the 16 columns start in different banks
@@ -56,7 +60,7 @@ struct SkinnyArgs {
 
 // FMT 0: f16 weights, 1: q8_0 weights.
 template <int FMT, bool STACKED>
-__global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) {
+__global__ __launch_bounds__(kThreads, 2) void skinny_mfma_kernel(SkinnyArgs p) {
     constexpr int kASets = STACKED ? 1 : 2;
     __shared__ __attribute__((aligned(16))) uint2 a_lds[2][kASets][8 * 64 * 2];                    // activation fragments of a step, two buffers
     __shared__ float tscale_s[2][16];                                   // factor that undoes each row's scaling of the step
@@ -77,37 +81,42 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
     // ---- weight addressing
     const int col = n0 + j < N ? n0 + j : N - 1;
     const uint16_t* w16 = nullptr;
-    const uint8_t* q_src[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    const uint8_t* q_base = nullptr;
+    uint32_t q_src[5] = {0, 0, 0, 0, 0};      // byte offsets of this lane's tile pieces from q_base (step 0)
     int q_dst[5] = {0, 0, 0, 0, 0};
     uint8_t* my_b = b_lds + (FMT == 1 ? wave * kQ8TileBytes : 0);
     if (FMT == 0) {
         w16 = static_cast<const uint16_t*>(p.W[z]) + (size_t)col * p.K + 8 * g;
     } else {
         const size_t col_stride = (size_t)(p.K >> 5) * 34;
-        const uint8_t* base = static_cast<const uint8_t*>(p.W[z]);
+        q_base = static_cast<const uint8_t*>(p.W[z]) + (size_t)n0 * col_stride;
 #pragma unroll
         for (int i = 0; i < 5; ++i) {
-            const int q = i * 64 + lane;          // 16-byte piece of the 16 x 272-byte tile
-            if (q < 272) {
-                const int c = q / 17, piece = q % 17;
-                const int cc = n0 + c < N ? n0 + c : N - 1;
-                q_src[i] = base + (size_t)cc * col_stride + 16 * piece;
-                q_dst[i] = c * kQ8ColStride + 16 * piece;
-            }
+            int q = i * 64 + lane;                // 16-byte piece of the 16 x 272-byte tile
+            if (q >= 272) q = lane;               // no such piece: repeat this lane's first one, so that no load sits
+                                                  // under a branch (a skipped load would make every wait conservative)
+            const int c = q / 17, piece = q % 17;
+            const int cc = n0 + c < N ? c : N - 1 - n0;
+            q_src[i] = (uint32_t)((size_t)cc * col_stride + 16 * piece);
+            q_dst[i] = c * kQ8ColStride + 16 * piece;
         }
     }
 
     // ---- activation addressing: thread (arow, acol) owns EPT consecutive k of row arow in every step:
     // k = 256 kt + EPT acol .. ; eight consecutive k form entry (MFMA i = k / 32, group (k / 8) % 4) of the fragments.
-    // Up to eight rows: a whole wave per row (4 elements per lane); above: 32 lanes per row (8 elements per lane).
-    constexpr int EPT = STACKED ? 4 : 8;
+    // Up to eight rows: 32 lanes per row (8 elements per lane); above: 16 lanes per row (16 elements per lane).
+    constexpr int EPT = STACKED ? 8 : 16;
     constexpr int TPR = kTileK / EPT;
+    static_assert(TPR * (STACKED ? 8 : 16) == kThreads, "one thread per EPT activations of a step");
     const int arow = tid / TPR, acol = tid % TPR;
     const bool a_live = arow < p.M;
     const float* a_ptr = p.A + (size_t)(a_live ? arow : 0) * p.K + EPT * acol;
-    const float* u_ptr = p.up ? p.up + (size_t)(a_live ? arow : 0) * p.K + EPT * acol : nullptr;
-    const uint16_t* nw16 = static_cast<const uint16_t*>(p.norm_w);
-    const float* nw32 = static_cast<const float*>(p.norm_w);
+    // SwiGLU partner or f32 norm weights; with neither, the activations themselves (loaded and ignored: the same
+    // loads are issued whatever the operand is)
+    const bool norm16 = p.norm_w && p.norm_dtype == 0u;
+    const float* b_ptr = p.up ? p.up + (size_t)(a_live ? arow : 0) * p.K + EPT * acol
+                              : (p.norm_w && !norm16 ? static_cast<const float*>(p.norm_w) + EPT * acol : a_ptr);
+    const uint16_t* nw16 = norm16 ? static_cast<const uint16_t*>(p.norm_w) + EPT * acol : nullptr;
     auto load_f32 = [&](const float* src, float (&v)[EPT]) {
 #pragma unroll
         for (int e = 0; e < EPT; e += 4) {
@@ -115,47 +124,47 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
             v[e] = x.x; v[e + 1] = x.y; v[e + 2] = x.z; v[e + 3] = x.w;
         }
     };
-    auto load_norm = [&](int k, float (&v)[EPT]) {
-        if (p.norm_dtype == 0u) {
-#pragma unroll
-            for (int e = 0; e < EPT; e += 4) {
-                const uint2 w = *reinterpret_cast<const uint2*>(nw16 + k + e);
-                v[e] = m40_h2f((uint16_t)(w.x & 0xffffu)); v[e + 1] = m40_h2f((uint16_t)(w.x >> 16));
-                v[e + 2] = m40_h2f((uint16_t)(w.y & 0xffffu)); v[e + 3] = m40_h2f((uint16_t)(w.y >> 16));
-            }
-        } else {
-            load_f32(nw32 + k, v);
-        }
-    };
     auto row_reduce_max = [&](float x) -> float {
-        if (STACKED) return m40_max64(x);
 #pragma unroll
-        for (int o = 1; o < 32; o <<= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+        for (int o = 1; o < TPR; o <<= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
         return x;
     };
 
     float fa[EPT], fb[EPT];    // this thread's activations of a step (and their SwiGLU partner or norm weights)
-    uint4 rb[8];               // f16: the eight 16-byte weight loads of a step; q8_0: five tile pieces
+    constexpr int NW = FMT == 0 ? 8 : 5;
+    uint4 rb[2][NW];           // weights of two steps in flight.  f16: eight 16-byte loads; q8_0: five tile pieces
     auto issue_a = [&](int kt) {
         load_f32(a_ptr + (size_t)kt * kTileK, fa);
-        if (u_ptr) load_f32(u_ptr + (size_t)kt * kTileK, fb);
-        else if (p.norm_w) load_norm(kt * kTileK + EPT * acol, fb);
+        if (norm16) {
+#pragma unroll
+            for (int e = 0; e < EPT; e += 4) {
+                const uint2 w = *reinterpret_cast<const uint2*>(nw16 + (size_t)kt * kTileK + e);
+                fb[e / 2] = __uint_as_float(w.x); fb[e / 2 + 1] = __uint_as_float(w.y);   // raw f16 pairs
+            }
+        } else {
+            load_f32(b_ptr + (size_t)kt * kTileK, fb);
+        }
     };
-    auto issue_w = [&](int kt) {
+    auto issue_w = [&](uint4 (&dst)[NW], int kt) {
         if (FMT == 0) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                rb[i] = m40_load_stream(reinterpret_cast<const uint4*>(w16 + (size_t)kt * kTileK + 32 * i));
+                dst[i] = m40_load_stream(reinterpret_cast<const uint4*>(w16 + (size_t)kt * kTileK + 32 * i));
         } else {
 #pragma unroll
             for (int i = 0; i < 5; ++i)
-                if (q_src[i]) rb[i] = m40_load_stream(reinterpret_cast<const uint4*>(q_src[i] + (size_t)kt * 272));
+                dst[i] = m40_load_stream(reinterpret_cast<const uint4*>(q_base + (size_t)kt * 272 + q_src[i]));
         }
     };
 
+    const int nsteps = kt1 - kt0;
     m40_float4 acc = {0.f, 0.f, 0.f, 0.f};
-    issue_w(kt0);              // weights of the first step are in flight during the prologue
+    // Order of issue, kept through the loop: activations of step s+1, then weights of step s+2.  A wait for the
+    // activations leaves the younger weight loads in flight; a wait for the weights of step s+1 leaves those of
+    // step s+2 in flight.
     issue_a(kt0);
+    issue_w(rb[0], kt0);
+    issue_w(rb[1], nsteps > 1 ? kt0 + 1 : kt0);      // a one-step slice loads its step twice (rare: K of 256 only)
 
     // RMS over the whole row (RMSNorm operand only)
     float rms = 1.0f;
@@ -167,12 +176,8 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
 #pragma unroll
             for (int e = 0; e < EPT; ++e) sq = fmaf(v[e], v[e], sq);
         }
-        if (STACKED) {
-            sq = m40_sum64(sq);
-        } else {
 #pragma unroll
-            for (int o = 1; o < 32; o <<= 1) sq += __shfl_xor(sq, o, 64);
-        }
+        for (int o = 1; o < TPR; o <<= 1) sq += __shfl_xor(sq, o, 64);
         rms = rsqrtf(sq / (float)p.K + p.eps);
     }
 
@@ -183,8 +188,9 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
         float mx = 0.0f;
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
-            float v = a_live ? fa[e] : 0.0f;
-            if (u_ptr) v = v / (1.0f + expf(-v)) * fb[e];
+            float v = fa[e];
+            if (p.up) v = v / (1.0f + expf(-v)) * fb[e];
+            else if (norm16) v = v * rms * m40_h2f((uint16_t)((__float_as_uint(fb[e / 2]) >> (16 * (e & 1))) & 0xffffu));
             else if (p.norm_w) v = v * rms * fb[e];
             if (!a_live) v = 0.0f;
             x[e] = v;
@@ -214,14 +220,14 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
             }
             hi[e / 2] = h2; lo[e / 2] = l2;
         }
-        const int k0 = EPT * acol;                                   // first k of this thread within the step
-        const int entry = (k0 >> 5) * 64 + ((k0 >> 3) & 3) * 16 + arow;
+        uint4* frag_hi = reinterpret_cast<uint4*>(a_lds[buf][0]);
+        uint4* frag_lo = reinterpret_cast<uint4*>(a_lds[buf][kASets - 1]);
 #pragma unroll
-        for (int e = 0; e < EPT / 4; ++e) {
-            const int sub = ((k0 >> 2) & 1) + e;                     // which half of the 8-half entry
-            a_lds[buf][0][entry * 2 + sub] = make_uint2(hi[2 * e], hi[2 * e + 1]);
-            if (STACKED) a_lds[buf][0][(entry + 8) * 2 + sub] = make_uint2(lo[2 * e], lo[2 * e + 1]);
-            else a_lds[buf][kASets - 1][entry * 2 + sub] = make_uint2(lo[2 * e], lo[2 * e + 1]);
+        for (int c = 0; c < EPT / 8; ++c) {
+            const int kk = EPT * acol + 8 * c;                       // first k of this eight within the step
+            const int entry = (kk >> 5) * 64 + ((kk >> 3) & 3) * 16 + arow;
+            frag_hi[entry] = make_uint4(hi[4 * c], hi[4 * c + 1], hi[4 * c + 2], hi[4 * c + 3]);
+            frag_lo[STACKED ? entry + 8 : entry] = make_uint4(lo[4 * c], lo[4 * c + 1], lo[4 * c + 2], lo[4 * c + 3]);
         }
         if (acol == 0) {
             tscale_s[buf][arow] = scale;
@@ -230,35 +236,31 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
     };
     convert(0);
 
-    for (int kt = kt0; kt < kt1; ++kt) {
-        const int buf = (kt - kt0) & 1;
-        uint4 wb[8];
-        if (FMT == 0) {
+    // One step.  BUF: which of the two fragment / weight buffers holds it; PREFETCH: steps s+1 (activations) and
+    // s+2 (weights) exist and are requested here; LAST: no step follows.
+    auto step = [&](auto buf_c, auto prefetch_c, auto last_c, int kt) {
+        constexpr int BUF = decltype(buf_c)::value;
+        constexpr bool PREFETCH = decltype(prefetch_c)::value;
+        constexpr bool LAST = decltype(last_c)::value;
+        if (FMT == 1) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) wb[i] = rb[i];
-        } else {
-#pragma unroll
-            for (int i = 0; i < 5; ++i)
-                if (q_src[i]) {
-                    uint32_t* dst = reinterpret_cast<uint32_t*>(my_b + q_dst[i]);      // 4-byte aligned only
-                    dst[0] = rb[i].x; dst[1] = rb[i].y; dst[2] = rb[i].z; dst[3] = rb[i].w;
-                }
+            for (int i = 0; i < 5; ++i) {
+                uint32_t* dst = reinterpret_cast<uint32_t*>(my_b + q_dst[i]);      // 4-byte aligned only
+                dst[0] = rb[BUF][i].x; dst[1] = rb[BUF][i].y; dst[2] = rb[BUF][i].z; dst[3] = rb[BUF][i].w;
+            }
         }
         __syncthreads();       // fragments of this step are complete; nobody still reads the other buffer
-        const bool more = kt + 1 < kt1;
-        if (more) {
-            issue_w(kt + 1);
-            issue_a(kt + 1);
-        }
+        if (!LAST) issue_a(kt + 1);
+        if (FMT == 1 && PREFETCH) issue_w(rb[BUF], kt + 2);
         m40_float4 tacc = {0.f, 0.f, 0.f, 0.f};
-        const uint4* a_hi_frag = reinterpret_cast<const uint4*>(a_lds[buf][0]);
-        const uint4* a_lo_frag = reinterpret_cast<const uint4*>(a_lds[buf][kASets - 1]);
+        const uint4* a_hi_frag = reinterpret_cast<const uint4*>(a_lds[BUF][0]);
+        const uint4* a_lo_frag = reinterpret_cast<const uint4*>(a_lds[BUF][kASets - 1]);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint4 a_hi = a_hi_frag[i * 64 + lane];
             if (FMT == 0) {
-                tacc = mfma16x16x32(a_hi, wb[i], tacc);
-                if (!STACKED) tacc = mfma16x16x32(a_lo_frag[i * 64 + lane], wb[i], tacc);
+                tacc = mfma16x16x32(a_hi, rb[BUF][i], tacc);
+                if (!STACKED) tacc = mfma16x16x32(a_lo_frag[i * 64 + lane], rb[BUF][i], tacc);
             } else {
                 const uint8_t* blk = my_b + j * kQ8ColStride + 34 * i;
                 const float d = m40_h2f(*reinterpret_cast<const uint16_t*>(blk));
@@ -286,9 +288,31 @@ __global__ __launch_bounds__(kThreads, 4) void skinny_mfma_kernel(SkinnyArgs p) 
                 for (int r = 0; r < 4; ++r) tacc[r] = fmaf(d, dblk[r], tacc[r]);
             }
         }
+        if (FMT == 0 && PREFETCH) issue_w(rb[BUF], kt + 2);   // the matrix cores have read this buffer
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] = fmaf(tscale_s[buf][4 * g + r], tacc[r], acc[r]);
-        if (more) convert(buf ^ 1);      // next step's fragments, while the other waves finish this one
+        for (int r = 0; r < 4; ++r) acc[r] = fmaf(tscale_s[BUF][4 * g + r], tacc[r], acc[r]);
+        if (!LAST) convert(BUF ^ 1);     // next step's fragments, while the other waves finish this one
+    };
+    {
+        using std::integral_constant;
+        const integral_constant<int, 0> b0; const integral_constant<int, 1> b1;
+        const integral_constant<bool, true> yes; const integral_constant<bool, false> no;
+        int s = 0;
+        for (; s + 3 < nsteps; s += 2) {          // both steps of a pair have a step two ahead
+            step(b0, yes, no, kt0 + s);
+            step(b1, yes, no, kt0 + s + 1);
+        }
+        const int rem = nsteps - s;               // 1, 2 or 3
+        if (rem == 3) {
+            step(b0, yes, no, kt0 + s);
+            step(b1, no, no, kt0 + s + 1);
+            step(b0, no, yes, kt0 + s + 2);
+        } else if (rem == 2) {
+            step(b0, no, no, kt0 + s);
+            step(b1, no, yes, kt0 + s + 1);
+        } else {
+            step(b0, no, yes, kt0 + s);
+        }
     }
     // lane (j, g) holds rows 4g + r of column j
     if (STACKED) {
@@ -446,7 +470,7 @@ __global__ __launch_bounds__(1024) void greedy_batch_kernel(GreedyBatchArgs a) {
 int pick_slices(int ntiles, int KT, int num_cus) {
     const long long groups = (ntiles + kWavesPerGroup - 1) / kWavesPerGroup;
     int s = 1;
-    while (s < 16 && groups * s < 2LL * num_cus && KT / (s * 2) >= 1) s *= 2;
+    while (s < 16 && groups * s < 3LL * num_cus && KT / (s * 2) >= 2) s *= 2;   // three workgroups fit a CU; two steps or more per slice
     return s > KT ? KT : s;
 }
 
