@@ -279,8 +279,8 @@ int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, 
               uint32_t group, uint32_t span) {
     constexpr uint32_t kRowsPerStep = kWaves * (64 / (HD / 8));   // token rows one workgroup covers per S
     M40StreamScratch& scr = ctx->scratch[stream_kind];
-    if (span > 512) {
-        // long rows: matrix-core kernel, chunks of a multiple of 128 tokens sized so the grid covers the CUs about twice
+    if (span > 512 && m40_aligned16(p.Q)) {
+        // long rows: matrix-core kernel (it reads q with 16-byte loads), chunks of a multiple of 128 tokens sized so the grid covers the CUs about twice
         p.subgroups = (group + 7) / 8;
         const uint64_t groups = (uint64_t)batch * p.kv_heads * p.subgroups;
         uint64_t chunk = ((uint64_t)span * groups + 2ull * ctx->num_cus - 1) / (2ull * ctx->num_cus);

@@ -42,7 +42,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_mfma_kernel(AttnParams p) {
     constexpr int PIECES = HD / 8;         // 16-byte pieces per row
     __shared__ __attribute__((aligned(16))) uint8_t v_lds[kWaves][kTile * RS];
     __shared__ __attribute__((aligned(16))) uint16_t p_lds[kWaves][16][40];      // rows of 80 bytes
-    __shared__ float red_s[kWaves];
     __shared__ float m_s[kWaves][8], l_s[kWaves][8];
     __shared__ float o_s[kWaves][8][HD];
 
@@ -93,12 +92,28 @@ __global__ __launch_bounds__(kThreads, 2) void attn_mfma_kernel(AttnParams p) {
     if (my_tiles_begin < ntiles) issue(my_tiles_begin);
 
     // ---- q fragments: power-of-two scaled, split into f16 hi + lo -----------------------------------------
+    // A-operand row rho = c16: head 2*(rho/4) + (rho%4)/2, part rho&1 (0 hi, 1 lo).  Every wave holds each q value
+    // of the group (twice: hi and lo lanes), so the largest magnitude needs no exchange between waves.  All loads
+    // go out together, behind the first tile's.
+    const uint32_t qhead = 2u * (uint32_t)(c16 >> 2) + (uint32_t)((c16 & 3) >> 1);
+    const bool q_live = qhead < gcount;
+    float qv[KS][8];
+    {
+        const float* qp = Qb + (size_t)(q_live ? qhead : 0u) * HD + 8 * g;
+#pragma unroll
+        for (int i = 0; i < KS; ++i) {
+            const float4 x = *reinterpret_cast<const float4*>(qp + 32 * i);
+            const float4 y = *reinterpret_cast<const float4*>(qp + 32 * i + 4);
+            qv[i][0] = x.x; qv[i][1] = x.y; qv[i][2] = x.z; qv[i][3] = x.w;
+            qv[i][4] = y.x; qv[i][5] = y.y; qv[i][6] = y.z; qv[i][7] = y.w;
+        }
+    }
     float qmax = 0.0f;
-    for (uint32_t e = tid; e < gcount * HD; e += kThreads) qmax = fmaxf(qmax, fabsf(Qb[e]));
+#pragma unroll
+    for (int i = 0; i < KS; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qmax = fmaxf(qmax, q_live ? fabsf(qv[i][j]) : 0.0f);
     qmax = m40_max64(qmax);
-    if (lane == 0) red_s[wave] = qmax;
-    __syncthreads();
-    qmax = fmaxf(fmaxf(red_s[0], red_s[1]), fmaxf(red_s[2], red_s[3]));
     float q_inv = 1.0f, q_scale = 1.0f;
     if (qmax > 0.0f && qmax < INFINITY) {
         int e;
@@ -109,25 +124,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_mfma_kernel(AttnParams p) {
         q_inv = ldexpf(1.0f, -e);
     }
     const float score_scale = (HD == 64 ? 0.125f : 0.08838834764831845f) * q_scale;
-    // A-operand row rho = c16: head 2*(rho/4) + (rho%4)/2, part rho&1 (0 hi, 1 lo)
     uint4 qf[KS];
     {
-        const uint32_t h = 2u * (uint32_t)(c16 >> 2) + (uint32_t)((c16 & 3) >> 1);
         const bool lo_part = (c16 & 1) != 0;
 #pragma unroll
         for (int i = 0; i < KS; ++i) {
             uint32_t w[4] = {0, 0, 0, 0};
-            if (h < gcount) {
-                const float* qp = Qb + (size_t)h * HD + 32 * i + 8 * g;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float a = qp[j] * q_inv;
-                    const _Float16 hi = static_cast<_Float16>(a);
-                    const _Float16 v = lo_part ? static_cast<_Float16>(a - static_cast<float>(hi)) : hi;
-                    w[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, v) << (16 * (j & 1));
-                }
+            for (int j = 0; j < 8; ++j) {
+                const float a = qv[i][j] * q_inv;
+                const _Float16 hi = static_cast<_Float16>(a);
+                const _Float16 v = lo_part ? static_cast<_Float16>(a - static_cast<float>(hi)) : hi;
+                w[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, v) << (16 * (j & 1));
             }
-            qf[i] = make_uint4(w[0], w[1], w[2], w[3]);
+            qf[i] = q_live ? make_uint4(w[0], w[1], w[2], w[3]) : make_uint4(0, 0, 0, 0);
         }
     }
 
