@@ -56,6 +56,8 @@ struct SkinnyArgs {
     size_t part_off[3];        // float offset of matrix z in `partial`; layout there [S][16][N z]
     float* partial;
     int nmat, M, K, S, direct;
+    int rms_deferred;          // RMSNorm operand: the kernel multiplies by A * norm_w only, and the kernel that adds the
+                               // slices scales each row by rsqrt(mean(A^2) + eps) (the product is linear in that factor)
 };
 
 // FMT 0: f16 weights, 1: q8_0 weights.
@@ -166,15 +168,20 @@ __global__ __launch_bounds__(kThreads, 2) void skinny_mfma_kernel(SkinnyArgs p) 
     issue_w(rb[0], kt0);
     issue_w(rb[1], nsteps > 1 ? kt0 + 1 : kt0);      // a one-step slice loads its step twice (rare: K of 256 only)
 
-    // RMS over the whole row (RMSNorm operand only)
+    // RMS over the whole row (RMSNorm operand whose scale is not left to the slice-adding kernel)
     float rms = 1.0f;
-    if (p.norm_w && a_live) {
+    if (p.norm_w && !p.rms_deferred && a_live) {
         float sq = 0.0f;
-        for (int k = 0; k < p.K; k += kTileK) {
-            float v[EPT];
-            load_f32(a_ptr + k, v);
+        for (int k = 0; k < p.K; k += 4 * kTileK) {
+            float v[4][EPT];
 #pragma unroll
-            for (int e = 0; e < EPT; ++e) sq = fmaf(v[e], v[e], sq);
+            for (int u = 0; u < 4; ++u) load_f32(a_ptr + (k + u * kTileK < p.K ? k + u * kTileK : k), v[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (k + u * kTileK < p.K) {
+#pragma unroll
+                    for (int e = 0; e < EPT; ++e) sq = fmaf(v[u][e], v[u][e], sq);
+                }
         }
 #pragma unroll
         for (int o = 1; o < TPR; o <<= 1) sq += __shfl_xor(sq, o, 64);
@@ -355,16 +362,42 @@ struct EpilogueArgs {
     const float* residual;
     int mode;
 };
+// rsqrt(mean(A[row]^2) + eps) by a 256-thread workgroup, the same value in every thread; fixed summation order.
+__device__ __forceinline__ float skinny_row_rms(const SkinnyArgs& g, int row) {
+    __shared__ float red_s[4];
+    const float* a = g.A + (size_t)row * g.K;
+    float sq = 0.0f;
+    for (int k0 = 0; k0 < g.K; k0 += 4096) {          // four 16-byte loads in flight per thread
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = k0 + u * 1024 + 4 * (int)threadIdx.x;
+            v[u] = k < g.K ? *reinterpret_cast<const float4*>(a + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            sq = fmaf(v[u].x, v[u].x, sq); sq = fmaf(v[u].y, v[u].y, sq);
+            sq = fmaf(v[u].z, v[u].z, sq); sq = fmaf(v[u].w, v[u].w, sq);
+        }
+    }
+    sq = m40_sum64(sq);
+    if ((threadIdx.x & 63u) == 0u) red_s[threadIdx.x >> 6] = sq;
+    __syncthreads();
+    sq = (red_s[0] + red_s[1]) + (red_s[2] + red_s[3]);
+    return rsqrtf(sq / (float)g.K + g.eps);
+}
+
 __global__ __launch_bounds__(256) void skinny_epilogue_kernel(EpilogueArgs e) {
     const int z = blockIdx.z, row = blockIdx.y;
     const int n = blockIdx.x * 256 + threadIdx.x;
+    const float rms = (e.g.norm_w && e.g.rms_deferred) ? skinny_row_rms(e.g, row) : 1.0f;
     if (n >= e.g.N[z]) return;
     if (e.mode == 1) {
-        const float gate = skinny_sum(e.g, 0, row, n), up = skinny_sum(e.g, 1, row, n);
+        const float gate = rms * skinny_sum(e.g, 0, row, n), up = rms * skinny_sum(e.g, 1, row, n);
         e.out[0][(size_t)row * e.g.N[0] + n] = gate / (1.0f + expf(-gate)) * up;
         return;
     }
-    float v = skinny_sum(e.g, z, row, n);
+    float v = rms * skinny_sum(e.g, z, row, n);
     if (e.bias) v = v + e.bias[n];
     if (e.residual) v = e.residual[(size_t)row * e.g.N[z] + n] + v;
     e.out[z][(size_t)row * e.g.N[z] + n] = v;
@@ -387,6 +420,7 @@ __global__ __launch_bounds__(256) void skinny_qkv_epilogue_kernel(QkvEpilogueArg
     const uint32_t half = e.head_dim / 2u;
     const uint32_t q_pairs = e.q_heads * half, kv_pairs = e.kv_heads * half;
     const uint32_t pair = blockIdx.x * 256u + threadIdx.x;
+    const float rms = (e.g.norm_w && e.g.rms_deferred) ? skinny_row_rms(e.g, (int)row) : 1.0f;
     if (pair >= q_pairs + 2u * kv_pairs) return;
     int which;
     uint32_t local;
@@ -397,7 +431,7 @@ __global__ __launch_bounds__(256) void skinny_qkv_epilogue_kernel(QkvEpilogueArg
     size_t i0, i1;
     m40_rope_pair(head, off, e.head_dim, which == 2 ? M40LLM_ROPE_LAYOUT_ADJACENT : e.rope_layout, &i0, &i1);
     const float* bias = which == 0 ? e.bq : (which == 1 ? e.bk : e.bv);
-    float y0 = skinny_sum(e.g, which, (int)row, (int)i0), y1 = skinny_sum(e.g, which, (int)row, (int)i1);
+    float y0 = rms * skinny_sum(e.g, which, (int)row, (int)i0), y1 = rms * skinny_sum(e.g, which, (int)row, (int)i1);
     if (bias) { y0 = y0 + bias[i0]; y1 = y1 + bias[i1]; }
     const uint32_t position = e.lens_dev[row];
     const uint32_t seq = e.ids_dev[row];
@@ -470,7 +504,8 @@ __global__ __launch_bounds__(1024) void greedy_batch_kernel(GreedyBatchArgs a) {
 int pick_slices(int ntiles, int KT, int num_cus) {
     const long long groups = (ntiles + kWavesPerGroup - 1) / kWavesPerGroup;
     int s = 1;
-    while (s < 16 && groups * s < 3LL * num_cus && KT / (s * 2) >= 2) s *= 2;   // three workgroups fit a CU; two steps or more per slice
+    // Measured on the batched decode step: about 1.5 workgroups per CU and at least two steps per slice.
+    while (s < 16 && groups * s * 2 < 3LL * num_cus && KT / (s * 2) >= 2) s *= 2;
     return s > KT ? KT : s;
 }
 
@@ -507,6 +542,7 @@ int launch_core(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind
     if ((size_t)S * 16 * n_total * sizeof(float) > sc.attn_partial_bytes && !(want_direct && S == 1)) return -2;
     a.S = S;
     a.direct = (want_direct && S == 1) ? 1 : 0;
+    a.rms_deferred = (pk.norm_w && !a.direct) ? 1 : 0;
     size_t off = 0;
     for (int z = 0; z < nmat; ++z) {
         a.part_off[z] = off;
