@@ -187,7 +187,7 @@ __global__ __launch_bounds__(512) void bs_attend_kernel(BsMulti multi) {
     const BsParams& p = multi.slot[blockIdx.z];
     constexpr int LPT = HD / 8, TPW = 64 / LPT, kWaves = 8;
     constexpr int S = kBsChunk / (kWaves * TPW);
-    __shared__ uint32_t pre[65];
+    __shared__ uint32_t pre[65], sel_s[64];
     __shared__ float red[kWaves][HD];
     __shared__ float wmax[kWaves], wsum[kWaves];
 
@@ -199,11 +199,11 @@ __global__ __launch_bounds__(512) void bs_attend_kernel(BsMulti multi) {
     const uint32_t count = p.counts[qh];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 
-    // pre[r] = first list position of the r-th selected block (exclusive prefix of the block lengths)
+    // pre[r] = first list position of the r-th selected block (exclusive prefix of the block lengths); sel_s[r] = its id
     if (wave == 0) {
-        uint32_t len = 0;
+        uint32_t len = 0, b = 0;
         if ((uint32_t)lane < count) {
-            const uint32_t b = p.sel[qh * 64 + lane];
+            b = p.sel[qh * 64 + lane];
             const uint32_t start = b * p.block_size;
             const uint32_t end = start + p.block_size < p.old_len ? start + p.block_size : p.old_len;
             len = end - start;
@@ -215,6 +215,7 @@ __global__ __launch_bounds__(512) void bs_attend_kernel(BsMulti multi) {
             if (lane >= o) incl += up;
         }
         pre[lane] = incl - len;
+        sel_s[lane] = b;
         if (lane == 63) pre[64] = incl;
     }
     __syncthreads();
@@ -225,40 +226,48 @@ __global__ __launch_bounds__(512) void bs_attend_kernel(BsMulti multi) {
     const size_t row_stride = (size_t)p.kv_heads * HD;
     const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
 
+    // Every list position of the chunk is turned into a token first (no memory access: the block table is in LDS),
+    // then all K / V / q4 / scale loads of the thread go out together with no branch around any of them: positions
+    // past the end repeat the last one, and the load that a token does not need reads a valid dummy address.
     uint4 kw[S], vw[S];
+    uint32_t qw[S];
+    float qs[S];
     bool valid[S], quant[S];
+    uint32_t tok[S], ring[S];
+    const uint32_t ring_mod = p.compressed ? p.recent_window : 0xffffffffu;     // t % 0xffffffff = t: dense cache rows
 #pragma unroll
     for (int s = 0; s < S; ++s) {
-        const uint32_t pos = cbeg + (uint32_t)((s * kWaves + wave) * TPW + tg);
+        uint32_t pos = cbeg + (uint32_t)((s * kWaves + wave) * TPW + tg);
         valid[s] = pos < cend;
-        quant[s] = false;
-        kw[s] = make_uint4(0, 0, 0, 0);
-        vw[s] = make_uint4(0, 0, 0, 0);
-        if (valid[s]) {
-            uint32_t t;
-            if (pos >= old_tokens) {
-                t = p.old_len + (pos - old_tokens);
-            } else {
-                uint32_t lo = 0, hi = count;          // largest r with pre[r] <= pos
-                while (hi - lo > 1u) {
-                    const uint32_t mid = (lo + hi) >> 1;
-                    if (pre[mid] <= pos) lo = mid; else hi = mid;
-                }
-                t = p.sel[qh * 64 + lo] * p.block_size + (pos - pre[lo]);
-            }
-            const uint16_t* kp;
-            if (t < p.old_len) kp = p.old_k + (size_t)t * row_stride;
-            else kp = p.new_k + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
-            kw[s] = *reinterpret_cast<const uint4*>(kp + (size_t)kvh * HD + 8 * c);
-            if (p.compressed && t < p.old_len) {
-                quant[s] = true;
-                vw[s].x = *reinterpret_cast<const uint32_t*>(p.q4_v + ((size_t)t * p.kv_heads + kvh) * (HD / 2) + 4 * c);
-                vw[s].y = __float_as_uint(p.q4_scale[(size_t)t * p.kv_heads + kvh]);
-            } else {
-                const uint16_t* vp = p.dense_v + (size_t)(p.compressed ? t % p.recent_window : t) * row_stride;
-                vw[s] = *reinterpret_cast<const uint4*>(vp + (size_t)kvh * HD + 8 * c);
-            }
+        pos = valid[s] ? pos : cend - 1u;
+        uint32_t lo = 0;                              // largest r < count with pre[r] <= pos (pre[0] = 0)
+#pragma unroll
+        for (uint32_t step = 32; step >= 1u; step >>= 1) {
+            const uint32_t mid = lo + step;
+            const uint32_t pm = pre[mid < 64u ? mid : 63u];
+            const bool take = (mid < count) & (pm <= pos);
+            lo = take ? mid : lo;
         }
+        const uint32_t t_old = sel_s[lo] * p.block_size + (pos - pre[lo]);
+        tok[s] = pos >= old_tokens ? p.old_len + (pos - old_tokens) : t_old;
+        ring[s] = tok[s] % ring_mod;
+    }
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const uint32_t t = tok[s];
+        const bool old = t < p.old_len;
+        const size_t ring_off = (size_t)ring[s] * row_stride;
+        const uint16_t* kp = (old ? p.old_k + (size_t)t * row_stride : p.new_k + ring_off) + (size_t)kvh * HD + 8 * c;
+        quant[s] = p.compressed && old;
+        const uint16_t* vp = quant[s] ? kp : p.dense_v + ring_off + (size_t)kvh * HD + 8 * c;
+        const uint32_t* q4p = quant[s]
+            ? reinterpret_cast<const uint32_t*>(p.q4_v + ((size_t)t * p.kv_heads + kvh) * (HD / 2) + 4 * c)
+            : reinterpret_cast<const uint32_t*>(kp);
+        const float* scp = quant[s] ? p.q4_scale + (size_t)t * p.kv_heads + kvh : reinterpret_cast<const float*>(kp);
+        kw[s] = *reinterpret_cast<const uint4*>(kp);
+        vw[s] = *reinterpret_cast<const uint4*>(vp);
+        qw[s] = *q4p;
+        qs[s] = *scp;
     }
     float q[8];
     {
@@ -296,8 +305,8 @@ __global__ __launch_bounds__(512) void bs_attend_kernel(BsMulti multi) {
         if (c == 0) lsum += e;
         float vf[8];
         if (quant[s]) {
-            const uint32_t packed = vw[s].x;
-            const float scale = __uint_as_float(vw[s].y);
+            const uint32_t packed = qw[s];
+            const float scale = qs[s];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int nib = (int)((packed >> (4 * j)) & 0xfu);
