@@ -289,3 +289,37 @@ def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc):
     assert stop >= 8
     assert np.array_equal(got[:32 + stop], want[:32 + stop]), (got[32:], want[32:], wgap)
     dm.close()
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_identity_model_repeats_the_last_prompt_token(ctx, mode):
+    """tests/e2e_decode_tokens_cpu.rs:13-58 (identity tiny model, tests/common/tiny_gguf.rs:43-45, 173-198, 263-288):
+    one-hot embedding rows, tied lm_head, zero Q/K/V and FFN matrices, identity O projection.  Every layer leaves the
+    hidden state alone, the output norm only rescales it, so greedy decoding repeats the last prompt token ('A' = 65)
+    for as long as it runs; here on every host path, and row-batched with one sequence per token."""
+    hd, heads = 64, 4
+    D = hd * heads          # 256: a multiple of the skinny GEMM's K step, so modes 1 and 2 take the row-batched fused path
+    cfg = dict(n_layers=2, d_model=D, q_heads=heads, kv_heads=heads, head_dim=hd, ffn=256, vocab=D, rms_eps=1e-5,
+               rope_base=10000.0, rope_scale=1.0, rope_layout=0, qkv_bias=False)
+    one = np.float16(1.0).view(np.uint16)
+    eye = np.zeros((D, D), dtype=np.uint16); eye[np.arange(D), np.arange(D)] = one
+    zeros = lambda n, k: np.zeros((n, k), dtype=np.uint16)
+    W = dict(wq=[], wk=[], wv=[], wo=[], wgate=[], wup=[], wdown=[], attn_norm=[], ffn_norm=[])
+    for _ in range(cfg["n_layers"]):
+        W["wq"].append(zeros(D, D)); W["wk"].append(zeros(D, D)); W["wv"].append(zeros(D, D)); W["wo"].append(eye.copy())
+        W["wgate"].append(zeros(256, D)); W["wup"].append(zeros(256, D)); W["wdown"].append(zeros(D, 256))
+        W["attn_norm"].append(np.ones(D, dtype=np.float32)); W["ffn_norm"].append(np.ones(D, dtype=np.float32))
+    W["out_norm"] = np.ones(D, dtype=np.float32)
+    W["lm_head"] = eye.copy(); W["tok_emb"] = W["lm_head"]
+    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=16, max_sequences=4)
+    dm.set_mode(mode)
+    ids, gaps = dm.decode_greedy(0, [1, 65], 4)              # BOS-like id, then 'A'
+    assert list(ids) == [1, 65, 65, 65, 65, 65]
+    assert np.all(gaps > 0.5)                                # the one-hot logit stands clear of the zeros
+    # rows 1..3 hold one prompt token each; three sequences step together and each repeats its own token
+    first = [7, 65, 100]
+    for r, t in enumerate(first):
+        dm.forward_token(1 + r, 0, t, want_hidden=False, want_logits=False)
+    bids, _ = dm.decode_batch_greedy([1, 2, 3], [1, 1, 1], first, 3)
+    assert bids.tolist() == [[7, 7, 7], [65, 65, 65], [100, 100, 100]]
+    dm.close()
