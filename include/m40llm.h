@@ -96,6 +96,14 @@ int m40llm_gemm_f16xf16_f32(M40llmCudaContext* ctx, const void* d_A_f16, const v
 /* A f16 x B f16 row-major -> f16, f32 accumulate (kernels.cu:5068-5103) */
 int m40llm_gemm_f16_storage_f32_compute(M40llmCudaContext* ctx, const void* d_A, const void* d_B,
                                         void* d_C, int M, int N, int K);
+/* GGUF f16 [N][K] -> f32 [K][N], then C[M,N] = A[M,K] x that operand (cuda/kernels.cu:5054-5066, 5197-5265; the
+ * reference multiplies with cublasSgemm, here a plain f32 kernel).  Prefill stream; the non-async forms block. */
+int m40llm_materialize_gguf_f16_to_f32_colmajor_nt(M40llmCudaContext* ctx, const void* d_B_f16,
+                                                   void* d_B_f32_colmajor_nt, int N, int K);
+int m40llm_gemm_f32xf32_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f32_colmajor_nt,
+                            void* d_C_f32, int M, int N, int K);
+int m40llm_gemm_f32xf32_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f32_colmajor_nt,
+                                  void* d_C_f32, int M, int N, int K);
 int m40llm_f16_to_f32(M40llmCudaContext* ctx, const void* d_in_f16, void* d_out_f32, size_t n);   /* :1129-1158 */
 int m40llm_q80_to_f32(M40llmCudaContext* ctx, const void* d_in_q80, void* d_out_f32, size_t n);   /* :1160-1173 */
 
@@ -381,9 +389,6 @@ int m40llm_ext_batched_greedy_step_async(M40llmCudaContext* ctx, const void* d_l
 const char* m40llm_ext_build_info(void);
 
 /* ---- present but unavailable (return -1, as cuda/stub.c does) ---------------------- */
-int m40llm_gemm_f32xf32_f32(M40llmCudaContext*, const void*, const void*, void*, int, int, int);
-int m40llm_gemm_f32xf32_f32_async(M40llmCudaContext*, const void*, const void*, void*, int, int, int);
-int m40llm_materialize_gguf_f16_to_f32_colmajor_nt(M40llmCudaContext*, const void*, void*, int, int);
 int m40llm_kvcache_build_q8_old_from_dense(M40llmCudaContext*, M40llmKVCache*, uint32_t, uint32_t, uint32_t);
 int m40llm_kvcache_build_compressed_from_dense(M40llmCudaContext*, M40llmKVCache*, const M40llmKVCache*, uint32_t);
 int m40llm_kvcache_debug_read_compressed_state(M40llmCudaContext*, M40llmKVCache*, uint32_t, uint32_t*,

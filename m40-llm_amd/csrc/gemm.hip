@@ -205,16 +205,18 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const AT* __restrict_
 // Row-major B[k*N + n]: a thread owns one output column for four rows, k ascending with one
 // accumulator per output (the reference's own order, kernels.cu:4999-5032); lanes read
 // consecutive n, so every B load is one contiguous 128-byte line per wave.
-template <typename AT, typename CT>
+template <typename AT, typename CT, typename BT = uint16_t>
 __global__ __launch_bounds__(256) void gemm_rowmajor_kernel(const AT* __restrict__ A,
-                                                            const uint16_t* __restrict__ B,
+                                                            const BT* __restrict__ B,
                                                             CT* __restrict__ C, int M, int N, int K) {
     const int col = blockIdx.x * 256 + threadIdx.x;
     const int row0 = blockIdx.y * 4;
     if (col >= N) return;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int k = 0; k < K; ++k) {
-        const float b = m40_h2f(B[(size_t)k * N + col]);
+        float b;
+        if constexpr (sizeof(BT) == 2) b = m40_h2f(B[(size_t)k * N + col]);
+        else b = B[(size_t)k * N + col];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = row0 + r < M ? row0 + r : M - 1;
@@ -481,6 +483,16 @@ int launch_q80_gemv(hipStream_t stream, const float* A, const float* up, const u
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
+// GGUF f16 weights [N][K] -> f32 [K][N] (the reference's "column-major NT" operand of its f32 x f32 route,
+// kernels.cu:5054-5066): consecutive threads write consecutive n.
+__global__ __launch_bounds__(256) void materialize_gguf_kernel(const uint16_t* __restrict__ B, float* __restrict__ Bt,
+                                                               int N, int K) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)N * K) return;
+    const size_t n = idx % (size_t)N, k = idx / (size_t)N;
+    Bt[idx] = m40_h2f(B[n * (size_t)K + k]);
+}
+
 int pick_mfma_shape(int ntiles, int KT, int* T, int* S) {
     // Aim for a few thousand waves in flight and >= 512 workgroups where N allows it.
     int s = 1;
@@ -588,6 +600,38 @@ int m40llm_gemm_f32xf16_f32(M40llmCudaContext* ctx, const void* d_A_f32, const v
         M, N, K);
     if (hipGetLastError() != hipSuccess) return -2;
     return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_materialize_gguf_f16_to_f32_colmajor_nt(M40llmCudaContext* ctx, const void* d_B_f16,
+                                                   void* d_B_f32_colmajor_nt, int N, int K) {
+    if (!ctx || !d_B_f16 || !d_B_f32_colmajor_nt) return -1;
+    if (N <= 0 || K <= 0) return -2;
+    (void)hipGetLastError();
+    const size_t total = (size_t)N * K;
+    materialize_gguf_kernel<<<(unsigned)((total + 255) / 256), 256, 0, ctx->prefill_stream>>>(
+        static_cast<const uint16_t*>(d_B_f16), static_cast<float*>(d_B_f32_colmajor_nt), N, K);
+    if (hipGetLastError() != hipSuccess) return -3;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -4;
+}
+
+// The reference routes this through cublasSgemm (kernels.cu:5217-5242); same operands, plain f32 accumulation here.
+int m40llm_gemm_f32xf32_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f32_colmajor_nt,
+                                  void* d_C_f32, int M, int N, int K) {
+    if (!ctx || !d_A_f32 || !d_B_f32_colmajor_nt || !d_C_f32) return -1;
+    if (M <= 0 || N <= 0 || K <= 0) return -2;
+    (void)hipGetLastError();
+    dim3 grid((N + 255) / 256, (M + 3) / 4);
+    gemm_rowmajor_kernel<float, float, float><<<grid, 256, 0, ctx->prefill_stream>>>(
+        static_cast<const float*>(d_A_f32), static_cast<const float*>(d_B_f32_colmajor_nt),
+        static_cast<float*>(d_C_f32), M, N, K);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int m40llm_gemm_f32xf32_f32(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f32_colmajor_nt,
+                            void* d_C_f32, int M, int N, int K) {
+    const int rc = m40llm_gemm_f32xf32_f32_async(ctx, d_A_f32, d_B_f32_colmajor_nt, d_C_f32, M, N, K);
+    if (rc != 0) return rc;
+    return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -4;
 }
 
 int m40llm_gemm_f16xf16_f32(M40llmCudaContext* ctx, const void* d_A_f16, const void* d_B_f16, void* d_C_f32,

@@ -7,9 +7,6 @@
 
 extern "C" {
 
-int m40llm_gemm_f32xf32_f32(M40llmCudaContext*, const void*, const void*, void*, int, int, int) { return M40_UNAVAILABLE; }
-int m40llm_gemm_f32xf32_f32_async(M40llmCudaContext*, const void*, const void*, void*, int, int, int) { return M40_UNAVAILABLE; }
-int m40llm_materialize_gguf_f16_to_f32_colmajor_nt(M40llmCudaContext*, const void*, void*, int, int) { return M40_UNAVAILABLE; }
 int m40llm_kvcache_build_q8_old_from_dense(M40llmCudaContext*, M40llmKVCache*, uint32_t, uint32_t, uint32_t) { return M40_UNAVAILABLE; }
 int m40llm_kvcache_build_compressed_from_dense(M40llmCudaContext*, M40llmKVCache*, const M40llmKVCache*, uint32_t) { return M40_UNAVAILABLE; }
 int m40llm_kvcache_debug_read_compressed_state(M40llmCudaContext*, M40llmKVCache*, uint32_t, uint32_t*, uint32_t*,

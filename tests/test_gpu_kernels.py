@@ -196,6 +196,15 @@ def test_gemm_known_answers(dev, orc):
     dev.call("m40llm_gemm_f16_storage_f32_compute", dA.ptr, dB.ptr, dC16.ptr, 2, 2, 2)
     assert np.array_equal(dC16.download(np.uint16, (2, 2)).view(np.float16).astype(np.float32), [[19, 22], [43, 50]])
     assert dev.lib.m40llm_gemm_f32xf16_gguf_f32(None, Af.ptr, Bg.ptr, dC.ptr, 1, 2, 3) == -1
+    # tests/gemm_mixed.rs:216-272: GGUF f16 weights materialised as f32 [K][N], then the f32 x f32 product
+    a = np.array([[1.0, -2.0, 3.0], [0.5, 4.0, -1.0]], dtype=np.float32)
+    b = np.array([0.25, 0.5, 0.75, -1.0, -1.25, 1.5, 2.0, -0.5, 0.125, 3.0, 2.5, -2.0], dtype=np.float32).reshape(4, 3)   # [N][K]
+    da, db, dbt, dc = dev.up(a), dev.up(f16bits(b)), dev.zeros(3 * 4 * 4), dev.zeros(2 * 4 * 4)
+    dev.call("m40llm_materialize_gguf_f16_to_f32_colmajor_nt", db.ptr, dbt.ptr, 4, 3)
+    assert np.array_equal(dbt.download(np.float32, (3, 4)), b.T)
+    dev.call("m40llm_gemm_f32xf32_f32", da.ptr, dbt.ptr, dc.ptr, 2, 4, 3)
+    assert np.array_equal(dc.download(np.float32, (2, 4)), a @ b.T)      # small dyadic values: exact
+    dev.call("m40llm_gemm_f32xf32_f32", da.ptr, dbt.ptr, dc.ptr, 0, 4, 3, expect=-2)
 
 
 @pytest.mark.parametrize("M,N,K", [
