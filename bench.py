@@ -9,7 +9,8 @@ ids, then greedy decode at batch 1.  Weights and KV cache are resident in HBM be
 
 Prints ONE JSON line: value = decoded tokens per second (whole job); roofline = the dominant kernel's algorithmic
 bytes per launch over its event-timed launch duration against 8 TB/s, plus its measured HBM traffic; cpu_baseline =
-the CPU oracle timed on this host on a short sample of the same workload.
+the CPU oracle timed on this host on a short sample of the same workload.  config.b8 carries the batch-8 half of the
+metric (Qwen2.5-3B-shaped model, 8 rows), measured in the same run.
 """
 import argparse
 import ctypes as C
@@ -106,6 +107,42 @@ def cpu_baseline(cfg, W, steps, threads):
                        f"(gcc -O2, {threads} thread{'s' if threads > 1 else ''})")
 
 
+def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
+    """The batch-8 half of the metric (BASELINE configs[2]): Qwen2.5-3B-shaped random-init model (36 layers, hidden
+    2048, 16 q / 2 kv heads, head_dim 128, FFN 11008, vocab 151936, biases, NeoX RoPE), 8 sequences with contexts
+    ~U[256, 4096] pre-filled with N(0,1) K/V, row-batched greedy decode on the fused graph path.  Four distinct random
+    layers are repeated over the 36 (each layer has its own device copy, so no layer finds its weights in a cache);
+    the embedding table is the lm_head matrix.  Reported beside the batch-1 value, never as it."""
+    cfg = dict(syn.QWEN25_3B)
+    B = 8
+    rng = np.random.default_rng(0)
+    lens = rng.integers(256, 4097, size=B).astype(np.uint32)
+    W = syn.make_weights(cfg, seed=0, unique_layers=4, tie_embeddings=True)
+    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=4096 + warmup + steps + 8, max_sequences=B)
+    dm.set_mode(2)
+    f16 = lambda a: np.ascontiguousarray(a.astype(np.float16).view(np.uint16))
+    dk = ctx.to_device(f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)))
+    dv = ctx.to_device(f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)))
+    for s in range(B):
+        for l in range(cfg["n_layers"]):
+            slot = dm.H.m40host_model_kv_slot(dm.h, s, l)
+            pkg.check(ctx.lib.m40llm_ext_kvcache_bulk_fill_f16(ctx.h, dm.kv_handle(), slot, dk.ptr, dv.ptr, int(lens[s])),
+                      "m40llm_ext_kvcache_bulk_fill_f16")
+    first = rng.integers(0, cfg["vocab"], size=B).astype(np.uint32)
+    ids, ms = dm.decode_batch_timed(np.arange(B), lens, first, warmup, steps)
+    D, F, V, L = cfg["d_model"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
+    KV = cfg["kv_heads"] * cfg["head_dim"]
+    wbytes = L * 2 * (D * (D + 2 * KV) + D * D + 3 * D * F) + 2 * V * D
+    kvbytes = int(lens.sum() + B * (warmup + steps / 2)) * L * KV * 2 * 2
+    dm.close()
+    dk.free(); dv.free()
+    ms_step = ms / steps
+    return {"workload": "Qwen2.5-3B-shaped random-init decode (BASELINE configs[2]), batch 8, contexts U[256,4096], "
+                        "row-batched greedy, fused + graph", "tok_s": B * steps / (ms / 1e3), "ms_per_step": ms_step,
+            "steps": steps, "warmup": warmup, "algorithmic_bytes_per_step": int(wbytes + kvbytes),
+            "whole_step_hbm_frac": (wbytes + kvbytes) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -117,6 +154,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--kernel-reps", type=int, default=10)
+    ap.add_argument("--no-b8", action="store_true", help="skip the batch-8 measurement reported in config.b8")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy through the library (calibrates rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings against a transfer of known size)")
@@ -183,9 +221,14 @@ def main():
                      "avg_launch_us": dom["avg_us"], "launches_timed": dom["launches"],
                      "algorithmic_bytes_per_launch": dom["bytes"]},
     }
+    dm.close()
+    if not args.no_b8 and not args.layers:
+        try:
+            out["config"]["b8"] = measure_b8(pkg, syn, ctx)
+        except Exception as e:     # the batch-1 line must still be printed
+            out["config"]["b8"] = {"error": repr(e)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, W, args.cpu_steps, 1)
-    dm.close()
     print(json.dumps(out))
 
 
