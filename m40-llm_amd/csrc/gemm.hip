@@ -406,7 +406,6 @@ __global__ __launch_bounds__(kQ80GemvThreads) void q80_gemv_kernel(Q80GemvArgs p
         }
     }
 
-    int ncols = 0;
     const int team_cols = team < p.N ? (p.N - team + nteams - 1) / nteams : 0;
     for (int i0 = 0; i0 < team_cols; i0 += kQ80GemvDepth) {
 #pragma unroll
@@ -439,7 +438,6 @@ __global__ __launch_bounds__(kQ80GemvThreads) void q80_gemv_kernel(Q80GemvArgs p
             }
         }
     }
-    (void)ncols;
     if (kw == 1) return;
     __syncthreads();
     // One thread per (team, column, row) adds the K-parts in a fixed order.

@@ -318,6 +318,28 @@ def test_q80_gemm_shapes_vs_oracle(dev, orc, M, N, K):
     close(got / scale, f64 / scale, 1e-4, 1e-5)
 
 
+def test_q80_gemv_random_shapes_vs_float64(dev):
+    """One and two rows over seeded random shapes: K = 64..16384 in steps of 64 (one to eight K parts per column,
+    partly filled parts, lanes without a block), N from 1 up (fewer columns than teams, column tails).  The matrix
+    buffer is exactly N * K/32 * 34 bytes, so a read outside it would land outside the allocation's payload."""
+    rng = np.random.default_rng(2024)
+    shapes = [(1, 1, 64), (2, 1, 128), (1, 17, 16384), (2, 5, 16320), (1, 3, 4160), (2, 2, 2112)]
+    for _ in range(18):
+        shapes.append((int(rng.integers(1, 3)), int(rng.integers(1, 400)), 64 * int(rng.integers(1, 130))))
+    for M, N, K in shapes:
+        d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
+        qs = rng.integers(-127, 128, size=(N, K // 32, 32)).astype(np.int8)
+        W = np.ascontiguousarray(np.stack([_q80_pack(d[i], qs[i]) for i in range(N)]))
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        dA, dW, dC = dev.up(A), dev.up(W), dev.zeros(M * N * 4)
+        dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dA.ptr, dW.ptr, dC.ptr, M, N, K)
+        got = dC.download(np.float32, (M, N))
+        f64 = A.astype(np.float64) @ (d.astype(np.float64)[:, :, None] * qs.astype(np.float64)).reshape(N, K).T
+        scale = np.abs(f64).max(axis=1, keepdims=True)
+        close(got / scale, f64 / scale, 1e-4, 1e-5)
+        dA.free(); dW.free(); dC.free()
+
+
 # ------------------------------------------------------------------ dense attention
 def _attention_case(dev, orc, qh, kvh, hd, L, k, v, q, max_seq=None, seq=0, batch=1):
     max_seq = max_seq or L
