@@ -24,18 +24,86 @@ constexpr int kWavesPerBlock = 4;
 
 // x -> LDS as normalised activations: a[k] = x[k] * scale * w[k], scale = 1/sqrt(sum(x^2)/K + eps).
 // Reduction order identical to rms_norm_kernel (elementwise.hip).
-__device__ __forceinline__ void stage_normed(const float* __restrict__ x, const void* __restrict__ w,
-                                             uint32_t w_dtype, float eps, int K, float* __restrict__ a_lds,
-                                             float* __restrict__ wave_sums) {
+//
+// In two halves so that the caller can request x and the norm weights first, then the GEMV weights, and only then
+// wait: loads return in issue order, so x arrives ahead of the weight stream and the whole prologue (sum of squares,
+// scaling, LDS, two barriers) runs while the weights are still in flight.  A batch is four 16-byte loads per thread
+// and array (K <= 4096 in one batch); longer rows take further batches inside stage_finish.
+constexpr int kStageBatch = 4;
+struct StageRegs {
+    float4 x[kStageBatch];
+    uint4 w[kStageBatch];      // raw bits: four f32 norm weights, or four f16 in .x/.y
+};
+
+__device__ __forceinline__ void stage_load(const float* __restrict__ x, const void* __restrict__ w, uint32_t w_dtype,
+                                           int K, int batch, StageRegs& r) {
+    const int n4 = K >> 2;
+    int idx[kStageBatch];
+#pragma unroll
+    for (int u = 0; u < kStageBatch; ++u) {
+        const int i = (batch * kStageBatch + u) * kThreads + (int)threadIdx.x;
+        idx[u] = i < n4 ? i : 0;                 // past the end: a valid address, ignored later (no load under a branch)
+    }
+#pragma unroll
+    for (int u = 0; u < kStageBatch; ++u) r.x[u] = reinterpret_cast<const float4*>(x)[idx[u]];
+    if (w_dtype == 0u) {
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) {
+            const uint2 h = reinterpret_cast<const uint2*>(w)[idx[u]];
+            r.w[u].x = h.x; r.w[u].y = h.y; r.w[u].z = 0u; r.w[u].w = 0u;
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < kStageBatch; ++u) r.w[u] = reinterpret_cast<const uint4*>(w)[idx[u]];
+    }
+}
+
+__device__ __forceinline__ void stage_sumsq(const StageRegs& r, int K, int batch, float& ss) {
+    const int n4 = K >> 2;
+#pragma unroll
+    for (int u = 0; u < kStageBatch; ++u) {
+        const int i = (batch * kStageBatch + u) * kThreads + (int)threadIdx.x;
+        if (i < n4) {
+            ss = fmaf(r.x[u].x, r.x[u].x, ss);
+            ss = fmaf(r.x[u].y, r.x[u].y, ss);
+            ss = fmaf(r.x[u].z, r.x[u].z, ss);
+            ss = fmaf(r.x[u].w, r.x[u].w, ss);
+        }
+    }
+}
+
+__device__ __forceinline__ void stage_store(const StageRegs& r, uint32_t w_dtype, int K, int batch, float scale,
+                                            float* __restrict__ a_lds) {
+    const int n4 = K >> 2;
+#pragma unroll
+    for (int u = 0; u < kStageBatch; ++u) {
+        const int i = (batch * kStageBatch + u) * kThreads + (int)threadIdx.x;
+        if (i < n4) {
+            float4 wv = make_float4(__uint_as_float(r.w[u].x), __uint_as_float(r.w[u].y), __uint_as_float(r.w[u].z),
+                                    __uint_as_float(r.w[u].w));
+            if (w_dtype == 0u) {
+                const uint32_t h0 = r.w[u].x, h1 = r.w[u].y;
+                wv = make_float4(m40_h2f((uint16_t)(h0 & 0xffffu)), m40_h2f((uint16_t)(h0 >> 16)),
+                                 m40_h2f((uint16_t)(h1 & 0xffffu)), m40_h2f((uint16_t)(h1 >> 16)));
+            }
+            reinterpret_cast<float4*>(a_lds)[i] = make_float4(r.x[u].x * scale * wv.x, r.x[u].y * scale * wv.y,
+                                                              r.x[u].z * scale * wv.z, r.x[u].w * scale * wv.w);
+        }
+    }
+}
+
+// `first` holds batch 0, loaded by the caller before its weight prefetch.
+__device__ __forceinline__ void stage_finish(const StageRegs& first, const float* __restrict__ x,
+                                             const void* __restrict__ w, uint32_t w_dtype, float eps, int K,
+                                             float* __restrict__ a_lds, float* __restrict__ wave_sums) {
     const int tid = threadIdx.x;
+    const int nbatch = ((K >> 2) + kStageBatch * kThreads - 1) / (kStageBatch * kThreads);
     float ss = 0.0f;
-    const float4* x4 = reinterpret_cast<const float4*>(x);
-    for (int i = tid; i < K / 4; i += kThreads) {
-        const float4 v = x4[i];
-        ss = fmaf(v.x, v.x, ss);
-        ss = fmaf(v.y, v.y, ss);
-        ss = fmaf(v.z, v.z, ss);
-        ss = fmaf(v.w, v.w, ss);
+    stage_sumsq(first, K, 0, ss);
+    for (int b = 1; b < nbatch; ++b) {
+        StageRegs r;
+        stage_load(x, w, w_dtype, K, b, r);
+        stage_sumsq(r, K, b, ss);
     }
     ss = m40_sum64(ss);
     if ((tid & 63) == 0) wave_sums[tid >> 6] = ss;
@@ -44,11 +112,11 @@ __device__ __forceinline__ void stage_normed(const float* __restrict__ x, const 
 #pragma unroll
     for (int i = 0; i < kWavesPerBlock; ++i) total += wave_sums[i];
     const float scale = 1.0f / sqrtf(total / static_cast<float>(K) + eps);
-    const uint16_t* w16 = reinterpret_cast<const uint16_t*>(w);
-    const float* w32 = reinterpret_cast<const float*>(w);
-    for (int i = tid; i < K; i += kThreads) {
-        const float wv = w_dtype == 0u ? m40_h2f(w16[i]) : w32[i];
-        a_lds[i] = x[i] * scale * wv;
+    stage_store(first, w_dtype, K, 0, scale, a_lds);
+    for (int b = 1; b < nbatch; ++b) {
+        StageRegs r;
+        stage_load(x, w, w_dtype, K, b, r);
+        stage_store(r, w_dtype, K, b, scale, a_lds);
     }
     __syncthreads();
 }
@@ -98,14 +166,16 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
     const float* bias = which == 0 ? p.bq : (which == 1 ? p.bk : p.bv);
     const uint4* bp[2] = {reinterpret_cast<const uint4*>(W + i0 * (size_t)K),
                           reinterpret_cast<const uint4*>(W + i1 * (size_t)K)};
-    // weights are requested first; the norm prologue runs while they are in flight
+    // x and the norm weights are requested first, then the GEMV weights; the norm prologue runs while those stream in
+    StageRegs xr;
+    stage_load(p.x, p.norm_w, p.norm_dtype, K, 0, xr);
     GemvRegs<2> regs;
     gemv_prefetch<2>(bp, 0, K >> 3, lane, regs);
     // the rotation angle does not depend on the data: evaluated while the weights are in flight
     const uint32_t position = p.position_dev ? *p.position_dev : p.position;
     float2 cs = make_float2(1.0f, 0.0f);
     if (which != 2) cs = m40_rope_cos_sin(position, off, p.head_dim, p.rope_base, p.rope_scale);
-    stage_normed(p.x, p.norm_w, p.norm_dtype, p.eps, K, a_lds, wave_sums);
+    stage_finish(xr, p.x, p.norm_w, p.norm_dtype, p.eps, K, a_lds, wave_sums);
     float d[2];
     gemv_accumulate<2>(bp, a_lds, 0, K >> 3, lane, regs, d);
     gemv_finish<2, 1>(d, nullptr, wave, lane);
@@ -166,9 +236,11 @@ __global__ __launch_bounds__(kThreads) void norm_gate_up_swiglu_kernel(const flo
     if (!live) j = F - 1;
     const uint4* bp[2] = {reinterpret_cast<const uint4*>(Wg + (size_t)j * K),
                           reinterpret_cast<const uint4*>(Wu + (size_t)j * K)};
+    StageRegs xr;
+    stage_load(x, norm_w, norm_dtype, K, 0, xr);
     GemvRegs<2> regs;
     gemv_prefetch<2>(bp, 0, K >> 3, lane, regs);
-    stage_normed(x, norm_w, norm_dtype, eps, K, a_lds, wave_sums);
+    stage_finish(xr, x, norm_w, norm_dtype, eps, K, a_lds, wave_sums);
     float d[2];
     gemv_accumulate<2>(bp, a_lds, 0, K >> 3, lane, regs, d);
     gemv_finish<2, 1>(d, nullptr, wave, lane);
@@ -200,9 +272,11 @@ __global__ __launch_bounds__(kThreads) void norm_gemv_kernel(const float* __rest
         const int col = (live && col0 + c < N) ? col0 + c : N - 1;
         bp[c] = reinterpret_cast<const uint4*>(W + (size_t)col * K);
     }
+    StageRegs xr;
+    stage_load(x, norm_w, norm_dtype, K, 0, xr);
     GemvRegs<COLS> regs;
     gemv_prefetch<COLS>(bp, 0, K >> 3, lane, regs);
-    stage_normed(x, norm_w, norm_dtype, eps, K, a_lds, wave_sums);
+    stage_finish(xr, x, norm_w, norm_dtype, eps, K, a_lds, wave_sums);
     float d[COLS];
     gemv_accumulate<COLS>(bp, a_lds, 0, K >> 3, lane, regs, d);
     gemv_finish<COLS, 1>(d, nullptr, wave, lane);
@@ -318,7 +392,7 @@ int m40llm_ext_fused_norm_qkv_rope_append_async(
     if (d_model == 0) return -3;
     const uint32_t D = d_model;
     if (!fast_ok(d_x_f32, d_wq_f16, (int)D) || !m40_aligned16(d_wk_f16) || !m40_aligned16(d_wv_f16) ||
-        (size_t)D * 4 > 60 * 1024)
+        !m40_aligned16(d_norm_w) || (size_t)D * 4 > 60 * 1024)
         return -6;
     QkvArgs p{};
     p.x = static_cast<const float*>(d_x_f32);
@@ -370,7 +444,9 @@ int m40llm_ext_fused_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const voi
     if (!ctx || !d_x_f32 || !d_norm_w || !d_wgate_f16 || !d_wup_f16 || !d_hid_f32) return -1;
     if (ffn <= 0 || d_model <= 0) return -2;
     if (norm_weight_dtype > 1) return -4;
-    if (!fast_ok(d_x_f32, d_wgate_f16, d_model) || !m40_aligned16(d_wup_f16) || (size_t)d_model * 4 > 60 * 1024) return -6;
+    if (!fast_ok(d_x_f32, d_wgate_f16, d_model) || !m40_aligned16(d_wup_f16) || !m40_aligned16(d_norm_w) ||
+        (size_t)d_model * 4 > 60 * 1024)
+        return -6;
     (void)hipGetLastError();
     norm_gate_up_swiglu_kernel<<<(ffn + 3) / 4, kThreads, (size_t)d_model * 4, ctx->decode_stream>>>(
         static_cast<const float*>(d_x_f32), d_norm_w, norm_weight_dtype, eps, static_cast<const uint16_t*>(d_wgate_f16),
@@ -385,7 +461,7 @@ int m40llm_ext_fused_norm_gemv_f32xf16_async(M40llmCudaContext* ctx, const void*
     if (!ctx || !d_x_f32 || !d_norm_w || !d_w_f16 || !d_out_f32) return -1;
     if (N <= 0 || K <= 0) return -2;
     if (norm_weight_dtype > 1) return -4;
-    if (!fast_ok(d_x_f32, d_w_f16, K) || (size_t)K * 4 > 60 * 1024) return -6;
+    if (!fast_ok(d_x_f32, d_w_f16, K) || !m40_aligned16(d_norm_w) || (size_t)K * 4 > 60 * 1024) return -6;
     (void)hipGetLastError();
     const float* x = static_cast<const float*>(d_x_f32);
     const uint16_t* W = static_cast<const uint16_t*>(d_w_f16);
