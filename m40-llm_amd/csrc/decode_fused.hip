@@ -209,15 +209,24 @@ __global__ __launch_bounds__(kThreads) void gemv_residual_kernel(const float* __
     for (int c = 0; c < COLS; ++c) bp[c] = reinterpret_cast<const uint4*>(W + (size_t)(col0 + c < N ? col0 + c : N - 1) * K);
     int c_begin, c_end;
     gemv_range<KSPLIT>(K, wave, &c_begin, &c_end);
+    // activations and residual first (cache hits), then the weight stream: nothing is requested after the weights
+    // (measured: with K split over the waves the early activation loads cost more than they save)
+    constexpr bool ACTS = KSPLIT == 1;
+    GemvActRegs acts;
+    if (ACTS) gemv_prefetch_acts(a, c_begin, c_end, lane, acts);
+    float res[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) res[c] = residual ? residual[col0 + c < N ? col0 + c : N - 1] : 0.0f;
     GemvRegs<COLS> regs;
     gemv_prefetch<COLS>(bp, c_begin, c_end, lane, regs);
     float d[COLS];
-    gemv_accumulate<COLS>(bp, a, c_begin, c_end, lane, regs, d);
+    if (ACTS) gemv_accumulate<COLS>(bp, a, c_begin, c_end, lane, regs, acts, d);
+    else gemv_accumulate<COLS>(bp, a, c_begin, c_end, lane, regs, d);
     gemv_finish<COLS, KSPLIT>(d, red, wave, lane);
     if (lane == 0 && (KSPLIT == 1 || wave == 0)) {
 #pragma unroll
         for (int c = 0; c < COLS; ++c)
-            if (col0 + c < N) out[col0 + c] = residual ? residual[col0 + c] + d[c] : d[c];
+            if (col0 + c < N) out[col0 + c] = residual ? res[c] + d[c] : d[c];
     }
 }
 

@@ -37,10 +37,14 @@ __global__ __launch_bounds__(256) void gemv_f32xf16_gguf_kernel(const float* __r
     }
     int c_begin, c_end;
     gemv_range<KSPLIT>(K, wave, &c_begin, &c_end);
+    constexpr bool ACTS = KSPLIT == 1;     // measured: with K split over the waves the early loads do not pay
+    GemvActRegs acts;
+    if (ACTS) gemv_prefetch_acts(A, c_begin, c_end, lane, acts);      // before the weights: they return first
     GemvRegs<COLS> regs;
     gemv_prefetch<COLS>(bp, c_begin, c_end, lane, regs);
     float acc[COLS];
-    gemv_accumulate<COLS>(bp, A, c_begin, c_end, lane, regs, acc);
+    if (ACTS) gemv_accumulate<COLS>(bp, A, c_begin, c_end, lane, regs, acts, acc);
+    else gemv_accumulate<COLS>(bp, A, c_begin, c_end, lane, regs, acc);
     gemv_finish<COLS, KSPLIT>(acc, red, wave, lane);
     if (lane == 0 && (KSPLIT == 1 || wave == 0)) {
 #pragma unroll

@@ -52,21 +52,40 @@ __device__ __forceinline__ void gemv_range(int K, int wave, int* c_begin, int* c
     }
 }
 
-// Issue the first kGemvPrefetch loads of every column (before any prologue that the caller runs).
+// Issue the first kGemvPrefetch loads of every column (before any prologue that the caller runs).  Chunks past the
+// end of the range re-read the range's first chunk and are ignored later, so no load sits under a per-lane branch
+// (waits count in issue order; a load that only some paths issue makes every later wait conservative).
 template <int COLS>
 __device__ __forceinline__ void gemv_prefetch(const uint4* const (&bp)[COLS], int c_begin, int c_end, int lane,
                                               GemvRegs<COLS>& r) {
 #pragma unroll
     for (int i = 0; i < kGemvPrefetch; ++i) {
-        const int kc = c_begin + lane + 64 * i;
+        if (c_begin + 64 * i >= c_end) break;           // the whole wave is past the end (uniform): nothing to request
+        int kc = c_begin + lane + 64 * i;
+        kc = kc < c_end ? kc : c_begin;
 #pragma unroll
-        for (int c = 0; c < COLS; ++c) r.w[i][c] = kc < c_end ? m40_load_stream(bp[c] + kc) : make_uint4(0, 0, 0, 0);
+        for (int c = 0; c < COLS; ++c) r.w[i][c] = m40_load_stream(bp[c] + kc);
     }
 }
 
-__device__ __forceinline__ void gemv_fma8(const uint4& w, const float* __restrict__ a, int kc, float& acc) {
-    const float4 a0 = *reinterpret_cast<const float4*>(a + 8 * kc);
-    const float4 a1 = *reinterpret_cast<const float4*>(a + 8 * kc + 4);
+// Activations of the prefetched chunks, read from global memory.  Callers issue this before gemv_prefetch: loads
+// return in issue order, so the activations (cache hits) are there when the first weights arrive.
+struct GemvActRegs {
+    float4 lo[kGemvPrefetch], hi[kGemvPrefetch];
+};
+__device__ __forceinline__ void gemv_prefetch_acts(const float* __restrict__ a, int c_begin, int c_end, int lane,
+                                                   GemvActRegs& r) {
+#pragma unroll
+    for (int i = 0; i < kGemvPrefetch; ++i) {
+        if (c_begin + 64 * i >= c_end) break;
+        int kc = c_begin + lane + 64 * i;
+        kc = kc < c_end ? kc : c_begin;
+        r.lo[i] = *reinterpret_cast<const float4*>(a + 8 * kc);
+        r.hi[i] = *reinterpret_cast<const float4*>(a + 8 * kc + 4);
+    }
+}
+
+__device__ __forceinline__ void gemv_fma8(const uint4& w, const float4& a0, const float4& a1, float& acc) {
     float f[8];
     m40_unpack8(w, f);
     acc = fmaf(a0.x, f[0], acc);
@@ -77,6 +96,23 @@ __device__ __forceinline__ void gemv_fma8(const uint4& w, const float* __restric
     acc = fmaf(a1.y, f[5], acc);
     acc = fmaf(a1.z, f[6], acc);
     acc = fmaf(a1.w, f[7], acc);
+}
+__device__ __forceinline__ void gemv_fma8(const uint4& w, const float* __restrict__ a, int kc, float& acc) {
+    gemv_fma8(w, *reinterpret_cast<const float4*>(a + 8 * kc), *reinterpret_cast<const float4*>(a + 8 * kc + 4), acc);
+}
+
+// Rest of the range beyond the prefetched chunks.
+template <int COLS>
+__device__ __forceinline__ void gemv_accumulate_tail(const uint4* const (&bp)[COLS], const float* __restrict__ a,
+                                                     int c_begin, int c_end, int lane, float (&acc)[COLS]) {
+#pragma unroll 2
+    for (int kc = c_begin + lane + 64 * kGemvPrefetch; kc < c_end; kc += 64) {
+        uint4 w[COLS];
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) w[c] = m40_load_stream(bp[c] + kc);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) gemv_fma8(w[c], a, kc, acc[c]);
+    }
 }
 
 // Consume the prefetched chunks, then the rest of the range.  `a` may point to global memory or LDS.
@@ -94,14 +130,25 @@ __device__ __forceinline__ void gemv_accumulate(const uint4* const (&bp)[COLS], 
             for (int c = 0; c < COLS; ++c) gemv_fma8(r.w[i][c], a, kc, acc[c]);
         }
     }
-#pragma unroll 2
-    for (int kc = c_begin + lane + 64 * kGemvPrefetch; kc < c_end; kc += 64) {
-        uint4 w[COLS];
+    gemv_accumulate_tail<COLS>(bp, a, c_begin, c_end, lane, acc);
+}
+
+// The same with the activations of the prefetched chunks already in registers (same arithmetic, same order).
+template <int COLS>
+__device__ __forceinline__ void gemv_accumulate(const uint4* const (&bp)[COLS], const float* __restrict__ a,
+                                                int c_begin, int c_end, int lane, const GemvRegs<COLS>& r,
+                                                const GemvActRegs& ar, float (&acc)[COLS]) {
 #pragma unroll
-        for (int c = 0; c < COLS; ++c) w[c] = m40_load_stream(bp[c] + kc);
+    for (int c = 0; c < COLS; ++c) acc[c] = 0.0f;
 #pragma unroll
-        for (int c = 0; c < COLS; ++c) gemv_fma8(w[c], a, kc, acc[c]);
+    for (int i = 0; i < kGemvPrefetch; ++i) {
+        const int kc = c_begin + lane + 64 * i;
+        if (kc < c_end) {
+#pragma unroll
+            for (int c = 0; c < COLS; ++c) gemv_fma8(r.w[i][c], ar.lo[i], ar.hi[i], acc[c]);
+        }
     }
+    gemv_accumulate_tail<COLS>(bp, a, c_begin, c_end, lane, acc);
 }
 
 // Lane butterfly, then (KSPLIT == 4) the four wave partials in wave order.  `red` is LDS of at
