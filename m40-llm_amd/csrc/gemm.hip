@@ -515,7 +515,7 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
     const bool fast = (K % 8 == 0) && m40_aligned16(A) && m40_aligned16(B);
     if (fast && M == 1) {
         const GemvShape g = gemv_pick_shape(N, K);
-        if (g.ksplit == 4) gemv_f32xf16_gguf_kernel<1, 4><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
+        if (g.ksplit == 4) gemv_f32xf16_gguf_kernel<2, 4><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else if (g.cols == 4) gemv_f32xf16_gguf_kernel<4, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else if (g.cols == 2) gemv_f32xf16_gguf_kernel<2, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else gemv_f32xf16_gguf_kernel<1, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);

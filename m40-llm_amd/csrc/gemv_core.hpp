@@ -25,8 +25,8 @@ static inline GemvShape gemv_pick_shape(int N, int K) {
     GemvShape s;
     s.ksplit = (N < 4096 && K >= 4096) ? 4 : 1;
     if (s.ksplit == 4) {
-        s.cols = 1;
-        s.blocks = N;
+        s.cols = 2;        // measured on the whole token: two columns per workgroup beat one and four
+        s.blocks = (N + s.cols - 1) / s.cols;
     } else {
         s.cols = N >= 16384 ? 4 : (N >= 6144 ? 2 : 1);
         s.blocks = (N + 4 * s.cols - 1) / (4 * s.cols);
