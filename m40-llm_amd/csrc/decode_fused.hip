@@ -100,10 +100,12 @@ __device__ __forceinline__ void stage_finish(const StageRegs& first, const float
     const int nbatch = ((K >> 2) + kStageBatch * kThreads - 1) / (kStageBatch * kThreads);
     float ss = 0.0f;
     stage_sumsq(first, K, 0, ss);
-    for (int b = 1; b < nbatch; ++b) {
-        StageRegs r;
-        stage_load(x, w, w_dtype, K, b, r);
-        stage_sumsq(r, K, b, ss);
+    if (nbatch > 1) {       // rows longer than one batch: kept apart so that the usual case has no loop with loads in it
+        for (int b = 1; b < nbatch; ++b) {
+            StageRegs r;
+            stage_load(x, w, w_dtype, K, b, r);
+            stage_sumsq(r, K, b, ss);
+        }
     }
     ss = m40_sum64(ss);
     if ((tid & 63) == 0) wave_sums[tid >> 6] = ss;
@@ -113,10 +115,12 @@ __device__ __forceinline__ void stage_finish(const StageRegs& first, const float
     for (int i = 0; i < kWavesPerBlock; ++i) total += wave_sums[i];
     const float scale = 1.0f / sqrtf(total / static_cast<float>(K) + eps);
     stage_store(first, w_dtype, K, 0, scale, a_lds);
-    for (int b = 1; b < nbatch; ++b) {
-        StageRegs r;
-        stage_load(x, w, w_dtype, K, b, r);
-        stage_store(r, w_dtype, K, b, scale, a_lds);
+    if (nbatch > 1) {
+        for (int b = 1; b < nbatch; ++b) {
+            StageRegs r;
+            stage_load(x, w, w_dtype, K, b, r);
+            stage_store(r, w_dtype, K, b, scale, a_lds);
+        }
     }
     __syncthreads();
 }
@@ -234,7 +238,7 @@ __global__ __launch_bounds__(kThreads) void gemv_residual_kernel(const float* __
 #pragma unroll
     for (int c = 0; c < COLS; ++c) res[c] = residual ? residual[col0 + c < N ? col0 + c : N - 1] : 0.0f;
     GemvRegs<COLS> regs;
-    gemv_prefetch<COLS>(bp, c_begin, c_end, lane, regs);
+    gemv_prefetch<COLS, KSPLIT != 1>(bp, c_begin, c_end, lane, regs);
     float d[COLS];
     if (ACTS) gemv_accumulate<COLS>(bp, a, c_begin, c_end, lane, regs, acts, d);
     else gemv_accumulate<COLS>(bp, a, c_begin, c_end, lane, regs, d);

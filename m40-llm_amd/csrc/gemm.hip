@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void gemv_f32xf16_gguf_kernel(const float* __r
     GemvActRegs acts;
     if (ACTS) gemv_prefetch_acts(A, c_begin, c_end, lane, acts);      // before the weights: they return first
     GemvRegs<COLS> regs;
-    gemv_prefetch<COLS>(bp, c_begin, c_end, lane, regs);
+    gemv_prefetch<COLS, KSPLIT != 1>(bp, c_begin, c_end, lane, regs);
     float acc[COLS];
     if (ACTS) gemv_accumulate<COLS>(bp, A, c_begin, c_end, lane, regs, acts, acc);
     else gemv_accumulate<COLS>(bp, A, c_begin, c_end, lane, regs, acc);

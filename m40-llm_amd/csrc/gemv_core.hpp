@@ -55,12 +55,14 @@ __device__ __forceinline__ void gemv_range(int K, int wave, int* c_begin, int* c
 // Issue the first kGemvPrefetch loads of every column (before any prologue that the caller runs).  Chunks past the
 // end of the range re-read the range's first chunk and are ignored later, so no load sits under a per-lane branch
 // (waits count in issue order; a load that only some paths issue makes every later wait conservative).
-template <int COLS>
+// SKIP_EMPTY: a slot that lies past the end for the whole wave is not requested at all (a uniform branch; used where
+// K is split over the waves and every load is awaited at once anyway).
+template <int COLS, bool SKIP_EMPTY = false>
 __device__ __forceinline__ void gemv_prefetch(const uint4* const (&bp)[COLS], int c_begin, int c_end, int lane,
                                               GemvRegs<COLS>& r) {
 #pragma unroll
     for (int i = 0; i < kGemvPrefetch; ++i) {
-        if (c_begin + 64 * i >= c_end) break;           // the whole wave is past the end (uniform): nothing to request
+        if (SKIP_EMPTY && c_begin + 64 * i >= c_end) break;
         int kc = c_begin + lane + 64 * i;
         kc = kc < c_end ? kc : c_begin;
 #pragma unroll
@@ -77,7 +79,6 @@ __device__ __forceinline__ void gemv_prefetch_acts(const float* __restrict__ a, 
                                                    GemvActRegs& r) {
 #pragma unroll
     for (int i = 0; i < kGemvPrefetch; ++i) {
-        if (c_begin + 64 * i >= c_end) break;
         int kc = c_begin + lane + 64 * i;
         kc = kc < c_end ? kc : c_begin;
         r.lo[i] = *reinterpret_cast<const float4*>(a + 8 * kc);
