@@ -339,16 +339,19 @@ __global__ __launch_bounds__(kThreads, 2) void skinny_mfma_kernel(SkinnyArgs p) 
     }
 }
 
-// sum over the K slices (ascending) of one output element
-__device__ __forceinline__ float skinny_sum(const SkinnyArgs& p, int z, int row, int n) {
+// The K slices of one output element.  Loading and adding are separate so that a kernel can request everything it
+// needs before it waits for anything; slices beyond S re-read slice 0 and are left out of the sum (no load sits under
+// a branch).  The sum runs over the slices in ascending order.
+__device__ __forceinline__ void skinny_load(const SkinnyArgs& p, int z, int row, int n, float (&part)[16]) {
     const float* src = p.partial + p.part_off[z] + (size_t)row * p.N[z] + n;
     const size_t slice_stride = (size_t)16 * p.N[z];
-    float part[16];
 #pragma unroll
-    for (int s = 0; s < 16; ++s) part[s] = s < p.S ? src[(size_t)s * slice_stride] : 0.0f;
+    for (int s = 0; s < 16; ++s) part[s] = src[(size_t)(s < p.S ? s : 0) * slice_stride];
+}
+__device__ __forceinline__ float skinny_add(const SkinnyArgs& p, const float (&part)[16]) {
     float v = 0.0f;
 #pragma unroll
-    for (int s = 0; s < 16; ++s) v += part[s];
+    for (int s = 0; s < 16; ++s) v += s < p.S ? part[s] : 0.0f;
     return v;
 }
 
@@ -362,6 +365,7 @@ struct EpilogueArgs {
     const float* residual;
     int mode;
 };
+
 // rsqrt(mean(A[row]^2) + eps) by a 256-thread workgroup, the same value in every thread; fixed summation order.
 __device__ __forceinline__ float skinny_row_rms(const SkinnyArgs& g, int row) {
     __shared__ float red_s[4];
@@ -372,7 +376,8 @@ __device__ __forceinline__ float skinny_row_rms(const SkinnyArgs& g, int row) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int k = k0 + u * 1024 + 4 * (int)threadIdx.x;
-            v[u] = k < g.K ? *reinterpret_cast<const float4*>(a + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+            v[u] = *reinterpret_cast<const float4*>(a + (k < g.K ? k : 0));
+            if (k >= g.K) v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -390,17 +395,26 @@ __device__ __forceinline__ float skinny_row_rms(const SkinnyArgs& g, int row) {
 __global__ __launch_bounds__(256) void skinny_epilogue_kernel(EpilogueArgs e) {
     const int z = blockIdx.z, row = blockIdx.y;
     const int n = blockIdx.x * 256 + threadIdx.x;
+    const int N = e.g.N[z];
+    const int nc = n < N ? n : N - 1;
+    // every load of the thread goes out before the first wait: slices of one matrix (mode 0) or of gate and up
+    // (mode 1; mode 0 reads its own slices twice rather than branch), bias and residual (or a stand-in address)
+    float pa[16], pb[16];
+    skinny_load(e.g, e.mode == 1 ? 0 : z, row, nc, pa);
+    skinny_load(e.g, e.mode == 1 ? 1 : z, row, nc, pb);
+    const float bias = *(e.bias ? e.bias + nc : e.g.partial);
+    const float res = *(e.residual ? e.residual + (size_t)row * N + nc : e.g.partial);
     const float rms = (e.g.norm_w && e.g.rms_deferred) ? skinny_row_rms(e.g, row) : 1.0f;
-    if (n >= e.g.N[z]) return;
+    if (n >= N) return;
     if (e.mode == 1) {
-        const float gate = rms * skinny_sum(e.g, 0, row, n), up = rms * skinny_sum(e.g, 1, row, n);
-        e.out[0][(size_t)row * e.g.N[0] + n] = gate / (1.0f + expf(-gate)) * up;
+        const float gate = rms * skinny_add(e.g, pa), up = rms * skinny_add(e.g, pb);
+        e.out[0][(size_t)row * N + n] = gate / (1.0f + expf(-gate)) * up;
         return;
     }
-    float v = rms * skinny_sum(e.g, z, row, n);
-    if (e.bias) v = v + e.bias[n];
-    if (e.residual) v = e.residual[(size_t)row * e.g.N[z] + n] + v;
-    e.out[z][(size_t)row * e.g.N[z] + n] = v;
+    float v = rms * skinny_add(e.g, pa);
+    if (e.bias) v = v + bias;
+    if (e.residual) v = res + v;
+    e.out[z][(size_t)row * N + n] = v;
 }
 
 // Q/K/V epilogue of a batched decode step: bias, RoPE at each row's position, q to its buffer, K and V (f16) into
@@ -419,9 +433,9 @@ __global__ __launch_bounds__(256) void skinny_qkv_epilogue_kernel(QkvEpilogueArg
     const uint32_t row = blockIdx.y;
     const uint32_t half = e.head_dim / 2u;
     const uint32_t q_pairs = e.q_heads * half, kv_pairs = e.kv_heads * half;
-    const uint32_t pair = blockIdx.x * 256u + threadIdx.x;
-    const float rms = (e.g.norm_w && e.g.rms_deferred) ? skinny_row_rms(e.g, (int)row) : 1.0f;
-    if (pair >= q_pairs + 2u * kv_pairs) return;
+    const uint32_t total = q_pairs + 2u * kv_pairs;
+    const uint32_t pair_raw = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t pair = pair_raw < total ? pair_raw : total - 1u;
     int which;
     uint32_t local;
     if (pair < q_pairs) { which = 0; local = pair; }
@@ -431,10 +445,17 @@ __global__ __launch_bounds__(256) void skinny_qkv_epilogue_kernel(QkvEpilogueArg
     size_t i0, i1;
     m40_rope_pair(head, off, e.head_dim, which == 2 ? M40LLM_ROPE_LAYOUT_ADJACENT : e.rope_layout, &i0, &i1);
     const float* bias = which == 0 ? e.bq : (which == 1 ? e.bk : e.bv);
-    float y0 = rms * skinny_sum(e.g, which, (int)row, (int)i0), y1 = rms * skinny_sum(e.g, which, (int)row, (int)i1);
-    if (bias) { y0 = y0 + bias[i0]; y1 = y1 + bias[i1]; }
+    // all loads first: slices of both elements, biases (or a stand-in address), the row's position and sequence id
+    float p0[16], p1[16];
+    skinny_load(e.g, which, (int)row, (int)i0, p0);
+    skinny_load(e.g, which, (int)row, (int)i1, p1);
+    const float b0 = *(bias ? bias + i0 : e.g.partial), b1 = *(bias ? bias + i1 : e.g.partial);
     const uint32_t position = e.lens_dev[row];
     const uint32_t seq = e.ids_dev[row];
+    const float rms = (e.g.norm_w && e.g.rms_deferred) ? skinny_row_rms(e.g, (int)row) : 1.0f;
+    if (pair_raw >= total) return;
+    float y0 = rms * skinny_add(e.g, p0), y1 = rms * skinny_add(e.g, p1);
+    if (bias) { y0 = y0 + b0; y1 = y1 + b1; }
     if (position >= e.max_seq_len || seq >= e.max_batch) return;
     if (which != 2) m40_rope_rotate(position, off, e.head_dim, e.rope_base, e.rope_scale, y0, y1, &y0, &y1);
     if (which == 0) {
