@@ -492,8 +492,31 @@ __global__ __launch_bounds__(1024) void greedy_batch_kernel(GreedyBatchArgs a) {
         if (oa > va || (oa == va && oi < ia)) { vb = fmaxf(va, ob); va = oa; ia = oi; }
         else vb = fmaxf(vb, oa);
     };
+    if ((a.n & 3u) == 0u && (reinterpret_cast<uintptr_t>(lg) & 15u) == 0u) {
+        // eight 16-byte loads per thread and batch, all requested before the first comparison; indices ascend within a
+        // thread, and ties between threads are settled by index in offer()
+        const float4* lg4 = reinterpret_cast<const float4*>(lg);
+        const uint32_t n4 = a.n >> 2;
+        for (uint32_t base = 0; base < n4; base += 8u * 1024u) {
+            float4 v[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8u; ++u) {
+                const uint32_t i = base + u * 1024u + threadIdx.x;
+                v[u] = lg4[i < n4 ? i : n4 - 1u];
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 8u; ++u) {
+                const uint32_t i = base + u * 1024u + threadIdx.x;
+                if (i < n4) {
+                    offer(v[u].x, -INFINITY, 4u * i); offer(v[u].y, -INFINITY, 4u * i + 1u);
+                    offer(v[u].z, -INFINITY, 4u * i + 2u); offer(v[u].w, -INFINITY, 4u * i + 3u);
+                }
+            }
+        }
+    } else {
 #pragma unroll 4
-    for (uint32_t i = threadIdx.x; i < a.n; i += 1024u) offer(lg[i], -INFINITY, i);
+        for (uint32_t i = threadIdx.x; i < a.n; i += 1024u) offer(lg[i], -INFINITY, i);
+    }
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
         const float oa = __shfl_xor(va, o, 64), ob = __shfl_xor(vb, o, 64);
