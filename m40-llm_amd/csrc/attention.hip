@@ -283,10 +283,10 @@ int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, 
         // long rows: matrix-core kernel (it reads q with 16-byte loads).  Chunks are a multiple of 128 tokens (one
         // 32-token tile per wave and pass) sized for about one workgroup per CU -- measured best at 32 K tokens (256
         // workgroups of 1024 tokens: 32 us against 36 us with twice as many half-sized ones) and on the batch-8 step
-        // -- rounded down unless that would put more than two workgroups on a CU.
+        // -- rounded to the nearest multiple, and up while more than two workgroups would land on a CU.
         p.subgroups = (group + 7) / 8;
         const uint64_t groups = (uint64_t)batch * p.kv_heads * p.subgroups;
-        uint64_t chunk = ((uint64_t)span * groups / ctx->num_cus) / 128 * 128;
+        uint64_t chunk = (((uint64_t)span * groups / ctx->num_cus) + 64) / 128 * 128;
         if (chunk < 128) chunk = 128;
         while (groups * ((span + chunk - 1) / chunk) > 2ull * ctx->num_cus) chunk += 128;
         if (chunk > 2048) chunk = 2048;
