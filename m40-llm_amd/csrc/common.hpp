@@ -95,6 +95,15 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
                                  const float* A, const uint16_t* B, float* C, int M, int N, int K);
 // skinny MFMA GEMM (skinny_mfma.hip): fmt 0 = f16 GGUF weights, 1 = q8_0 blocks.  `up` != null multiplies
 // silu(A) by it while packing; W1/C1 give an optional second matrix of the same shape.
+// Row-batched vector-ALU GEMV (rows_gemv.hip): up to eight rows, K <= 2048, epilogue in the same kernel.
+bool m40_rows_gemv_supported(int rows, int K);
+int m40_rows_gemv_residual(hipStream_t stream, const float* a, const uint16_t* W, const float* residual, float* out,
+                           int rows, int N, int K);
+int m40_rows_norm_qkv(hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
+                      uint32_t rows, const float* x, const void* norm_w, uint32_t norm_dtype, float eps,
+                      const uint16_t* wq, const uint16_t* wk, const uint16_t* wv, const float* bq, const float* bk,
+                      const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
+                      uint32_t rope_layout, float* q_out);
 bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
 int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);

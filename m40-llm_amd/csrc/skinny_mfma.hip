@@ -672,6 +672,14 @@ int m40llm_ext_batched_norm_qkv_rope_append_async(
     if (!rows_ok(ctx, (int)rows, (int)d_model)) return -6;
     if (!m40_aligned16(d_wq_f16) || !m40_aligned16(d_wk_f16) || !m40_aligned16(d_wv_f16)) return -6;
     (void)hipGetLastError();
+    // up to eight rows and K <= 2048: vector-ALU kernel with the whole epilogue inside (one launch instead of two)
+    if (m40_rows_gemv_supported((int)rows, (int)d_model) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
+        return m40_rows_norm_qkv(ctx->decode_stream, kv, seq_ids_dev, seq_lens_dev, rows, static_cast<const float*>(d_x_f32),
+                                 d_norm_w, norm_weight_dtype, eps, static_cast<const uint16_t*>(d_wq_f16),
+                                 static_cast<const uint16_t*>(d_wk_f16), static_cast<const uint16_t*>(d_wv_f16),
+                                 static_cast<const float*>(d_bq_f32), static_cast<const float*>(d_bk_f32),
+                                 static_cast<const float*>(d_bv_f32), d_model, q_heads, freq_base, freq_scale, rope_layout,
+                                 static_cast<float*>(d_q_out_f32));
     const int QN = (int)(q_heads * kv->head_dim), KN = (int)(kv->num_heads * kv->head_dim);
     PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
     const void* W[3] = {d_wq_f16, d_wk_f16, d_wv_f16};
@@ -699,6 +707,10 @@ int m40llm_ext_batched_gemm_residual_f32xf16_async(M40llmCudaContext* ctx, const
     if (N <= 0 || K <= 0) return -2;
     if (!rows_ok(ctx, (int)rows, K) || !m40_aligned16(d_w_f16)) return -6;
     (void)hipGetLastError();
+    if (m40_rows_gemv_supported((int)rows, K) && m40_aligned16(d_a_f32))
+        return m40_rows_gemv_residual(ctx->decode_stream, static_cast<const float*>(d_a_f32),
+                                      static_cast<const uint16_t*>(d_w_f16), static_cast<const float*>(d_residual_f32),
+                                      static_cast<float*>(d_out_f32), (int)rows, N, K);
     PackSpec pk{static_cast<const float*>(d_a_f32), nullptr, nullptr, 0, 0.0f};
     const void* W[1] = {d_w_f16};
     const int Ns[1] = {N};
