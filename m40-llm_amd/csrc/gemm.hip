@@ -519,6 +519,9 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
         else if (g.cols == 4) gemv_f32xf16_gguf_kernel<4, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else if (g.cols == 2) gemv_f32xf16_gguf_kernel<2, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else gemv_f32xf16_gguf_kernel<1, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
+    } else if (fast && N <= 8192 && m40_rows_gemv_supported(M, K)) {
+        // few columns: the vector-ALU row kernel needs no K split and no second launch
+        return m40_rows_gemv_residual(stream, A, B, nullptr, C, M, N, K);
     } else if (fast && m40_skinny_supported(ctx, stream_kind, M, N, K, 0)) {
         return m40_launch_skinny(ctx, stream, stream_kind, 0, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     } else if (fast && K % 64 == 0 && (size_t)K * 64 <= ctx->scratch[stream_kind].gemm_pack_bytes - 256) {

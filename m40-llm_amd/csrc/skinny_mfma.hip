@@ -707,7 +707,7 @@ int m40llm_ext_batched_gemm_residual_f32xf16_async(M40llmCudaContext* ctx, const
     if (N <= 0 || K <= 0) return -2;
     if (!rows_ok(ctx, (int)rows, K) || !m40_aligned16(d_w_f16)) return -6;
     (void)hipGetLastError();
-    if (m40_rows_gemv_supported((int)rows, K) && m40_aligned16(d_a_f32))
+    if (N <= 8192 && m40_rows_gemv_supported((int)rows, K) && m40_aligned16(d_a_f32))
         return m40_rows_gemv_residual(ctx->decode_stream, static_cast<const float*>(d_a_f32),
                                       static_cast<const uint16_t*>(d_w_f16), static_cast<const float*>(d_residual_f32),
                                       static_cast<float*>(d_out_f32), (int)rows, N, K);
