@@ -125,13 +125,6 @@ __device__ __forceinline__ void stage_finish(const StageRegs& first, const float
     __syncthreads();
 }
 
-__device__ __forceinline__ void stage_plain(const float* __restrict__ x, int K, float* __restrict__ a_lds) {
-    const float4* x4 = reinterpret_cast<const float4*>(x);
-    float4* a4 = reinterpret_cast<float4*>(a_lds);
-    for (int i = threadIdx.x; i < K / 4; i += kThreads) a4[i] = x4[i];
-    __syncthreads();
-}
-
 struct QkvArgs {
     const float* x;
     const void* norm_w;
