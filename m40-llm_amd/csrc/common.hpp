@@ -39,7 +39,17 @@ struct M40llmCudaContext {
     hipEvent_t decode_waits_prefill_event;
     M40StreamScratch scratch[2];   // [stream_kind]
     int num_cus;
+    // RoPE pair frequencies base^(-2 i / head_dim), i < head_dim / 2, filled on the device on first use of a
+    // (head_dim, base) on a stream: kM40RopeSlots tables of kM40RopeTableLen floats per stream
+    float* rope_tables;
+    struct { float base; uint32_t head_dim; uint32_t ready; } rope_slots[2][4];
 };
+constexpr int kM40RopeSlots = 4;
+constexpr int kM40RopeTableLen = 256;
+// Table of a (head_dim, base) for kernels launched on `stream` (of kind stream_kind), or nullptr (head_dim too large,
+// no free slot, or the stream is being captured and the table does not exist yet): callers then evaluate the power.
+const float* m40_rope_inv_freq_table(M40llmCudaContext* ctx, uint32_t stream_kind, hipStream_t stream, uint32_t head_dim,
+                                     float base);
 
 struct M40llmKVCache {
     // dense storage, f16 [seq][token][kv_head][head_dim]
@@ -99,7 +109,7 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
 bool m40_rows_gemv_supported(int rows, int K);
 int m40_rows_gemv_residual(hipStream_t stream, const float* a, const uint16_t* W, const float* residual, float* out,
                            int rows, int N, int K);
-int m40_rows_norm_qkv(hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
+int m40_rows_norm_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
                       uint32_t rows, const float* x, const void* norm_w, uint32_t norm_dtype, float eps,
                       const uint16_t* wq, const uint16_t* wk, const uint16_t* wv, const float* bq, const float* bk,
                       const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
@@ -226,17 +236,24 @@ __device__ __forceinline__ void m40_rope_pair(uint32_t head, uint32_t off, uint3
 // that rotates (standalone RoPE, the rotating KV appends, the fused QKV kernel) must produce the same
 // bits for the same input, and the compiler's choices inside the inlined trigonometric code were seen
 // to differ by an ulp between call sites.
-__device__ __noinline__ static float2 m40_rope_cos_sin(uint32_t position, uint32_t off, uint32_t head_dim, float base,
-                                                       float scale) {
-    const float pos = static_cast<float>(position) * scale;
+__device__ __noinline__ static float m40_rope_inv_freq(uint32_t off, uint32_t head_dim, float base) {
     // The per-pair frequency is evaluated in double and rounded once: theta multiplies it by
     // the position, so a one-ulp difference in a float powf would grow to ~position * 2^-23
     // radians.  The rounded double result equals the host libm's powf for the bases and
     // exponents in use.
     const float exponent = -2.0f * static_cast<float>(off) / static_cast<float>(head_dim);
-    const float inv_freq = static_cast<float>(pow(static_cast<double>(base), static_cast<double>(exponent)));
+    return static_cast<float>(pow(static_cast<double>(base), static_cast<double>(exponent)));
+}
+// cos/sin at `position` for a pair whose frequency is already known (from m40_rope_inv_freq or from the context's
+// table of the same values).
+__device__ __noinline__ static float2 m40_rope_cos_sin_freq(uint32_t position, float inv_freq, float scale) {
+    const float pos = static_cast<float>(position) * scale;
     const float theta = pos * inv_freq;
     return make_float2(cosf(theta), sinf(theta));
+}
+__device__ __forceinline__ float2 m40_rope_cos_sin(uint32_t position, uint32_t off, uint32_t head_dim, float base,
+                                                   float scale) {
+    return m40_rope_cos_sin_freq(position, m40_rope_inv_freq(off, head_dim, base), scale);
 }
 __device__ __forceinline__ void m40_rope_apply(float2 cs, float x0, float x1, float* y0, float* y1) {
     // explicit fused multiply-adds: the same rounding in every kernel that inlines this rotation

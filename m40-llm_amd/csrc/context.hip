@@ -31,7 +31,35 @@ bool alloc_scratch(M40StreamScratch& s) {
     return true;
 }
 
+// inv_freq[i] = base^(-2 i / head_dim) by the expression every rotating kernel uses when it has no table
+__global__ void rope_table_kernel(float* table, uint32_t head_dim, float base) {
+    const uint32_t i = threadIdx.x;
+    if (i < head_dim / 2u) table[i] = m40_rope_inv_freq(i, head_dim, base);
+}
+
 }  // namespace
+
+const float* m40_rope_inv_freq_table(M40llmCudaContext* ctx, uint32_t stream_kind, hipStream_t stream, uint32_t head_dim,
+                                     float base) {
+    if (!ctx || !ctx->rope_tables || stream_kind > 1u || head_dim / 2u > (uint32_t)kM40RopeTableLen || head_dim < 2u)
+        return nullptr;
+    float* tables = ctx->rope_tables + (size_t)stream_kind * kM40RopeSlots * kM40RopeTableLen;
+    int free_slot = -1;
+    for (int i = 0; i < kM40RopeSlots; ++i) {
+        auto& slot = ctx->rope_slots[stream_kind][i];
+        if (slot.ready && slot.head_dim == head_dim && slot.base == base) return tables + (size_t)i * kM40RopeTableLen;
+        if (!slot.ready && free_slot < 0) free_slot = i;
+    }
+    if (free_slot < 0) return nullptr;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone) return nullptr;
+    float* table = tables + (size_t)free_slot * kM40RopeTableLen;
+    rope_table_kernel<<<1, kM40RopeTableLen, 0, stream>>>(table, head_dim, base);
+    if (hipGetLastError() != hipSuccess) return nullptr;
+    auto& slot = ctx->rope_slots[stream_kind][free_slot];
+    slot.base = base; slot.head_dim = head_dim; slot.ready = 1u;
+    return table;
+}
 
 extern "C" {
 
@@ -67,6 +95,11 @@ M40llmCudaContext* m40llm_create_context(int device_id) {
         m40llm_destroy_context(ctx);
         return nullptr;
     }
+    if (hipMalloc(&ctx->rope_tables, sizeof(float) * 2 * kM40RopeSlots * kM40RopeTableLen) != hipSuccess) {
+        ctx->rope_tables = nullptr;
+        m40llm_destroy_context(ctx);
+        return nullptr;
+    }
     hipDeviceProp_t prop;
     ctx->num_cus = 256;
     if (hipGetDeviceProperties(&prop, selected) == hipSuccess && prop.multiProcessorCount > 0) {
@@ -82,6 +115,7 @@ void m40llm_destroy_context(M40llmCudaContext* ctx) {
     if (ctx->prefill_stream) (void)hipStreamSynchronize(ctx->prefill_stream);
     free_scratch(ctx->scratch[0]);
     free_scratch(ctx->scratch[1]);
+    if (ctx->rope_tables) (void)hipFree(ctx->rope_tables);
     if (ctx->prefill_waits_decode_event) (void)hipEventDestroy(ctx->prefill_waits_decode_event);
     if (ctx->decode_waits_prefill_event) (void)hipEventDestroy(ctx->decode_waits_prefill_event);
     if (ctx->prefill_stream) (void)hipStreamDestroy(ctx->prefill_stream);

@@ -181,6 +181,7 @@ struct RowsQkvArgs {
     const uint32_t* ids_dev; const uint32_t* lens_dev;
     uint32_t rows, d_model, max_seq_len, max_batch, q_heads, kv_heads, head_dim, rope_layout, norm_dtype;
     float eps, rope_base, rope_scale;
+    const float* rope_table;      // pair frequencies of (head_dim, rope_base), or null
 };
 
 // RMSNorm of every row, Q/K/V projections, bias, RoPE at each row's position, q out, K/V (f16) into the cache rows.
@@ -230,11 +231,15 @@ __global__ __launch_bounds__(kThreads) void rows_norm_qkv_kernel(RowsQkvArgs p) 
     const uint32_t position = p.lens_dev[e_rowc];
     const uint32_t seq = p.ids_dev[e_rowc];
     const float b0 = *(bias ? bias + e_i0 : p.x), b1 = *(bias ? bias + e_i1 : p.x);
+    float inv_freq = p.rope_table ? p.rope_table[e_off] : 0.0f;
     GemvRegs<kCols> regs;
     gemv_prefetch<kCols>(bp, 0, K >> 3, lane, regs);
     // the rotation angle does not depend on the projections: evaluated while the weights are in flight
     float2 cs = make_float2(1.0f, 0.0f);
-    if (e_which != 2) cs = m40_rope_cos_sin(position, e_off, p.head_dim, p.rope_base, p.rope_scale);
+    if (e_which != 2) {
+        if (!p.rope_table) inv_freq = m40_rope_inv_freq(e_off, p.head_dim, p.rope_base);
+        cs = m40_rope_cos_sin_freq(position, inv_freq, p.rope_scale);
+    }
     rows_stage(xr, true, p.norm_dtype, p.eps, (int)p.rows, K, a_lds, wave_sums);
     float acc[kCols][kRows];
     rows_dot(regs, a_lds, K, lane, acc);
@@ -272,7 +277,7 @@ int m40_rows_gemv_residual(hipStream_t stream, const float* a, const uint16_t* W
     return hipGetLastError() == hipSuccess ? 0 : -7;
 }
 
-int m40_rows_norm_qkv(hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
+int m40_rows_norm_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
                       uint32_t rows, const float* x, const void* norm_w, uint32_t norm_dtype, float eps,
                       const uint16_t* wq, const uint16_t* wk, const uint16_t* wv, const float* bq, const float* bk,
                       const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
@@ -287,6 +292,7 @@ int m40_rows_norm_qkv(hipStream_t stream, const M40llmKVCache* kv, const uint32_
     p.rows = rows; p.d_model = d_model; p.max_seq_len = kv->max_seq_len; p.max_batch = kv->max_batch_size;
     p.q_heads = q_heads; p.kv_heads = kv->num_heads; p.head_dim = kv->head_dim; p.rope_layout = rope_layout;
     p.norm_dtype = norm_dtype; p.eps = eps; p.rope_base = rope_base; p.rope_scale = rope_scale;
+    p.rope_table = m40_rope_inv_freq_table(ctx, 1, stream, kv->head_dim, rope_base);
     const uint32_t pairs = (q_heads + 2u * kv->num_heads) * (kv->head_dim / 2u);
     const uint32_t blocks = (pairs + (kCols / 2) * kWaves - 1u) / ((kCols / 2) * kWaves);
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rows_norm_qkv_kernel),
