@@ -210,7 +210,8 @@ def test_gemm_known_answers(dev, orc):
 @pytest.mark.parametrize("M,N,K", [
     (1, 2048, 2048), (1, 256, 2048), (1, 5632, 2048), (1, 2048, 5632), (1, 32000, 2048),   # TinyLlama shapes
     (1, 11008, 2048), (1, 2048, 11008),                                                        # Qwen2.5-3B shapes
-    (2, 2048, 2048), (4, 256, 2048), (8, 2048, 2048), (8, 11008, 2048), (8, 2048, 11008),     # batched (MFMA, stacked)
+    (2, 2048, 2048), (4, 256, 2048), (8, 2048, 2048), (7, 333, 1024), (8, 8192, 256), (6, 4100, 2048),   # row-batched vector-ALU kernel
+    (8, 11008, 2048), (8, 2048, 11008), (3, 9000, 2048), (8, 512, 4096),                       # batched (MFMA, stacked)
     (16, 2048, 2048), (9, 4096, 4096), (16, 300, 14336),                                       # MFMA, two fragment sets
     (20, 520, 1024),                                                                           # more than one row tile
     (1, 37, 300), (3, 37, 300), (5, 7, 8), (1, 50, 2056),                                      # odd shapes: generic / tails
