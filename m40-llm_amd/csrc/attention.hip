@@ -379,14 +379,24 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
 
 // Reads the (ids, lens) pair of a batched call back to the host for validation, as the reference
 // does before launching (cuda/kernels.cu:4721-4754); returns the largest length.
-static int validate_batch(const M40llmKVCache* kv, const uint32_t* ids_dev, const uint32_t* lens_dev,
-                          uint32_t batch, uint32_t* max_len) {
-    uint32_t stack_ids[64], stack_lens[64];
-    uint32_t* ids = batch <= 64 ? stack_ids : new uint32_t[batch];
-    uint32_t* lens = batch <= 64 ? stack_lens : new uint32_t[batch];
+// The reference copies both metadata arrays to the host and validates them before it launches (kernels.cu:4723-4754).
+// Here the copies are ordered on the decode stream (they see whatever earlier decode-stream work wrote) and land in
+// the context's pinned staging words: two asynchronous copies and one wait.
+static int validate_batch(M40llmCudaContext* ctx, const M40llmKVCache* kv, const uint32_t* ids_dev,
+                          const uint32_t* lens_dev, uint32_t batch, uint32_t* max_len) {
+    uint32_t *ids, *lens;
+    const bool staged = ctx->host_staging && 2u * batch <= (uint32_t)kM40HostStagingWords;
+    if (staged) {
+        ids = ctx->host_staging;
+        lens = ctx->host_staging + batch;
+    } else {
+        ids = new uint32_t[batch];
+        lens = new uint32_t[batch];
+    }
     int rc = 0;
-    if (hipMemcpy(lens, lens_dev, (size_t)batch * 4, hipMemcpyDeviceToHost) != hipSuccess ||
-        hipMemcpy(ids, ids_dev, (size_t)batch * 4, hipMemcpyDeviceToHost) != hipSuccess) {
+    if (hipMemcpyAsync(lens, lens_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, ctx->decode_stream) != hipSuccess ||
+        hipMemcpyAsync(ids, ids_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, ctx->decode_stream) != hipSuccess ||
+        hipStreamSynchronize(ctx->decode_stream) != hipSuccess) {
         (void)hipGetLastError();
         rc = -7;
     }
@@ -396,7 +406,7 @@ static int validate_batch(const M40llmKVCache* kv, const uint32_t* ids_dev, cons
         else if (lens[i] == 0 || lens[i] > kv->max_seq_len) rc = -8;
         else if (lens[i] > mx) mx = lens[i];
     }
-    if (batch > 64) { delete[] ids; delete[] lens; }
+    if (!staged) { delete[] ids; delete[] lens; }
     *max_len = mx;
     return rc;
 }
@@ -507,7 +517,7 @@ static int batched_impl(M40llmCudaContext* ctx, const M40llmKVCache* kv, const u
     if (kv->head_dim != 64 && kv->head_dim != 128) return -6;
     if (!kv->d_k || !kv->d_v) return -6;
     uint32_t max_len = 0;
-    int rc = validate_batch(kv, seq_ids_dev, seq_lens_dev, batch_size, &max_len);
+    int rc = validate_batch(ctx, kv, seq_ids_dev, seq_lens_dev, batch_size, &max_len);
     if (rc != 0) return rc;
     if (max_len == 0) return -8;
     M40AttnArgs a{};

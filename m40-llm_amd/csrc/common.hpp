@@ -42,8 +42,10 @@ struct M40llmCudaContext {
     // RoPE pair frequencies base^(-2 i / head_dim), i < head_dim / 2, filled on the device on first use of a
     // (head_dim, base) on a stream: kM40RopeSlots tables of kM40RopeTableLen floats per stream
     float* rope_tables;
+    uint32_t* host_staging;        // pinned, kM40HostStagingWords words: device metadata read back for validation
     struct { float base; uint32_t head_dim; uint32_t ready; } rope_slots[2][4];
 };
+constexpr int kM40HostStagingWords = 2048;
 constexpr int kM40RopeSlots = 4;
 constexpr int kM40RopeTableLen = 256;
 // Table of a (head_dim, base) for kernels launched on `stream` (of kind stream_kind), or nullptr (head_dim too large,

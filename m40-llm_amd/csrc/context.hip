@@ -100,6 +100,11 @@ M40llmCudaContext* m40llm_create_context(int device_id) {
         m40llm_destroy_context(ctx);
         return nullptr;
     }
+    if (hipHostMalloc(reinterpret_cast<void**>(&ctx->host_staging), sizeof(uint32_t) * kM40HostStagingWords, hipHostMallocDefault) != hipSuccess) {
+        ctx->host_staging = nullptr;
+        m40llm_destroy_context(ctx);
+        return nullptr;
+    }
     hipDeviceProp_t prop;
     ctx->num_cus = 256;
     if (hipGetDeviceProperties(&prop, selected) == hipSuccess && prop.multiProcessorCount > 0) {
@@ -116,6 +121,7 @@ void m40llm_destroy_context(M40llmCudaContext* ctx) {
     free_scratch(ctx->scratch[0]);
     free_scratch(ctx->scratch[1]);
     if (ctx->rope_tables) (void)hipFree(ctx->rope_tables);
+    if (ctx->host_staging) (void)hipHostFree(ctx->host_staging);
     if (ctx->prefill_waits_decode_event) (void)hipEventDestroy(ctx->prefill_waits_decode_event);
     if (ctx->decode_waits_prefill_event) (void)hipEventDestroy(ctx->decode_waits_prefill_event);
     if (ctx->prefill_stream) (void)hipStreamDestroy(ctx->prefill_stream);
