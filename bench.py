@@ -8,7 +8,8 @@ greedy sample.  Workload at N=1: the TinyLlama-1.1B-shaped random-init model of 
 ids, then greedy decode at batch 1.  Weights and KV cache are resident in HBM before the timed region.
 
 Prints ONE JSON line: value = decoded tokens per second (whole job); roofline = the dominant kernel's algorithmic
-bytes per launch over its event-timed launch duration against 8 TB/s, plus its measured HBM traffic; cpu_baseline =
+bytes per launch over its event-timed launch duration against 8 TB/s, plus its measured HBM traffic and the time of a
+kernel that only reads the same number of bytes in one launch (the practical ceiling on this box); cpu_baseline =
 the CPU oracle timed on this host on a short sample of the same workload.  config.b8 carries the batch-8 half of the
 metric (Qwen2.5-3B-shaped model, 8 rows), measured in the same run.
 """
@@ -143,6 +144,32 @@ def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
             "whole_step_hbm_frac": (wbytes + kvbytes) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
 
 
+def plain_read_yardstick(pkg, ctx, nbytes):
+    """Fastest of a few workgroup counts for a plain one-launch read of nbytes (rotating over cold buffers): what a
+    bandwidth-bound kernel of this size can reach on this box, launch ramp and tail included."""
+    nbuf = int(max(2, min(24, (1 << 30) // nbytes)))
+    bufs = [ctx.alloc(nbytes) for _ in range(nbuf)]
+    out = ctx.alloc(2048 * 4)
+    e0, e1 = ctx.event(), ctx.event()
+    best = None
+    for wgs in (256, 512, 1024, 2048, 4096):
+        reps = 3 * nbuf
+        for i in range(nbuf + reps):
+            if i == nbuf:
+                ctx.sync(1)
+                ctx.record(e0, 1)
+            pkg.check(ctx.lib.m40llm_ext_read_probe_async(ctx.h, bufs[i % nbuf].ptr, nbytes, wgs, out.ptr),
+                      "m40llm_ext_read_probe_async")
+        ctx.record(e1, 1)
+        us = ctx.elapsed_ms(e0, e1) * 1e3 / reps
+        if best is None or us < best["us"]:
+            best = {"us": us, "workgroups": wgs}
+    for b in bufs:
+        b.free()
+    out.free()
+    return best
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,6 +227,7 @@ def main():
         src.free(); dst.free()
     dom = measure_dominant_kernel(pkg, ctx, dm, cfg, args.kernel_reps, mode)
     achieved = dom["bytes"] / (dom["avg_us"] * 1e-6) / 1e9
+    yard = plain_read_yardstick(pkg, ctx, dom["bytes"])
     token_bytes = algorithmic_bytes_per_token(cfg)
     out = {
         "metric": "decode tok/s at B=1 and B=8; attn+GEMV HBM GB/s as % of MI355X peak",
@@ -219,7 +247,10 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(dom["kernel"]), "kernel": dom["kernel"],
                      "shape": dom["shape"],
                      "avg_launch_us": dom["avg_us"], "launches_timed": dom["launches"],
-                     "algorithmic_bytes_per_launch": dom["bytes"]},
+                     "algorithmic_bytes_per_launch": dom["bytes"],
+                     # a kernel that only reads the same number of bytes, one launch, fastest of five grid sizes
+                     "plain_read_us": yard["us"], "plain_read_workgroups": yard["workgroups"],
+                     "frac_of_plain_read": yard["us"] / dom["avg_us"]},
     }
     dm.close()
     if not args.no_b8 and not args.layers:

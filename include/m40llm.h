@@ -312,6 +312,12 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
  * writes the top-1 minus top-2 gap to out_gap_dev (may be NULL).  Decode stream. */
 int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t rows,
                                 size_t n, uint32_t* out_idx_dev, float* out_gap_dev);
+/* Bandwidth yardstick (no counterpart in the reference): reads `bytes` (16-byte aligned start) of device memory
+ * once, `workgroups` (<= 65536) workgroups of 256 threads each owning a contiguous range, and xors every 32-bit word
+ * read into d_out_u32[0 .. 2047] (word = workgroup index modulo 2048; not cleared by the call).  One launch on the
+ * decode stream; the benchmarks time it beside the kernels it bounds. */
+int m40llm_ext_read_probe_async(M40llmCudaContext* ctx, const void* d_src, size_t bytes, uint32_t workgroups,
+                                uint32_t* d_out_u32);
 /* Fused batch-1 decode-step entry points (decode stream, asynchronous).  They compute exactly what the
  * reference's per-op call sequence computes (src/infer/forward.rs:304-662), several steps per launch:
  *   steps 1-5: RMSNorm -> Q/K/V projections (+bias) -> RoPE(Q) -> d_q_out; RoPE(K) and V -> f16 append at the

@@ -169,6 +169,32 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
     }
 }
 
+// Reads n16 16-byte words and folds them into one word per workgroup: the plain HBM read stream of one launch, as a
+// yardstick for the bandwidth-bound kernels (nothing else is computed).  A workgroup owns a contiguous range and
+// walks it with four streaming loads per thread in flight, like a wave of the GEMV walks its columns.
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict__ src, size_t n16, uint32_t* __restrict__ out) {
+    const size_t per = (n16 + gridDim.x - 1) / gridDim.x;
+    const size_t begin = (size_t)blockIdx.x * per;
+    const size_t end = begin + per < n16 ? begin + per : n16;
+    uint32_t acc = 0u;
+    for (size_t base = begin + threadIdx.x; base < end; base += 4u * 256u) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t i = base + (size_t)u * 256u;
+            v[u] = m40_load_stream(src + (i < end ? i : base));
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t w = v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+            acc ^= base + (size_t)u * 256u < end ? w : 0u;         // a stand-in load past the end does not count
+        }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) acc ^= (uint32_t)__shfl_xor((int)acc, o, 64);
+    if ((threadIdx.x & 63u) == 0u) atomicXor(&out[blockIdx.x & 2047u], acc);
+}
+
 inline int blocks_for(size_t n) { return (int)((n + kThreads - 1) / kThreads); }
 
 }  // namespace
@@ -356,6 +382,15 @@ int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32
     (void)hipGetLastError();
     argmax_kernel<<<rows, 1024, 0, ctx->decode_stream>>>(static_cast<const float*>(d_logits_f32), n,
                                                          out_idx_dev, out_gap_dev);
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_read_probe_async(M40llmCudaContext* ctx, const void* d_src, size_t bytes, uint32_t workgroups,
+                                uint32_t* d_out_u32) {
+    if (!ctx || !d_src || !d_out_u32) return -1;
+    if (bytes < 16 || workgroups == 0 || workgroups > 65536u || (reinterpret_cast<uintptr_t>(d_src) & 15u) != 0u) return -2;
+    (void)hipGetLastError();
+    read_probe_kernel<<<workgroups, 256, 0, ctx->decode_stream>>>(static_cast<const uint4*>(d_src), bytes / 16, d_out_u32);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -1,6 +1,6 @@
 """Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
 
-    python m40-llm_amd/kernel_bench.py [--only attn,gemv,gemm8,q80,bsel] [--json out.jsonl]
+    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8] [--json out.jsonl]
 
 Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
 events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
@@ -38,7 +38,7 @@ class Bench:
         if rc != 0:
             raise m40.M40Error(name, rc)
 
-    def time(self, name, shape, algo_bytes, launch, n_variants, stream=1, reps=None, warm=None):
+    def time(self, name, shape, algo_bytes, launch, n_variants, stream=1, reps=None, warm=None, quiet=False):
         """launch(i) enqueues one launch on variant i; returns microseconds per launch."""
         reps = reps or max(2 * n_variants, 64)
         warm = warm or max(n_variants, 8)
@@ -55,7 +55,8 @@ class Bench:
         row = dict(kernel=name, shape=shape, us_per_launch=round(us, 3), algorithmic_bytes=int(algo_bytes),
                    gbs=round(gbs, 1), frac=round(gbs / PEAK_GBS, 4), launches=reps, buffers=n_variants)
         self.rows.append(row)
-        print(f"{name:34s} {shape:44s} {us:9.2f} us {gbs:8.1f} GB/s  frac {gbs / PEAK_GBS:6.3f}", flush=True)
+        if not quiet:
+            print(f"{name:34s} {shape:44s} {us:9.2f} us {gbs:8.1f} GB/s  frac {gbs / PEAK_GBS:6.3f}", flush=True)
         return us
 
 
@@ -105,6 +106,29 @@ def bench_attention(b: Bench):
            lambda i: b.call("m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async", kv.h, ids[i].ptr, lens_m1.ptr, 1, B,
                             4096, q.ptr, qh, out.ptr), nset)
     kv.destroy()
+
+
+def bench_read_probe(b: Bench):
+    """Plain read of N bytes in one launch: what a bandwidth-bound kernel of that size can at best reach on this box."""
+    out = b.ctx.alloc(2048 * 4)
+    for label, nbytes in (("O projection weights (TinyLlama)", 2048 * 2048 * 2), ("down weights (TinyLlama)", 2048 * 5632 * 2),
+                          ("gate + up weights (TinyLlama)", 2 * 2048 * 5632 * 2), ("gate + up weights (Qwen2.5-3B)", 2 * 2048 * 11008 * 2),
+                          ("lm_head weights (TinyLlama)", 32000 * 2048 * 2), ("K + V, 32768 tokens x 8 heads x 128", 32768 * 8 * 128 * 2 * 2)):
+        nbuf = n_rot(nbytes, budget=2 << 30, cap=48)
+        bufs = [b.ctx.alloc(nbytes) for _ in range(nbuf)]
+        best = None
+        for wgs in (256, 512, 1024, 2048, 4096, 8192):          # the fastest split is the yardstick
+            rows_before = len(b.rows)
+            us = b.time("plain read, one launch", f"{label}: {nbytes / 1e6:.1f} MB, {wgs} workgroups", nbytes,
+                        lambda i: b.call("m40llm_ext_read_probe_async", bufs[i].ptr, nbytes, wgs, out.ptr), nbuf, quiet=True)
+            row = b.rows.pop(rows_before)
+            if best is None or us < best["us_per_launch"]:
+                best = row
+        b.rows.append(best)
+        print(f"{best['kernel']:34s} {best['shape']:44s} {best['us_per_launch']:9.2f} us {best['gbs']:8.1f} GB/s  frac {best['frac']:6.3f}",
+              flush=True)
+        for x in bufs:
+            x.free()
 
 
 def bench_gemv(b: Bench, M: int):
@@ -232,13 +256,15 @@ def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="attn,gemv,gemm8,q80,bsel,decode8")
+    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
     which = set(args.only.split(","))
     b = Bench()
     print(b.lib.m40llm_ext_build_info().decode() if hasattr(b.lib, "m40llm_ext_build_info") else "")
+    if "read" in which:
+        bench_read_probe(b)
     if "attn" in which:
         bench_attention(b)
     if "gemv" in which:

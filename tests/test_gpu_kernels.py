@@ -489,3 +489,17 @@ def test_argmax_extension(dev, orc):
         srt = np.sort(x[r])
         assert gap[r] == srt[-1] - srt[-2]
     assert idx[3] == 77 and gap[3] == 0.0
+
+
+def test_read_probe_xor(dev):
+    # the bandwidth yardstick reads every 16-byte word exactly once: the xor over all words must match
+    rng = np.random.default_rng(11)
+    for n16, wgs in ((1, 1), (255, 3), (2048 * 8 + 3, 7), (700001, 512), (700001, 4096)):
+        x = rng.integers(0, 2 ** 32, size=n16 * 4, dtype=np.uint32)
+        dx, out = dev.up(x), dev.up(np.zeros(2048, dtype=np.uint32))
+        dev.call("m40llm_ext_read_probe_async", dx.ptr, n16 * 16, wgs, out.ptr)
+        dev.sync()
+        assert np.bitwise_xor.reduce(out.download(np.uint32, (2048,))) == np.bitwise_xor.reduce(x)
+    assert dev.lib.m40llm_ext_read_probe_async(dev.h, dx.ptr, 8, 1, out.ptr) == -2
+    assert dev.lib.m40llm_ext_read_probe_async(dev.h, dx.ptr, 64, 0, out.ptr) == -2
+    assert dev.lib.m40llm_ext_read_probe_async(dev.h, None, 64, 1, out.ptr) == -1
