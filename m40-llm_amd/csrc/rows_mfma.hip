@@ -1,0 +1,291 @@
+// Row-batched projections (up to eight activation rows, K = 2048) against f16 GGUF weights [N][K] on the matrix
+// cores, one launch per projection, for the wide matrices of a batched decode step (gate/up, lm_head).
+//
+// The split-K kernel of skinny_mfma.hip converts a step of activations per barrier and needs a second launch to add
+// its slices.  Here the workgroups are persistent: each converts the eight rows once into f16 hi + lo MFMA fragments
+// for the whole of K (64 KB of LDS, per-row power-of-two scale, RMSNorm weights folded in), then walks its share of
+// the column tiles.  A tile's K range is split over the four waves (16 MFMA steps each), so a wave requests a whole
+// tile quarter -- sixteen 16-byte loads per lane -- at once and keeps two tiles in flight; the waves' partial sums
+// meet in LDS in wave order and the first wave writes the result (residual, bias or SwiGLU applied), so nothing is
+// left for a second launch and no result depends on timing.
+//
+// SwiGLU form: a tile is eight gate columns and the eight up columns of the same index, so that gate and up of an
+// output element come out of one MFMA accumulator tile, eight lanes apart.
+//
+// Reference semantics: RMSNorm cuda/kernels.cu:770-807, f32 x f16 GGUF product :5037-5052, SwiGLU :869-880; call
+// order of the batched layer src/infer/forward.rs:1831-2136.
+#include "common.hpp"
+
+#include <type_traits>
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+constexpr int kRows = 8;
+constexpr int kK = 2048;                      // the one K this kernel is built for
+constexpr int kSteps = kK / 32 / kWaves;      // MFMA k-steps per wave and tile: 16
+constexpr int kFragBytes = (kK / 32) * 64 * 16;   // 64 KB: [k-step][lane] 16-byte A-operand entries
+constexpr int kStageRow = kK / kWaves * 2 + 16;   // LDS bytes per column of a wave's weight tile quarter: 1 KB + 16 (spreads the columns over the banks)
+constexpr int kStageBytes = 16 * kStageRow;       // per wave
+constexpr int kDynamicLds = kFragBytes + kWaves * kStageBytes;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ m40_float4 mfma16x16x32(const uint4& a, const uint4& b, m40_float4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(m40_half8, a),
+                                                  __builtin_bit_cast(m40_half8, b), c, 0, 0, 0);
+}
+
+struct RowsMfmaArgs {
+    const float* x;            // [rows][K]
+    const void* norm_w;        // RMSNorm weights, or null
+    uint32_t norm_dtype;       // 0 f16, 1 f32
+    float eps;
+    const uint16_t* W0;        // [N][K]
+    const uint16_t* W1;        // SwiGLU: the up matrix
+    float* out;                // [rows][N]
+    int rows, N, units;        // units: 16-column tiles (plain) or 8-column gate/up tiles (SwiGLU)
+};
+
+template <bool SWIGLU>
+__global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t frag_bytes[];
+    uint4* a_frag = reinterpret_cast<uint4*>(frag_bytes);
+    uint8_t* stage = frag_bytes + kFragBytes + (threadIdx.x >> 6) * kStageBytes;     // this wave's weight tile quarter
+    __shared__ float red_s[2][kWaves][4][64];      // the waves' tile sums, two tiles deep
+    __shared__ float row_scale_s[kRows];           // undoes the row's power-of-two scale, times the RMSNorm factor
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int j = lane & 15, g = lane >> 4;
+    const int u_begin = (int)((long long)blockIdx.x * p.units / gridDim.x);
+    const int u_end = (int)((long long)(blockIdx.x + 1) * p.units / gridDim.x);
+    const int n_units = u_end - u_begin;
+
+    // Weight loads are whole 1 KB runs: instruction i of a wave reads the wave's K quarter of column i of the tile,
+    // 16 bytes per lane.  (Reading the MFMA operand layout straight from memory -- 16 columns x 64 bytes per
+    // instruction, 4 KB apart -- streams a third slower: measured 26.5 us against 18.2 us for these 90 MB.)  The
+    // operand layout is produced by a pass through the wave's own LDS tile.
+    // No load under a branch: a tile past the workgroup's range re-reads the first 16 bytes of its first tile.
+    uint4 b0[kSteps], b1[kSteps];
+    auto issue = [&](uint4 (&b)[kSteps], int local) {
+        const bool live = local < n_units;
+        const int unit = u_begin + (live ? local : 0);
+        const int lane_off = live ? 8 * lane : 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            int col;
+            const uint16_t* W = p.W0;
+            if (SWIGLU) {
+                col = 8 * unit + (i & 7);
+                if (i & 8) W = p.W1;
+            } else {
+                col = 16 * unit + i;
+            }
+            col = col < p.N ? col : p.N - 1;
+            b[i] = *reinterpret_cast<const uint4*>(W + (size_t)col * kK + wave * (kK / kWaves) + lane_off);
+        }
+    };
+    issue(b0, 0);
+
+    // ---- the eight rows -> f16 hi + lo fragments, once -------------------------------------------------------
+    // Thread (row = tid / 32, l = tid % 32) owns the 8-element chunks l, l + 32, ... of its row, so a row lives in
+    // one half-wave and its maximum and sum of squares need no LDS.
+    {
+        const int row = tid >> 5, l = tid & 31;
+        const bool live = row < p.rows;
+        const float* xr = p.x + (size_t)(live ? row : 0) * kK;
+        float v[8][8];
+        float sq = 0.0f;            // sum of squares of the raw row (RMSNorm only)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float4 a = reinterpret_cast<const float4*>(xr)[2 * (l + 32 * c)];
+            const float4 b = reinterpret_cast<const float4*>(xr)[2 * (l + 32 * c) + 1];
+            v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
+            v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
+        }
+        // norm weights: every load of a branch goes out before its first use (one round trip, not one per chunk)
+        if (p.norm_w && p.norm_dtype == 0u) {
+            uint4 wq[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wq[c] = reinterpret_cast<const uint4*>(p.norm_w)[l + 32 * c];
+            float sq0 = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                float w[8];
+                m40_unpack8(wq[c], w);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { sq0 = fmaf(v[c][e], v[c][e], sq0); v[c][e] *= w[e]; }
+            }
+            sq = sq0;
+        } else if (p.norm_w) {
+            float4 wa[8], wb[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                wa[c] = reinterpret_cast<const float4*>(p.norm_w)[2 * (l + 32 * c)];
+                wb[c] = reinterpret_cast<const float4*>(p.norm_w)[2 * (l + 32 * c) + 1];
+            }
+            float sq0 = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const float w[8] = {wa[c].x, wa[c].y, wa[c].z, wa[c].w, wb[c].x, wb[c].y, wb[c].z, wb[c].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { sq0 = fmaf(v[c][e], v[c][e], sq0); v[c][e] *= w[e]; }
+            }
+            sq = sq0;
+        }
+        float mx = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (!live) v[c][e] = 0.0f;
+                mx = fmaxf(mx, fabsf(v[c][e]));
+            }
+#pragma unroll
+        for (int o = 1; o < 32; o <<= 1) {
+            sq += __shfl_xor(sq, o, 64);
+            mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        }
+        float scale = 1.0f, inv_scale = 1.0f;
+        if (mx > 0.0f && mx < INFINITY) {
+            int ex;
+            (void)frexpf(mx, &ex);        // mx = f * 2^ex, f in [0.5, 1)
+            ex -= 11;                     // scaled maximum in [2^10, 2^11)
+            ex = ex < -100 ? -100 : (ex > 100 ? 100 : ex);
+            scale = ldexpf(1.0f, ex);
+            inv_scale = ldexpf(1.0f, -ex);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            uint32_t hi[4], lo[4];
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                uint32_t h2 = 0, l2 = 0;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const float s = v[c][e + q] * inv_scale;
+                    const _Float16 h = static_cast<_Float16>(s);
+                    const _Float16 lw = static_cast<_Float16>(s - static_cast<float>(h));
+                    h2 |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * q);
+                    l2 |= (uint32_t)__builtin_bit_cast(uint16_t, lw) << (16 * q);
+                }
+                hi[e / 2] = h2; lo[e / 2] = l2;
+            }
+            const int chunk = l + 32 * c;                              // k = 8 chunk .. +7
+            const int entry = (chunk >> 2) * 64 + (chunk & 3) * 16 + row;   // A operand: lane = 16 (k / 8 % 4) + row
+            a_frag[entry] = make_uint4(hi[0], hi[1], hi[2], hi[3]);          // rows 0..7: hi parts
+            a_frag[entry + 8] = make_uint4(lo[0], lo[1], lo[2], lo[3]);      // rows 8..15: lo parts
+        }
+        if (l == 0) row_scale_s[row] = scale * (p.norm_w ? rsqrtf(sq / (float)kK + p.eps) : 1.0f);
+    }
+    issue(b1, 1);
+    __syncthreads();
+
+    // ---- tiles -------------------------------------------------------------------------------------------------
+    // tile quarter: registers -> LDS (column-major as loaded) -> MFMA B operand (lane (j, g): 16 bytes of column j)
+    auto to_lds = [&](const uint4 (&b)[kSteps]) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)      // built from the elements: a whole-struct copy would keep the array in scratch memory
+            *reinterpret_cast<u32x4*>(stage + i * kStageRow + 16 * lane) = u32x4{b[i].x, b[i].y, b[i].z, b[i].w};
+        __builtin_amdgcn_wave_barrier();
+    };
+    auto compute = [&](int parity) {
+        m40_float4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < kSteps; ++i) {
+            const uint4 bw = *reinterpret_cast<const uint4*>(stage + j * kStageRow + 64 * i + 16 * g);
+            acc = mfma16x16x32(a_frag[(kSteps * wave + i) * 64 + lane], bw, acc);
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            acc[r] += __shfl_xor(acc[r], 32, 64);       // hi rows (g 0, 1) + lo rows (g 2, 3)
+            red_s[parity][wave][r][lane] = acc[r];
+        }
+    };
+    // After the barrier every thread can form any element of the tile from red_s.  Thread t writes element t modulo
+    // the tile's live elements, so every thread stores exactly once (some twice the same value to the same address):
+    // no store sits under a branch, and the waits of the loop stay exact.
+    constexpr int kTileCols = SWIGLU ? 8 : 16;
+    const int n_out = kTileCols * p.rows;
+    const int e_out = tid % n_out, e_row = e_out / kTileCols, e_j = e_out % kTileCols;
+    const int e_lane = 16 * (e_row >> 2) + e_j, e_r = e_row & 3;
+    auto tile_sum = [&](int parity, int ln) {
+        return ((red_s[parity][0][e_r][ln] + red_s[parity][1][e_r][ln]) + red_s[parity][2][e_r][ln]) + red_s[parity][3][e_r][ln];
+    };
+    auto finish = [&](int local, int parity) {
+        const int unit = u_begin + local;
+        const float s = row_scale_s[e_row];
+        int col = kTileCols * unit + e_j;
+        col = col < p.N ? col : p.N - 1;          // a column past the end was computed from the last column's weights
+        float v = tile_sum(parity, e_lane) * s;
+        if (SWIGLU) {
+            const float up = tile_sum(parity, e_lane + 8) * s;
+            v = v / (1.0f + expf(-v)) * up;
+        }
+        p.out[(size_t)e_row * p.N + col] = v;
+    };
+    // One tile from register set b; PREFETCH: tile local + 2 exists and is requested into the same set.
+    auto tile = [&](uint4 (&b)[kSteps], auto prefetch_c, int local, int parity) {
+        to_lds(b);
+        if (decltype(prefetch_c)::value) issue(b, local + 2);
+        compute(parity);
+        __syncthreads();
+        finish(local, parity);
+    };
+    {
+        const std::integral_constant<bool, true> yes;
+        const std::integral_constant<bool, false> no;
+        int local = 0;
+        for (; local + 3 < n_units; local += 2) {        // both tiles of a pair have a tile two ahead
+            tile(b0, yes, local, 0);
+            tile(b1, yes, local + 1, 1);
+        }
+        const int rem = n_units - local;                  // 1, 2 or 3
+        if (rem == 3) {
+            tile(b0, yes, local, 0);
+            tile(b1, no, local + 1, 1);
+            tile(b0, no, local + 2, 0);
+        } else if (rem == 2) {
+            tile(b0, no, local, 0);
+            tile(b1, no, local + 1, 1);
+        } else {
+            tile(b0, no, local, 0);
+        }
+    }
+}
+
+template <bool SWIGLU>
+int launch(M40llmCudaContext* ctx, hipStream_t stream, const RowsMfmaArgs& a) {
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rows_mfma_kernel<SWIGLU>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDynamicLds);
+    if (attr != hipSuccess) return -7;
+    int grid = ctx->num_cus;           // one workgroup per CU: 138 KB of LDS each
+    if (grid > a.units) grid = a.units;
+    rows_mfma_kernel<SWIGLU><<<grid, kThreads, kDynamicLds, stream>>>(a);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
+
+}  // namespace
+
+bool m40_rows_mfma_supported(int rows, int K) { return rows >= 1 && rows <= kRows && K == kK; }
+
+int m40_rows_mfma_swiglu(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
+                         float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K) {
+    if (!m40_rows_mfma_supported(rows, K) || ffn <= 0) return -6;
+    if (!m40_aligned16(x) || !m40_aligned16(wgate) || !m40_aligned16(wup) || (norm_w && !m40_aligned16(norm_w))) return -6;
+    RowsMfmaArgs a{};
+    a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = wgate; a.W1 = wup; a.out = out;
+    a.rows = rows; a.N = ffn; a.units = (ffn + 7) / 8;
+    return launch<true>(ctx, stream, a);
+}
+
+int m40_rows_mfma_plain(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
+                        float eps, const uint16_t* W, float* out, int rows, int N, int K) {
+    if (!m40_rows_mfma_supported(rows, K) || N <= 0) return -6;
+    if (!m40_aligned16(x) || !m40_aligned16(W) || (norm_w && !m40_aligned16(norm_w))) return -6;
+    RowsMfmaArgs a{};
+    a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = W; a.out = out; a.rows = rows; a.N = N; a.units = (N + 15) / 16;
+    return launch<false>(ctx, stream, a);
+}

@@ -732,6 +732,11 @@ int m40llm_ext_batched_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const v
     if (norm_weight_dtype > 1) return -4;
     if (!rows_ok(ctx, (int)rows, d_model) || !m40_aligned16(d_wgate_f16) || !m40_aligned16(d_wup_f16)) return -6;
     (void)hipGetLastError();
+    // up to eight rows and K = 2048: persistent kernel with the SwiGLU inside (one launch instead of two)
+    if (m40_rows_mfma_supported((int)rows, d_model) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
+        return m40_rows_mfma_swiglu(ctx, ctx->decode_stream, static_cast<const float*>(d_x_f32), d_norm_w, norm_weight_dtype,
+                                    eps, static_cast<const uint16_t*>(d_wgate_f16), static_cast<const uint16_t*>(d_wup_f16),
+                                    static_cast<float*>(d_hid_f32), (int)rows, ffn, d_model);
     PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
     const void* W[2] = {d_wgate_f16, d_wup_f16};
     const int Ns[2] = {ffn, ffn};
@@ -750,6 +755,9 @@ int m40llm_ext_batched_norm_gemm_f32xf16_async(M40llmCudaContext* ctx, const voi
     if (norm_weight_dtype > 1) return -4;
     if (!rows_ok(ctx, (int)rows, K) || !m40_aligned16(d_w_f16)) return -6;
     (void)hipGetLastError();
+    if (m40_rows_mfma_supported((int)rows, K) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
+        return m40_rows_mfma_plain(ctx, ctx->decode_stream, static_cast<const float*>(d_x_f32), d_norm_w, norm_weight_dtype, eps,
+                                   static_cast<const uint16_t*>(d_w_f16), static_cast<float*>(d_out_f32), (int)rows, N, K);
     PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
     const void* W[1] = {d_w_f16};
     const int Ns[1] = {N};

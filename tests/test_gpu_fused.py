@@ -221,6 +221,50 @@ def test_batched_gemm_residual_and_norm_gate_up_vs_oracle(dev, orc, rows):
     dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", hid.ptr, dwd.ptr, dx.ptr, out.ptr, rows, D, F - 64, expect=-6)
 
 
+@pytest.mark.parametrize("rows,F,V,norm_dtype", [(1, 1004, 1000, 1), (5, 2056, 4099, 0), (8, 5632, 20011, 1)])
+def test_batched_projections_at_k2048_vs_oracle(dev, orc, rows, F, V, norm_dtype):
+    # d_model 2048 with up to eight rows takes the persistent matrix-core kernel: gate/up + SwiGLU with column tails
+    # (F not a multiple of 8), lm_head-style norm + product (V not a multiple of 16), and a wide residual product
+    rng = np.random.default_rng(100 + rows)
+    D = 2048
+    x = _rows_case(rng, rows, D)
+    nw = (1 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    if norm_dtype == 0:
+        nw = nw.astype(np.float16).astype(np.float32)
+    dnw = dev.up(f16bits(nw) if norm_dtype == 0 else nw)
+    wg = f16bits(rng.standard_normal((F, D)) * 0.03); wu = f16bits(rng.standard_normal((F, D)) * 0.03)
+    dx, dwg, dwu = dev.up(x), dev.up(wg), dev.up(wu)
+    hid = dev.zeros(rows * F * 4)
+    dev.call("m40llm_ext_batched_norm_gate_up_swiglu_async", dx.ptr, dnw.ptr, norm_dtype, 1e-5, dwg.ptr, dwu.ptr, hid.ptr, rows, F, D)
+    dev.sync()
+    xn = orc.rms_norm(x, 1e-5, nw, 1)
+    want_h = orc.swiglu(orc.gemm("f32xf16_gguf", xn, wg, rows, F, D), orc.gemm("f32xf16_gguf", xn, wu, rows, F, D))
+    got_h = hid.download(np.float32, (rows, F))
+    sc = np.abs(want_h).max(axis=1, keepdims=True)
+    close(got_h / sc, want_h / sc)
+    # norm + product (the lm_head call)
+    wv = f16bits(rng.standard_normal((V, D)) * 0.03)
+    dwv, logits = dev.up(wv), dev.zeros(rows * V * 4)
+    dev.call("m40llm_ext_batched_norm_gemm_f32xf16_async", dx.ptr, dnw.ptr, norm_dtype, 1e-5, dwv.ptr, logits.ptr, rows, V, D)
+    dev.sync()
+    want = orc.gemm("f32xf16_gguf", xn, wv, rows, V, D)
+    got = logits.download(np.float32, (rows, V))
+    sc = np.abs(want).max(axis=1, keepdims=True)
+    close(got / sc, want / sc)
+    for r in range(rows):
+        assert int(np.argmax(got[r])) == int(np.argmax(want[r]))
+    # product + residual, in place, wider than the vector-ALU kernel takes (N > 8192)
+    if V > 8192:
+        res = rng.standard_normal((rows, V)).astype(np.float32)
+        dres = dev.up(res)
+        dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", dx.ptr, dwv.ptr, dres.ptr, dres.ptr, rows, V, D)
+        dev.sync()
+        want = res + orc.gemm("f32xf16_gguf", x, wv, rows, V, D)
+        got = dres.download(np.float32, (rows, V))
+        sc = np.abs(want).max(axis=1, keepdims=True)
+        close(got / sc, want / sc)
+
+
 @pytest.mark.parametrize("qh,kvh,hd,layout,bias,rows", [(8, 2, 64, 0, False, 5), (4, 2, 128, 1, True, 8), (4, 1, 128, 1, True, 12)])
 def test_batched_norm_qkv_rope_append_vs_oracle(dev, orc, qh, kvh, hd, layout, bias, rows):
     rng = np.random.default_rng(qh + rows)
