@@ -122,6 +122,12 @@ int m40_rows_mfma_swiglu(M40llmCudaContext* ctx, hipStream_t stream, const float
                          float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K);
 int m40_rows_mfma_plain(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
                         float eps, const uint16_t* W, float* out, int rows, int N, int K);
+bool m40_rows_mfma_qkv_supported(int rows, int K, uint32_t head_dim);
+int m40_rows_mfma_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev,
+                      const uint32_t* lens_dev, uint32_t rows, const float* x, const void* norm_w, uint32_t norm_dtype, float eps,
+                      const uint16_t* wq, const uint16_t* wk, const uint16_t* wv, const float* bq, const float* bk,
+                      const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
+                      uint32_t rope_layout, float* q_out);
 bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
 int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);

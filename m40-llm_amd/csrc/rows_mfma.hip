@@ -31,6 +31,8 @@ constexpr int kStageBytes = 16 * kStageRow;       // per wave
 constexpr int kDynamicLds = kFragBytes + kWaves * kStageBytes;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ m40_float4 mfma16x16x32(const uint4& a, const uint4& b, m40_float4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(m40_half8, a),
@@ -46,10 +48,44 @@ struct RowsMfmaArgs {
     const uint16_t* W1;        // SwiGLU: the up matrix
     float* out;                // [rows][N]
     int rows, N, units;        // units: 16-column tiles (plain) or 8-column gate/up tiles (SwiGLU)
+    // Q/K/V form: W0 / W1 / W2 are the three matrices; a tile is 16 columns of one head that hold eight whole rotation
+    // pairs (split-half layout: eight columns and their partners half a head further on)
+    const uint16_t* W2;
+    const float *bq, *bk, *bv;
+    float* q_out;                 // [rows][q_heads * head_dim]
+    uint16_t* k_cache; uint16_t* v_cache; uint32_t* seq_map;
+    const uint32_t* ids_dev; const uint32_t* lens_dev;
+    const float* rope_table;      // pair frequencies of (head_dim, rope_base), or null
+    uint32_t max_seq_len, max_batch, q_heads, kv_heads, head_dim, rope_layout;
+    float rope_base, rope_scale;
 };
 
-template <bool SWIGLU>
+// Column i (0..15) of Q/K/V tile `unit`: which matrix, and the column inside it.
+struct QkvTile {
+    int which, head, tt;          // tt: tile inside the head
+    bool split;                   // split-half pairs: columns 8 tt + i and head_dim / 2 + 8 tt + i
+};
+__device__ __forceinline__ QkvTile qkv_tile(const RowsMfmaArgs& p, int unit) {
+    const int tph = (int)p.head_dim / 16;
+    const int qt = (int)p.q_heads * tph, kt = (int)p.kv_heads * tph;
+    QkvTile t;
+    t.which = unit < qt ? 0 : (unit < qt + kt ? 1 : 2);
+    const int local = unit - (t.which == 0 ? 0 : (t.which == 1 ? qt : qt + kt));
+    t.head = local / tph;
+    t.tt = local % tph;
+    t.split = t.which != 2 && p.rope_layout == M40LLM_ROPE_LAYOUT_NEOX;
+    return t;
+}
+__device__ __forceinline__ int qkv_col(const RowsMfmaArgs& p, const QkvTile& t, int i) {
+    const int hd = (int)p.head_dim;
+    return t.split ? t.head * hd + (i & 8 ? hd / 2 : 0) + 8 * t.tt + (i & 7) : t.head * hd + 16 * t.tt + i;
+}
+
+// MODE 0: out = x W^T; 1: SwiGLU of gate and up; 2: Q/K/V with bias, RoPE and cache append
+template <int MODE>
 __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) {
+    constexpr bool SWIGLU = MODE == 1;
+    constexpr bool QKV = MODE == 2;
     extern __shared__ __attribute__((aligned(16))) uint8_t frag_bytes[];
     uint4* a_frag = reinterpret_cast<uint4*>(frag_bytes);
     uint8_t* stage = frag_bytes + kFragBytes + (threadIdx.x >> 6) * kStageBytes;     // this wave's weight tile quarter
@@ -79,14 +115,52 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
             if (SWIGLU) {
                 col = 8 * unit + (i & 7);
                 if (i & 8) W = p.W1;
+                col = col < p.N ? col : p.N - 1;
+            } else if (QKV) {
+                const QkvTile t = qkv_tile(p, unit);
+                col = qkv_col(p, t, i);
+                W = t.which == 0 ? p.W0 : (t.which == 1 ? p.W1 : p.W2);
             } else {
                 col = 16 * unit + i;
+                col = col < p.N ? col : p.N - 1;
             }
-            col = col < p.N ? col : p.N - 1;
             b[i] = *reinterpret_cast<const uint4*>(W + (size_t)col * kK + wave * (kK / kWaves) + lane_off);
         }
     };
-    issue(b0, 0);
+    // the tile element this thread writes (see `finish`)
+    constexpr int kTileCols = SWIGLU ? 8 : 16;      // output columns of a tile
+    const int n_out = kTileCols * p.rows;
+    const int e_out = tid % n_out, e_row = e_out / kTileCols, e_j = e_out % kTileCols;
+    const int e_lane = 16 * (e_row >> 2) + e_j, e_r = e_row & 3;
+
+    // Q/K/V form: what the thread's element needs besides the product -- its column and its partner's, biases, the
+    // row's position and sequence, the pair's frequency.  Requested for the first tile before anything else, so that
+    // the rotation is ready when the product is.
+    struct QkvOperands {
+        int which, col, partner_j;
+        bool second;
+        uint32_t position, seq;
+        float bias_own, bias_other, inv_freq;
+    };
+    auto qkv_operands = [&](int unit) {
+        QkvOperands o;
+        const QkvTile t = qkv_tile(p, unit);
+        o.which = t.which;
+        o.col = qkv_col(p, t, e_j);
+        o.partner_j = t.split ? e_j ^ 8 : e_j ^ 1;
+        o.second = t.split ? (e_j & 8) != 0 : (e_j & 1) != 0;
+        const uint32_t off = t.split ? (uint32_t)(8 * t.tt + (e_j & 7)) : (uint32_t)((16 * t.tt + e_j) >> 1);
+        const float* bias = t.which == 0 ? p.bq : (t.which == 1 ? p.bk : p.bv);
+        o.position = p.lens_dev[e_row];
+        o.seq = p.ids_dev[e_row];
+        o.bias_own = bias ? bias[o.col] : 0.0f;
+        o.bias_other = bias ? bias[qkv_col(p, t, o.partner_j)] : 0.0f;
+        o.inv_freq = p.rope_table ? p.rope_table[off] : m40_rope_inv_freq(off, p.head_dim, p.rope_base);
+        return o;
+    };
+    QkvOperands first_ops{};
+    float2 first_cs = make_float2(1.0f, 0.0f);
+    if (QKV) first_ops = qkv_operands(u_begin);
 
     // ---- the eight rows -> f16 hi + lo fragments, once -------------------------------------------------------
     // Thread (row = tid / 32, l = tid % 32) owns the 8-element chunks l, l + 32, ... of its row, so a row lives in
@@ -104,6 +178,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
             v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
             v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
         }
+        issue(b0, 0);       // behind the rows (returns are in order: the rows, cache-resident, are not kept waiting)
         // norm weights: every load of a branch goes out before its first use (one round trip, not one per chunk)
         if (p.norm_w && p.norm_dtype == 0u) {
             uint4 wq[8];
@@ -161,16 +236,11 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
             uint32_t hi[4], lo[4];
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
-                uint32_t h2 = 0, l2 = 0;
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const float s = v[c][e + q] * inv_scale;
-                    const _Float16 h = static_cast<_Float16>(s);
-                    const _Float16 lw = static_cast<_Float16>(s - static_cast<float>(h));
-                    h2 |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * q);
-                    l2 |= (uint32_t)__builtin_bit_cast(uint16_t, lw) << (16 * q);
-                }
-                hi[e / 2] = h2; lo[e / 2] = l2;
+                const f32x2 s2 = {v[c][e] * inv_scale, v[c][e + 1] * inv_scale};
+                const f16x2 h2 = __builtin_convertvector(s2, f16x2);                       // one packed conversion
+                const f16x2 l2 = __builtin_convertvector(s2 - __builtin_convertvector(h2, f32x2), f16x2);
+                hi[e / 2] = __builtin_bit_cast(uint32_t, h2);
+                lo[e / 2] = __builtin_bit_cast(uint32_t, l2);
             }
             const int chunk = l + 32 * c;                              // k = 8 chunk .. +7
             const int entry = (chunk >> 2) * 64 + (chunk & 3) * 16 + row;   // A operand: lane = 16 (k / 8 % 4) + row
@@ -179,6 +249,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
         }
         if (l == 0) row_scale_s[row] = scale * (p.norm_w ? rsqrtf(sq / (float)kK + p.eps) : 1.0f);
     }
+    if (QKV && first_ops.which != 2) first_cs = m40_rope_cos_sin_freq(first_ops.position, first_ops.inv_freq, p.rope_scale);
     issue(b1, 1);
     __syncthreads();
 
@@ -207,16 +278,33 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
     // After the barrier every thread can form any element of the tile from red_s.  Thread t writes element t modulo
     // the tile's live elements, so every thread stores exactly once (some twice the same value to the same address):
     // no store sits under a branch, and the waits of the loop stay exact.
-    constexpr int kTileCols = SWIGLU ? 8 : 16;
-    const int n_out = kTileCols * p.rows;
-    const int e_out = tid % n_out, e_row = e_out / kTileCols, e_j = e_out % kTileCols;
-    const int e_lane = 16 * (e_row >> 2) + e_j, e_r = e_row & 3;
     auto tile_sum = [&](int parity, int ln) {
         return ((red_s[parity][0][e_r][ln] + red_s[parity][1][e_r][ln]) + red_s[parity][2][e_r][ln]) + red_s[parity][3][e_r][ln];
     };
     auto finish = [&](int local, int parity) {
         const int unit = u_begin + local;
         const float s = row_scale_s[e_row];
+        if (QKV) {
+            const QkvOperands o = local == 0 ? first_ops : qkv_operands(unit);
+            float own = tile_sum(parity, e_lane) * s + o.bias_own;
+            const float other = tile_sum(parity, (e_lane & ~15) + o.partner_j) * s + o.bias_other;
+            if (o.position >= p.max_seq_len || o.seq >= p.max_batch) return;
+            if (o.which != 2) {
+                const float2 cs = local == 0 ? first_cs : m40_rope_cos_sin_freq(o.position, o.inv_freq, p.rope_scale);
+                float r0, r1;
+                m40_rope_apply(cs, o.second ? other : own, o.second ? own : other, &r0, &r1);
+                own = o.second ? r1 : r0;
+            }
+            if (o.which == 0) {
+                p.q_out[(size_t)e_row * p.q_heads * p.head_dim + o.col] = own;
+            } else {
+                const size_t ept = (size_t)p.kv_heads * p.head_dim;
+                uint16_t* dst = (o.which == 1 ? p.k_cache : p.v_cache) + ((size_t)o.seq * p.max_seq_len + o.position) * ept;
+                dst[o.col] = m40_f2h(own);
+                if (o.which == 1 && o.col == 0) p.seq_map[o.seq] = o.position + 1u;
+            }
+            return;
+        }
         int col = kTileCols * unit + e_j;
         col = col < p.N ? col : p.N - 1;          // a column past the end was computed from the last column's weights
         float v = tile_sum(parity, e_lane) * s;
@@ -256,14 +344,14 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
     }
 }
 
-template <bool SWIGLU>
+template <int MODE>
 int launch(M40llmCudaContext* ctx, hipStream_t stream, const RowsMfmaArgs& a) {
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rows_mfma_kernel<SWIGLU>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rows_mfma_kernel<MODE>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kDynamicLds);
     if (attr != hipSuccess) return -7;
     int grid = ctx->num_cus;           // one workgroup per CU: 138 KB of LDS each
     if (grid > a.units) grid = a.units;
-    rows_mfma_kernel<SWIGLU><<<grid, kThreads, kDynamicLds, stream>>>(a);
+    rows_mfma_kernel<MODE><<<grid, kThreads, kDynamicLds, stream>>>(a);
     return hipGetLastError() == hipSuccess ? 0 : -7;
 }
 
@@ -278,7 +366,7 @@ int m40_rows_mfma_swiglu(M40llmCudaContext* ctx, hipStream_t stream, const float
     RowsMfmaArgs a{};
     a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = wgate; a.W1 = wup; a.out = out;
     a.rows = rows; a.N = ffn; a.units = (ffn + 7) / 8;
-    return launch<true>(ctx, stream, a);
+    return launch<1>(ctx, stream, a);
 }
 
 int m40_rows_mfma_plain(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
@@ -287,5 +375,28 @@ int m40_rows_mfma_plain(M40llmCudaContext* ctx, hipStream_t stream, const float*
     if (!m40_aligned16(x) || !m40_aligned16(W) || (norm_w && !m40_aligned16(norm_w))) return -6;
     RowsMfmaArgs a{};
     a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = W; a.out = out; a.rows = rows; a.N = N; a.units = (N + 15) / 16;
-    return launch<false>(ctx, stream, a);
+    return launch<0>(ctx, stream, a);
+}
+
+bool m40_rows_mfma_qkv_supported(int rows, int K, uint32_t head_dim) {
+    return m40_rows_mfma_supported(rows, K) && head_dim >= 16 && head_dim % 16 == 0;
+}
+
+int m40_rows_mfma_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKVCache* kv, const uint32_t* ids_dev,
+                      const uint32_t* lens_dev, uint32_t rows, const float* x, const void* norm_w, uint32_t norm_dtype, float eps,
+                      const uint16_t* wq, const uint16_t* wk, const uint16_t* wv, const float* bq, const float* bk,
+                      const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
+                      uint32_t rope_layout, float* q_out) {
+    if (!m40_rows_mfma_qkv_supported((int)rows, (int)d_model, kv->head_dim)) return -6;
+    if (!m40_aligned16(x) || !m40_aligned16(norm_w) || !m40_aligned16(wq) || !m40_aligned16(wk) || !m40_aligned16(wv)) return -6;
+    RowsMfmaArgs a{};
+    a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = wq; a.W1 = wk; a.W2 = wv;
+    a.bq = bq; a.bk = bk; a.bv = bv; a.q_out = q_out; a.k_cache = kv->d_k; a.v_cache = kv->d_v; a.seq_map = kv->d_seq_map;
+    a.ids_dev = ids_dev; a.lens_dev = lens_dev;
+    a.rope_table = m40_rope_inv_freq_table(ctx, 1, stream, kv->head_dim, rope_base);
+    a.max_seq_len = kv->max_seq_len; a.max_batch = kv->max_batch_size; a.q_heads = q_heads; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.rope_layout = rope_layout; a.rope_base = rope_base; a.rope_scale = rope_scale;
+    a.rows = (int)rows; a.N = (int)((q_heads + 2u * kv->num_heads) * kv->head_dim);
+    a.units = a.N / 16;
+    return launch<2>(ctx, stream, a);
 }

@@ -675,6 +675,14 @@ int m40llm_ext_batched_norm_qkv_rope_append_async(
     if (!rows_ok(ctx, (int)rows, (int)d_model)) return -6;
     if (!m40_aligned16(d_wq_f16) || !m40_aligned16(d_wk_f16) || !m40_aligned16(d_wv_f16)) return -6;
     (void)hipGetLastError();
+    // up to eight rows and K = 2048: persistent matrix-core kernel with the whole epilogue inside
+    if (m40_rows_mfma_qkv_supported((int)rows, (int)d_model, kv->head_dim) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
+        return m40_rows_mfma_qkv(ctx, ctx->decode_stream, kv, seq_ids_dev, seq_lens_dev, rows, static_cast<const float*>(d_x_f32),
+                                 d_norm_w, norm_weight_dtype, eps, static_cast<const uint16_t*>(d_wq_f16),
+                                 static_cast<const uint16_t*>(d_wk_f16), static_cast<const uint16_t*>(d_wv_f16),
+                                 static_cast<const float*>(d_bq_f32), static_cast<const float*>(d_bk_f32),
+                                 static_cast<const float*>(d_bv_f32), d_model, q_heads, freq_base, freq_scale, rope_layout,
+                                 static_cast<float*>(d_q_out_f32));
     // up to eight rows and K <= 2048: vector-ALU kernel with the whole epilogue inside (one launch instead of two)
     if (m40_rows_gemv_supported((int)rows, (int)d_model) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
         return m40_rows_norm_qkv(ctx, ctx->decode_stream, kv, seq_ids_dev, seq_lens_dev, rows, static_cast<const float*>(d_x_f32),

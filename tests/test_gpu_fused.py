@@ -265,7 +265,10 @@ def test_batched_projections_at_k2048_vs_oracle(dev, orc, rows, F, V, norm_dtype
         close(got / sc, want / sc)
 
 
-@pytest.mark.parametrize("qh,kvh,hd,layout,bias,rows", [(8, 2, 64, 0, False, 5), (4, 2, 128, 1, True, 8), (4, 1, 128, 1, True, 12)])
+@pytest.mark.parametrize("qh,kvh,hd,layout,bias,rows", [
+    (8, 2, 64, 0, False, 5), (4, 2, 128, 1, True, 8), (4, 1, 128, 1, True, 12),
+    # d_model 2048 with up to eight rows: the persistent matrix-core kernel (adjacent and split-half pairs, with and without bias)
+    (32, 4, 64, 0, False, 5), (16, 2, 128, 1, True, 8), (32, 8, 64, 1, True, 1), (16, 4, 128, 0, True, 3)])
 def test_batched_norm_qkv_rope_append_vs_oracle(dev, orc, qh, kvh, hd, layout, bias, rows):
     rng = np.random.default_rng(qh + rows)
     D = qh * hd
@@ -306,6 +309,10 @@ def test_batched_norm_qkv_rope_append_vs_oracle(dev, orc, qh, kvh, hd, layout, b
         close(gk.view(np.float16).astype(np.float32) / sk, want_k / sk, 2e-3, 1e-3)       # f16 storage
         sv = np.abs(v[r]).max()
         close(gv.view(np.float16).astype(np.float32) / sv, v[r] / sv, 2e-3, 1e-3)
+        # nothing but the row's own position was written
+        if pos + 1 < S:
+            ok, _ = kv.read_token(seq, pos + 1)
+            assert not ok.any()
     kv.destroy()
 
 
