@@ -250,7 +250,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
         if (l == 0) row_scale_s[row] = scale * (p.norm_w ? rsqrtf(sq / (float)kK + p.eps) : 1.0f);
     }
     if (QKV && first_ops.which != 2) first_cs = m40_rope_cos_sin_freq(first_ops.position, first_ops.inv_freq, p.rope_scale);
-    issue(b1, 1);
+    if (!QKV) issue(b1, 1);            // the Q/K/V form has one tile per workgroup
     __syncthreads();
 
     // ---- tiles -------------------------------------------------------------------------------------------------
@@ -285,12 +285,12 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
         const int unit = u_begin + local;
         const float s = row_scale_s[e_row];
         if (QKV) {
-            const QkvOperands o = local == 0 ? first_ops : qkv_operands(unit);
+            const QkvOperands& o = first_ops;          // one tile per workgroup in this form (checked by the host)
             float own = tile_sum(parity, e_lane) * s + o.bias_own;
             const float other = tile_sum(parity, (e_lane & ~15) + o.partner_j) * s + o.bias_other;
             if (o.position >= p.max_seq_len || o.seq >= p.max_batch) return;
             if (o.which != 2) {
-                const float2 cs = local == 0 ? first_cs : m40_rope_cos_sin_freq(o.position, o.inv_freq, p.rope_scale);
+                const float2 cs = first_cs;
                 float r0, r1;
                 m40_rope_apply(cs, o.second ? other : own, o.second ? own : other, &r0, &r1);
                 own = o.second ? r1 : r0;
@@ -322,7 +322,9 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
         __syncthreads();
         finish(local, parity);
     };
-    {
+    if (QKV) {
+        tile(b0, std::integral_constant<bool, false>{}, 0, 0);
+    } else {
         const std::integral_constant<bool, true> yes;
         const std::integral_constant<bool, false> no;
         int local = 0;
@@ -388,6 +390,8 @@ int m40_rows_mfma_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKV
                       const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
                       uint32_t rope_layout, float* q_out) {
     if (!m40_rows_mfma_qkv_supported((int)rows, (int)d_model, kv->head_dim)) return -6;
+    // one tile per workgroup: the rotation angle of a thread's element is computed once, ahead of the product
+    if ((int)((q_heads + 2u * kv->num_heads) * kv->head_dim / 16u) > ctx->num_cus) return -6;
     if (!m40_aligned16(x) || !m40_aligned16(norm_w) || !m40_aligned16(wq) || !m40_aligned16(wk) || !m40_aligned16(wv)) return -6;
     RowsMfmaArgs a{};
     a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = wq; a.W1 = wk; a.W2 = wv;

@@ -676,7 +676,8 @@ int m40llm_ext_batched_norm_qkv_rope_append_async(
     if (!m40_aligned16(d_wq_f16) || !m40_aligned16(d_wk_f16) || !m40_aligned16(d_wv_f16)) return -6;
     (void)hipGetLastError();
     // up to eight rows and K = 2048: persistent matrix-core kernel with the whole epilogue inside
-    if (m40_rows_mfma_qkv_supported((int)rows, (int)d_model, kv->head_dim) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
+    if (m40_rows_mfma_qkv_supported((int)rows, (int)d_model, kv->head_dim) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w) &&
+        (int)((q_heads + 2u * kv->num_heads) * kv->head_dim / 16u) <= ctx->num_cus)
         return m40_rows_mfma_qkv(ctx, ctx->decode_stream, kv, seq_ids_dev, seq_lens_dev, rows, static_cast<const float*>(d_x_f32),
                                  d_norm_w, norm_weight_dtype, eps, static_cast<const uint16_t*>(d_wq_f16),
                                  static_cast<const uint16_t*>(d_wk_f16), static_cast<const uint16_t*>(d_wv_f16),

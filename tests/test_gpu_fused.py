@@ -265,6 +265,32 @@ def test_batched_projections_at_k2048_vs_oracle(dev, orc, rows, F, V, norm_dtype
         close(got / sc, want / sc)
 
 
+@pytest.mark.parametrize("rows,N,K", [(8, 2048, 11008), (5, 512, 5632), (3, 1000, 2304), (1, 2048, 4096), (8, 40, 8192)])
+def test_batched_down_projection_k_chunks_vs_oracle(dev, orc, rows, N, K):
+    # down-projection shapes (K > 2048, K slices summed with the residual by the slice-adding launch, in place; column
+    # tail; fewer column tiles than the chip has CUs)
+    rng = np.random.default_rng(rows + K)
+    a = _rows_case(rng, rows, K)
+    w = f16bits(rng.standard_normal((N, K)) * 0.03)
+    res = rng.standard_normal((rows, N)).astype(np.float32)
+    da, dw, dres = dev.up(a), dev.up(w), dev.up(res)
+    dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", da.ptr, dw.ptr, dres.ptr, dres.ptr, rows, N, K)
+    dev.sync()
+    want = res + orc.gemm("f32xf16_gguf", a, w, rows, N, K)
+    got = dres.download(np.float32, (rows, N))
+    sc = np.abs(want).max(axis=1, keepdims=True)
+    close(got / sc, want / sc)
+    # a second call with other inputs through the same scratch slices, no residual
+    a2 = _rows_case(rng, rows, K)
+    da2, out = dev.up(a2), dev.zeros(rows * N * 4)
+    dev.call("m40llm_ext_batched_gemm_residual_f32xf16_async", da2.ptr, dw.ptr, None, out.ptr, rows, N, K)
+    dev.sync()
+    want = orc.gemm("f32xf16_gguf", a2, w, rows, N, K)
+    got = out.download(np.float32, (rows, N))
+    sc = np.abs(want).max(axis=1, keepdims=True)
+    close(got / sc, want / sc)
+
+
 @pytest.mark.parametrize("qh,kvh,hd,layout,bias,rows", [
     (8, 2, 64, 0, False, 5), (4, 2, 128, 1, True, 8), (4, 1, 128, 1, True, 12),
     # d_model 2048 with up to eight rows: the persistent matrix-core kernel (adjacent and split-half pairs, with and without bias)
