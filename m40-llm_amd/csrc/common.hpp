@@ -42,6 +42,9 @@ struct M40llmCudaContext {
     // RoPE pair frequencies base^(-2 i / head_dim), i < head_dim / 2, filled on the device on first use of a
     // (head_dim, base) on a stream: kM40RopeSlots tables of kM40RopeTableLen floats per stream
     float* rope_tables;
+    // beside every frequency table: the rotation of each pair at the position last asked for, as {position bits, cos,
+    // sin, scale bits} (16 bytes, written and read whole); a decode step computes the angles once, in its first layer
+    float4* rope_cs;
     uint32_t* host_staging;        // pinned, kM40HostStagingWords words: device metadata read back for validation
     struct { float base; uint32_t head_dim; uint32_t ready; } rope_slots[2][4];
 };
@@ -117,6 +120,8 @@ int m40_rows_norm_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKV
                       const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
                       uint32_t rope_layout, float* q_out);
 // rows_mfma.hip: persistent matrix-core kernel for up to eight rows and K = 2048, epilogue inside (one launch)
+// the {position, cos, sin, scale} entries that belong to a table returned by m40_rope_inv_freq_table (or null)
+float4* m40_rope_cs_cache(M40llmCudaContext* ctx, const float* table);
 bool m40_rows_mfma_supported(int rows, int K);
 int m40_rows_mfma_swiglu(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
                          float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K);

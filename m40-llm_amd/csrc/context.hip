@@ -39,6 +39,11 @@ __global__ void rope_table_kernel(float* table, uint32_t head_dim, float base) {
 
 }  // namespace
 
+float4* m40_rope_cs_cache(M40llmCudaContext* ctx, const float* table) {
+    if (!ctx || !table || !ctx->rope_tables || !ctx->rope_cs) return nullptr;
+    return ctx->rope_cs + (table - ctx->rope_tables);
+}
+
 const float* m40_rope_inv_freq_table(M40llmCudaContext* ctx, uint32_t stream_kind, hipStream_t stream, uint32_t head_dim,
                                      float base) {
     if (!ctx || !ctx->rope_tables || stream_kind > 1u || head_dim / 2u > (uint32_t)kM40RopeTableLen || head_dim < 2u)
@@ -100,6 +105,11 @@ M40llmCudaContext* m40llm_create_context(int device_id) {
         m40llm_destroy_context(ctx);
         return nullptr;
     }
+    const size_t cs_bytes = sizeof(float4) * 2 * kM40RopeSlots * kM40RopeTableLen;
+    if (hipMalloc(reinterpret_cast<void**>(&ctx->rope_cs), cs_bytes) != hipSuccess || hipMemset(ctx->rope_cs, 0xff, cs_bytes) != hipSuccess) {
+        m40llm_destroy_context(ctx);       // 0xff: no entry matches a position
+        return nullptr;
+    }
     if (hipHostMalloc(reinterpret_cast<void**>(&ctx->host_staging), sizeof(uint32_t) * kM40HostStagingWords, hipHostMallocDefault) != hipSuccess) {
         ctx->host_staging = nullptr;
         m40llm_destroy_context(ctx);
@@ -121,6 +131,7 @@ void m40llm_destroy_context(M40llmCudaContext* ctx) {
     free_scratch(ctx->scratch[0]);
     free_scratch(ctx->scratch[1]);
     if (ctx->rope_tables) (void)hipFree(ctx->rope_tables);
+    if (ctx->rope_cs) (void)hipFree(ctx->rope_cs);
     if (ctx->host_staging) (void)hipHostFree(ctx->host_staging);
     if (ctx->prefill_waits_decode_event) (void)hipEventDestroy(ctx->prefill_waits_decode_event);
     if (ctx->decode_waits_prefill_event) (void)hipEventDestroy(ctx->decode_waits_prefill_event);

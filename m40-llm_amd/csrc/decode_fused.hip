@@ -136,6 +136,7 @@ struct QkvArgs {
     uint32_t* seq_map_entry;
     const uint32_t* position_dev;
     const float* rope_table;   // pair frequencies of (head_dim, rope_base), or null: the kernel evaluates the power
+    float4* rope_cs;           // with rope_table: {position bits, cos, sin, scale bits} per pair, kept from launch to launch
     uint32_t position, max_seq_len;
     uint32_t d_model, q_heads, kv_heads, head_dim, rope_layout, norm_dtype;
     float eps, rope_base, rope_scale;
@@ -178,8 +179,12 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
     // position and pair frequencies are requested with x, ahead of the weights
     const uint32_t position = p.position_dev ? *p.position_dev : p.position;
     float inv_freq[PAIRS];
+    float4 kept[PAIRS];        // the pair's rotation as left by an earlier launch (the step's first layer)
 #pragma unroll
-    for (int q = 0; q < PAIRS; ++q) inv_freq[q] = p.rope_table ? p.rope_table[off[q]] : 0.0f;
+    for (int q = 0; q < PAIRS; ++q) {
+        inv_freq[q] = p.rope_table ? p.rope_table[off[q]] : 0.0f;
+        kept[q] = p.rope_cs ? p.rope_cs[off[q]] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
     GemvRegs<2 * PAIRS> regs;
     gemv_prefetch<2 * PAIRS>(bp, 0, K >> 3, lane, regs);
     // the rotation angle does not depend on the data: evaluated while the weights are in flight
@@ -188,8 +193,17 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
     for (int q = 0; q < PAIRS; ++q) {
         cs[q] = make_float2(1.0f, 0.0f);
         if (which[q] != 2) {
-            if (!p.rope_table) inv_freq[q] = m40_rope_inv_freq(off[q], p.head_dim, p.rope_base);
-            cs[q] = m40_rope_cos_sin_freq(position, inv_freq[q], p.rope_scale);
+            // The angle depends on the position only: all layers of a step share it.  An entry is 16 bytes, stored and
+            // loaded whole, and carries its own position and scale, so a reader takes it only when it is this step's.
+            const bool hit = p.rope_cs && __float_as_uint(kept[q].x) == position && __float_as_uint(kept[q].w) == __float_as_uint(p.rope_scale);
+            if (hit) {
+                cs[q] = make_float2(kept[q].y, kept[q].z);
+            } else {
+                if (!p.rope_table) inv_freq[q] = m40_rope_inv_freq(off[q], p.head_dim, p.rope_base);
+                cs[q] = m40_rope_cos_sin_freq(position, inv_freq[q], p.rope_scale);
+                if (p.rope_cs && which[q] == 0 && local[q] < half && lane == 0)      // the waves of q head 0 keep it
+                    p.rope_cs[off[q]] = make_float4(__uint_as_float(position), cs[q].x, cs[q].y, p.rope_scale);
+            }
         }
     }
     stage_finish(xr, p.x, p.norm_w, p.norm_dtype, p.eps, K, a_lds, wave_sums);
@@ -454,6 +468,7 @@ int m40llm_ext_fused_norm_qkv_rope_append_async(
     p.rope_layout = rope_layout; p.norm_dtype = norm_weight_dtype;
     p.eps = eps; p.rope_base = freq_base; p.rope_scale = freq_scale;
     p.rope_table = m40_rope_inv_freq_table(ctx, 1, ctx->decode_stream, kv->head_dim, freq_base);
+    p.rope_cs = m40_rope_cs_cache(ctx, p.rope_table);
     const uint32_t pairs = (q_heads + 2u * kv->num_heads) * (kv->head_dim / 2u);
     (void)hipGetLastError();
     // one pair per wave: two per wave measured 3 % slower on the whole token at 1280 pairs
