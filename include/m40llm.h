@@ -21,7 +21,7 @@
  *     mutex around every FFI call, src/cuda.rs:1121-1137).
  *
  * Symbols of the reference that lie outside the decode hot path (staged / q8 /
- * lossy-summary attention modes, prefill attention, cuBLAS-only GEMM, persistent
+ * lossy-summary attention modes, cuBLAS-only GEMM, persistent
  * decode prototype, telemetry readers) are exported and return their
  * "unavailable" code exactly as cuda/stub.c does (-1), so a binding that declares
  * all of them still links.  They are listed at the end of this header.
@@ -304,6 +304,25 @@ int m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async(
  * q4 V + scales for positions < seq_len - recent_window and ring rows for the rest. */
 int m40llm_ext_kvcache_bulk_fill_f16(M40llmCudaContext* ctx, M40llmKVCache* kv, uint32_t seq_id,
                                      const void* k_dev_f16, const void* v_dev_f16, uint32_t seq_len);
+/* Packed variable-length causal prefill attention, all f32 (cuda/kernels.cu:3749-3835, entry points :4834-4977;
+ * declared src/cuda.rs:619-648; CPU restatement tests/attention_prefill_varlen.rs:27-76).
+ * Q and Out: [total_q][q_heads][head_dim]; K and V: [total_kv][kv_heads][head_dim]; sequence b owns q_lens[b] query
+ * tokens from q_offsets[b] and kv_lens[b] keys from kv_offsets[b] (token units, device arrays); query q_idx attends
+ * keys 0 .. kv_len - q_len + q_idx.  Prefill stream.  The lengths are read back and validated on the host before the
+ * launch in both forms, as in the reference; only the first form waits for the kernel.
+ * -1 null argument, -2 batch 0, -3 head counts, -9 head_dim not 64 / 128, -7 read-back failed,
+ * -8 a length is 0, q_len > kv_len or kv_len > 8192, -4 launch (or 16-byte misaligned Q/K/V), -5 synchronise. */
+int m40llm_attention_prefill_f32_gqa_varlen(M40llmCudaContext* ctx, const void* q_dev_f32, const void* k_dev_f32,
+                                            const void* v_dev_f32, const uint32_t* q_offsets_dev,
+                                            const uint32_t* kv_offsets_dev, const uint32_t* q_lens_dev,
+                                            const uint32_t* kv_lens_dev, uint32_t batch_size, uint32_t q_heads,
+                                            uint32_t kv_heads, uint32_t head_dim, void* out_dev_f32);
+int m40llm_attention_prefill_f32_gqa_varlen_async(M40llmCudaContext* ctx, const void* q_dev_f32, const void* k_dev_f32,
+                                                  const void* v_dev_f32, const uint32_t* q_offsets_dev,
+                                                  const uint32_t* kv_offsets_dev, const uint32_t* q_lens_dev,
+                                                  const uint32_t* kv_lens_dev, uint32_t batch_size, uint32_t q_heads,
+                                                  uint32_t kv_heads, uint32_t head_dim, void* out_dev_f32);
+
 /* raw views of the compressed cache for tests: which = 0 old_k, 1 q4_v, 2 q4_scale, 3 recent_k,
  * 4 recent_v, 5 seq_map; copies `bytes` from byte offset `offset` to the host */
 int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t which,
@@ -423,13 +442,6 @@ int m40llm_attention_last_token_f32_gqa_block_summary_lossy_async(
     uint32_t, uint32_t, void*);
 int m40llm_attention_last_token_f32_gqa_compressed_recent_only_async(
     M40llmCudaContext*, const M40llmKVCache*, uint32_t, const void*, uint32_t, uint32_t, void*);
-int m40llm_attention_prefill_f32_gqa_varlen(M40llmCudaContext*, const void*, const void*, const void*,
-                                            const uint32_t*, const uint32_t*, const uint32_t*,
-                                            const uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t, void*);
-int m40llm_attention_prefill_f32_gqa_varlen_async(M40llmCudaContext*, const void*, const void*, const void*,
-                                                  const uint32_t*, const uint32_t*, const uint32_t*,
-                                                  const uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t,
-                                                  void*);
 int m40llm_start_persistent_decode(M40llmCudaContext*);
 int m40llm_stop_persistent_decode(M40llmCudaContext*);
 int m40llm_persistent_decode_submit_vec(M40llmCudaContext*, const void*, void*, uint32_t, float, float,

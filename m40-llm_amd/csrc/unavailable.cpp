@@ -52,16 +52,6 @@ int m40llm_attention_last_token_f32_gqa_compressed_recent_only_async(M40llmCudaC
                                                                      const void*, uint32_t, uint32_t, void*) {
     return M40_UNAVAILABLE;
 }
-int m40llm_attention_prefill_f32_gqa_varlen(M40llmCudaContext*, const void*, const void*, const void*, const uint32_t*,
-                                            const uint32_t*, const uint32_t*, const uint32_t*, uint32_t, uint32_t,
-                                            uint32_t, uint32_t, void*) {
-    return M40_UNAVAILABLE;
-}
-int m40llm_attention_prefill_f32_gqa_varlen_async(M40llmCudaContext*, const void*, const void*, const void*,
-                                                  const uint32_t*, const uint32_t*, const uint32_t*, const uint32_t*,
-                                                  uint32_t, uint32_t, uint32_t, uint32_t, void*) {
-    return M40_UNAVAILABLE;
-}
 int m40llm_start_persistent_decode(M40llmCudaContext*) { return M40_UNAVAILABLE; }
 int m40llm_stop_persistent_decode(M40llmCudaContext*) { return M40_UNAVAILABLE; }
 int m40llm_persistent_decode_submit_vec(M40llmCudaContext*, const void*, void*, uint32_t, float, float, uint32_t,

@@ -1,6 +1,6 @@
 """Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
 
-    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8] [--json out.jsonl]
+    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill] [--json out.jsonl]
 
 Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
 events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
@@ -131,6 +131,45 @@ def bench_read_probe(b: Bench):
             x.free()
 
 
+PEAK_F32_MATRIX_TFLOPS = 157.3
+
+
+def bench_prefill(b: Bench):
+    """Packed variable-length causal prefill attention (all f32): arithmetic-bound, so the yardstick is the f32
+    matrix-instruction peak; flops = 4 * head_dim per visible (query, key) pair and q head."""
+    rng = np.random.default_rng(0)
+    cases = [("qh32 kvh4 hd64, one sequence of 512", 32, 4, 64, [512]), ("qh32 kvh4 hd64, one sequence of 4096", 32, 4, 64, [4096]),
+             ("qh16 kvh2 hd128, one sequence of 4096", 16, 2, 128, [4096]),
+             ("qh16 kvh2 hd128, 8 sequences U[256,4096]", 16, 2, 128, [int(x) for x in rng.integers(256, 4097, size=8)])]
+    for label, qh, kvh, hd, lens in cases:
+        n = sum(lens)
+        q = b.ctx.to_device(rng.standard_normal((n, qh, hd), dtype=np.float32))
+        k = b.ctx.to_device(rng.standard_normal((n, kvh, hd), dtype=np.float32))
+        v = b.ctx.to_device(rng.standard_normal((n, kvh, hd), dtype=np.float32))
+        out = b.ctx.alloc(n * qh * hd * 4)
+        lens_np = np.asarray(lens, dtype=np.uint32)
+        offs = np.concatenate([[0], np.cumsum(lens_np)[:-1]]).astype(np.uint32)
+        dl, do = b.ctx.to_device(lens_np), b.ctx.to_device(offs)
+        pairs = sum(L * (L + 1) // 2 for L in lens)
+        flops = 4.0 * hd * pairs * qh
+        reps, warm = 6, 2
+        for i in range(warm + reps):
+            if i == warm:
+                b.ctx.sync(0)
+                b.ctx.record(b.e0, 0)
+            b.call("m40llm_attention_prefill_f32_gqa_varlen_async", q.ptr, k.ptr, v.ptr, do.ptr, do.ptr, dl.ptr, dl.ptr, len(lens), qh, kvh,
+                   hd, out.ptr)
+        b.ctx.record(b.e1, 0)
+        us = b.ctx.elapsed_ms(b.e0, b.e1) * 1e3 / reps
+        tf = flops / us / 1e6
+        b.rows.append(dict(kernel="attention_prefill_gqa_varlen", shape=label, us_per_launch=round(us, 2), flops=flops,
+                           tflops=round(tf, 2), frac_f32_matrix_peak=round(tf / PEAK_F32_MATRIX_TFLOPS, 4), launches=reps))
+        print(f"{'attention_prefill_gqa_varlen':34s} {label:44s} {us:9.1f} us {tf:8.1f} TFLOP/s  frac {tf / PEAK_F32_MATRIX_TFLOPS:6.3f} of the f32 matrix peak",
+              flush=True)
+        for x in (q, k, v, out, dl, do):
+            x.free()
+
+
 def bench_gemv(b: Bench, M: int):
     rng = np.random.default_rng(1)
     shapes = [(2048, 2048), (256, 2048), (5632, 2048), (2048, 5632), (32000, 2048)] if M == 1 else \
@@ -256,7 +295,7 @@ def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8")
+    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
@@ -277,6 +316,8 @@ def main():
         bench_block_select(b)
     if "decode8" in which:
         bench_decode_batch(b, mode=args.decode_mode)
+    if "prefill" in which:
+        bench_prefill(b)
     if args.json:
         with open(args.json, "w") as f:
             for r in b.rows:

@@ -419,6 +419,62 @@ void orc_attention_last_token_gqa_batched(const uint16_t* K, const uint16_t* V,
 }
 
 /* ------------------------------------------------------------------------ */
+/* Packed variable-length causal prefill attention, all f32.                   */
+/* Reference: cuda/kernels.cu:3749-3835 (kernel: query q_idx of sequence b      */
+/* attends keys 0 .. kv_len - q_len + q_idx; three passes; p = exp / denom      */
+/* before the weighted sum), argument checks and their codes :4834-4895, CPU    */
+/* restatement tests/attention_prefill_varlen.rs:27-76.  Q and Out are          */
+/* [total_q][q_heads][hd], K and V [total_kv][kv_heads][hd]; offsets in tokens. */
+/* ------------------------------------------------------------------------ */
+int orc_attention_prefill_gqa_varlen(const float* q, const float* k, const float* v,
+                                     const uint32_t* q_offsets, const uint32_t* kv_offsets,
+                                     const uint32_t* q_lens, const uint32_t* kv_lens, uint32_t batch,
+                                     uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float* out) {
+    if (!q || !k || !v || !q_offsets || !kv_offsets || !q_lens || !kv_lens || !out) return -1;
+    if (batch == 0) return -2;
+    if (q_heads == 0 || kv_heads == 0 || q_heads % kv_heads != 0) return -3;
+    if (head_dim != 64 && head_dim != 128) return -9;
+    for (uint32_t b = 0; b < batch; ++b)
+        if (q_lens[b] == 0 || kv_lens[b] == 0 || q_lens[b] > kv_lens[b] || kv_lens[b] > 8192) return -8;
+    const uint32_t group = q_heads / kv_heads;
+    const float inv_sqrt = orc_inv_sqrt_head_dim(head_dim);
+#pragma omp parallel for schedule(dynamic) if (batch > 1)
+    for (uint32_t b = 0; b < batch; ++b) {
+        float* scores = (float*)malloc(sizeof(float) * kv_lens[b]);
+        for (uint32_t qi = 0; qi < q_lens[b]; ++qi) {
+            const uint32_t causal_end = kv_lens[b] - q_lens[b] + qi;
+            for (uint32_t h = 0; h < q_heads; ++h) {
+                const uint32_t kvh = h / group;
+                const float* qh = q + ((size_t)(q_offsets[b] + qi) * q_heads + h) * head_dim;
+                float max_score = -1e30f;
+                for (uint32_t t = 0; t <= causal_end; ++t) {
+                    const float* kh = k + ((size_t)(kv_offsets[b] + t) * kv_heads + kvh) * head_dim;
+                    float dot = 0.0f;
+                    for (uint32_t d = 0; d < head_dim; ++d) dot += qh[d] * kh[d];
+                    const float s = dot * inv_sqrt;
+                    scores[t] = s;
+                    if (s > max_score) max_score = s;
+                }
+                float denom = 0.0f;
+                for (uint32_t t = 0; t <= causal_end; ++t) denom += expf(scores[t] - max_score);
+                if (!(denom > 0.0f)) denom = 1.0f;
+                float* oh = out + ((size_t)(q_offsets[b] + qi) * q_heads + h) * head_dim;
+                for (uint32_t d = 0; d < head_dim; ++d) {
+                    float acc = 0.0f;
+                    for (uint32_t t = 0; t <= causal_end; ++t) {
+                        const float* vh = v + ((size_t)(kv_offsets[b] + t) * kv_heads + kvh) * head_dim;
+                        acc += (expf(scores[t] - max_score) / denom) * vh[d];
+                    }
+                    oh[d] = acc;
+                }
+            }
+        }
+        free(scores);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
 /* fp16-K / q4-V compressed cache.                                           */
 /* Layout: cuda/kernels.cu:5357-5385, :5435-5543; append/evict :6108-6250     */
 /* with kernels :2230-2311, ring write :5786-5790.                            */

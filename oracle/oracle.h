@@ -74,6 +74,12 @@ void orc_attention_last_token_gqa_batched(const uint16_t* K, const uint16_t* V,
                                           uint32_t head_dim, const uint32_t* seq_ids,
                                           const uint32_t* seq_lens, uint32_t batch,
                                           const float* q, uint32_t q_heads, float* out);
+/* packed variable-length causal prefill attention, all f32 (cuda/kernels.cu:3749-3835, :4834-4895); returns the
+ * reference's argument-check codes (-1, -2, -3, -9, -8) or 0 */
+int orc_attention_prefill_gqa_varlen(const float* q, const float* k, const float* v,
+                                     const uint32_t* q_offsets, const uint32_t* kv_offsets,
+                                     const uint32_t* q_lens, const uint32_t* kv_lens, uint32_t batch,
+                                     uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, float* out);
 float orc_inv_sqrt_head_dim(uint32_t head_dim);
 
 /* ---- fp16-K / q4-V compressed cache --------------------------------------- */

@@ -96,6 +96,7 @@ def lib() -> C.CDLL:
     sig("orc_kv_append_f32_rope_k", None, vp, vp, u32, u32, u32, u32, u32, vp, vp, f32, f32, u32)
     sig("orc_attention_last_token_gqa", None, vp, vp, u32, u32, u32, u32, vp, u32, u32, vp)
     sig("orc_attention_last_token_gqa_batched", None, vp, vp, u32, u32, u32, vp, vp, u32, vp, u32, vp)
+    sig("orc_attention_prefill_gqa_varlen", C.c_int, vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, vp)
     sig("orc_inv_sqrt_head_dim", f32, u32)
     sig("orc_ckv_create", C.POINTER(OrcCkv), u32, u32, u32, u32, u32, u32)
     sig("orc_ckv_destroy", None, C.POINTER(OrcCkv))
@@ -222,6 +223,24 @@ def attention(K, V, max_seq_len, kv_heads, head_dim, seq, q, q_heads, seq_len):
     lib().orc_attention_last_token_gqa(ptr(K), ptr(V), max_seq_len, kv_heads, head_dim, seq,
                                        ptr(q), q_heads, seq_len, ptr(out))
     return out
+
+
+def prefill_offsets(lens):
+    """exclusive prefix of token counts (u32), as the reference's batch metadata builds it (src/infer/batch.rs:276-355)"""
+    lens = np.asarray(lens, dtype=np.uint32)
+    return np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.uint32)
+
+
+def attention_prefill(q, k, v, q_lens, kv_lens, q_heads, kv_heads, head_dim):
+    """q [total_q, q_heads, hd], k/v [total_kv, kv_heads, hd], all f32 -> (rc, out like q)"""
+    q = np.ascontiguousarray(q, dtype=np.float32); k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    ql = np.ascontiguousarray(q_lens, dtype=np.uint32); kl = np.ascontiguousarray(kv_lens, dtype=np.uint32)
+    qo, ko = prefill_offsets(ql), prefill_offsets(kl)
+    out = np.zeros_like(q)
+    rc = lib().orc_attention_prefill_gqa_varlen(ptr(q), ptr(k), ptr(v), ptr(qo), ptr(ko), ptr(ql), ptr(kl), len(ql),
+                                                q_heads, kv_heads, head_dim, ptr(out))
+    return rc, out
 
 
 def attention_batched(K, V, max_seq_len, kv_heads, head_dim, seq_ids, seq_lens, q, q_heads):

@@ -503,3 +503,71 @@ def test_read_probe_xor(dev):
     assert dev.lib.m40llm_ext_read_probe_async(dev.h, dx.ptr, 8, 1, out.ptr) == -2
     assert dev.lib.m40llm_ext_read_probe_async(dev.h, dx.ptr, 64, 0, out.ptr) == -2
     assert dev.lib.m40llm_ext_read_probe_async(dev.h, None, 64, 1, out.ptr) == -1
+
+
+# ------------------------------------------------------------------ packed varlen prefill attention
+def _prefill_call(dev, orc, q, k, v, ql, kl, qh, kvh, hd, sync_form=True, expect=0):
+    dq, dk, dv = dev.up(q), dev.up(k), dev.up(v)
+    dqo, dko = dev.up(orc.prefill_offsets(ql)), dev.up(orc.prefill_offsets(kl))
+    dql, dkl = dev.up(np.asarray(ql, dtype=np.uint32)), dev.up(np.asarray(kl, dtype=np.uint32))
+    out = dev.zeros(q.nbytes)
+    name = "m40llm_attention_prefill_f32_gqa_varlen" if sync_form else "m40llm_attention_prefill_f32_gqa_varlen_async"
+    dev.call(name, dq.ptr, dk.ptr, dv.ptr, dqo.ptr, dko.ptr, dql.ptr, dkl.ptr, len(ql), qh, kvh, hd, out.ptr, expect=expect)
+    if not sync_form:
+        dev.ctx.sync(0)
+    return out.download(np.float32, q.shape)
+
+
+def _modular(n, mul, mod, scale, offset):
+    i = np.arange(n, dtype=np.int64)
+    return ((i * mul % mod).astype(np.float32) * np.float32(scale) + np.float32(offset)).astype(np.float32)
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+def test_prefill_varlen_reference_fixture(dev, orc, hd):
+    # tests/attention_prefill_varlen.rs:93-131: (q 3, kv 3), (q 2, kv 5), (q 1, kv 4); 4 q heads, 2 kv heads
+    ql, kl, qh, kvh = [3, 2, 1], [3, 5, 4], 4, 2
+    q = _modular(sum(ql) * qh * hd, 17, 251, 0.0011, -0.13).reshape(sum(ql), qh, hd)
+    k = _modular(sum(kl) * kvh * hd, 23, 263, 0.0009, -0.09).reshape(sum(kl), kvh, hd)
+    v = _modular(sum(kl) * kvh * hd, 29, 269, 0.0013, -0.17).reshape(sum(kl), kvh, hd)
+    rc, want = orc.attention_prefill(q, k, v, ql, kl, qh, kvh, hd)
+    assert rc == 0
+    for sync_form in (True, False):
+        close(_prefill_call(dev, orc, q, k, v, ql, kl, qh, kvh, hd, sync_form), want)
+
+
+@pytest.mark.parametrize("qh,kvh,hd,ql,kl", [
+    (4, 2, 64, [1], [1]),                                   # one token
+    (6, 2, 64, [4, 1, 7], [4, 9, 10]),                      # full prefill, one-token decode, chunked prefill
+    (8, 2, 128, [70, 33, 64], [70, 97, 64]),                # query tiles with tails, key tiles with tails
+    (32, 4, 64, [300, 17], [300, 529]),                     # config-1 heads, several query tiles
+    (3, 3, 128, [129], [1000]),                             # 871 cached keys ahead of the queries
+    (16, 2, 128, [5, 5, 5, 5, 5], [8192, 5, 37, 64, 65]),   # the longest allowed key range
+])
+def test_prefill_varlen_random_vs_oracle(dev, orc, qh, kvh, hd, ql, kl):
+    rng = np.random.default_rng(len(ql) + hd)
+    q = rng.standard_normal((sum(ql), qh, hd)).astype(np.float32)
+    k = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+    v = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+    rc, want = orc.attention_prefill(q, k, v, ql, kl, qh, kvh, hd)
+    assert rc == 0
+    got = _prefill_call(dev, orc, q, k, v, ql, kl, qh, kvh, hd, sync_form=False)
+    close(got, want)
+    # the first query of a full prefill sees one key: that V row, exactly
+    if ql[0] == kl[0]:
+        assert np.array_equal(got[0], np.repeat(v[0], qh // kvh, axis=0))
+
+
+def test_prefill_varlen_argument_checks(dev, orc):
+    rng = np.random.default_rng(0)
+    qh, kvh, hd, ql, kl = 4, 2, 64, [2, 3], [2, 5]
+    q = rng.standard_normal((5, qh, hd)).astype(np.float32)
+    k = rng.standard_normal((7, kvh, hd)).astype(np.float32)
+    _prefill_call(dev, orc, q, k, k, ql, kl, qh, kvh, 32, expect=-9)
+    _prefill_call(dev, orc, q, k, k, ql, kl, 5, 2, hd, expect=-3)
+    _prefill_call(dev, orc, q, k, k, [2, 6], kl, qh, kvh, hd, expect=-8)       # more queries than keys
+    _prefill_call(dev, orc, q, k, k, [2, 0], kl, qh, kvh, hd, expect=-8)
+    _prefill_call(dev, orc, q, k, k, ql, [2, 8193], qh, kvh, hd, expect=-8)
+    dq = dev.up(q)
+    assert dev.lib.m40llm_attention_prefill_f32_gqa_varlen(dev.h, dq.ptr, dq.ptr, dq.ptr, dq.ptr, dq.ptr, dq.ptr, dq.ptr, 0, qh, kvh, hd, dq.ptr) == -2
+    assert dev.lib.m40llm_attention_prefill_f32_gqa_varlen(dev.h, None, dq.ptr, dq.ptr, dq.ptr, dq.ptr, dq.ptr, dq.ptr, 1, qh, kvh, hd, dq.ptr) == -1

@@ -53,7 +53,7 @@ def test_unavailable_symbols_report_minus_one_without_a_device():
     lib = m40.native()
     assert lib.m40llm_start_persistent_decode(None) == -1
     assert lib.m40llm_gemm_f32xf32_f32_async(None, None, None, None, 1, 1, 1) == -1
-    assert lib.m40llm_attention_prefill_f32_gqa_varlen(None, None, None, None, None, None, None, None, 1, 1, 1, 64, None) == -1
+    assert lib.m40llm_attention_prefill_f32_gqa_varlen(None, None, None, None, None, None, None, None, 1, 1, 1, 64, None) == -1   # null arguments
     # argument checks that run before any device work
     assert lib.m40llm_device_malloc(None, 16, None) == -1
     assert lib.m40llm_gemm_f32xf16_gguf_f32(None, None, None, None, 1, 1, 1) == -1

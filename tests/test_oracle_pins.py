@@ -580,3 +580,66 @@ def test_layer_single_token_context_is_v(orc):
     g = xn @ f(W["wgate"][0]).T; u = xn @ f(W["wup"][0]).T
     want = x1 + (g / (1 + np.exp(-g)) * u) @ f(W["wdown"][0]).T
     assert np.allclose(out, want, rtol=2e-3, atol=2e-3)
+
+
+# ---------------------------------------------------------------- packed varlen prefill attention
+def _f64_prefill(q, k, v, q_lens, kv_lens, qh, kvh, hd):
+    out = np.zeros(q.shape, dtype=np.float64)
+    qo = np.concatenate([[0], np.cumsum(q_lens)[:-1]]); ko = np.concatenate([[0], np.cumsum(kv_lens)[:-1]])
+    g = qh // kvh
+    for b in range(len(q_lens)):
+        for qi in range(q_lens[b]):
+            end = kv_lens[b] - q_lens[b] + qi
+            for h in range(qh):
+                kk = k[ko[b]:ko[b] + end + 1, h // g].astype(np.float64)
+                vv = v[ko[b]:ko[b] + end + 1, h // g].astype(np.float64)
+                s = kk @ q[qo[b] + qi, h].astype(np.float64) / np.sqrt(hd)
+                p = np.exp(s - s.max()); p /= p.sum()
+                out[qo[b] + qi, h] = p @ vv
+    return out
+
+
+def _modular_fixture(n, spec):
+    i = np.arange(n, dtype=np.int64)
+    return ((i * spec["mul"] % spec["mod"]).astype(np.float32) * np.float32(spec["scale"]) + np.float32(spec["offset"])).astype(np.float32)
+
+
+def test_prefill_varlen_reference_fixture_vs_float64(orc):
+    import json, os
+    g = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_literals.json")))["attention_prefill_varlen"]
+    ql = [s["query_len"] for s in g["sequences"]]; kl = [s["kv_len"] for s in g["sequences"]]
+    qh, kvh = g["q_heads"], g["kv_heads"]
+    for hd in g["head_dims"]:
+        q = _modular_fixture(sum(ql) * qh * hd, g["q"]).reshape(sum(ql), qh, hd)
+        k = _modular_fixture(sum(kl) * kvh * hd, g["k"]).reshape(sum(kl), kvh, hd)
+        v = _modular_fixture(sum(kl) * kvh * hd, g["v"]).reshape(sum(kl), kvh, hd)
+        rc, got = orc.attention_prefill(q, k, v, ql, kl, qh, kvh, hd)
+        assert rc == 0
+        assert np.allclose(got, _f64_prefill(q, k, v, ql, kl, qh, kvh, hd), rtol=1e-5, atol=1e-6)
+
+
+def test_prefill_varlen_invariants_and_codes(orc):
+    rng = np.random.default_rng(5)
+    qh, kvh, hd = 6, 2, 64
+    ql, kl = [4, 1, 7], [4, 9, 10]          # full prefill, one-token decode, chunked prefill (3 cached tokens)
+    q = rng.standard_normal((sum(ql), qh, hd)).astype(np.float32)
+    k = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float16).astype(np.float32)
+    rc, got = orc.attention_prefill(q, k, v, ql, kl, qh, kvh, hd)
+    assert rc == 0
+    assert np.allclose(got, _f64_prefill(q, k, v, ql, kl, qh, kvh, hd), rtol=1e-5, atol=1e-6)
+    # the first query of a full prefill sees one key: its output is that V row, exactly
+    assert np.array_equal(got[0], np.repeat(v[0], qh // kvh, axis=0))
+    # a one-token sequence is last-token attention over its keys (the decode oracle on the same f16-exact values)
+    K16 = np.ascontiguousarray(k[4:13].astype(np.float16).view(np.uint16)[None]); V16 = np.ascontiguousarray(v[4:13].astype(np.float16).view(np.uint16)[None])
+    want = orc.attention(K16, V16, 9, kvh, hd, 0, q[4].reshape(-1), qh, 9)
+    assert np.allclose(got[4].reshape(-1), want, rtol=1e-6, atol=1e-7)
+    # the batch is the sequences one by one
+    rc1, solo = orc.attention_prefill(q[5:], k[13:], v[13:], [7], [10], qh, kvh, hd)
+    assert rc1 == 0 and np.array_equal(solo, got[5:])
+    # argument checks of cuda/kernels.cu:4849-4887
+    assert orc.attention_prefill(q, k, v, ql, kl, qh, kvh, 32)[0] == -9
+    assert orc.attention_prefill(q, k, v, ql, kl, 5, 2, hd)[0] == -3
+    assert orc.attention_prefill(q, k, v, [4, 1, 11], kl, qh, kvh, hd)[0] == -8      # query longer than its keys
+    assert orc.attention_prefill(q, k, v, [4, 0, 7], kl, qh, kvh, hd)[0] == -8
+    assert orc.attention_prefill(q, k, v, [4, 1, 7], [4, 9, 8193], qh, kvh, hd)[0] == -8
