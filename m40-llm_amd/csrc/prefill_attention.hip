@@ -139,22 +139,28 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             s0 = mfma16x16x4(qa[s], k_lds[j * KSTR + 4 * s + g], s0);
             s1 = mfma16x16x4(qa[s], k_lds[(16 + j) * KSTR + 4 * s + g], s1);
         }
-        float p0[4], p1[4];
+        float p0[4], p1[4], f[4];
+        bool moved = false;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const bool a0 = key0 + (uint32_t)j <= row_end[r], a1 = key0 + 16u + (uint32_t)j <= row_end[r];
             const float x0 = a0 ? s0[r] * inv_sqrt : -INFINITY, x1 = a1 ? s1[r] * inv_sqrt : -INFINITY;
             const float n = fmaxf(m_run[r], row_max16(fmaxf(x0, x1)));
             // no maximum yet: the old state weighs nothing; a masked key weighs nothing
-            const float f = m_run[r] == -INFINITY ? 0.0f : expf(m_run[r] - n);
-            p0[r] = a0 ? expf(x0 - n) : 0.0f;
-            p1[r] = a1 ? expf(x1 - n) : 0.0f;
-            l_run[r] = fmaf(l_run[r], f, p0[r] + p1[r]);
+            f[r] = m_run[r] == -INFINITY ? 0.0f : __expf(m_run[r] - n);
+            p0[r] = a0 ? __expf(x0 - n) : 0.0f;
+            p1[r] = a1 ? __expf(x1 - n) : 0.0f;
+            l_run[r] = fmaf(l_run[r], f[r], p0[r] + p1[r]);
+            moved = moved || m_run[r] != n;
             m_run[r] = n;
-#pragma unroll
-            for (int d = 0; d < DT; ++d) O[d][r] *= f;
             my_p[(4 * g + r) * PSTR + j] = p0[r];
             my_p[(4 * g + r) * PSTR + 16 + j] = p1[r];
+        }
+        if (__any(moved)) {               // the accumulators are only rescaled when some row's maximum rose
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) O[d][r] *= f[r];
         }
         __builtin_amdgcn_wave_barrier();
         // O += P . V: A = P[query j][key 4 s + g], B = V[key 4 s + g][column 16 d + j]
