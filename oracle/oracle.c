@@ -12,6 +12,7 @@
  *   f16 conversion ........ numpy float16 (independent RNE), all 65536 codes
  *   KV layout ............. reference literal index(1,2,2,4)=104
  *   attention ............. float64 softmax, L=1 / equal-K invariants, closed-form fixtures
+ *   prefill attention ..... float64 softmax on the reference's fixture; one-key, one-token and per-sequence invariants
  *   q4 V .................. brute-force quantiser, byte-accounting literals 8192/2048/128
  *   block selection ....... brute-force sort on tiny inputs, "all blocks selected == dense"
  *   GEMM .................. reference known answers [19,22;43,50], [40,46]; float64 matmul
