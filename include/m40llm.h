@@ -337,6 +337,13 @@ int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32
  * decode stream; the benchmarks time it beside the kernels it bounds. */
 int m40llm_ext_read_probe_async(M40llmCudaContext* ctx, const void* d_src, size_t bytes, uint32_t workgroups,
                                 uint32_t* d_out_u32);
+/* Weight-file ingestion: `num_bytes` of the file at `path`, from byte `file_offset`, into one new device allocation
+ * (*out_device_ptr, released with m40llm_device_free).  Replaces read-the-file + m40llm_upload_weights
+ * (src/infer/load.rs:27-40, kernels.cu:1264-1290): positional reads into two pinned staging buffers overlap the
+ * copies to the device, and nothing the size of the file is held in host memory.  Blocks until the data is resident.
+ * -1 null argument, -2 device / allocation, -3 copy, -6 the file cannot be opened or the range is not inside it. */
+int m40llm_ext_upload_file_range(M40llmCudaContext* ctx, const char* path, uint64_t file_offset, uint64_t num_bytes,
+                                 void** out_device_ptr);
 /* Fused batch-1 decode-step entry points (decode stream, asynchronous).  They compute exactly what the
  * reference's per-op call sequence computes (src/infer/forward.rs:304-662), several steps per launch:
  *   steps 1-5: RMSNorm -> Q/K/V projections (+bias) -> RoPE(Q) -> d_q_out; RoPE(K) and V -> f16 append at the

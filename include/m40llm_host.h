@@ -155,6 +155,41 @@ int m40host_model_decode_batch_greedy(M40HostModel* model, const uint32_t* seque
                                       const uint32_t* first_tokens, uint32_t rows, uint32_t steps, uint32_t* ids_out,
                                       float* gaps_out);
 
+/* ---- GGUF ingestion (src/gguf.rs:172-329, src/infer/load.rs:10-92, src/infer/tensor_views.rs:29-117,
+ *      src/infer/types.rs:114-242, src/infer/mapping.rs:95-540, src/infer/embeddings.rs:14-143) -------------- */
+typedef struct M40HostGguf M40HostGguf;                 /* a parsed file header: no device, no tensor data */
+typedef struct M40HostGgufWeights M40HostGgufWeights;   /* a file whose data section is resident on the device */
+/* Parse magic, version, metadata and tensor descriptors (load_gguf).  NULL + m40host_last_error() when the file is
+ * not GGUF, is truncated, or holds an unknown value type.  _parse does the same for a header held in memory. */
+M40HostGguf* m40host_gguf_open(const char* path);
+M40HostGguf* m40host_gguf_parse(const void* bytes, size_t n);
+void m40host_gguf_close(M40HostGguf* gguf);
+/* Everything the host layer derives from the header, as one JSON object: version, data_offset, file_len, metadata
+ * (arrays cut to their first 32 elements, with "len"), tensors, then "config" (ModelConfig::from_metadata), "views"
+ * (byte_offset, nbytes, strides per tensor), "layers" (per layer, the tensor chosen for each role of map_standard_layer,
+ * or {"error": message}), "lm_head" (map_lm_head: name, d_model, vocab, tied) and "output_norm"; a stage that the reference
+ * would reject appears as "<stage>_error" with the reference's message instead.  Returns the size needed including
+ * the terminating zero; writes at most `capacity` bytes. */
+size_t m40host_gguf_describe_json(const M40HostGguf* gguf, char* buf, size_t capacity);
+/* Where one token's embedding starts in the data section, its length and the table's ggml dtype code
+ * (embeddings.rs:33-60).  -1 + last_error for a token outside the vocabulary or an unsupported dtype. */
+int m40host_gguf_embedding_row(const M40HostGguf* gguf, uint64_t token_id, uint64_t* byte_offset, uint64_t* row_bytes,
+                               uint32_t* dtype_raw);
+/* LoadedModel::from_gguf: parse, validate every tensor against the data section, then stream the data section into
+ * one device allocation (m40llm_ext_upload_file_range).  Nothing is allocated when validation fails. */
+M40HostGgufWeights* m40host_gguf_load(M40llmCudaContext* ctx, const char* path);
+void m40host_gguf_weights_free(M40HostGgufWeights* weights);     /* after every model made from it is destroyed */
+uint64_t m40host_gguf_weights_len(const M40HostGgufWeights* weights);
+const void* m40host_gguf_weights_base(const M40HostGgufWeights* weights);
+/* device address of a tensor = base + its offset in the data section; NULL + last_error for an unknown name */
+const void* m40host_gguf_tensor_ptr(const M40HostGgufWeights* weights, const char* name);
+/* load_token_embedding_to_f32: F16 rows widened, Q8_0 rows dequantised (d * q), both on the device */
+int m40host_gguf_load_token_embedding_f32(const M40HostGgufWeights* weights, uint64_t token_id, void* d_out_f32);
+/* A decoder that reads the file's tensors in place (validate_full_layer_decode, then the model of
+ * m40host_model_create).  max_seq_len 0 = the file's context_length; kv_cfg NULL = dense cache. */
+M40HostModel* m40host_model_from_gguf(M40HostGgufWeights* weights, uint32_t max_seq_len, uint32_t max_sequences,
+                                      const M40HostKvConfig* kv_cfg);
+
 #ifdef __cplusplus
 }
 #endif

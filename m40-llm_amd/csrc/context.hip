@@ -2,10 +2,17 @@
 // Reference behaviour: cuda/kernels.cu:276-680, 1245-1292.
 #include "common.hpp"
 
+#include <fcntl.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <cerrno>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <new>
+#include <thread>
 
 namespace {
 
@@ -229,6 +236,95 @@ int m40llm_upload_weights(M40llmCudaContext* ctx, const void* host_ptr, size_t n
     if (hipMemcpy(d_ptr, host_ptr, num_bytes, hipMemcpyHostToDevice) != hipSuccess) {
         (void)hipFree(d_ptr);
         return -3;
+    }
+    *out_device_ptr = d_ptr;
+    return 0;
+}
+
+// A byte range of a file into one new device allocation.  The range is read with positional reads into two
+// pinned staging buffers by a few threads while the previous buffer's copy to the device is still in flight, so
+// disk (or page cache) and the host-to-device link overlap; nothing the size of the file is ever held in host
+// memory.  Replaces the reference's read-whole-file + upload_weights sequence (src/infer/load.rs:27-40,
+// kernels.cu:1264-1290) for weight files.
+int m40llm_ext_upload_file_range(M40llmCudaContext* ctx, const char* path, uint64_t file_offset, uint64_t num_bytes,
+                                 void** out_device_ptr) {
+    if (!ctx || !path || !out_device_ptr) return -1;
+    if (m40_ensure_device(ctx) != 0) return -2;
+    const int fd = ::open(path, O_RDONLY | O_CLOEXEC);
+    if (fd < 0) return -6;
+    struct stat st {};
+    if (::fstat(fd, &st) != 0 || st.st_size < 0 || file_offset > static_cast<uint64_t>(st.st_size) ||
+        num_bytes > static_cast<uint64_t>(st.st_size) - file_offset) {
+        ::close(fd);
+        return -6;
+    }
+    constexpr uint64_t kStage = 64ull << 20;
+    constexpr int kReaders = 4;
+    void* d_ptr = nullptr;
+    void* stage[2] = {nullptr, nullptr};
+    hipEvent_t done[2] = {nullptr, nullptr};
+    int rc = 0;
+    if (hipMalloc(&d_ptr, num_bytes ? num_bytes : 4) != hipSuccess) {
+        (void)hipGetLastError();
+        ::close(fd);
+        return -2;
+    }
+    const uint64_t stage_bytes = num_bytes < kStage ? (num_bytes ? num_bytes : 4) : kStage;
+    for (int i = 0; i < 2 && rc == 0; ++i) {
+        if (hipHostMalloc(&stage[i], stage_bytes, hipHostMallocDefault) != hipSuccess ||
+            hipEventCreateWithFlags(&done[i], hipEventDisableTiming) != hipSuccess)
+            rc = -2;
+    }
+    hipStream_t stream = ctx->prefill_stream;
+    bool used[2] = {false, false};
+    int which = 0;
+    for (uint64_t at = 0; at < num_bytes && rc == 0; at += stage_bytes, which ^= 1) {
+        const uint64_t n = num_bytes - at < stage_bytes ? num_bytes - at : stage_bytes;
+        if (used[which] && hipEventSynchronize(done[which]) != hipSuccess) {
+            rc = -3;
+            break;
+        }
+        std::atomic<bool> short_read{false};
+        auto read_part = [&](int part) {
+            const uint64_t per = (n + kReaders - 1) / kReaders;
+            uint64_t lo = per * part, hi = lo + per < n ? lo + per : n;
+            while (lo < hi) {
+                const ssize_t got = ::pread(fd, static_cast<char*>(stage[which]) + lo, hi - lo, static_cast<off_t>(file_offset + at + lo));
+                if (got <= 0) {
+                    if (got < 0 && errno == EINTR) continue;
+                    short_read = true;
+                    return;
+                }
+                lo += static_cast<uint64_t>(got);
+            }
+        };
+        {
+            std::thread readers[kReaders - 1];
+            for (int t = 1; t < kReaders; ++t) readers[t - 1] = std::thread(read_part, t);
+            read_part(0);
+            for (auto& t : readers) t.join();
+        }
+        if (short_read) {
+            rc = -6;
+            break;
+        }
+        if (hipMemcpyAsync(static_cast<char*>(d_ptr) + at, stage[which], n, hipMemcpyHostToDevice, stream) != hipSuccess ||
+            hipEventRecord(done[which], stream) != hipSuccess) {
+            rc = -3;
+            break;
+        }
+        used[which] = true;
+    }
+    if (hipStreamSynchronize(stream) != hipSuccess && rc == 0) rc = -3;
+    for (int i = 0; i < 2; ++i) {
+        if (done[i]) (void)hipEventDestroy(done[i]);
+        if (stage[i]) (void)hipHostFree(stage[i]);
+    }
+    ::close(fd);
+    if (rc != 0) {
+        (void)hipFree(d_ptr);
+        (void)hipGetLastError();
+        return rc;
     }
     *out_device_ptr = d_ptr;
     return 0;

@@ -8,6 +8,7 @@
 
 #include "decode.hpp"
 #include "decode_batch.hpp"
+#include "gguf_loader.hpp"
 #include "kv_compression.hpp"
 #include "kv_selection.hpp"
 #include "model.hpp"
@@ -74,6 +75,13 @@ struct PlanHolder {
 
 struct M40HostModel {
     std::unique_ptr<DecodeModel> m;
+};
+struct M40HostGguf {
+    gguf::Model model;
+    std::string json;
+};
+struct M40HostGgufWeights {
+    std::unique_ptr<GgufWeights> w;
 };
 
 extern "C" {
@@ -375,6 +383,102 @@ int m40host_model_decode_batch_greedy(M40HostModel* m, const uint32_t* seq_ids, 
                                       float* gaps_out) {
     return guarded(
         [&]() -> int { m->m->decode_batch_greedy(seq_ids, kv_lens, first_tokens, rows, steps, ids_out, gaps_out); return 0; }, -100);
+}
+
+// ---- GGUF ingestion ------------------------------------------------------------------------------------
+M40HostGguf* m40host_gguf_open(const char* path) {
+    return guarded(
+        [&]() -> M40HostGguf* {
+            if (!path) throw std::invalid_argument("null path");
+            gguf::MappedFile file(path);
+            auto g = std::make_unique<M40HostGguf>();
+            g->model = gguf::parse(file.data(), file.size());
+            g->json = gguf::describe_json(g->model);
+            return g.release();
+        },
+        nullptr);
+}
+M40HostGguf* m40host_gguf_parse(const void* bytes, size_t n) {
+    return guarded(
+        [&]() -> M40HostGguf* {
+            if (!bytes && n) throw std::invalid_argument("null bytes");
+            auto g = std::make_unique<M40HostGguf>();
+            g->model = gguf::parse(static_cast<const uint8_t*>(bytes), n);
+            g->json = gguf::describe_json(g->model);
+            return g.release();
+        },
+        nullptr);
+}
+void m40host_gguf_close(M40HostGguf* g) { delete g; }
+size_t m40host_gguf_describe_json(const M40HostGguf* g, char* buf, size_t capacity) {
+    if (!g) return 0;
+    if (buf && capacity) {
+        const size_t n = g->json.size() < capacity - 1 ? g->json.size() : capacity - 1;
+        std::memcpy(buf, g->json.data(), n);
+        buf[n] = 0;
+    }
+    return g->json.size() + 1;
+}
+int m40host_gguf_embedding_row(const M40HostGguf* g, uint64_t token_id, uint64_t* byte_offset, uint64_t* row_bytes,
+                               uint32_t* dtype_raw) {
+    return guarded(
+        [&]() -> int {
+            if (!g) throw std::invalid_argument("null handle");
+            const gguf::Config cfg = gguf::config_from_metadata(g->model.metadata, g->model.tensors);
+            if (g->model.data_offset > g->model.file_len) throw gguf::Error("GGUF data_offset beyond file size");
+            const gguf::Views views = gguf::build_views(g->model.tensors, g->model.file_len - g->model.data_offset);
+            const gguf::EmbeddingRow r = gguf::embedding_row(views, cfg, token_id);
+            if (byte_offset) *byte_offset = r.byte_offset;
+            if (row_bytes) *row_bytes = r.row_bytes;
+            if (dtype_raw) *dtype_raw = r.dtype;
+            return 0;
+        },
+        -1);
+}
+
+M40HostGgufWeights* m40host_gguf_load(M40llmCudaContext* ctx, const char* path) {
+    return guarded(
+        [&]() -> M40HostGgufWeights* {
+            if (!ctx || !path) throw std::invalid_argument("null argument");
+            auto h = std::make_unique<M40HostGgufWeights>();
+            h->w = std::make_unique<GgufWeights>(ctx, path);
+            return h.release();
+        },
+        nullptr);
+}
+void m40host_gguf_weights_free(M40HostGgufWeights* w) { delete w; }
+uint64_t m40host_gguf_weights_len(const M40HostGgufWeights* w) { return w ? w->w->weights_len() : 0; }
+const void* m40host_gguf_weights_base(const M40HostGgufWeights* w) { return w ? w->w->base() : nullptr; }
+const void* m40host_gguf_tensor_ptr(const M40HostGgufWeights* w, const char* name) {
+    return guarded(
+        [&]() -> const void* {
+            if (!w || !name) throw std::invalid_argument("null argument");
+            const void* p = w->w->tensor_ptr(name);
+            if (!p) throw gguf::Error(std::string("no tensor named '") + name + "'");
+            return p;
+        },
+        nullptr);
+}
+int m40host_gguf_load_token_embedding_f32(const M40HostGgufWeights* w, uint64_t token_id, void* d_out_f32) {
+    return guarded(
+        [&]() -> int {
+            if (!w) throw std::invalid_argument("null handle");
+            w->w->load_token_embedding_f32(token_id, d_out_f32);
+            return 0;
+        },
+        -1);
+}
+M40HostModel* m40host_model_from_gguf(M40HostGgufWeights* w, uint32_t max_seq_len, uint32_t max_sequences,
+                                      const M40HostKvConfig* kv_cfg) {
+    return guarded(
+        [&]() -> M40HostModel* {
+            if (!w) throw std::invalid_argument("null handle");
+            const KvCompressionConfig k = kv_cfg ? to_cpp(*kv_cfg) : KvCompressionConfig::dense_reference();
+            auto h = std::make_unique<M40HostModel>();
+            h->m = w->w->make_model(max_seq_len, max_sequences, k);
+            return h.release();
+        },
+        nullptr);
 }
 
 }  // extern "C"
