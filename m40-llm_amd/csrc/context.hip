@@ -258,8 +258,8 @@ int m40llm_ext_upload_file_range(M40llmCudaContext* ctx, const char* path, uint6
         ::close(fd);
         return -6;
     }
-    constexpr uint64_t kStage = 64ull << 20;
-    constexpr int kReaders = 4;
+    constexpr uint64_t kStage = 16ull << 20;
+    constexpr int kReaders = 8;
     void* d_ptr = nullptr;
     void* stage[2] = {nullptr, nullptr};
     hipEvent_t done[2] = {nullptr, nullptr};

@@ -129,3 +129,55 @@ class GgufWeights:
                    rope_scale=c["rope_freq_scale"], rope_layout=c["rope_layout"],
                    qkv_bias=self.info["layers"][0].get("bq") is not None)
         return GgufModel(self, h, cfg, max_seq_len or c["context_length"], max_sequences)
+
+
+def write_model_file(path: str, cfg: dict, W: dict, arch: str = "llama", alignment: int = 32) -> int:
+    """Stream a synthetic decoder (the weight dictionary of synthetic.make_weights) to `path` as a GGUF v3 file with
+    llama.cpp's tensor names (blk.N.*, token_embd, output_norm, output); shapes are written fastest dimension first
+    ([K, N] for a projection with N output columns).  Returns the file size.  Used by the load benchmark; nothing is
+    converted: the f16 arrays go to the file as they are."""
+    import struct
+
+    def s(x: str) -> bytes:
+        raw = x.encode()
+        return struct.pack("<Q", len(raw)) + raw
+
+    kvs = [s("general.architecture") + struct.pack("<I", 8) + s(arch)]
+    for key, val in (("block_count", cfg["n_layers"]), ("embedding_length", cfg["d_model"]), ("attention.head_count", cfg["q_heads"]),
+                     ("attention.head_count_kv", cfg["kv_heads"]), ("context_length", cfg.get("context_length", 2048)),
+                     ("feed_forward_length", cfg["ffn"]), ("vocab_size", cfg["vocab"])):
+        kvs.append(s(f"{arch}.{key}") + struct.pack("<II", 4, val))
+    for key, val in (("attention.layer_norm_rms_epsilon", cfg["rms_eps"]), ("rope.freq_base", cfg["rope_base"])):
+        kvs.append(s(f"{arch}.{key}") + struct.pack("<If", 6, val))
+    tensors = [("token_embd.weight", W["tok_emb"], 1)]
+    for l in range(cfg["n_layers"]):
+        tensors.append((f"blk.{l}.attn_norm.weight", W["attn_norm"][l], 0))
+        for role, name in (("wq", "attn_q"), ("wk", "attn_k"), ("wv", "attn_v")):
+            tensors.append((f"blk.{l}.{name}.weight", W[role][l], 1))
+        if cfg.get("qkv_bias"):
+            for role, name in (("bq", "attn_q"), ("bk", "attn_k"), ("bv", "attn_v")):
+                tensors.append((f"blk.{l}.{name}.bias", W[role][l], 0))
+        tensors.append((f"blk.{l}.attn_output.weight", W["wo"][l], 1))
+        tensors.append((f"blk.{l}.ffn_norm.weight", W["ffn_norm"][l], 0))
+        for role, name in (("wgate", "ffn_gate"), ("wup", "ffn_up"), ("wdown", "ffn_down")):
+            tensors.append((f"blk.{l}.{name}.weight", W[role][l], 1))
+    tensors.append(("output_norm.weight", W["out_norm"], 0))
+    if W["lm_head"] is not W["tok_emb"]:
+        tensors.append(("output.weight", W["lm_head"], 1))
+    head = b"GGUF" + struct.pack("<IQQ", 3, len(tensors), len(kvs)) + b"".join(kvs)
+    offsets, at = [], 0
+    for name, a, dt in tensors:
+        at += -at % alignment
+        offsets.append(at)
+        at += a.nbytes
+        shape = list(a.shape)[::-1]
+        head += s(name) + struct.pack("<I", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape) + struct.pack("<IQ", dt, offsets[-1])
+    with open(path, "wb") as f:
+        f.write(head)
+        f.write(b"\0" * (-len(head) % alignment))
+        pos = 0
+        for (name, a, dt), off in zip(tensors, offsets):
+            f.write(b"\0" * (off - pos))
+            f.write(np.ascontiguousarray(a).data)
+            pos = off + a.nbytes
+        return f.tell()

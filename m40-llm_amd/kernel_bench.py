@@ -1,6 +1,6 @@
 """Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
 
-    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill] [--json out.jsonl]
+    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf] [--json out.jsonl]
 
 Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
 events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
@@ -170,6 +170,51 @@ def bench_prefill(b: Bench):
             x.free()
 
 
+def bench_gguf_load(b: Bench):
+    """Weight-file ingestion: a TinyLlama-1.1B-shaped f16 GGUF file (synthetic weights, ~2.2 GB) from the page cache
+    into HBM through m40host_gguf_load (parse + validate + streamed upload), beside the reference's sequence on the
+    same file (read the whole file into host memory, then m40llm_upload_weights; src/infer/load.rs:11-40), and the
+    decode rate of a model assembled from the loaded file.  Bound: the host-to-device link, not HBM."""
+    import ctypes as C
+    import tempfile
+    import time
+    gg = importlib.import_module("m40-llm_amd.gguf")
+    syn = importlib.import_module("m40-llm_amd.synthetic")
+    cfg = dict(syn.TINYLLAMA_1B, context_length=2048)
+    W = syn.make_weights(cfg, seed=0, unique_layers=2)
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "tinyllama_shape_f16.gguf")
+        size = gg.write_model_file(path, cfg, W)
+        del W
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            gw = gg.GgufWeights(b.ctx, path)
+            times.append(time.perf_counter() - t0)
+            if len(times) < 3:
+                gw.close()
+        best = min(times)
+        t0 = time.perf_counter()
+        blob = np.fromfile(path, dtype=np.uint8)
+        p = C.c_void_p()
+        m40.check(b.lib.m40llm_upload_weights(b.ctx.h, blob.ctypes.data_as(C.c_void_p), blob.nbytes, C.byref(p)), "m40llm_upload_weights")
+        t_ref = time.perf_counter() - t0
+        b.lib.m40llm_device_free(b.ctx.h, p)
+        del blob
+        gm = gw.model(max_seq_len=256, max_sequences=1)
+        gm.set_mode(2)
+        ids, ms = gm.decode_timed(0, [1, 2, 3, 4], 8, 64)
+        gm.close()
+        gw.close()
+    row = dict(kernel="gguf load (parse, validate, streamed upload)", shape=f"TinyLlama-1.1B shape, f16, {size / 1e9:.2f} GB file",
+               seconds=round(best, 4), gb_per_s=round(size / best / 1e9, 2), read_then_upload_seconds=round(t_ref, 4),
+               read_then_upload_gb_per_s=round(size / t_ref / 1e9, 2), decode_tok_s_from_file=round(64e3 / ms, 1))
+    b.rows.append(row)
+    print(f"{'gguf load':34s} {row['shape']:44s} {best * 1e3:9.1f} ms {row['gb_per_s']:8.2f} GB/s file->HBM   "
+          f"(read whole file + upload_weights: {t_ref * 1e3:.1f} ms, {row['read_then_upload_gb_per_s']:.2f} GB/s); "
+          f"decode from the loaded file {row['decode_tok_s_from_file']:.1f} tok/s", flush=True)
+
+
 def bench_gemv(b: Bench, M: int):
     rng = np.random.default_rng(1)
     shapes = [(2048, 2048), (256, 2048), (5632, 2048), (2048, 5632), (32000, 2048)] if M == 1 else \
@@ -295,7 +340,7 @@ def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill")
+    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
@@ -318,6 +363,8 @@ def main():
         bench_decode_batch(b, mode=args.decode_mode)
     if "prefill" in which:
         bench_prefill(b)
+    if "gguf" in which:
+        bench_gguf_load(b)
     if args.json:
         with open(args.json, "w") as f:
             for r in b.rows:

@@ -56,7 +56,7 @@ def test_embedding_rows_reference_cases(ctx, tmpfile):
 
 
 def test_data_section_is_resident_byte_for_byte_across_staging_buffers(ctx, tmpfile):
-    # 150 MiB of random bytes in three tensors: more than two 64 MiB staging buffers, offsets that are not
+    # 150 MiB of random bytes in three tensors: many rounds through the two staging buffers, offsets that are not
     # multiples of the buffer size
     rng = np.random.default_rng(0)
     sizes = [(1 << 20) * 70 + 6, (1 << 20) * 3, (1 << 20) * 77 + 2]
