@@ -337,6 +337,26 @@ int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32
  * decode stream; the benchmarks time it beside the kernels it bounds. */
 int m40llm_ext_read_probe_async(M40llmCudaContext* ctx, const void* d_src, size_t bytes, uint32_t workgroups,
                                 uint32_t* d_out_u32);
+/* Prefill, steps between the Q/K/V projections and the attention for a packed batch of prompts, one launch instead
+ * of three per token (src/infer/forward.rs:2349-2396: append_token_f32_rope_k_at_layout + rope_f32_inplace_layout on
+ * the Q row + on the K row, per token).  Rows are packed sequence after sequence (sequence i holds q_lens_host[i]
+ * rows); row j of sequence i is the token at position start_pos_host[i] + j (start_pos_host NULL = 0) of cache slot
+ * seq_slots_host[i].  d_q [rows][q_heads][head_dim] and d_k [rows][kv_heads][head_dim] are rotated in place (f32);
+ * the rotated K and d_v are cast to f16 into the cache, and the slot's length becomes start + len.  With the three
+ * bias vectors (all or none) Q, K and V first receive their bias in place (the per-row residual adds of
+ * forward.rs:149-160).  Bit-identical to the per-token calls.  Dense caches, at most 64 sequences, distinct slots.  Decode stream.
+ * -1 null, -2 batch / slot / q_heads / layout, -3/-4 cache geometry, -5 past max_seq_len, -7 empty sequence,
+ * -8 a slot named twice, -9 compressed cache, -6 launch. */
+int m40llm_ext_prefill_rope_append_async(M40llmCudaContext* ctx, M40llmKVCache* kv, void* d_q_f32, void* d_k_f32,
+                                         void* d_v_f32, uint32_t batch, const uint32_t* seq_slots_host,
+                                         const uint32_t* q_lens_host, const uint32_t* start_pos_host, uint32_t q_heads,
+                                         float freq_base, float freq_scale, uint32_t rope_layout, const void* d_bq_f32,
+                                         const void* d_bk_f32, const void* d_bv_f32);
+/* embedding rows of `rows` (<= 65535) token ids held on the device (f16 table [vocab][d_model]) -> f32 [rows][d_model];
+ * the row form of m40llm_ext_embed_token_dev_async (src/infer/forward.rs:2241-2250 loads them one blocking call per
+ * token).  Decode stream. */
+int m40llm_ext_embed_rows_async(M40llmCudaContext* ctx, const void* d_table_f16, const uint32_t* tokens_dev, uint32_t rows,
+                                uint32_t vocab, uint32_t d_model, void* d_out_f32);
 /* Weight-file ingestion: `num_bytes` of the file at `path`, from byte `file_offset`, into one new device allocation
  * (*out_device_ptr, released with m40llm_device_free).  Replaces read-the-file + m40llm_upload_weights
  * (src/infer/load.rs:27-40, kernels.cu:1264-1290): positional reads into two pinned staging buffers overlap the

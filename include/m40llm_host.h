@@ -154,6 +154,13 @@ int m40host_model_forward_batched(M40HostModel* model, const uint32_t* sequence_
 int m40host_model_decode_batch_greedy(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
                                       const uint32_t* first_tokens, uint32_t rows, uint32_t steps, uint32_t* ids_out,
                                       float* gaps_out);
+/* Packed prefill of `batch` prompts (forward_prefill_all_layers_varlen_for_sequences, src/infer/forward.rs:2153-2600):
+ * tokens holds the prompts one after the other (lens[i] ids each); every sequence starts at position 0 of its cache
+ * slots, which afterwards hold lens[i] tokens.  Dense cache, head_dim 64 or 128, at most 64 prompts and 65535 tokens
+ * per call.  hidden_last_host [batch][d_model] and logits_last_host [batch][vocab] receive the last token of each
+ * prompt; either may be NULL. */
+int m40host_model_forward_prefill(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* lens,
+                                  const uint32_t* tokens, uint32_t batch, float* hidden_last_host, float* logits_last_host);
 
 /* ---- GGUF ingestion (src/gguf.rs:172-329, src/infer/load.rs:10-92, src/infer/tensor_views.rs:29-117,
  *      src/infer/types.rs:114-242, src/infer/mapping.rs:95-540, src/infer/embeddings.rs:14-143) -------------- */

@@ -366,10 +366,10 @@ __global__ __launch_bounds__(kThreads) void embed_token_dev_kernel(const uint16_
                                                                    const uint32_t* __restrict__ token_dev,
                                                                    uint32_t vocab, uint32_t d_model,
                                                                    float* __restrict__ out) {
-    uint32_t tok = *token_dev;
+    uint32_t tok = token_dev[blockIdx.y];
     if (tok >= vocab) tok = vocab - 1;
     const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-    if (i < d_model) out[i] = m40_h2f(table[(size_t)tok * d_model + i]);
+    if (i < d_model) out[(size_t)blockIdx.y * d_model + i] = m40_h2f(table[(size_t)tok * d_model + i]);
 }
 
 // Device-side greedy bookkeeping.  state: [0] position, [1] step, [2] current token,
@@ -548,6 +548,16 @@ int m40llm_ext_embed_token_dev_async(M40llmCudaContext* ctx, const void* d_table
     (void)hipGetLastError();
     embed_token_dev_kernel<<<(d_model + kThreads - 1) / kThreads, kThreads, 0, ctx->decode_stream>>>(
         static_cast<const uint16_t*>(d_table_f16), token_dev, vocab, d_model, static_cast<float*>(d_out_f32));
+    return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_embed_rows_async(M40llmCudaContext* ctx, const void* d_table_f16, const uint32_t* tokens_dev, uint32_t rows,
+                                uint32_t vocab, uint32_t d_model, void* d_out_f32) {
+    if (!ctx || !d_table_f16 || !tokens_dev || !d_out_f32) return -1;
+    if (vocab == 0 || d_model == 0 || rows == 0 || rows > 65535u) return -2;
+    (void)hipGetLastError();
+    embed_token_dev_kernel<<<dim3((d_model + kThreads - 1) / kThreads, rows), kThreads, 0, ctx->decode_stream>>>(
+        static_cast<const uint16_t*>(d_table_f16), tokens_dev, vocab, d_model, static_cast<float*>(d_out_f32));
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -67,6 +67,74 @@ __global__ __launch_bounds__(kThreads) void dense_append_f16_kernel(
     if (idx == 0) seq_map[seq_id] = position + 1u;
 }
 
+// Prefill: RoPE of Q and K (in place, f32, for the attention that follows) and the cast of the rotated K and of V
+// into the dense cache, for every row of a packed batch in one launch.  One workgroup per row; the row's sequence
+// is found in the by-value table (at most kPrefillSeqs sequences).  Same rotation function and the same inverse
+// frequencies as the per-token appends and the standalone RoPE, so the bits agree with the per-token call sequence
+// (reference: src/infer/forward.rs:2349-2396, three launches per token and layer).
+constexpr int kPrefillSeqs = 64;
+struct PrefillSeqTable {
+    uint32_t n;
+    uint32_t slot[kPrefillSeqs], q_off[kPrefillSeqs], len[kPrefillSeqs], start[kPrefillSeqs];
+};
+
+__global__ __launch_bounds__(kThreads) void prefill_rope_append_kernel(
+    float* __restrict__ q, float* __restrict__ k, float* __restrict__ v, uint16_t* __restrict__ k_base,
+    uint16_t* __restrict__ v_base, uint32_t* __restrict__ seq_map, PrefillSeqTable t, uint32_t q_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t max_seq_len, const float* __restrict__ inv_freq_table,
+    float freq_base, float freq_scale, uint32_t layout, const float* __restrict__ bq, const float* __restrict__ bk,
+    const float* __restrict__ bv) {
+    const uint32_t row = blockIdx.x;
+    uint32_t s = 0;
+    for (uint32_t i = 1; i < t.n; ++i)
+        if (row >= t.q_off[i]) s = i;
+    const uint32_t local = row - t.q_off[s];
+    const uint32_t position = t.start[s] + local;
+    const uint32_t slot = t.slot[s];
+    const uint32_t half_dim = head_dim / 2u;
+    const uint32_t q_pairs = q_heads * half_dim, kv_pairs = kv_heads * half_dim;
+    float* q_row = q + (size_t)row * q_heads * head_dim;
+    float* k_row = k + (size_t)row * kv_heads * head_dim;
+    float* v_row = v + (size_t)row * kv_heads * head_dim;
+    const size_t ept = (size_t)kv_heads * head_dim;
+    uint16_t* k_out = k_base + ((size_t)slot * max_seq_len + position) * ept;
+    uint16_t* v_out = v_base + ((size_t)slot * max_seq_len + position) * ept;
+    for (uint32_t idx = threadIdx.x; idx < q_pairs + kv_pairs; idx += kThreads) {
+        const bool is_q = idx < q_pairs;
+        const uint32_t p = is_q ? idx : idx - q_pairs;
+        const uint32_t off = p % half_dim, head = p / half_dim;
+        size_t i0, i1;
+        m40_rope_pair(head, off, head_dim, layout, &i0, &i1);
+        const float f = inv_freq_table ? inv_freq_table[off] : m40_rope_inv_freq(off, head_dim, freq_base);
+        const float2 cs = m40_rope_cos_sin_freq(position, f, freq_scale);
+        float* x = is_q ? q_row : k_row;
+        const float* bias = is_q ? bq : bk;
+        float x0 = x[i0], x1 = x[i1];
+        if (bias) {   // the bias add of the per-row sequence (forward.rs:149-160), before the rotation
+            x0 = x0 + bias[i0];
+            x1 = x1 + bias[i1];
+        }
+        float y0, y1;
+        m40_rope_apply(cs, x0, x1, &y0, &y1);
+        x[i0] = y0;
+        x[i1] = y1;
+        if (!is_q) {
+            float v0 = v_row[i0], v1 = v_row[i1];
+            if (bv) {
+                v0 = v0 + bv[i0];
+                v1 = v1 + bv[i1];
+                v_row[i0] = v0;
+                v_row[i1] = v1;
+            }
+            k_out[i0] = m40_f2h(y0);
+            k_out[i1] = m40_f2h(y1);
+            v_out[i0] = m40_f2h(v0);
+            v_out[i1] = m40_f2h(v1);
+        }
+    }
+    if (threadIdx.x == 0 && local + 1u == t.len[s]) seq_map[slot] = position + 1u;
+}
+
 // Compressed append: one wave per kv head.  Phase 1 reads the ring row that is about to be
 // overwritten into registers and, when position >= W, evicts it to old index position-W
 // (K copied, V quantised to 4 bits with one f32 scale per token-head).  Phase 2, after a
@@ -461,6 +529,46 @@ int m40llm_kvcache_append_token_f32_rope_k_at_layout_async(M40llmCudaContext* ct
         static_cast<const float*>(k_dev_f32), static_cast<const float*>(v_dev_f32), kv->d_k, kv->d_v,
         kv->d_seq_map, seq_id, kv->max_seq_len, kv->num_heads, kv->head_dim, position, nullptr, freq_base,
         freq_scale, rope_layout, 0, 0);
+    return hipGetLastError() == hipSuccess ? 0 : -6;
+}
+
+int m40llm_ext_prefill_rope_append_async(M40llmCudaContext* ctx, M40llmKVCache* kv, void* d_q_f32, void* d_k_f32,
+                                         void* d_v_f32, uint32_t batch, const uint32_t* seq_slots_host,
+                                         const uint32_t* q_lens_host, const uint32_t* start_pos_host, uint32_t q_heads,
+                                         float freq_base, float freq_scale, uint32_t rope_layout, const void* d_bq_f32,
+                                         const void* d_bk_f32, const void* d_bv_f32) {
+    if (!ctx || !kv || !d_q_f32 || !d_k_f32 || !d_v_f32 || !seq_slots_host || !q_lens_host) return -1;
+    const int n_bias = (d_bq_f32 != nullptr) + (d_bk_f32 != nullptr) + (d_bv_f32 != nullptr);
+    if (n_bias != 0 && n_bias != 3) return -2;
+    if (kv->compressed || !kv->d_k || !kv->d_v) return -9;
+    if (batch == 0 || batch > (uint32_t)kPrefillSeqs || q_heads == 0) return -2;
+    if (kv->head_dim == 0 || kv->num_heads == 0) return -3;
+    if (kv->head_dim % 2 != 0) return -4;
+    if (rope_layout > M40LLM_ROPE_LAYOUT_NEOX) return -2;
+    PrefillSeqTable t{};
+    t.n = batch;
+    uint64_t rows = 0;
+    for (uint32_t i = 0; i < batch; ++i) {
+        const uint32_t start = start_pos_host ? start_pos_host[i] : 0u;
+        if (seq_slots_host[i] >= kv->max_batch_size) return -2;
+        if (q_lens_host[i] == 0) return -7;
+        if ((uint64_t)start + q_lens_host[i] > kv->max_seq_len) return -5;
+        for (uint32_t j = 0; j < i; ++j)
+            if (seq_slots_host[j] == seq_slots_host[i]) return -8;   // two sequences of one call would race on a slot
+        t.slot[i] = seq_slots_host[i];
+        t.q_off[i] = (uint32_t)rows;
+        t.len[i] = q_lens_host[i];
+        t.start[i] = start;
+        rows += q_lens_host[i];
+        if (rows > 0x7fffffffull) return -2;
+    }
+    hipStream_t stream = ctx->decode_stream;
+    const float* table = m40_rope_inv_freq_table(ctx, 1, stream, kv->head_dim, freq_base);
+    (void)hipGetLastError();
+    prefill_rope_append_kernel<<<(unsigned)rows, kThreads, 0, stream>>>(
+        static_cast<float*>(d_q_f32), static_cast<float*>(d_k_f32), static_cast<float*>(d_v_f32), kv->d_k, kv->d_v,
+        kv->d_seq_map, t, q_heads, kv->num_heads, kv->head_dim, kv->max_seq_len, table, freq_base, freq_scale, rope_layout,
+        static_cast<const float*>(d_bq_f32), static_cast<const float*>(d_bk_f32), static_cast<const float*>(d_bv_f32));
     return hipGetLastError() == hipSuccess ? 0 : -6;
 }
 

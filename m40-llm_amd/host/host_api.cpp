@@ -385,6 +385,26 @@ int m40host_model_decode_batch_greedy(M40HostModel* m, const uint32_t* seq_ids, 
         [&]() -> int { m->m->decode_batch_greedy(seq_ids, kv_lens, first_tokens, rows, steps, ids_out, gaps_out); return 0; }, -100);
 }
 
+int m40host_model_forward_prefill(M40HostModel* m, const uint32_t* seq_ids, const uint32_t* lens, const uint32_t* tokens,
+                                  uint32_t batch, float* hidden_last_host, float* logits_last_host) {
+    return guarded(
+        [&]() -> int {
+            if (!m || !seq_ids || !lens || !tokens) throw std::invalid_argument("null argument");
+            DecodeModel& d = *m->m;
+            const float* h = d.forward_prefill(seq_ids, lens, tokens, batch);
+            const size_t D = d.config().d_model, V = d.config().vocab;
+            size_t row = 0;
+            for (uint32_t i = 0; i < batch; ++i) {
+                row += lens[i];
+                const float* last = h + (row - 1) * D;
+                if (hidden_last_host) M40H_TRY(m40llm_memcpy_d2h(d.ctx(), hidden_last_host + i * D, last, D * 4));
+                if (logits_last_host) d.logits_from_hidden(last, logits_last_host + i * V);
+            }
+            return 0;
+        },
+        -100);
+}
+
 // ---- GGUF ingestion ------------------------------------------------------------------------------------
 M40HostGguf* m40host_gguf_open(const char* path) {
     return guarded(

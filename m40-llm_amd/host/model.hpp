@@ -74,6 +74,7 @@ public:
     void reset() { if (p_) m40llm_device_free(ctx_, p_); p_ = nullptr; }
     void* ptr() const { return p_; }
     float* f32(size_t off = 0) const { return static_cast<float*>(p_) + off; }
+    uint32_t* u32(size_t off = 0) const { return static_cast<uint32_t*>(p_) + off; }
     size_t bytes() const { return bytes_; }
 
 private:
@@ -98,6 +99,26 @@ struct ForwardWorkspace {
         logits = DeviceBuf(c, R * (size_t)m.vocab * 4);
         argmax_idx = DeviceBuf(c, R * 4); argmax_gap = DeviceBuf(c, R * 4); positions = DeviceBuf(c, R * 4 * 2);
         rows = want_rows;
+    }
+};
+
+struct PrefillWorkspace {   // activations of a packed prefill: no per-row logits
+    uint32_t rows = 0, batch = 0;
+    DeviceBuf xn, q, k, v, att, y, x1, gate, up, hid, a, b, tokens, offsets, lens;
+    void ensure(M40llmCudaContext* c, const ModelConfig& m, uint32_t want_rows, uint32_t want_batch) {
+        if (want_rows > rows) {
+            const size_t D = m.d_model, KV = (size_t)m.kv_heads * m.head_dim, F = m.ffn, R = want_rows;
+            xn = DeviceBuf(c, R * D * 4); q = DeviceBuf(c, R * D * 4); k = DeviceBuf(c, R * KV * 4); v = DeviceBuf(c, R * KV * 4);
+            att = DeviceBuf(c, R * D * 4); y = DeviceBuf(c, R * D * 4); x1 = DeviceBuf(c, R * D * 4);
+            gate = DeviceBuf(c, R * F * 4); up = DeviceBuf(c, R * F * 4); hid = DeviceBuf(c, R * F * 4);
+            a = DeviceBuf(c, R * D * 4); b = DeviceBuf(c, R * D * 4);
+            tokens = DeviceBuf(c, R * 4);
+            rows = want_rows;
+        }
+        if (want_batch > batch) {
+            offsets = DeviceBuf(c, (size_t)want_batch * 4); lens = DeviceBuf(c, (size_t)want_batch * 4);
+            batch = want_batch;
+        }
     }
 };
 
@@ -366,6 +387,79 @@ public:
                                               (int)cfg_.d_model));
         M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_PREFILL));
         M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits, ws_.logits.ptr(), (size_t)cfg_.vocab * 4));
+    }
+
+    // ---- packed prefill of several prompts ---------------------------------------------------------
+    // All tokens of all prompts as rows of one batch (forward.rs:2153-2600): per layer the projections are GEMMs over
+    // every row, RoPE + bias + the f16 KV append run as one launch, and the attention is the packed causal prefill
+    // kernel.  Each sequence starts at position 0 of its (cleared) cache slots.  Returns the hidden rows
+    // [total rows][d_model] on the device; row offsets are the running sum of `lens`.
+    const float* forward_prefill(const uint32_t* seq_ids, const uint32_t* lens, const uint32_t* tokens, uint32_t batch) {
+        if (batch == 0) throw std::invalid_argument("batched prefill requires at least one item");
+        if (kvcfg_.is_enabled()) throw std::invalid_argument("batched prefill requires the dense KV cache");
+        if (cfg_.head_dim != 64 && cfg_.head_dim != 128)
+            throw std::invalid_argument("batched prefill attention currently requires head_dim=64 or 128, got " +
+                                        std::to_string(cfg_.head_dim));   // forward.rs:2177-2182
+        uint64_t total = 0;
+        std::vector<uint32_t> offsets(batch);
+        for (uint32_t i = 0; i < batch; ++i) {
+            if (lens[i] == 0) throw std::invalid_argument("batched prefill item has empty prompt");
+            if (lens[i] > cfg_.max_seq_len) throw std::out_of_range("prompt longer than max_seq_len");
+            (void)kv_slot(seq_ids[i], cfg_.n_layers - 1);
+            offsets[i] = (uint32_t)total;
+            total += lens[i];
+        }
+        if (total > 65535u) throw std::invalid_argument("batched prefill is limited to 65535 rows per call");
+        const uint32_t rows = (uint32_t)total;
+        for (uint32_t r = 0; r < rows; ++r)
+            if (tokens[r] >= cfg_.vocab) throw std::out_of_range("token id out of range");
+        pws_.ensure(ctx_, cfg_, rows, batch);
+        const uint32_t D = cfg_.d_model, KV = cfg_.kv_heads * cfg_.head_dim, F = cfg_.ffn;
+        const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
+        M40H_TRY(m40llm_stream_synchronize(ctx_, DEC));   // the tables below are rewritten: nothing may still read them
+        M40H_TRY(m40llm_stream_synchronize(ctx_, PRE));
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, pws_.tokens.ptr(), tokens, (size_t)rows * 4));
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, pws_.offsets.ptr(), offsets.data(), (size_t)batch * 4));
+        M40H_TRY(m40llm_memcpy_h2d(ctx_, pws_.lens.ptr(), lens, (size_t)batch * 4));
+        float* a = pws_.a.f32();
+        float* b = pws_.b.f32();
+        M40H_TRY(m40llm_ext_embed_rows_async(ctx_, tok_emb_, pws_.tokens.u32(), rows, cfg_.vocab, D, a));
+        std::vector<uint32_t> slots(batch);
+        const uint32_t* d_off = pws_.offsets.u32();
+        const uint32_t* d_len = pws_.lens.u32();
+        for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
+            const LayerWeights& w = layers_[l];
+            for (uint32_t i = 0; i < batch; ++i) slots[i] = kv_slot(seq_ids[i], l);
+            M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, a, w.attn_norm, pws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wq, pws_.q.ptr(), (int)rows, (int)D, (int)D));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wk, pws_.k.ptr(), (int)rows, (int)KV, (int)D));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wv, pws_.v.ptr(), (int)rows, (int)KV, (int)D));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_ext_prefill_rope_append_async(ctx_, kv_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), batch, slots.data(), lens,
+                                                          nullptr, cfg_.q_heads, cfg_.rope_base, cfg_.rope_scale, cfg_.rope_layout,
+                                                          cfg_.has_qkv_bias ? w.bq : nullptr, cfg_.has_qkv_bias ? w.bk : nullptr,
+                                                          cfg_.has_qkv_bias ? w.bv : nullptr));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_attention_prefill_f32_gqa_varlen_async(ctx_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), d_off, d_off, d_len, d_len,
+                                                                   batch, cfg_.q_heads, cfg_.kv_heads, cfg_.head_dim, pws_.att.ptr()));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.att.ptr(), w.wo, pws_.y.ptr(), (int)rows, (int)D, (int)D));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, a, pws_.y.ptr(), pws_.x1.ptr(), (size_t)rows * D));
+            M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, pws_.x1.ptr(), w.ffn_norm, pws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wgate, pws_.gate.ptr(), (int)rows, (int)F, (int)D));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wup, pws_.up.ptr(), (int)rows, (int)F, (int)D));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_swiglu_f32_async(ctx_, pws_.gate.ptr(), pws_.up.ptr(), pws_.hid.ptr(), (size_t)rows * F));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.hid.ptr(), w.wdown, pws_.y.ptr(), (int)rows, (int)D, (int)F));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, pws_.x1.ptr(), pws_.y.ptr(), b, (size_t)rows * D));
+            std::swap(a, b);
+        }
+        M40H_TRY(m40llm_stream_synchronize(ctx_, DEC));
+        return a;
     }
 
     // Greedy decode of one sequence: prompt tokens from start_pos, then n_gen sampled tokens
@@ -738,6 +832,7 @@ private:
     KvCompressionConfig kvcfg_;
     M40llmKVCache* kv_ = nullptr;
     ForwardWorkspace ws_;
+    PrefillWorkspace pws_;
     uint32_t mode_ = 0;
     DeviceBuf state_;
     DeviceBuf top2_;

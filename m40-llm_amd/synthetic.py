@@ -177,6 +177,19 @@ class DeviceModel:
                  "m40host_model_decode_batch_greedy")
         return ids, gaps
 
+    def forward_prefill(self, seq_ids, prompts, want_logits=True):
+        """Packed prefill of several prompts; returns the last token's hidden state and logits per prompt."""
+        s = np.ascontiguousarray(seq_ids, dtype=np.uint32)
+        lens = np.ascontiguousarray([len(p) for p in prompts], dtype=np.uint32)
+        toks = np.ascontiguousarray(np.concatenate([np.asarray(p, dtype=np.uint32) for p in prompts]))
+        hid = np.empty((len(s), self.cfg["d_model"]), dtype=np.float32)
+        log = np.empty((len(s), self.cfg["vocab"]), dtype=np.float32) if want_logits else None
+        self._ok(self.H.m40host_model_forward_prefill(self.h, s.ctypes.data_as(C.c_void_p), lens.ctypes.data_as(C.c_void_p),
+                                                      toks.ctypes.data_as(C.c_void_p), len(s), hid.ctypes.data_as(C.c_void_p),
+                                                      log.ctypes.data_as(C.c_void_p) if want_logits else None),
+                 "m40host_model_forward_prefill")
+        return hid, log
+
     def decode_timed(self, seq, prompt, warmup, steps):
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
         ids = np.zeros(len(prompt) + warmup + steps, dtype=np.uint32)
