@@ -133,6 +133,9 @@ int m40_rows_mfma_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKV
                       const uint16_t* wq, const uint16_t* wk, const uint16_t* wv, const float* bq, const float* bk,
                       const float* bv, uint32_t d_model, uint32_t q_heads, float rope_base, float rope_scale,
                       uint32_t rope_layout, float* q_out);
+// many-row f32 x f16 GEMM on 128 x 128 tiles (gemm_tiled.hip): M > 32, K a multiple of 32, 16-byte aligned operands
+bool m40_gemm_tiled_supported(const void* A, const void* B, int M, int N, int K);
+int m40_launch_gemm_tiled(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K);
 bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
 int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);

@@ -1,6 +1,6 @@
 """Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
 
-    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf] [--json out.jsonl]
+    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd] [--json out.jsonl]
 
 Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
 events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
@@ -215,6 +215,33 @@ def bench_gguf_load(b: Bench):
           f"decode from the loaded file {row['decode_tok_s_from_file']:.1f} tok/s", flush=True)
 
 
+def bench_prefill_forward(b: Bench):
+    """Whole prefill forward (every layer, packed prompts) of the TinyLlama-1.1B shape through the host layer:
+    tokens per second and the matrix-instruction rate of the projections (2 * rows * weight elements per layer;
+    f16 instructions on hi/lo-split f32 activations, so the bound is half the 2.5 PFLOP/s f16 peak)."""
+    import time
+    syn = importlib.import_module("m40-llm_amd.synthetic")
+    cfg = dict(syn.TINYLLAMA_1B)
+    W = syn.make_weights(cfg, seed=0, unique_layers=2)
+    dm = syn.DeviceModel(b.ctx, cfg, W, max_seq_len=4096, max_sequences=8)
+    del W
+    rng = np.random.default_rng(0)
+    per_layer = cfg["d_model"] * (2 * cfg["d_model"] + 2 * cfg["kv_heads"] * cfg["head_dim"] + 3 * cfg["ffn"])
+    for label, lens in (("one prompt of 512", [512]), ("one prompt of 4096", [4096]), ("8 prompts U[256,4096]", [int(x) for x in rng.integers(256, 4097, size=8)])):
+        prompts = [rng.integers(0, cfg["vocab"], size=n).tolist() for n in lens]
+        seqs = list(range(len(lens)))
+        dm.forward_prefill(seqs, prompts, want_logits=False)          # warm (workspace, tables)
+        t0 = time.perf_counter()
+        dm.forward_prefill(seqs, prompts, want_logits=False)
+        dt = time.perf_counter() - t0
+        rows = sum(lens)
+        tf = 2.0 * rows * per_layer * cfg["n_layers"] / dt / 1e12
+        b.rows.append(dict(kernel="prefill forward, TinyLlama-1.1B shape", shape=label, rows=rows, ms=round(dt * 1e3, 2),
+                           tok_s=round(rows / dt, 1), projection_tflops=round(tf, 1)))
+        print(f"{'prefill forward (22 layers)':34s} {label:44s} {dt * 1e3:9.1f} ms {rows / dt:10.0f} tok/s   projections {tf:6.1f} TFLOP/s", flush=True)
+    dm.close()
+
+
 def bench_gemv(b: Bench, M: int):
     rng = np.random.default_rng(1)
     shapes = [(2048, 2048), (256, 2048), (5632, 2048), (2048, 5632), (32000, 2048)] if M == 1 else \
@@ -340,7 +367,7 @@ def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf")
+    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
@@ -365,6 +392,8 @@ def main():
         bench_prefill(b)
     if "gguf" in which:
         bench_gguf_load(b)
+    if "pfwd" in which:
+        bench_prefill_forward(b)
     if args.json:
         with open(args.json, "w") as f:
             for r in b.rows:

@@ -176,6 +176,25 @@ def test_kv_append_rope_k_fused_equals_standalone(dev, orc, layout):
 
 
 # ------------------------------------------------------------------ GEMM family
+@pytest.mark.parametrize("M,N,K", [(33, 16, 32), (100, 200, 2048), (128, 256, 2048), (300, 136, 5632), (257, 2048, 64)])
+def test_gemm_many_rows_vs_oracle(dev, orc, M, N, K):
+    # the 128 x 128-tile matrix-core GEMM behind m40llm_gemm_f32xf16_gguf_f32 for M > 32 (prefill): ragged tiles in
+    # both directions, one and many K steps
+    rng = np.random.default_rng(M * 7 + N)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    A[1, :8] *= 1e-6                      # tiny activations keep their value through the low part
+    B = f16bits(rng.standard_normal((N, K)) * 0.05)
+    got = dev.gemm_gguf(A, B, M, N, K)
+    want = orc.gemm("f32xf16_gguf", A, B, M, N, K)
+    close(got, want)
+    # values beyond the f16 range must not turn into infinities
+    A[0, ::7] = 1.2e5
+    got = dev.gemm_gguf(A, B, M, N, K)
+    assert np.isfinite(got).all()
+    close(got[0], orc.gemm("f32xf16_gguf", A, B, M, N, K)[0], 2e-3, 2e-3 * np.abs(got[0]).max())
+    close(got[1:], want[1:])
+
+
 def test_gemm_known_answers(dev, orc):
     A = f16bits([[1, 2], [3, 4]]); B = f16bits([[5, 6], [7, 8]])
     dA, dB, dC = dev.up(A), dev.up(B), dev.zeros(16)
