@@ -29,6 +29,8 @@ struct M40StreamScratch {
     size_t attn_partial_bytes;
     void* select;            // block scores / selected ids / counts of the block-select path
     size_t select_bytes;
+    void* tiled_pack;        // f16 high / low planes of the activations of the many-row GEMM; grown on demand
+    size_t tiled_pack_bytes;
 };
 
 struct M40llmCudaContext {
@@ -135,7 +137,11 @@ int m40_rows_mfma_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKV
                       uint32_t rope_layout, float* q_out);
 // many-row f32 x f16 GEMM on 128 x 128 tiles (gemm_tiled.hip): M > 32, K a multiple of 32, 16-byte aligned operands
 bool m40_gemm_tiled_supported(const void* A, const void* B, int M, int N, int K);
-int m40_launch_gemm_tiled(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K);
+int m40_launch_gemm_tiled(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint16_t* B,
+                          float* C, int M, int N, int K);
+// up to three weight matrices over the same activations in one launch; 1 = declined (no packing buffer), else 0 / -2
+int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, int M, int K,
+                                int n_mats, const uint16_t* const* B, const int* N, float* const* C);
 bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
 int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);

@@ -24,6 +24,7 @@ void free_scratch(M40StreamScratch& s) {
     if (s.gemm_pack) (void)hipFree(s.gemm_pack);
     if (s.attn_partial) (void)hipFree(s.attn_partial);
     if (s.select) (void)hipFree(s.select);
+    if (s.tiled_pack) (void)hipFree(s.tiled_pack);
     s = M40StreamScratch{};
 }
 

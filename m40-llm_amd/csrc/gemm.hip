@@ -520,8 +520,11 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
         else if (g.cols == 2) gemv_f32xf16_gguf_kernel<2, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
         else gemv_f32xf16_gguf_kernel<1, 1><<<g.blocks, 256, 0, stream>>>(A, B, C, N, K);
     } else if (fast && m40_gemm_tiled_supported(A, B, M, N, K)) {
-        // many rows (prefill): one pass over the weights for all rows
-        return m40_launch_gemm_tiled(stream, A, B, C, M, N, K);
+        // many rows (prefill): one pass over the weights for all rows; declined (1) only when its packing buffer
+        // cannot be provided, then the skinny kernels take the rows 16 at a time
+        const int rc = m40_launch_gemm_tiled(ctx, stream, stream_kind, A, B, C, M, N, K);
+        if (rc != 1) return rc;
+        return m40_launch_skinny(ctx, stream, stream_kind, 0, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     } else if (fast && N <= 8192 && m40_rows_gemv_supported(M, K)) {
         // few columns: the vector-ALU row kernel needs no K split and no second launch
         return m40_rows_gemv_residual(stream, A, B, nullptr, C, M, N, K);

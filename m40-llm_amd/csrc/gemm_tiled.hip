@@ -3,86 +3,112 @@
 // beyond what the skinny kernels serve in one pass, where they would stream the weights once per 16 rows.
 //
 // Tiling: a workgroup of 4 waves owns a 128 x 128 tile of C and walks K in steps of 32.  Per step the 128 x 32 block
-// of A is read as f32, split exactly into an f16 high part and an f16 low part (a = hi + lo up to 2^-22 relative),
-// and written to LDS with the 128 x 32 block of B; each wave then computes its 64 x 64 quarter with
+// of A, split exactly into an f16 high part and an f16 low part (a = hi + lo up to 2^-22 relative), is written to
+// LDS with the 128 x 32 block of B; each wave then computes its 64 x 64 quarter with
 // v_mfma_f32_16x16x32_f16, once with the high and once with the low part, so the products carry the f32 activations'
-// precision.  Global loads for step k+1 are issued before the arithmetic of step k and land in the other LDS buffer
-// after it: one barrier per step.
+// precision.  The global loads of the next three steps are in flight (three rotating register sets) while a step
+// computes from one LDS buffer and the following step's data moves into the other: one barrier per step.
+//
+// The split is done once per call by a packing pass (A -> two f16 planes in a per-stream buffer that grows on
+// demand), so the 128 x 128 tiles along N do not each repeat it.  When the buffer cannot be grown (the stream is being
+// captured) the launch is declined and the caller falls back to the skinny kernels.  Several weight matrices that
+// share A (Q/K/V, gate/up) can be served by one packing pass and one launch.
 #include "common.hpp"
 
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBM = 128, kBN = 128, kBK = 32;
 constexpr int kStride = kBK + 8;                 // halves per LDS row: 80 B, conflict-free 16-byte fragment reads
 constexpr int kTileHalves = kBM * kStride;       // one 128 x 32 operand block
 constexpr int kBufHalves = 3 * kTileHalves;      // A high, A low, B
 constexpr int kThreads = 256;
+constexpr int kMaxMats = 3;
 
-struct StepRegs {
-    float4 a[4];   // 16 consecutive f32 of one A row
-    uint4 b[2];    // 16 consecutive f16 of one B column
+// Up to three weight matrices that share the activations (Q/K/V, gate/up): their column tiles are laid side by side.
+struct TiledMats {
+    int n;
+    const uint16_t* B[kMaxMats];
+    float* C[kMaxMats];
+    int N[kMaxMats];
+    int tile_start[kMaxMats + 1];   // first column tile of each matrix; [n] = total
 };
 
-__device__ __forceinline__ void split16(const float4 (&a)[4], half8 (&hi)[2], half8 (&lo)[2]) {
+struct StepRegs {   // one K step of one thread: rows lrow and lrow + 64, 16 bytes (8 halves) of each
+    uint4 ah[2], al[2], b[2];
+};
+
+// A [total] f32 -> hi [total] f16, lo [total] f16 (a = hi + lo up to 2^-22 relative); 8 elements per thread
+__global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __restrict__ A, _Float16* __restrict__ hi,
+                                                               _Float16* __restrict__ lo, size_t total8) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total8) return;
+    const float4 x0 = reinterpret_cast<const float4*>(A)[2 * i], x1 = reinterpret_cast<const float4*>(A)[2 * i + 1];
+    const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+    half8 h, l;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float x[4] = {a[i].x, a[i].y, a[i].z, a[i].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            // clamped to the f16 range: a value beyond +-65504 keeps its sign and loses precision instead of becoming
-            // an infinity (and its low part a NaN)
-            const float xc = fminf(fmaxf(x[j], -65504.0f), 65504.0f);
-            const _Float16 h = static_cast<_Float16>(xc);
-            const _Float16 l = static_cast<_Float16>(fminf(fmaxf(x[j] - static_cast<float>(h), -65504.0f), 65504.0f));
-            hi[i >> 1][(i & 1) * 4 + j] = h;
-            lo[i >> 1][(i & 1) * 4 + j] = l;
-        }
+    for (int j = 0; j < 8; ++j) {
+        // clamped to the f16 range: a value beyond +-65504 keeps its sign and loses precision instead of becoming an
+        // infinity (and its low part a NaN)
+        const float xc = fminf(fmaxf(x[j], -65504.0f), 65504.0f);
+        h[j] = static_cast<_Float16>(xc);
+        l[j] = static_cast<_Float16>(fminf(fmaxf(x[j] - static_cast<float>(h[j]), -65504.0f), 65504.0f));
     }
+    reinterpret_cast<half8*>(hi)[i] = h;
+    reinterpret_cast<half8*>(lo)[i] = l;
 }
 
-__global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(const float* __restrict__ A,
-                                                                              const uint16_t* __restrict__ B,
-                                                                              float* __restrict__ C, int M, int N, int K,
-                                                                              int tiles_n) {
+__global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(const _Float16* __restrict__ A_hi,
+                                                                              const _Float16* __restrict__ A_lo,
+                                                                              TiledMats mats, int M, int K) {
     extern __shared__ __align__(16) _Float16 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const int tiles_n = mats.tile_start[mats.n];
+    const int tile_m = blockIdx.x / tiles_n;
+    int tile_n = blockIdx.x % tiles_n;
+    int mat = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMats; ++i)
+        if (i < mats.n && tile_n >= mats.tile_start[i]) mat = i;
+    tile_n -= mats.tile_start[mat];
+    const uint16_t* __restrict__ B = mats.B[mat];
+    float* __restrict__ C = mats.C[mat];
+    const int N = mats.N[mat];
     const int m0 = tile_m * kBM, n0 = tile_n * kBN;
-    // loader role: row (or column) tid / 2, k half tid % 2
-    const int lrow = tid >> 1, lhalf = tid & 1;
-    const int a_row = m0 + lrow < M ? m0 + lrow : M - 1;     // clamped: rows beyond M are computed and never stored
-    const int b_col = n0 + lrow < N ? n0 + lrow : N - 1;
-    const float* a_src = A + (size_t)a_row * K + lhalf * 16;
-    const uint16_t* b_src = B + (size_t)b_col * K + lhalf * 16;
+    // loader role: four lanes cover the 64 bytes one row contributes to a step, so a wave's load instruction touches
+    // 16 rows (16 cache lines) instead of 32; each thread serves rows lrow and lrow + 64
+    const int lrow = tid >> 2, lchunk = tid & 3;
+    size_t a_off[2], b_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int ar = m0 + lrow + 64 * i < M ? m0 + lrow + 64 * i : M - 1;   // clamped: computed, never stored
+        const int bc = n0 + lrow + 64 * i < N ? n0 + lrow + 64 * i : N - 1;
+        a_off[i] = (size_t)ar * K + lchunk * 8;
+        b_off[i] = (size_t)bc * K + lchunk * 8;
+    }
     const int steps = K / kBK;
 
     auto issue = [&](StepRegs& r, int step) {
-        const float4* ap = reinterpret_cast<const float4*>(a_src + (size_t)step * kBK);
-        const uint4* bp = reinterpret_cast<const uint4*>(b_src + (size_t)step * kBK);
+        const size_t k = (size_t)step * kBK;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r.a[i] = ap[i];
-        r.b[0] = bp[0];
-        r.b[1] = bp[1];
+        for (int i = 0; i < 2; ++i) {
+            r.ah[i] = *reinterpret_cast<const uint4*>(A_hi + a_off[i] + k);
+            r.al[i] = *reinterpret_cast<const uint4*>(A_lo + a_off[i] + k);
+            r.b[i] = *reinterpret_cast<const uint4*>(B + b_off[i] + k);
+        }
     };
     auto to_lds = [&](const StepRegs& r, int buf) {
-        _Float16* base = lds + buf * kBufHalves;
-        half8 hi[2], lo[2];
-        split16(r.a, hi, lo);
-        _Float16* ah = base + lrow * kStride + lhalf * 16;
-        _Float16* al = ah + kTileHalves;
-        _Float16* bb = ah + 2 * kTileHalves;
-        *reinterpret_cast<half8*>(ah) = hi[0];
-        *reinterpret_cast<half8*>(ah + 8) = hi[1];
-        *reinterpret_cast<half8*>(al) = lo[0];
-        *reinterpret_cast<half8*>(al + 8) = lo[1];
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        *reinterpret_cast<u32x4*>(bb) = u32x4{r.b[0].x, r.b[0].y, r.b[0].z, r.b[0].w};
-        *reinterpret_cast<u32x4*>(bb + 8) = u32x4{r.b[1].x, r.b[1].y, r.b[1].z, r.b[1].w};
+        _Float16* base = lds + buf * kBufHalves + lrow * kStride + lchunk * 8;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            _Float16* p = base + i * 64 * kStride;
+            *reinterpret_cast<u32x4*>(p) = u32x4{r.ah[i].x, r.ah[i].y, r.ah[i].z, r.ah[i].w};
+            *reinterpret_cast<u32x4*>(p + kTileHalves) = u32x4{r.al[i].x, r.al[i].y, r.al[i].z, r.al[i].w};
+            *reinterpret_cast<u32x4*>(p + 2 * kTileHalves) = u32x4{r.b[i].x, r.b[i].y, r.b[i].z, r.b[i].w};
+        }
     };
 
     floatx4 acc[4][4];
@@ -104,25 +130,40 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
         for (int mt = 0; mt < 4; ++mt) {
             const half8 hi = *reinterpret_cast<const half8*>(ah + mt * 16 * kStride);
             const half8 lo = *reinterpret_cast<const half8*>(ah + kTileHalves + mt * 16 * kStride);
+            // the four high-part products first, then the four low-part ones: two instructions on one accumulator are
+            // four instructions apart instead of back to back
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, bf[nt], acc[mt][nt], 0, 0, 0);
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, bf[nt], acc[mt][nt], 0, 0, 0);
-            }
+            for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, bf[nt], acc[mt][nt], 0, 0, 0);
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, bf[nt], acc[mt][nt], 0, 0, 0);
         }
     };
 
-    StepRegs regs;
-    issue(regs, 0);
-    to_lds(regs, 0);
+    // Three register sets keep the loads of the next three steps in flight (a step's arithmetic is several times
+    // shorter than the memory latency); the sets rotate with the step, so the loop is unrolled by three.
+    StepRegs r0, r1, r2;
+    const int last = steps - 1;
+    issue(r0, 0);
+    issue(r1, 1 < last ? 1 : last);
+    issue(r2, 2 < last ? 2 : last);
+    to_lds(r0, 0);
     __syncthreads();
-    for (int s = 0; s < steps; ++s) {
-        const int next = s + 1 < steps ? s + 1 : s;     // the last step reloads its own block: no branch around loads
-        issue(regs, next);
+    // step s: reload the set that step s consumed with step s + 3 (clamped: no branch around loads), compute from the
+    // current LDS buffer, move step s + 1 into the other buffer
+    auto step = [&](StepRegs& reload, const StepRegs& next, int s) {
+        issue(reload, s + 3 < last ? s + 3 : last);
         compute(s & 1);
-        to_lds(regs, (s + 1) & 1);
+        to_lds(next, (s + 1) & 1);
         __syncthreads();
+    };
+    int s = 0;
+    for (; s + 3 <= steps; s += 3) {
+        step(r0, r1, s);
+        step(r1, r2, s + 1);
+        step(r2, r0, s + 2);
     }
+    if (s < steps) step(r0, r1, s);
+    if (s + 1 < steps) step(r1, r2, s + 1);
 
     // D fragment: lane holds rows 4 * (lane / 16) + r, column lane % 16 of each 16 x 16 tile
     const int out_col = lane & 15, out_row = (lane >> 4) * 4;
@@ -145,21 +186,56 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
 
 bool m40_gemm_tiled_supported(const void* A, const void* B, int M, int N, int K) {
     return M > 32 && N >= 16 && K >= kBK && K % kBK == 0 && m40_aligned16(A) && m40_aligned16(B) &&
-           ((long long)((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN)) <= 0x7fffffffll;
+           ((long long)((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN)) <= 0x3fffffffll;
 }
 
-int m40_launch_gemm_tiled(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K) {
-    if (!m40_gemm_tiled_supported(A, B, M, N, K)) return -2;
-    static bool attr_set = false;
-    constexpr size_t lds_bytes = 2 * kBufHalves * sizeof(_Float16);   // 61440
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_f32xf16_gguf_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
-            return -2;
-        attr_set = true;
+// Returns 1 when the activations' packing buffer cannot be provided (the stream is being captured and the buffer is
+// too small, or the allocation fails): the caller then uses another kernel.
+int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, int M, int K,
+                                int n_mats, const uint16_t* const* B, const int* N, float* const* C) {
+    if (!ctx || stream_kind > 1u || n_mats < 1 || n_mats > kMaxMats) return -2;
+    TiledMats mats{};
+    mats.n = n_mats;
+    long long tiles_n = 0;
+    for (int i = 0; i < n_mats; ++i) {
+        if (!m40_gemm_tiled_supported(A, B[i], M, N[i], K) || !C[i]) return -2;
+        mats.B[i] = B[i];
+        mats.C[i] = C[i];
+        mats.N[i] = N[i];
+        mats.tile_start[i] = (int)tiles_n;
+        tiles_n += (N[i] + kBN - 1) / kBN;
     }
-    const int tiles_m = (M + kBM - 1) / kBM, tiles_n = (N + kBN - 1) / kBN;
+    mats.tile_start[n_mats] = (int)tiles_n;
+    const long long tiles_m = (M + kBM - 1) / kBM;
+    if (tiles_m * tiles_n > 0x7fffffffll) return -2;
+    constexpr size_t lds_bytes = 2 * kBufHalves * sizeof(_Float16);   // 61440
+    // two f16 planes of A in the stream's packing buffer, grown on demand (never while the stream is being captured)
+    M40StreamScratch& sc = ctx->scratch[stream_kind];
+    const size_t need = (size_t)M * K * 4;
+    if (sc.tiled_pack_bytes < need) {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone) return 1;
+        if (hipStreamSynchronize(stream) != hipSuccess) return -2;
+        if (sc.tiled_pack) (void)hipFree(sc.tiled_pack);
+        sc.tiled_pack = nullptr;
+        sc.tiled_pack_bytes = 0;
+        const size_t want = need + need / 4;
+        if (hipMalloc(&sc.tiled_pack, want) != hipSuccess) {
+            (void)hipGetLastError();
+            return 1;
+        }
+        sc.tiled_pack_bytes = want;
+    }
     (void)hipGetLastError();
-    gemm_tiled_f32xf16_gguf_kernel<<<tiles_m * tiles_n, kThreads, lds_bytes, stream>>>(A, B, C, M, N, K, tiles_n);
+    _Float16* hi = static_cast<_Float16*>(sc.tiled_pack);
+    _Float16* lo = hi + (size_t)M * K;
+    const size_t total8 = (size_t)M * K / 8;
+    pack_hilo_planes_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(A, hi, lo, total8);
+    gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles_m * tiles_n), kThreads, lds_bytes, stream>>>(hi, lo, mats, M, K);
     return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+int m40_launch_gemm_tiled(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint16_t* B,
+                          float* C, int M, int N, int K) {
+    return m40_launch_gemm_tiled_multi(ctx, stream, stream_kind, A, M, K, 1, &B, &N, &C);
 }

@@ -1,6 +1,6 @@
 """Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
 
-    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd] [--json out.jsonl]
+    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN] [--json out.jsonl]
 
 Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
 events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
@@ -215,6 +215,36 @@ def bench_gguf_load(b: Bench):
           f"decode from the loaded file {row['decode_tok_s_from_file']:.1f} tok/s", flush=True)
 
 
+PEAK_F16_MATRIX_TFLOPS = 2500.0
+
+
+def bench_gemm_many_rows(b: Bench):
+    """The many-row GEMM of the prefill path (f32 activations split into two f16 parts: two matrix instructions per
+    product tile).  Useful rate = 2 M N K / time; the instruction rate is twice that and is what the 2.5 PFLOP/s f16
+    peak bounds."""
+    rng = np.random.default_rng(3)
+    for M, N, K in ((4096, 2048, 2048), (4096, 256, 2048), (4096, 5632, 2048), (4096, 2048, 5632), (512, 5632, 2048), (16384, 11008, 2048)):
+        A = b.ctx.to_device(rng.standard_normal((M, K), dtype=np.float32))
+        W = b.ctx.to_device(f16(rng.standard_normal((N, K), dtype=np.float32) * 0.02))
+        Cb = b.ctx.alloc(M * N * 4)
+        reps, warm = 10, 2
+        for i in range(warm + reps):
+            if i == warm:
+                b.ctx.sync(1)
+                b.ctx.record(b.e0, 1)
+            b.call("m40llm_ext_gemm_f32xf16_gguf_f32_async", A.ptr, W.ptr, Cb.ptr, M, N, K, 1)
+        b.ctx.record(b.e1, 1)
+        us = b.ctx.elapsed_ms(b.e0, b.e1) * 1e3 / reps
+        tf = 2.0 * M * N * K / us / 1e6
+        b.rows.append(dict(kernel="gemm_f32xf16_gguf many rows", shape=f"M={M} N={N} K={K}", us_per_launch=round(us, 2),
+                           useful_tflops=round(tf, 1), instruction_tflops=round(2 * tf, 1),
+                           frac_f16_matrix_peak=round(2 * tf / PEAK_F16_MATRIX_TFLOPS, 4)))
+        print(f"{'gemm_f32xf16_gguf many rows':34s} {f'M={M} N={N} K={K}':44s} {us:9.1f} us {tf:8.1f} TFLOP/s useful, {2 * tf:7.1f} issued  "
+              f"frac {2 * tf / PEAK_F16_MATRIX_TFLOPS:6.3f} of the f16 matrix peak", flush=True)
+        for x in (A, W, Cb):
+            x.free()
+
+
 def bench_prefill_forward(b: Bench):
     """Whole prefill forward (every layer, packed prompts) of the TinyLlama-1.1B shape through the host layer:
     tokens per second and the matrix-instruction rate of the projections (2 * rows * weight elements per layer;
@@ -367,7 +397,7 @@ def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd")
+    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
@@ -392,6 +422,8 @@ def main():
         bench_prefill(b)
     if "gguf" in which:
         bench_gguf_load(b)
+    if "gemmN" in which:
+        bench_gemm_many_rows(b)
     if "pfwd" in which:
         bench_prefill_forward(b)
     if args.json:
