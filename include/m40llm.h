@@ -280,6 +280,15 @@ int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_
 int m40llm_ext_gemm_f32xf16_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32,
                                            const void* d_B_f16, void* d_C_f32, int M, int N, int K,
                                            uint32_t stream_kind);
+/* One to three f16 weight matrices (GGUF order) applied to the same f32 activations A [M][K]: C_i [M][N_i] = A x B_i,
+ * each exactly what m40llm_gemm_f32xf16_gguf_f32 computes.  The reference issues these as separate GEMMs
+ * (qkv_project_f32xf16_gguf_f32_async and the gate/up pair, src/infer/forward.rs:2326-2338, 2471-2490); with many rows
+ * they share one pass that splits A into f16 planes and one launch.  Unused matrix slots are NULL / 0.  Asynchronous on
+ * `stream_kind`. */
+int m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(M40llmCudaContext* ctx, const void* d_A_f32, int M, int K, int n_mats,
+                                                 const void* d_B0_f16, int N0, void* d_C0_f32, const void* d_B1_f16, int N1,
+                                                 void* d_C1_f32, const void* d_B2_f16, int N2, void* d_C2_f32,
+                                                 uint32_t stream_kind);
 /* Per-q-head selection of the block-select path, computed by the same kernels that the
  * attention entry points run (the reference's debug selector covers q-head 0 only).
  * out_blocks_host: [q_heads][64] (0xffffffff beyond the count), out_counts_host: [q_heads],

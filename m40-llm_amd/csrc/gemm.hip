@@ -561,6 +561,23 @@ int m40_launch_gemm_f32xf16_gguf(M40llmCudaContext* ctx, hipStream_t stream, uin
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
+// Up to three f16 weight matrices applied to the same activations.  Many rows: one packing pass and one launch of
+// the tiled kernel; otherwise (or when that declines) one GEMM per matrix.
+static int launch_multi_f32xf16(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, int M, int K,
+                                int n_mats, const uint16_t* const* B, const int* N, float* const* C) {
+    bool tiled = (K % 8 == 0);
+    for (int i = 0; i < n_mats && tiled; ++i) tiled = m40_gemm_tiled_supported(A, B[i], M, N[i], K);
+    if (tiled) {
+        const int rc = m40_launch_gemm_tiled_multi(ctx, stream, stream_kind, A, M, K, n_mats, B, N, C);
+        if (rc != 1) return rc;
+    }
+    for (int i = 0; i < n_mats; ++i) {
+        const int rc = m40_launch_gemm_f32xf16_gguf(ctx, stream, stream_kind, A, B[i], C[i], M, N[i], K);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
 static int launch_q80(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint8_t* B,
                       float* C, int M, int N, int K) {
     if (m40_aligned16(B) && m40_aligned16(A) && q80_gemv_supported(M, N, K))
@@ -588,6 +605,26 @@ int m40llm_gemm_f32xf16_gguf_f32(M40llmCudaContext* ctx, const void* d_A_f32, co
                                           M, N, K);
     if (rc != 0) return rc;
     return hipStreamSynchronize(ctx->prefill_stream) == hipSuccess ? 0 : -3;
+}
+
+int m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(M40llmCudaContext* ctx, const void* d_A_f32, int M, int K, int n_mats,
+                                                 const void* d_B0_f16, int N0, void* d_C0_f32, const void* d_B1_f16, int N1,
+                                                 void* d_C1_f32, const void* d_B2_f16, int N2, void* d_C2_f32,
+                                                 uint32_t stream_kind) {
+    if (!ctx || !d_A_f32) return -1;
+    if (n_mats < 1 || n_mats > 3 || M <= 0 || K <= 0) return -2;
+    const uint16_t* B[3] = {static_cast<const uint16_t*>(d_B0_f16), static_cast<const uint16_t*>(d_B1_f16),
+                            static_cast<const uint16_t*>(d_B2_f16)};
+    float* C[3] = {static_cast<float*>(d_C0_f32), static_cast<float*>(d_C1_f32), static_cast<float*>(d_C2_f32)};
+    const int N[3] = {N0, N1, N2};
+    for (int i = 0; i < n_mats; ++i) {
+        if (!B[i] || !C[i]) return -1;
+        if (N[i] <= 0) return -2;
+    }
+    if (m40_ensure_device(ctx) != 0) return -2;
+    hipStream_t stream = m40_select_stream(ctx, stream_kind);
+    if (!stream) return -3;
+    return launch_multi_f32xf16(ctx, stream, stream_kind, static_cast<const float*>(d_A_f32), M, K, n_mats, B, N, C);
 }
 
 int m40llm_ext_gemm_f32xf16_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16,

@@ -67,8 +67,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
     extern __shared__ __align__(16) _Float16 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles_n = mats.tile_start[mats.n];
-    const int tile_m = blockIdx.x / tiles_n;
-    int tile_n = blockIdx.x % tiles_n;
+    // Workgroups are dealt to the eight dies in turn.  Renumbered so that each die owns a contiguous band of tile
+    // rows: its L2 then holds one eighth of A (and streams B) instead of every die reading all of A.
+    const int per_die = (int)gridDim.x / 8;
+    const int logical = (int)blockIdx.x < per_die * 8 ? ((int)blockIdx.x % 8) * per_die + (int)blockIdx.x / 8 : (int)blockIdx.x;
+    const int tile_m = logical / tiles_n;
+    int tile_n = logical % tiles_n;
     int mat = 0;
 #pragma unroll
     for (int i = 1; i < kMaxMats; ++i)

@@ -432,9 +432,8 @@ public:
             for (uint32_t i = 0; i < batch; ++i) slots[i] = kv_slot(seq_ids[i], l);
             M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, a, w.attn_norm, pws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wq, pws_.q.ptr(), (int)rows, (int)D, (int)D));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wk, pws_.k.ptr(), (int)rows, (int)KV, (int)D));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wv, pws_.v.ptr(), (int)rows, (int)KV, (int)D));
+            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(ctx_, pws_.xn.ptr(), (int)rows, (int)D, 3, w.wq, (int)D, pws_.q.ptr(),
+                                                                  w.wk, (int)KV, pws_.k.ptr(), w.wv, (int)KV, pws_.v.ptr(), PRE));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
             M40H_TRY(m40llm_ext_prefill_rope_append_async(ctx_, kv_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), batch, slots.data(), lens,
                                                           nullptr, cfg_.q_heads, cfg_.rope_base, cfg_.rope_scale, cfg_.rope_layout,
@@ -443,17 +442,17 @@ public:
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
             M40H_TRY(m40llm_attention_prefill_f32_gqa_varlen_async(ctx_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), d_off, d_off, d_len, d_len,
                                                                    batch, cfg_.q_heads, cfg_.kv_heads, cfg_.head_dim, pws_.att.ptr()));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.att.ptr(), w.wo, pws_.y.ptr(), (int)rows, (int)D, (int)D));
+            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx_, pws_.att.ptr(), w.wo, pws_.y.ptr(), (int)rows, (int)D, (int)D, PRE));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
             M40H_TRY(m40llm_residual_add_f32_async(ctx_, a, pws_.y.ptr(), pws_.x1.ptr(), (size_t)rows * D));
             M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, pws_.x1.ptr(), w.ffn_norm, pws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wgate, pws_.gate.ptr(), (int)rows, (int)F, (int)D));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.xn.ptr(), w.wup, pws_.up.ptr(), (int)rows, (int)F, (int)D));
+            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(ctx_, pws_.xn.ptr(), (int)rows, (int)D, 2, w.wgate, (int)F,
+                                                                  pws_.gate.ptr(), w.wup, (int)F, pws_.up.ptr(), nullptr, 0, nullptr, PRE));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
             M40H_TRY(m40llm_swiglu_f32_async(ctx_, pws_.gate.ptr(), pws_.up.ptr(), pws_.hid.ptr(), (size_t)rows * F));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
-            M40H_TRY(m40llm_gemm_f32xf16_gguf_f32(ctx_, pws_.hid.ptr(), w.wdown, pws_.y.ptr(), (int)rows, (int)D, (int)F));
+            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx_, pws_.hid.ptr(), w.wdown, pws_.y.ptr(), (int)rows, (int)D, (int)F, PRE));
             M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
             M40H_TRY(m40llm_residual_add_f32_async(ctx_, pws_.x1.ptr(), pws_.y.ptr(), b, (size_t)rows * D));
             std::swap(a, b);

@@ -176,6 +176,30 @@ def test_kv_append_rope_k_fused_equals_standalone(dev, orc, layout):
 
 
 # ------------------------------------------------------------------ GEMM family
+@pytest.mark.parametrize("M", [5, 200])
+def test_gemm_multi_matrix_equals_separate_calls(dev, M):
+    # Q/K/V-shaped and gate/up-shaped groups over shared activations: bit-identical to one GEMM per matrix, for few rows
+    # (one GEMM per matrix inside) and many rows (one tiled launch)
+    rng = np.random.default_rng(M)
+    K, Ns = 256, (384, 64, 136)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    Bs = [f16bits(rng.standard_normal((n, K)) * 0.05) for n in Ns]
+    dA, dB = dev.up(A), [dev.up(b) for b in Bs]
+    for n_mats in (1, 2, 3):
+        outs = [dev.zeros(M * n * 4) for n in Ns]
+        args = []
+        for i in range(3):
+            args += [dB[i].ptr, Ns[i], outs[i].ptr] if i < n_mats else [None, 0, None]
+        dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_multi_async", dA.ptr, M, K, n_mats, *args, 1)
+        dev.sync()
+        for i in range(n_mats):
+            want = dev.gemm_gguf(A, Bs[i], M, Ns[i], K)
+            assert np.array_equal(outs[i].download(np.float32, (M, Ns[i])).view(np.uint32), want.view(np.uint32)), (n_mats, i)
+    z = dev.zeros(16)
+    dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_multi_async", dA.ptr, M, K, 4, dB[0].ptr, 8, z.ptr, None, 0, None, None, 0, None, 1, expect=-2)
+    dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_multi_async", dA.ptr, M, K, 2, dB[0].ptr, 8, z.ptr, None, 8, None, None, 0, None, 1, expect=-1)
+
+
 @pytest.mark.parametrize("M,N,K", [(33, 16, 32), (100, 200, 2048), (128, 256, 2048), (300, 136, 5632), (257, 2048, 64)])
 def test_gemm_many_rows_vs_oracle(dev, orc, M, N, K):
     # the 128 x 128-tile matrix-core GEMM behind m40llm_gemm_f32xf16_gguf_f32 for M > 32 (prefill): ragged tiles in
