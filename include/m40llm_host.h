@@ -162,6 +162,44 @@ int m40host_model_decode_batch_greedy(M40HostModel* model, const uint32_t* seque
 int m40host_model_forward_prefill(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* lens,
                                   const uint32_t* tokens, uint32_t batch, float* hidden_last_host, float* logits_last_host);
 
+/* ---- continuous-batching decode scheduler (src/server.rs:203-770 without HTTP, tokenizer and channels) ---------- */
+typedef struct M40HostScheduler M40HostScheduler;
+typedef struct M40HostTickReport {
+    uint32_t prefill_rows, prefill_tokens, decode_rows, completed, cancelled, failed;
+} M40HostTickReport;
+/* Engine callbacks for a scheduler that is not tied to a model (tests, other back ends): fill one row of `vocab`
+ * logits per item; return 0, or nonzero to fail every request of the call. */
+typedef int (*m40host_sched_prefill_fn)(void* user, const uint32_t* sequence_ids, const uint32_t* lens, const uint32_t* tokens,
+                                        uint32_t batch, float* logits_out);
+typedef int (*m40host_sched_decode_fn)(void* user, const uint32_t* sequence_ids, const uint32_t* kv_lens, const uint32_t* tokens,
+                                       uint32_t rows, float* logits_out);
+/* sequence_slots 0 (or above the model's max_sequences) = the model's max_sequences.  Prompts are prefilled with the
+ * packed prefill forward when the model can (dense cache, head_dim 64 / 128), token by token otherwise; decode ticks
+ * run one batched step with the fused kernels in the model's host mode 1 / 2. */
+M40HostScheduler* m40host_scheduler_create_for_model(M40HostModel* model, uint32_t sequence_slots);
+M40HostScheduler* m40host_scheduler_create_with_engine(uint32_t vocab, uint32_t max_seq_len, uint32_t sequence_slots,
+                                                       m40host_sched_prefill_fn prefill_fn, m40host_sched_decode_fn decode_fn,
+                                                       void* user);
+void m40host_scheduler_destroy(M40HostScheduler* scheduler);
+/* enqueue_scheduler_request: leases a sequence slot (FIFO pool) or fails with "decode batching requires a sequence
+ * lease"; max_tokens < 0 = the context length; top_k < 0 / top_p <= 0 = none (top_k 1 = greedy).  Returns the request
+ * id (1, 2, ...) or -1. */
+int64_t m40host_scheduler_submit(M40HostScheduler* scheduler, const uint32_t* prompt, size_t n_prompt, int64_t max_tokens,
+                                 const uint32_t* stop_ids, size_t n_stop, float temperature, int64_t top_k, float top_p,
+                                 uint64_t seed);
+int m40host_scheduler_cancel(M40HostScheduler* scheduler, uint64_t request_id);   /* 1 if the request was active */
+/* one scheduler tick: cancelled requests leave, finished ones are reported, pending prompts are prefilled together and
+ * sample their first token, every other request takes one batched decode step */
+int m40host_scheduler_tick(M40HostScheduler* scheduler, M40HostTickReport* report);
+/* 0 unknown, 1 pending prefill, 2 decoding, 3 complete, 4 cancelled, 5 failed */
+uint32_t m40host_scheduler_state(M40HostScheduler* scheduler, uint64_t request_id);
+uint32_t m40host_scheduler_sequence_of(M40HostScheduler* scheduler, uint64_t request_id);   /* 0xffffffff when not active */
+size_t m40host_scheduler_active(M40HostScheduler* scheduler);
+size_t m40host_scheduler_available_slots(M40HostScheduler* scheduler);
+/* generated ids so far (any state): returns their number, writes at most `capacity` */
+int64_t m40host_scheduler_generated(M40HostScheduler* scheduler, uint64_t request_id, uint32_t* ids_out, size_t capacity);
+size_t m40host_scheduler_error(M40HostScheduler* scheduler, uint64_t request_id, char* buf, size_t capacity);
+
 /* ---- GGUF ingestion (src/gguf.rs:172-329, src/infer/load.rs:10-92, src/infer/tensor_views.rs:29-117,
  *      src/infer/types.rs:114-242, src/infer/mapping.rs:95-540, src/infer/embeddings.rs:14-143) -------------- */
 typedef struct M40HostGguf M40HostGguf;                 /* a parsed file header: no device, no tensor data */

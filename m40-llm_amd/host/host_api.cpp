@@ -13,6 +13,7 @@
 #include "kv_selection.hpp"
 #include "model.hpp"
 #include "sampling.hpp"
+#include "scheduler.hpp"
 
 using namespace m40host;
 
@@ -75,6 +76,9 @@ struct PlanHolder {
 
 struct M40HostModel {
     std::unique_ptr<DecodeModel> m;
+};
+struct M40HostScheduler {
+    std::unique_ptr<DecodeScheduler> s;
 };
 struct M40HostGguf {
     gguf::Model model;
@@ -499,6 +503,142 @@ M40HostModel* m40host_model_from_gguf(M40HostGgufWeights* w, uint32_t max_seq_le
             return h.release();
         },
         nullptr);
+}
+
+// ---- continuous-batching decode scheduler -----------------------------------------------------------------
+M40HostScheduler* m40host_scheduler_create_for_model(M40HostModel* model, uint32_t sequence_slots) {
+    return guarded(
+        [&]() -> M40HostScheduler* {
+            if (!model) throw std::invalid_argument("null model");
+            DecodeModel* d = model->m.get();
+            const ModelConfig& c = d->config();
+            if (sequence_slots == 0 || sequence_slots > c.max_sequences) sequence_slots = c.max_sequences;
+            SchedulerEngine e;
+            e.vocab = c.vocab;
+            e.max_seq_len = c.max_seq_len;
+            e.prefill = [d](const std::vector<SchedulerPrefillItem>& items, float* logits_out) {
+                const ModelConfig& cfg = d->config();
+                if (d->packed_prefill_available()) {
+                    for (size_t i0 = 0; i0 < items.size();) {   // at most 64 prompts and 65535 rows per packed call
+                        std::vector<uint32_t> seqs, lens, toks;
+                        size_t i = i0;
+                        while (i < items.size() && seqs.size() < 64 && toks.size() + items[i].len <= 65535u) {
+                            seqs.push_back(items[i].sequence_id);
+                            lens.push_back(items[i].len);
+                            toks.insert(toks.end(), items[i].tokens, items[i].tokens + items[i].len);
+                            ++i;
+                        }
+                        if (i == i0) throw std::invalid_argument("prompt longer than one packed prefill call takes");
+                        const float* h = d->forward_prefill(seqs.data(), lens.data(), toks.data(), (uint32_t)seqs.size());
+                        size_t row = 0;
+                        for (size_t j = 0; j < seqs.size(); ++j) {
+                            row += lens[j];
+                            d->logits_from_hidden(h + (row - 1) * cfg.d_model, logits_out + (i0 + j) * (size_t)cfg.vocab);
+                        }
+                        i0 = i;
+                    }
+                } else {   // token by token (DecodeSchedulerRequest::step, server.rs:300-329)
+                    for (size_t i = 0; i < items.size(); ++i) {
+                        const float* h = nullptr;
+                        for (uint32_t p = 0; p < items[i].len; ++p) h = d->forward_token(items[i].sequence_id, p, items[i].tokens[p]);
+                        d->logits_from_hidden(h, logits_out + i * (size_t)cfg.vocab);
+                    }
+                }
+            };
+            e.decode = [d](const std::vector<SchedulerDecodeItem>& items, float* logits_out) {
+                std::vector<uint32_t> seqs, lens, toks;
+                for (const auto& it : items) {
+                    seqs.push_back(it.sequence_id);
+                    lens.push_back(it.kv_len);
+                    toks.push_back(it.token);
+                }
+                d->batched_step_logits(seqs.data(), lens.data(), toks.data(), (uint32_t)items.size(), logits_out);
+            };
+            auto h = std::make_unique<M40HostScheduler>();
+            h->s = std::make_unique<DecodeScheduler>(std::move(e), sequence_slots);
+            return h.release();
+        },
+        nullptr);
+}
+M40HostScheduler* m40host_scheduler_create_with_engine(uint32_t vocab, uint32_t max_seq_len, uint32_t sequence_slots,
+                                                       m40host_sched_prefill_fn prefill_fn, m40host_sched_decode_fn decode_fn,
+                                                       void* user) {
+    return guarded(
+        [&]() -> M40HostScheduler* {
+            if (!prefill_fn || !decode_fn) throw std::invalid_argument("null engine callback");
+            SchedulerEngine e;
+            e.vocab = vocab;
+            e.max_seq_len = max_seq_len;
+            e.prefill = [prefill_fn, user](const std::vector<SchedulerPrefillItem>& items, float* logits_out) {
+                std::vector<uint32_t> seqs, lens, toks;
+                for (const auto& it : items) {
+                    seqs.push_back(it.sequence_id);
+                    lens.push_back(it.len);
+                    toks.insert(toks.end(), it.tokens, it.tokens + it.len);
+                }
+                if (prefill_fn(user, seqs.data(), lens.data(), toks.data(), (uint32_t)items.size(), logits_out) != 0)
+                    throw std::runtime_error("prefill callback reported an error");
+            };
+            e.decode = [decode_fn, user](const std::vector<SchedulerDecodeItem>& items, float* logits_out) {
+                std::vector<uint32_t> seqs, lens, toks;
+                for (const auto& it : items) {
+                    seqs.push_back(it.sequence_id);
+                    lens.push_back(it.kv_len);
+                    toks.push_back(it.token);
+                }
+                if (decode_fn(user, seqs.data(), lens.data(), toks.data(), (uint32_t)items.size(), logits_out) != 0)
+                    throw std::runtime_error("decode callback reported an error");
+            };
+            auto h = std::make_unique<M40HostScheduler>();
+            h->s = std::make_unique<DecodeScheduler>(std::move(e), sequence_slots);
+            return h.release();
+        },
+        nullptr);
+}
+void m40host_scheduler_destroy(M40HostScheduler* s) { delete s; }
+int64_t m40host_scheduler_submit(M40HostScheduler* s, const uint32_t* prompt, size_t n_prompt, int64_t max_tokens,
+                                 const uint32_t* stop_ids, size_t n_stop, float temperature, int64_t top_k, float top_p,
+                                 uint64_t seed) {
+    return guarded(
+        [&]() -> int64_t {
+            if (!s) throw std::invalid_argument("null scheduler");
+            SamplerConfig c;
+            c.temperature = temperature;
+            if (top_k >= 0) c.top_k = (size_t)top_k;
+            if (top_p > 0.0f) c.top_p = top_p;
+            c.seed = seed;
+            std::vector<uint32_t> stops(stop_ids, stop_ids + (stop_ids ? n_stop : 0));
+            return (int64_t)s->s->submit(prompt, n_prompt, max_tokens >= 0 ? std::optional<size_t>((size_t)max_tokens) : std::nullopt,
+                                         std::move(stops), c);
+        },
+        -1);
+}
+int m40host_scheduler_cancel(M40HostScheduler* s, uint64_t request_id) { return s && s->s->cancel(request_id) ? 1 : 0; }
+int m40host_scheduler_tick(M40HostScheduler* s, M40HostTickReport* report) {
+    return guarded(
+        [&]() -> int {
+            if (!s) throw std::invalid_argument("null scheduler");
+            const SchedulerTickReport r = s->s->tick();
+            if (report) *report = M40HostTickReport{r.prefill_rows, r.prefill_tokens, r.decode_rows, r.completed, r.cancelled, r.failed};
+            return 0;
+        },
+        -1);
+}
+uint32_t m40host_scheduler_state(M40HostScheduler* s, uint64_t request_id) { return s ? (uint32_t)s->s->state(request_id) : 0; }
+uint32_t m40host_scheduler_sequence_of(M40HostScheduler* s, uint64_t request_id) { return s ? s->s->sequence_of(request_id) : 0xffffffffu; }
+size_t m40host_scheduler_active(M40HostScheduler* s) { return s ? s->s->active() : 0; }
+size_t m40host_scheduler_available_slots(M40HostScheduler* s) { return s ? s->s->available_slots() : 0; }
+int64_t m40host_scheduler_generated(M40HostScheduler* s, uint64_t request_id, uint32_t* ids_out, size_t capacity) {
+    if (!s) return -1;
+    const std::vector<uint32_t> g = s->s->generated(request_id);
+    for (size_t i = 0; i < g.size() && i < capacity; ++i) ids_out[i] = g[i];
+    return (int64_t)g.size();
+}
+size_t m40host_scheduler_error(M40HostScheduler* s, uint64_t request_id, char* buf, size_t capacity) {
+    if (!s) return 0;
+    const std::string e = s->s->error_of(request_id);
+    put_err(buf, capacity, e);
+    return e.size();
 }
 
 }  // extern "C"

@@ -394,6 +394,7 @@ public:
     // every row, RoPE + bias + the f16 KV append run as one launch, and the attention is the packed causal prefill
     // kernel.  Each sequence starts at position 0 of its (cleared) cache slots.  Returns the hidden rows
     // [total rows][d_model] on the device; row offsets are the running sum of `lens`.
+    bool packed_prefill_available() const { return !kvcfg_.is_enabled() && (cfg_.head_dim == 64 || cfg_.head_dim == 128); }
     const float* forward_prefill(const uint32_t* seq_ids, const uint32_t* lens, const uint32_t* tokens, uint32_t batch) {
         if (batch == 0) throw std::invalid_argument("batched prefill requires at least one item");
         if (kvcfg_.is_enabled()) throw std::invalid_argument("batched prefill requires the dense KV cache");
@@ -571,7 +572,8 @@ public:
     // Per step: every layer as five fused calls on the decode stream, output norm + lm_head, then the greedy pick,
     // the length increment and the next embedding on the device.  Nothing is read back until the end.
     bool batched_fused_available(uint32_t rows) const {
-        return !kvcfg_.is_enabled() && rows >= 1 && rows <= 16 && cfg_.d_model % 256 == 0 && cfg_.ffn % 256 == 0;
+        return !kvcfg_.is_enabled() && rows >= 1 && rows <= 16 && cfg_.d_model % 256 == 0 && cfg_.ffn % 256 == 0 &&
+               (cfg_.head_dim == 64 || cfg_.head_dim == 128);   // the lengths-on-device attention serves these two
     }
     void batched_layer_fused(uint32_t l, const uint32_t* slots_dev, const uint32_t* lens_dev, uint32_t rows, uint32_t hint,
                              const float* d_x, float* d_out) {
@@ -604,6 +606,69 @@ public:
                                                       static_cast<uint32_t*>(bids_.ptr()), static_cast<float*>(bgaps_.ptr()),
                                                       tok_emb_, cfg_.d_model, hidden));
     }
+    // One decode step for `rows` sequences (token r at position kv_lens[r] of sequence seq_ids[r]) with the logits of
+    // every row brought to the host: what a serving loop that samples on the host needs per tick
+    // (forward_one_token_all_layers_batched_for_sequences + logits_after_batched_forward, src/server.rs:664-711).
+    // Fused kernels in groups of up to 16 rows when the host mode allows them, the reference's sequence otherwise.
+    void batched_step_logits(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* tokens, uint32_t rows,
+                             float* host_logits) {
+        if (rows == 0) throw std::invalid_argument("empty batch");
+        for (uint32_t r = 0; r < rows; ++r) {
+            if (kv_lens[r] + 1 > cfg_.max_seq_len) throw std::out_of_range("sequence would exceed max_seq_len");
+            if (seq_ids[r] >= cfg_.max_sequences) throw std::out_of_range("sequence id out of range");
+            if (tokens[r] >= cfg_.vocab) throw std::out_of_range("token id out of range");
+        }
+        const bool batched_attention = !kvcfg_.is_enabled() && (cfg_.head_dim == 64 || cfg_.head_dim == 128);
+        if (rows == 1 || !batched_attention) {
+            // one request, or a cache / head size the batched attention does not serve: request by request
+            // (scheduler_can_use_batched_attention -> DecodeSchedulerRequest::step, src/server.rs:457-480, 649-661)
+            for (uint32_t r = 0; r < rows; ++r) {
+                const float* h = forward_token(seq_ids[r], kv_lens[r], tokens[r]);
+                logits_from_hidden(h, host_logits + (size_t)r * cfg_.vocab);
+            }
+            return;
+        }
+        if (!(mode_ >= 1 && batched_fused_available(rows < 16 ? rows : 16))) {
+            const float* hidden = forward_batched(seq_ids, kv_lens, tokens, rows);
+            logits_from_hidden_rows(hidden, rows, host_logits);
+            return;
+        }
+        for (uint32_t r0 = 0; r0 < rows; r0 += 16) {
+            const uint32_t n = rows - r0 < 16 ? rows - r0 : 16;
+            ws_.ensure(ctx_, cfg_, n);
+            std::vector<uint32_t> table((size_t)cfg_.n_layers * n + 2 * n);   // slots per layer, then lengths, then tokens
+            uint32_t longest = 0;
+            for (uint32_t l = 0; l < cfg_.n_layers; ++l)
+                for (uint32_t r = 0; r < n; ++r) table[(size_t)l * n + r] = kv_slot(seq_ids[r0 + r], l);
+            for (uint32_t r = 0; r < n; ++r) {
+                table[(size_t)cfg_.n_layers * n + r] = kv_lens[r0 + r];
+                table[(size_t)cfg_.n_layers * n + n + r] = tokens[r0 + r];
+                longest = kv_lens[r0 + r] > longest ? kv_lens[r0 + r] : longest;
+            }
+            sync_all();   // the table buffer of the previous group may still be read
+            if (tick_table_cap_ < table.size()) {
+                tick_table_ = DeviceBuf(ctx_, table.size() * 4);
+                tick_table_cap_ = table.size();
+            }
+            M40H_TRY(m40llm_memcpy_h2d(ctx_, tick_table_.ptr(), table.data(), table.size() * 4));
+            const uint32_t* slots = tick_table_.u32();
+            const uint32_t* lens = tick_table_.u32((size_t)cfg_.n_layers * n);
+            const uint32_t* toks = tick_table_.u32((size_t)cfg_.n_layers * n + n);
+            float* a = ws_.scratch_a.f32();
+            float* b = ws_.scratch_b.f32();
+            M40H_TRY(m40llm_ext_embed_rows_async(ctx_, tok_emb_, toks, n, cfg_.vocab, cfg_.d_model, a));
+            const uint32_t hint = len_hint_for(longest);
+            for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
+                batched_layer_fused(l, slots + (size_t)l * n, lens, n, hint, a, b);
+                std::swap(a, b);
+            }
+            M40H_TRY(m40llm_ext_batched_norm_gemm_f32xf16_async(ctx_, a, out_norm_, cfg_.norm_weight_dtype, cfg_.rms_eps, lm_head_,
+                                                                ws_.logits.ptr(), n, (int)cfg_.vocab, (int)cfg_.d_model));
+            M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
+            M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits + (size_t)r0 * cfg_.vocab, ws_.logits.ptr(), (size_t)n * cfg_.vocab * 4));
+        }
+    }
+
     // Returns false when a pick was a near-tie (the caller then repeats the decode on the host-sampled path).
     bool decode_batch_device(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens, uint32_t rows,
                              uint32_t warmup, uint32_t steps, uint32_t* ids_out, float* gaps_out, double* elapsed_ms) {
@@ -838,6 +903,8 @@ private:
     static constexpr uint32_t kTop2Capacity = 1u << 16;
     uint32_t state_cap_ = 0;
     DeviceBuf bslots_, blens_, bstate_, bids_, bgaps_;
+    DeviceBuf tick_table_;
+    size_t tick_table_cap_ = 0;
     M40llmCudaGraphExec* bgraph_ = nullptr;
     uint32_t bgraph_rows_ = 0, bgraph_hint_ = 0;
     M40llmCudaGraphExec* graph_ = nullptr;
