@@ -1,6 +1,6 @@
 """Per-kernel throughput of the decode hot path on one MI355X, against the HBM roofline.
 
-    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN] [--json out.jsonl]
+    python m40-llm_amd/kernel_bench.py [--only read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN,sched] [--json out.jsonl]
 
 Every case launches through the C-ABI library on its decode (or prefill) stream and is timed with
 events recorded on that same stream: `reps` launches between two events, inputs rotated over enough
@@ -272,6 +272,45 @@ def bench_prefill_forward(b: Bench):
     dm.close()
 
 
+def bench_scheduler(b: Bench):
+    """Continuous batching end to end (TinyLlama-1.1B shape, synthetic weights): 32 requests with prompts of 64-512
+    tokens and 64 new tokens each through 8 sequence slots, host-sampled greedy; beside the same requests served one
+    after the other on one slot."""
+    import time
+    syn = importlib.import_module("m40-llm_amd.synthetic")
+    sch = importlib.import_module("m40-llm_amd.scheduler")
+    cfg = dict(syn.TINYLLAMA_1B)
+    W = syn.make_weights(cfg, seed=0, unique_layers=2, std=0.02, emb_std=1.0)
+    dm = syn.DeviceModel(b.ctx, cfg, W, max_seq_len=1024, max_sequences=8)
+    del W
+    dm.set_mode(2)
+    rng = np.random.default_rng(1)
+    reqs = [rng.integers(0, cfg["vocab"], size=int(n)).tolist() for n in rng.integers(64, 513, size=32)]
+    new_tokens = 64
+    for label, slots in (("8 slots, continuous batching", 8), ("1 slot, one request at a time", 1)):
+        s = sch.Scheduler.for_model(dm, slots)
+        pending = list(reqs)
+        warm = s.submit(reqs[0][:16], max_tokens=4)          # graph capture, workspaces
+        s.run_until_idle()
+        assert s.state(warm) == "complete"
+        t0 = time.perf_counter()
+        ticks = 0
+        while pending or s.active():
+            while pending and s.available_slots():
+                s.submit(pending.pop(0), max_tokens=new_tokens)
+            s.tick()
+            ticks += 1
+        dt = time.perf_counter() - t0
+        gen = len(reqs) * new_tokens
+        prompt_tokens = sum(len(r) for r in reqs)
+        b.rows.append(dict(kernel="decode scheduler, TinyLlama-1.1B shape", shape=label, requests=len(reqs), prompt_tokens=prompt_tokens,
+                           generated=gen, seconds=round(dt, 3), generated_tok_s=round(gen / dt, 1), ticks=ticks))
+        print(f"{'decode scheduler':34s} {label:44s} {dt * 1e3:9.1f} ms {gen / dt:10.1f} generated tok/s   ({len(reqs)} requests, "
+              f"{prompt_tokens} prompt tokens, {ticks} ticks)", flush=True)
+        s.close()
+    dm.close()
+
+
 def bench_gemv(b: Bench, M: int):
     rng = np.random.default_rng(1)
     shapes = [(2048, 2048), (256, 2048), (5632, 2048), (2048, 5632), (32000, 2048)] if M == 1 else \
@@ -397,7 +436,7 @@ def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN")
+    ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN,sched")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
     args = ap.parse_args()
@@ -426,6 +465,8 @@ def main():
         bench_gemm_many_rows(b)
     if "pfwd" in which:
         bench_prefill_forward(b)
+    if "sched" in which:
+        bench_scheduler(b)
     if args.json:
         with open(args.json, "w") as f:
             for r in b.rows:
