@@ -1,18 +1,23 @@
-// Packed variable-length causal prefill attention for gfx950, all f32 (the step before decode).
+// Packed variable-length causal prefill attention for gfx950, f32 in and out (the step before decode).
 //
 // Q and Out are [total_q][q_heads][hd], K and V [total_kv][kv_heads][hd]; sequence b owns q_lens[b] query tokens from
 // q_offsets[b] and kv_lens[b] keys from kv_offsets[b]; query q_idx attends keys 0 .. kv_len - q_len + q_idx.
 //
 // The reference walks every key once per (query, head) with one workgroup each (cuda/kernels.cu:3749-3835).  Here a
 // workgroup owns 64 consecutive queries of one q head (four waves x 16 queries) and streams the sequence's keys in
-// tiles of 32 through LDS, so a key row is fetched once per 64 queries.  Both products run on the f32 matrix
-// instruction v_mfma_f32_16x16x4_f32 (inputs stay f32: no split, no rounding of K or V):
-//   scores  S[query][key] = sum_d Q[query][d] K[key][d]   A = Q (kept in registers for the whole kernel), B = K tile
-//   output  O[query][d]  += sum_key P[query][key] V[key][d]   A = softmax weights (through a 2 KB LDS tile per wave,
-//           which turns the accumulator layout into the A-operand layout), B = V tile
+// tiles of 32 through LDS, so a key row is fetched once per 64 queries.  Both products run on v_mfma_f32_16x16x32_f16
+// with every f32 operand split exactly into an f16 high and an f16 low part (x = hi + lo to 2^-22): a product is
+// three instructions, hi hi + lo hi + hi lo (the lo lo term is below 2^-22 of the operands' magnitudes), which is
+// five times the rate of the f32 matrix instruction for the same product at f32-level accuracy:
+//   scores  S[query][key] = sum_d Q[query][d] K[key][d]   A = Q (two f16 parts, in registers for the whole kernel),
+//           B = K tile (two f16 planes in LDS)
+//   output  O[query][d]  += sum_key P[query][key] V[key][d]   A = softmax weights (two f16 planes through a small LDS
+//           tile per wave, which turns the accumulator layout into the A-operand layout), B = V tile, stored
+//           transposed [d][key] so that eight consecutive keys are one 16-byte read
 // with a running maximum per query (the rows of a lane's accumulators are the same four queries in both products,
 // so the rescaling needs no exchange).  The result is the same softmax as the reference's three passes
-// (p = exp(s - max) / sum), within f32 rounding.
+// (p = exp(s - max) / sum), within f32 rounding.  Operands beyond the f16 range (|x| > 65504) are not supported by the
+// split (none occur after RMSNorm-scaled projections; the decode-side attention has no such limit).
 //
 // Reference: kernel cuda/kernels.cu:3749-3835; entry points, argument checks and their codes :4834-4977
 // (lengths are read back to the host and validated before the launch, also in the _async form).
@@ -25,10 +30,14 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kQTile = 16 * kWaves;      // queries per workgroup
-constexpr int kKTile = 32;               // keys per LDS tile
+constexpr int kKTile = 32;               // keys per LDS tile = the K depth of one matrix instruction of the P . V product
 
-__device__ __forceinline__ m40_float4 mfma16x16x4(float a, float b, m40_float4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ m40_float4 mfma32(half8 a, half8 b, m40_float4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 __device__ __forceinline__ float row_max16(float x) {     // over the 16 lanes of a row group
     x = fmaxf(x, m40_dpp_f<M40_DPP_XOR1>(x));
@@ -36,6 +45,12 @@ __device__ __forceinline__ float row_max16(float x) {     // over the 16 lanes o
     x = fmaxf(x, m40_dpp_f<M40_DPP_HALF_MIRROR>(x));
     x = fmaxf(x, m40_dpp_f<M40_DPP_MIRROR>(x));
     return x;
+}
+// x = hi + lo with both parts f16: exact to about 2^-22 relative for values inside the f16 range
+__device__ __forceinline__ void split(float x, _Float16* hi, _Float16* lo) {
+    const _Float16 h = static_cast<_Float16>(x);
+    *hi = h;
+    *lo = static_cast<_Float16>(x - static_cast<float>(h));
 }
 
 struct PrefillArgs {
@@ -46,15 +61,16 @@ struct PrefillArgs {
 
 template <int HD>
 __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
-    constexpr int KS = HD / 4;             // MFMA k-steps of a score tile
+    constexpr int KS = HD / 32;            // matrix-instruction k-steps of a score tile
     constexpr int DT = HD / 16;            // 16-column output tiles
-    constexpr int KSTR = HD + 4;           // LDS floats per K row: key j, group g -> bank 4 j + g
-    constexpr int VSTR = HD + 16;          // LDS floats per V row: key group g, column j -> bank 16 g + j
-    constexpr int PSTR = kKTile + 4;       // LDS floats per row of a wave's weight tile
-    constexpr int LD4 = kKTile * HD / 4 / kThreads;      // float4 loads per thread and tile, for K and for V
-    __shared__ __attribute__((aligned(16))) float k_lds[kKTile * KSTR];
-    __shared__ __attribute__((aligned(16))) float v_lds[kKTile * VSTR];
-    __shared__ float p_lds[kWaves][16 * PSTR];
+    constexpr int KSTR = HD + 8;           // LDS halves per K row: 16-byte fragment reads of 16 keys hit 64 distinct banks
+    constexpr int VSTR = kKTile + 8;       // LDS halves per row of the transposed V tile [column][key]
+    constexpr int PSTR = kKTile + 8;       // LDS halves per row of a wave's weight tile
+    constexpr int KLD = kKTile * HD / 4 / kThreads;        // float4 loads of K per thread and tile
+    constexpr int VLD = kKTile / 2 * HD / 4 / kThreads;    // key pairs x float4 columns of V per thread and tile
+    __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][kKTile * KSTR];   // [hi, lo][key][d]
+    __shared__ __attribute__((aligned(16))) _Float16 v_lds[2][HD * VSTR];       // [hi, lo][d][key]
+    __shared__ __attribute__((aligned(16))) _Float16 p_lds[kWaves][2][16 * PSTR];
 
     const uint32_t b = blockIdx.z, h = blockIdx.y;
     const uint32_t q_len = p.q_lens[b], kv_len = p.kv_lens[b];
@@ -68,15 +84,26 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     const uint32_t wg_last_q = q0 + kQTile - 1 < q_len - 1 ? q0 + kQTile - 1 : q_len - 1;
     const uint32_t n_tiles = (shift + wg_last_q) / kKTile + 1;    // key tiles this workgroup walks
 
-    // ---- this wave's 16 queries: A operand of the score product, lane (query j, k group g) holds Q[j][4 s + g]
+    // ---- this wave's 16 queries: A operand of the score product, lane (query j, k group g) holds
+    //      Q[j][32 s + 8 g .. + 7] as a high and a low f16 part
     const uint32_t wq0 = q0 + 16u * wave;                         // first query of the wave
     const bool wave_live = wq0 < q_len;
     const uint32_t my_q = wq0 + j < q_len ? wq0 + j : q_len - 1;  // a query past the end repeats the last one (not stored)
-    float qa[KS];
+    half8 qh[KS], ql[KS];
     {
-        const float* qp = p.Q + ((size_t)(p.q_offsets[b] + my_q) * p.q_heads + h) * HD + g;
+        const float* qp = p.Q + ((size_t)(p.q_offsets[b] + my_q) * p.q_heads + h) * HD + 8 * g;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) qa[s] = qp[4 * s];
+        for (int s = 0; s < KS; ++s) {
+            const float4 x0 = *reinterpret_cast<const float4*>(qp + 32 * s), x1 = *reinterpret_cast<const float4*>(qp + 32 * s + 4);
+            const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                _Float16 a, c;
+                split(x[i], &a, &c);
+                qh[s][i] = a;
+                ql[s][i] = c;
+            }
+        }
     }
     // queries of this lane's accumulator rows: 4 g + r; their last visible key
     uint32_t row_end[4];
@@ -87,31 +114,68 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     }
     const uint32_t wave_end = shift + (wq0 + 15u < q_len ? wq0 + 15u : q_len - 1);    // last key any query of the wave sees
 
-    // ---- K / V tile loads: thread t moves float4 t, t + 256, ... of the tile's [32][HD] block
+    // ---- K / V tile loads.  K: thread t moves float4 t, t + 256, ... of the tile's [32][HD] block.  V: a thread takes
+    //      the same four columns of two adjacent keys, so that the transposed tile is written two keys (one 32-bit
+    //      word) at a time.
     const float* Kb = p.K + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
     const float* Vb = p.V + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
     const size_t row_stride = (size_t)p.kv_heads * HD;
-    float4 kreg[LD4], vreg[LD4];
+    float4 kreg[KLD], vreg[VLD][2];
     auto issue = [&](uint32_t tile) {
 #pragma unroll
-        for (int u = 0; u < LD4; ++u) {
+        for (int u = 0; u < KLD; ++u) {
             const int f = u * kThreads + tid;                     // float4 index inside the tile
             const uint32_t key_in = (uint32_t)(f / (HD / 4)), c4 = (uint32_t)(f % (HD / 4));
             uint32_t key = tile * kKTile + key_in;
             key = key < kv_len ? key : kv_len - 1;                // past the sequence: a valid row, masked later
             kreg[u] = *reinterpret_cast<const float4*>(Kb + (size_t)key * row_stride + 4 * c4);
-            vreg[u] = *reinterpret_cast<const float4*>(Vb + (size_t)key * row_stride + 4 * c4);
+        }
+#pragma unroll
+        for (int u = 0; u < VLD; ++u) {
+            const int f = u * kThreads + tid;
+            const uint32_t pair = (uint32_t)(f / (HD / 4)), c4 = (uint32_t)(f % (HD / 4));
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                uint32_t key = tile * kKTile + 2u * pair + (uint32_t)e;
+                key = key < kv_len ? key : kv_len - 1;
+                vreg[u][e] = *reinterpret_cast<const float4*>(Vb + (size_t)key * row_stride + 4 * c4);
+            }
         }
     };
     auto to_lds = [&]() {
 #pragma unroll
-        for (int u = 0; u < LD4; ++u) {
+        for (int u = 0; u < KLD; ++u) {
             const int f = u * kThreads + tid;
             const int key_in = f / (HD / 4), c4 = f % (HD / 4);
-            float* kd = k_lds + key_in * KSTR + 4 * c4;
-            kd[0] = kreg[u].x; kd[1] = kreg[u].y; kd[2] = kreg[u].z; kd[3] = kreg[u].w;
-            float* vd = v_lds + key_in * VSTR + 4 * c4;
-            vd[0] = vreg[u].x; vd[1] = vreg[u].y; vd[2] = vreg[u].z; vd[3] = vreg[u].w;
+            const float x[4] = {kreg[u].x, kreg[u].y, kreg[u].z, kreg[u].w};
+            half4 hi, lo;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                _Float16 a, c;
+                split(x[i], &a, &c);
+                hi[i] = a;
+                lo[i] = c;
+            }
+            *reinterpret_cast<half4*>(&k_lds[0][key_in * KSTR + 4 * c4]) = hi;
+            *reinterpret_cast<half4*>(&k_lds[1][key_in * KSTR + 4 * c4]) = lo;
+        }
+#pragma unroll
+        for (int u = 0; u < VLD; ++u) {
+            const int f = u * kThreads + tid;
+            const int pair = f / (HD / 4), c4 = f % (HD / 4);
+            const float x0[4] = {vreg[u][0].x, vreg[u][0].y, vreg[u][0].z, vreg[u][0].w};
+            const float x1[4] = {vreg[u][1].x, vreg[u][1].y, vreg[u][1].z, vreg[u][1].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                half2v hi, lo;
+                _Float16 a, c;
+                split(x0[i], &a, &c);
+                hi[0] = a; lo[0] = c;
+                split(x1[i], &a, &c);
+                hi[1] = a; lo[1] = c;
+                *reinterpret_cast<half2v*>(&v_lds[0][(4 * c4 + i) * VSTR + 2 * pair]) = hi;
+                *reinterpret_cast<half2v*>(&v_lds[1][(4 * c4 + i) * VSTR + 2 * pair]) = lo;
+            }
         }
     };
     issue(0);
@@ -122,7 +186,8 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     for (int r = 0; r < 4; ++r) { m_run[r] = -INFINITY; l_run[r] = 0.0f; }
 #pragma unroll
     for (int d = 0; d < DT; ++d) O[d] = m40_float4{0.f, 0.f, 0.f, 0.f};
-    float* my_p = p_lds[wave];
+    _Float16* my_ph = p_lds[wave][0];
+    _Float16* my_pl = p_lds[wave][1];
 
     for (uint32_t tile = 0; tile < n_tiles; ++tile) {
         __syncthreads();                  // the previous tile has been read by every wave
@@ -132,14 +197,24 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         const uint32_t key0 = tile * kKTile;
         if (!wave_live || key0 > wave_end) continue;              // nothing of this tile is visible to the wave
 
-        // scores of the two 16-key halves: lane (key j, g) gets rows 4 g + r
+        // scores of the two 16-key halves: lane (key j, g) gets rows 4 g + r.  q . k = qh kh + ql kh + qh kl
+        // (the ql kl term is below 2^-22 of |q| |k|)
         m40_float4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            s0 = mfma16x16x4(qa[s], k_lds[j * KSTR + 4 * s + g], s0);
-            s1 = mfma16x16x4(qa[s], k_lds[(16 + j) * KSTR + 4 * s + g], s1);
+            const int off = 32 * s + 8 * g;
+            const half8 k0h = *reinterpret_cast<const half8*>(&k_lds[0][j * KSTR + off]);
+            const half8 k0l = *reinterpret_cast<const half8*>(&k_lds[1][j * KSTR + off]);
+            const half8 k1h = *reinterpret_cast<const half8*>(&k_lds[0][(16 + j) * KSTR + off]);
+            const half8 k1l = *reinterpret_cast<const half8*>(&k_lds[1][(16 + j) * KSTR + off]);
+            s0 = mfma32(qh[s], k0h, s0);
+            s1 = mfma32(qh[s], k1h, s1);
+            s0 = mfma32(ql[s], k0h, s0);
+            s1 = mfma32(ql[s], k1h, s1);
+            s0 = mfma32(qh[s], k0l, s0);
+            s1 = mfma32(qh[s], k1l, s1);
         }
-        float p0[4], p1[4], f[4];
+        float f[4];
         bool moved = false;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -148,13 +223,18 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             const float n = fmaxf(m_run[r], row_max16(fmaxf(x0, x1)));
             // no maximum yet: the old state weighs nothing; a masked key weighs nothing
             f[r] = m_run[r] == -INFINITY ? 0.0f : __expf(m_run[r] - n);
-            p0[r] = a0 ? __expf(x0 - n) : 0.0f;
-            p1[r] = a1 ? __expf(x1 - n) : 0.0f;
-            l_run[r] = fmaf(l_run[r], f[r], p0[r] + p1[r]);
+            const float p0 = a0 ? __expf(x0 - n) : 0.0f;
+            const float p1 = a1 ? __expf(x1 - n) : 0.0f;
+            l_run[r] = fmaf(l_run[r], f[r], p0 + p1);
             moved = moved || m_run[r] != n;
             m_run[r] = n;
-            my_p[(4 * g + r) * PSTR + j] = p0[r];
-            my_p[(4 * g + r) * PSTR + 16 + j] = p1[r];
+            _Float16 a, c;
+            split(p0, &a, &c);
+            my_ph[(4 * g + r) * PSTR + j] = a;
+            my_pl[(4 * g + r) * PSTR + j] = c;
+            split(p1, &a, &c);
+            my_ph[(4 * g + r) * PSTR + 16 + j] = a;
+            my_pl[(4 * g + r) * PSTR + 16 + j] = c;
         }
         if (__any(moved)) {               // the accumulators are only rescaled when some row's maximum rose
 #pragma unroll
@@ -163,15 +243,18 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
                 for (int r = 0; r < 4; ++r) O[d][r] *= f[r];
         }
         __builtin_amdgcn_wave_barrier();
-        // O += P . V: A = P[query j][key 4 s + g], B = V[key 4 s + g][column 16 d + j]
-        float pa[kKTile / 4];
-#pragma unroll
-        for (int s = 0; s < kKTile / 4; ++s) pa[s] = my_p[j * PSTR + 4 * s + g];
+        // O += P . V over the tile's 32 keys in one k-step: A = P[query j][key 8 g .. + 7], B = V^T[column 16 d + j][key 8 g .. + 7];
+        // p v = ph vh + pl vh + ph vl
+        const half8 ph = *reinterpret_cast<const half8*>(&my_ph[j * PSTR + 8 * g]);
+        const half8 pl = *reinterpret_cast<const half8*>(&my_pl[j * PSTR + 8 * g]);
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
-#pragma unroll
-            for (int s = 0; s < kKTile / 4; ++s) O[d] = mfma16x16x4(pa[s], v_lds[(4 * s + g) * VSTR + 16 * d + j], O[d]);
+            const half8 vh = *reinterpret_cast<const half8*>(&v_lds[0][(16 * d + j) * VSTR + 8 * g]);
+            const half8 vl = *reinterpret_cast<const half8*>(&v_lds[1][(16 * d + j) * VSTR + 8 * g]);
+            O[d] = mfma32(ph, vh, O[d]);
+            O[d] = mfma32(pl, vh, O[d]);
+            O[d] = mfma32(ph, vl, O[d]);
         }
     }
 

@@ -596,9 +596,11 @@ def test_prefill_varlen_random_vs_oracle(dev, orc, qh, kvh, hd, ql, kl):
     assert rc == 0
     got = _prefill_call(dev, orc, q, k, v, ql, kl, qh, kvh, hd, sync_form=False)
     close(got, want)
-    # the first query of a full prefill sees one key: that V row, exactly
+    # the first query of a full prefill sees one key: that V row, to what the two-part f16 split of V carries
+    # (22 bits, and no finer than the f16 subnormal spacing 2^-24 for the low part)
     if ql[0] == kl[0]:
-        assert np.array_equal(got[0], np.repeat(v[0], qh // kvh, axis=0))
+        want0 = np.repeat(v[0], qh // kvh, axis=0)
+        assert np.all(np.abs(got[0] - want0) <= 2.0 ** -22 * np.abs(want0) + 2.0 ** -24)
 
 
 def test_prefill_varlen_argument_checks(dev, orc):
