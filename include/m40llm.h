@@ -320,7 +320,9 @@ int m40llm_ext_kvcache_bulk_fill_f16(M40llmCudaContext* ctx, M40llmKVCache* kv, 
  * keys 0 .. kv_len - q_len + q_idx.  Prefill stream.  The lengths are read back and validated on the host before the
  * launch in both forms, as in the reference; only the first form waits for the kernel.
  * -1 null argument, -2 batch 0, -3 head counts, -9 head_dim not 64 / 128, -7 read-back failed,
- * -8 a length is 0, q_len > kv_len or kv_len > 8192, -4 launch (or 16-byte misaligned Q/K/V), -5 synchronise. */
+ * -8 a length is 0, q_len > kv_len or kv_len > 8192, or the key ranges of the sequences are not laid out one after the
+ * other in batch order (kv_offsets[b + 1] >= kv_offsets[b] + kv_lens[b]: how packed batches are built; this
+ * implementation packs K and V by sequence), -4 launch, allocation or 16-byte misaligned Q/K/V, -5 synchronise. */
 int m40llm_attention_prefill_f32_gqa_varlen(M40llmCudaContext* ctx, const void* q_dev_f32, const void* k_dev_f32,
                                             const void* v_dev_f32, const uint32_t* q_offsets_dev,
                                             const uint32_t* kv_offsets_dev, const uint32_t* q_lens_dev,

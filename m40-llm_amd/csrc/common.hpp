@@ -31,6 +31,8 @@ struct M40StreamScratch {
     size_t select_bytes;
     void* tiled_pack;        // f16 high / low planes of the activations of the many-row GEMM; grown on demand
     size_t tiled_pack_bytes;
+    void* attn_planes;       // f16 high / low planes of K and V^T for the prefill attention; grown on demand
+    size_t attn_planes_bytes;
 };
 
 struct M40llmCudaContext {

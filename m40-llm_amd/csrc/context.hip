@@ -25,6 +25,7 @@ void free_scratch(M40StreamScratch& s) {
     if (s.attn_partial) (void)hipFree(s.attn_partial);
     if (s.select) (void)hipFree(s.select);
     if (s.tiled_pack) (void)hipFree(s.tiled_pack);
+    if (s.attn_planes) (void)hipFree(s.attn_planes);
     s = M40StreamScratch{};
 }
 

@@ -55,9 +55,50 @@ __device__ __forceinline__ void split(float x, _Float16* hi, _Float16* lo) {
 
 struct PrefillArgs {
     const float* Q; const float* K; const float* V; float* Out;
+    const _Float16* planes;     // per padded 32-key tile and kv head: K hi [32][HD], K lo, V^T hi [HD][32], V^T lo
+    uint32_t plane_tiles;       // padded tiles in total (sequence b starts at tile kv_offsets[b] / 32 + b ... see pack)
     const uint32_t* q_offsets; const uint32_t* kv_offsets; const uint32_t* q_lens; const uint32_t* kv_lens;
     uint32_t q_heads, kv_heads;
 };
+
+// First padded tile of sequence b in the packed planes: every sequence starts on a tile boundary of its own, so a
+// sequence gets one tile of slack (rows_before / 32 rounded down, plus b).
+__device__ __forceinline__ uint32_t first_tile_of(uint32_t kv_offset, uint32_t b) { return kv_offset / kKTile + b; }
+
+// K and V of one 32-key tile and kv head -> two f16 planes each, V transposed, in the order the attention kernel copies
+// them to LDS.  Done once per call so that the 64-query workgroups (and the q heads of a group) do not each repeat the
+// split.  Keys past the sequence end are written as zeros (they are masked anyway).
+template <int HD>
+__global__ __launch_bounds__(kThreads) void prefill_pack_kv_kernel(PrefillArgs p) {
+    __shared__ float vt[kKTile][HD + 1];
+    const uint32_t b = blockIdx.z, kvh = blockIdx.y, tile = blockIdx.x;
+    const uint32_t kv_len = p.kv_lens[b];
+    if (tile * kKTile >= kv_len) return;
+    const float* Kb = p.K + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
+    const float* Vb = p.V + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
+    const size_t row_stride = (size_t)p.kv_heads * HD;
+    _Float16* out = const_cast<_Float16*>(p.planes) + ((size_t)(first_tile_of(p.kv_offsets[b], b) + tile) * p.kv_heads + kvh) * (4 * kKTile * HD);
+    _Float16* kh = out, *kl = out + kKTile * HD, *vh = out + 2 * kKTile * HD, *vl = out + 3 * kKTile * HD;
+    for (int e = threadIdx.x; e < kKTile * HD; e += kThreads) {
+        const int key_in = e / HD, d = e % HD;
+        const uint32_t key = tile * kKTile + key_in;
+        const bool live = key < kv_len;
+        const float kx = live ? Kb[(size_t)key * row_stride + d] : 0.0f;
+        vt[key_in][d] = live ? Vb[(size_t)key * row_stride + d] : 0.0f;
+        _Float16 a, c;
+        split(kx, &a, &c);
+        kh[e] = a;
+        kl[e] = c;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < kKTile * HD; e += kThreads) {
+        const int d = e / kKTile, key_in = e % kKTile;
+        _Float16 a, c;
+        split(vt[key_in][d], &a, &c);
+        vh[e] = a;
+        vl[e] = c;
+    }
+}
 
 template <int HD>
 __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
@@ -66,8 +107,6 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     constexpr int KSTR = HD + 8;           // LDS halves per K row: 16-byte fragment reads of 16 keys hit 64 distinct banks
     constexpr int VSTR = kKTile + 8;       // LDS halves per row of the transposed V tile [column][key]
     constexpr int PSTR = kKTile + 8;       // LDS halves per row of a wave's weight tile
-    constexpr int KLD = kKTile * HD / 4 / kThreads;        // float4 loads of K per thread and tile
-    constexpr int VLD = kKTile / 2 * HD / 4 / kThreads;    // key pairs x float4 columns of V per thread and tile
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][kKTile * KSTR];   // [hi, lo][key][d]
     __shared__ __attribute__((aligned(16))) _Float16 v_lds[2][HD * VSTR];       // [hi, lo][d][key]
     __shared__ __attribute__((aligned(16))) _Float16 p_lds[kWaves][2][16 * PSTR];
@@ -114,67 +153,34 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     }
     const uint32_t wave_end = shift + (wq0 + 15u < q_len ? wq0 + 15u : q_len - 1);    // last key any query of the wave sees
 
-    // ---- K / V tile loads.  K: thread t moves float4 t, t + 256, ... of the tile's [32][HD] block.  V: a thread takes
-    //      the same four columns of two adjacent keys, so that the transposed tile is written two keys (one 32-bit
-    //      word) at a time.
-    const float* Kb = p.K + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
-    const float* Vb = p.V + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
-    const size_t row_stride = (size_t)p.kv_heads * HD;
-    float4 kreg[KLD], vreg[VLD][2];
+    // ---- K / V tile loads: 16-byte pieces of the packed f16 planes (prefill_pack_kv_kernel), straight into LDS
+    constexpr int PIECES = kKTile * HD / 8 / kThreads;           // per plane and thread: 1 (HD 64) or 2 (HD 128)
+    const _Float16* tile_base = p.planes + ((size_t)first_tile_of(p.kv_offsets[b], b) * p.kv_heads + kvh) * (4 * kKTile * HD);
+    const size_t tile_stride = (size_t)p.kv_heads * (4 * kKTile * HD);
+    uint4 kreg[2][PIECES], vreg[2][PIECES];
     auto issue = [&](uint32_t tile) {
+        const _Float16* t = tile_base + (size_t)tile * tile_stride;
 #pragma unroll
-        for (int u = 0; u < KLD; ++u) {
-            const int f = u * kThreads + tid;                     // float4 index inside the tile
-            const uint32_t key_in = (uint32_t)(f / (HD / 4)), c4 = (uint32_t)(f % (HD / 4));
-            uint32_t key = tile * kKTile + key_in;
-            key = key < kv_len ? key : kv_len - 1;                // past the sequence: a valid row, masked later
-            kreg[u] = *reinterpret_cast<const float4*>(Kb + (size_t)key * row_stride + 4 * c4);
-        }
+        for (int u = 0; u < PIECES; ++u) {
+            const int c = u * kThreads + tid;
 #pragma unroll
-        for (int u = 0; u < VLD; ++u) {
-            const int f = u * kThreads + tid;
-            const uint32_t pair = (uint32_t)(f / (HD / 4)), c4 = (uint32_t)(f % (HD / 4));
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                uint32_t key = tile * kKTile + 2u * pair + (uint32_t)e;
-                key = key < kv_len ? key : kv_len - 1;
-                vreg[u][e] = *reinterpret_cast<const float4*>(Vb + (size_t)key * row_stride + 4 * c4);
+            for (int pl = 0; pl < 2; ++pl) {
+                kreg[pl][u] = *reinterpret_cast<const uint4*>(t + pl * kKTile * HD + 8 * c);
+                vreg[pl][u] = *reinterpret_cast<const uint4*>(t + (2 + pl) * kKTile * HD + 8 * c);
             }
         }
     };
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     auto to_lds = [&]() {
 #pragma unroll
-        for (int u = 0; u < KLD; ++u) {
-            const int f = u * kThreads + tid;
-            const int key_in = f / (HD / 4), c4 = f % (HD / 4);
-            const float x[4] = {kreg[u].x, kreg[u].y, kreg[u].z, kreg[u].w};
-            half4 hi, lo;
+        for (int u = 0; u < PIECES; ++u) {
+            const int c = u * kThreads + tid;
+            const int key_in = c / (HD / 8), kpart = c % (HD / 8);     // K plane [key][HD]
+            const int d = c / (kKTile / 8), vpart = c % (kKTile / 8);  // V^T plane [d][32 keys]
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                _Float16 a, c;
-                split(x[i], &a, &c);
-                hi[i] = a;
-                lo[i] = c;
-            }
-            *reinterpret_cast<half4*>(&k_lds[0][key_in * KSTR + 4 * c4]) = hi;
-            *reinterpret_cast<half4*>(&k_lds[1][key_in * KSTR + 4 * c4]) = lo;
-        }
-#pragma unroll
-        for (int u = 0; u < VLD; ++u) {
-            const int f = u * kThreads + tid;
-            const int pair = f / (HD / 4), c4 = f % (HD / 4);
-            const float x0[4] = {vreg[u][0].x, vreg[u][0].y, vreg[u][0].z, vreg[u][0].w};
-            const float x1[4] = {vreg[u][1].x, vreg[u][1].y, vreg[u][1].z, vreg[u][1].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                half2v hi, lo;
-                _Float16 a, c;
-                split(x0[i], &a, &c);
-                hi[0] = a; lo[0] = c;
-                split(x1[i], &a, &c);
-                hi[1] = a; lo[1] = c;
-                *reinterpret_cast<half2v*>(&v_lds[0][(4 * c4 + i) * VSTR + 2 * pair]) = hi;
-                *reinterpret_cast<half2v*>(&v_lds[1][(4 * c4 + i) * VSTR + 2 * pair]) = lo;
+            for (int pl = 0; pl < 2; ++pl) {
+                *reinterpret_cast<u32x4*>(&k_lds[pl][key_in * KSTR + 8 * kpart]) = u32x4{kreg[pl][u].x, kreg[pl][u].y, kreg[pl][u].z, kreg[pl][u].w};
+                *reinterpret_cast<u32x4*>(&v_lds[pl][d * VSTR + 8 * vpart]) = u32x4{vreg[pl][u].x, vreg[pl][u].y, vreg[pl][u].z, vreg[pl][u].w};
             }
         }
     };
@@ -214,20 +220,19 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             s0 = mfma32(qh[s], k0l, s0);
             s1 = mfma32(qh[s], k1l, s1);
         }
-        float f[4];
+        float f[4], psum[4];
         bool moved = false;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const bool a0 = key0 + (uint32_t)j <= row_end[r], a1 = key0 + 16u + (uint32_t)j <= row_end[r];
             const float x0 = a0 ? s0[r] * inv_sqrt : -INFINITY, x1 = a1 ? s1[r] * inv_sqrt : -INFINITY;
             const float n = fmaxf(m_run[r], row_max16(fmaxf(x0, x1)));
-            // no maximum yet: the old state weighs nothing; a masked key weighs nothing
-            f[r] = m_run[r] == -INFINITY ? 0.0f : __expf(m_run[r] - n);
-            const float p0 = a0 ? __expf(x0 - n) : 0.0f;
+            const float p0 = a0 ? __expf(x0 - n) : 0.0f;                 // a masked key weighs nothing
             const float p1 = a1 ? __expf(x1 - n) : 0.0f;
-            l_run[r] = fmaf(l_run[r], f[r], p0 + p1);
             moved = moved || m_run[r] != n;
+            f[r] = m_run[r];                                             // the old maximum, turned into a factor below
             m_run[r] = n;
+            psum[r] = p0 + p1;
             _Float16 a, c;
             split(p0, &a, &c);
             my_ph[(4 * g + r) * PSTR + j] = a;
@@ -236,12 +241,20 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             my_ph[(4 * g + r) * PSTR + 16 + j] = a;
             my_pl[(4 * g + r) * PSTR + 16 + j] = c;
         }
-        if (__any(moved)) {               // the accumulators are only rescaled when some row's maximum rose
+        if (__any(moved)) {               // sums and accumulators are only rescaled when some row's maximum rose
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // no maximum yet: the old state weighs nothing
+                f[r] = f[r] == -INFINITY ? 0.0f : __expf(f[r] - m_run[r]);
+                l_run[r] *= f[r];
+            }
 #pragma unroll
             for (int d = 0; d < DT; ++d)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) O[d][r] *= f[r];
         }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) l_run[r] += psum[r];
         __builtin_amdgcn_wave_barrier();
         // O += P . V over the tile's 32 keys in one k-step: A = P[query j][key 8 g .. + 7], B = V^T[column 16 d + j][key 8 g .. + 7];
         // p v = ph vh + pl vh + ph vl
@@ -297,10 +310,42 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
     a.Out = static_cast<float*>(out);
     a.q_offsets = q_offsets; a.kv_offsets = kv_offsets; a.q_lens = q_lens; a.kv_lens = kv_lens;
     a.q_heads = q_heads; a.kv_heads = kv_heads;
+    // f16 planes of K and V (prefill_pack_kv_kernel) in the prefill stream's buffer, grown on demand.  The packed
+    // layout needs the sequences' key ranges to lie one after the other (offsets non-decreasing with the batch index,
+    // no overlap), which is how packed batches are built; anything else is refused.
+    std::vector<uint32_t> offs(batch);
+    if (hipMemcpy(offs.data(), kv_offsets, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
+    uint64_t end_prev = 0;
+    for (uint32_t i = 0; i < batch; ++i) {
+        if (offs[i] < end_prev) return -8;
+        end_prev = (uint64_t)offs[i] + host[batch + i];
+    }
+    const uint64_t plane_tiles = (offs[batch - 1] / kKTile + (batch - 1)) + (host[2 * (size_t)batch - 1] + kKTile - 1) / kKTile;
+    const size_t need = (size_t)plane_tiles * kv_heads * 4 * kKTile * head_dim * sizeof(_Float16);
+    M40StreamScratch& sc = ctx->scratch[0];
+    if (sc.attn_planes_bytes < need) {
+        if (hipStreamSynchronize(ctx->prefill_stream) != hipSuccess) return -5;
+        if (sc.attn_planes) (void)hipFree(sc.attn_planes);
+        sc.attn_planes = nullptr;
+        sc.attn_planes_bytes = 0;
+        if (hipMalloc(&sc.attn_planes, need + need / 4) != hipSuccess) {
+            (void)hipGetLastError();
+            return -4;
+        }
+        sc.attn_planes_bytes = need + need / 4;
+    }
+    a.planes = static_cast<const _Float16*>(sc.attn_planes);
+    a.plane_tiles = (uint32_t)plane_tiles;
     (void)hipGetLastError();
+    const dim3 pack_grid((max_kv + kKTile - 1) / kKTile, kv_heads, batch);
     const dim3 grid((max_q + kQTile - 1) / kQTile, q_heads, batch);
-    if (head_dim == 64) prefill_attn_kernel<64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
-    else prefill_attn_kernel<128><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+    if (head_dim == 64) {
+        prefill_pack_kv_kernel<64><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        prefill_attn_kernel<64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+    } else {
+        prefill_pack_kv_kernel<128><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        prefill_attn_kernel<128><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+    }
     if (hipGetLastError() != hipSuccess) return -4;
     if (synchronize && hipStreamSynchronize(ctx->prefill_stream) != hipSuccess) return -5;
     return 0;
