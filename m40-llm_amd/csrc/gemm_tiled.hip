@@ -22,7 +22,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBM = 128, kBN = 128, kBK = 32;
-constexpr int kStride = kBK + 8;                 // halves per LDS row: 80 B, conflict-free 16-byte fragment reads
+constexpr int kStride = kBK;                     // halves per LDS row: 64 B, no padding; 16-byte chunks are swizzled (below)
 constexpr int kTileHalves = kBM * kStride;       // one 128 x 32 operand block
 constexpr int kBufHalves = 3 * kTileHalves;      // A high, A low, B
 constexpr int kThreads = 256;
@@ -104,8 +104,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
             r.b[i] = *reinterpret_cast<const uint4*>(B + b_off[i] + k);
         }
     };
+    // LDS rows are 64 bytes = four 16-byte chunks; chunk c of row r is stored at position c ^ ((r / 4) % 4), so that
+    // the 16-byte fragment reads of rows r and r + 4 (same banks without the swizzle) fall into different banks, with
+    // no padding: 48 KB per workgroup
     auto to_lds = [&](const StepRegs& r, int buf) {
-        _Float16* base = lds + buf * kBufHalves + lrow * kStride + lchunk * 8;
+        _Float16* base = lds + buf * kBufHalves + lrow * kStride + ((lchunk ^ ((lrow >> 2) & 3)) * 8);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             _Float16* p = base + i * 64 * kStride;
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
         for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int wm = wave >> 1, wn = wave & 1;
-    const int frag_row = lane & 15, frag_k = (lane >> 4) * 8;
+    const int frag_row = lane & 15, frag_k = ((lane >> 4) ^ ((frag_row >> 2) & 3)) * 8;   // swizzled chunk of this lane's k group
     auto compute = [&](int buf) {
         const _Float16* base = lds + buf * kBufHalves;
         const _Float16* ah = base + (wm * 64 + frag_row) * kStride + frag_k;
@@ -144,7 +147,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
     };
 
     // Three register sets keep the loads of the next three steps in flight (a step's arithmetic is several times
-    // shorter than the memory latency); the sets rotate with the step, so the loop is unrolled by three.
+    // shorter than the memory latency); the sets rotate with the step, so the loop is unrolled by three.  (Two sets and
+    // three workgroups per CU measured the same on large shapes and slower on small grids.)
     StepRegs r0, r1, r2;
     const int last = steps - 1;
     issue(r0, 0);
@@ -212,7 +216,7 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
     mats.tile_start[n_mats] = (int)tiles_n;
     const long long tiles_m = (M + kBM - 1) / kBM;
     if (tiles_m * tiles_n > 0x7fffffffll) return -2;
-    constexpr size_t lds_bytes = 2 * kBufHalves * sizeof(_Float16);   // 61440
+    constexpr size_t lds_bytes = 2 * kBufHalves * sizeof(_Float16);   // 49152
     // two f16 planes of A in the stream's packing buffer, grown on demand (never while the stream is being captured)
     M40StreamScratch& sc = ctx->scratch[stream_kind];
     const size_t need = (size_t)M * K * 4;
