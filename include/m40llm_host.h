@@ -175,7 +175,8 @@ typedef int (*m40host_sched_decode_fn)(void* user, const uint32_t* sequence_ids,
                                        uint32_t rows, float* logits_out);
 /* sequence_slots 0 (or above the model's max_sequences) = the model's max_sequences.  Prompts are prefilled with the
  * packed prefill forward when the model can (dense cache, head_dim 64 / 128), token by token otherwise; decode ticks
- * run one batched step with the fused kernels in the model's host mode 1 / 2. */
+ * run one batched step with the fused kernels in the model's host mode 1 / 2; requests with top_k = 1 and no top_p get
+ * their token from the device-side argmax unless the top two logits are a near tie (then from the host sampler). */
 M40HostScheduler* m40host_scheduler_create_for_model(M40HostModel* model, uint32_t sequence_slots);
 M40HostScheduler* m40host_scheduler_create_with_engine(uint32_t vocab, uint32_t max_seq_len, uint32_t sequence_slots,
                                                        m40host_sched_prefill_fn prefill_fn, m40host_sched_decode_fn decode_fn,

@@ -554,6 +554,17 @@ M40HostScheduler* m40host_scheduler_create_for_model(M40HostModel* model, uint32
                 }
                 d->batched_step_logits(seqs.data(), lens.data(), toks.data(), (uint32_t)items.size(), logits_out);
             };
+            e.decode_pick = [d](const std::vector<SchedulerDecodeItem>& items, const uint8_t* greedy, float* logits_out,
+                                uint32_t* picks_out, uint8_t* picked_out) {
+                std::vector<uint32_t> seqs, lens, toks;
+                for (const auto& it : items) {
+                    seqs.push_back(it.sequence_id);
+                    lens.push_back(it.kv_len);
+                    toks.push_back(it.token);
+                }
+                d->batched_step_logits(seqs.data(), lens.data(), toks.data(), (uint32_t)items.size(), logits_out, greedy, picks_out,
+                                       picked_out);
+            };
             auto h = std::make_unique<M40HostScheduler>();
             h->s = std::make_unique<DecodeScheduler>(std::move(e), sequence_slots);
             return h.release();

@@ -610,8 +610,13 @@ public:
     // every row brought to the host: what a serving loop that samples on the host needs per tick
     // (forward_one_token_all_layers_batched_for_sequences + logits_after_batched_forward, src/server.rs:664-711).
     // Fused kernels in groups of up to 16 rows when the host mode allows them, the reference's sequence otherwise.
+    // greedy / picks / picked (all null, or all given): rows marked greedy get their token picked on the device (first
+    // index of the maximum, as a top_k = 1 sampler picks) when the top-1 / top-2 logit gap clears the tie guard; such
+    // rows set picked[r] = 1 and their logits are not copied.  Every other row receives its logits.
     void batched_step_logits(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* tokens, uint32_t rows,
-                             float* host_logits) {
+                             float* host_logits, const uint8_t* greedy = nullptr, uint32_t* picks = nullptr,
+                             uint8_t* picked = nullptr) {
+        if (picked) std::fill(picked, picked + rows, (uint8_t)0);
         if (rows == 0) throw std::invalid_argument("empty batch");
         for (uint32_t r = 0; r < rows; ++r) {
             if (kv_lens[r] + 1 > cfg_.max_seq_len) throw std::out_of_range("sequence would exceed max_seq_len");
@@ -664,8 +669,28 @@ public:
             }
             M40H_TRY(m40llm_ext_batched_norm_gemm_f32xf16_async(ctx_, a, out_norm_, cfg_.norm_weight_dtype, cfg_.rms_eps, lm_head_,
                                                                 ws_.logits.ptr(), n, (int)cfg_.vocab, (int)cfg_.d_model));
+            bool any_greedy = false;
+            for (uint32_t r = 0; r < n && greedy && picks && picked; ++r) any_greedy = any_greedy || greedy[r0 + r];
+            std::vector<uint32_t> idx(n);
+            std::vector<float> gap(n, 0.0f);
+            if (any_greedy) {
+                M40H_TRY(m40llm_ext_argmax_f32_async(ctx_, ws_.logits.ptr(), n, cfg_.vocab, ws_.argmax_idx.u32(),
+                                                     ws_.argmax_gap.f32()));
+            }
             M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
-            M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits + (size_t)r0 * cfg_.vocab, ws_.logits.ptr(), (size_t)n * cfg_.vocab * 4));
+            if (any_greedy) {
+                M40H_TRY(m40llm_memcpy_d2h(ctx_, idx.data(), ws_.argmax_idx.ptr(), (size_t)n * 4));
+                M40H_TRY(m40llm_memcpy_d2h(ctx_, gap.data(), ws_.argmax_gap.ptr(), (size_t)n * 4));
+            }
+            for (uint32_t r = 0; r < n; ++r) {
+                if (any_greedy && greedy[r0 + r] && gap[r] >= kGreedyTieGuard) {
+                    picks[r0 + r] = idx[r];
+                    picked[r0 + r] = 1;
+                } else {
+                    M40H_TRY(m40llm_memcpy_d2h(ctx_, host_logits + (size_t)(r0 + r) * cfg_.vocab, ws_.logits.f32((size_t)r * cfg_.vocab),
+                                               (size_t)cfg_.vocab * 4));
+                }
+            }
         }
     }
 

@@ -13,7 +13,8 @@
 //                   (prepare_batch_token :331-348, finish_batch_token :406-433);
 //   a request that finishes in a tick is reported then (send_complete), its lease dropped (slot to the back of the
 //   free list, src/decode_batch.rs:75-85).
-// The engine that runs the model is behind two callbacks, so the scheduling logic can be exercised without a GPU.
+// The engine that runs the model is behind two callbacks (and an optional third that lets the engine pick the token of
+// greedy requests itself), so the scheduling logic can be exercised without a GPU.
 #pragma once
 
 #include <cstdint>
@@ -49,6 +50,12 @@ struct SchedulerEngine {
     // logits_out: one row of `vocab` floats per item (the last prompt token's logits / the new token's logits)
     std::function<void(const std::vector<SchedulerPrefillItem>&, float* logits_out)> prefill;
     std::function<void(const std::vector<SchedulerDecodeItem>&, float* logits_out)> decode;
+    // Optional.  Like decode, but rows flagged greedy (their sampler keeps only the top token) may be decided by the
+    // engine: it stores the first index of the row's maximum in picks_out[r] and sets picked_out[r] = 1, and then need
+    // not fill that row's logits (a model does so on the device when the top two logits are not a near tie).
+    std::function<void(const std::vector<SchedulerDecodeItem>&, const uint8_t* greedy, float* logits_out, uint32_t* picks_out,
+                       uint8_t* picked_out)>
+        decode_pick;
 };
 
 enum class SchedulerRequestState : uint32_t { Unknown = 0, PendingPrefill = 1, Decoding = 2, Complete = 3, Cancelled = 4, Failed = 5 };
@@ -178,8 +185,8 @@ private:
     }
 
     // sample from a logits row, push the token, then complete or stay active (finish_prefill / finish_batch_token)
-    void sample_and_route(std::unique_ptr<Request> r, const float* logits, SchedulerTickReport& rep) {
-        const uint32_t next = static_cast<uint32_t>(r->sampler.sample(logits, engine_.vocab));
+    void sample_and_route(std::unique_ptr<Request> r, const float* logits, SchedulerTickReport& rep, const uint32_t* pick = nullptr) {
+        const uint32_t next = pick ? *pick : static_cast<uint32_t>(r->sampler.sample(logits, engine_.vocab));
         r->ids.push_back(next);
         r->generated.push_back(next);
         if (r->stopping.should_stop(r->generated)) {
@@ -236,8 +243,19 @@ private:
             items.push_back({r->lease.sequence_id(), (uint32_t)r->processed, r->ids[r->processed]});
         rep.decode_rows = (uint32_t)ready.size();
         logits_.resize(items.size() * (size_t)engine_.vocab);
+        std::vector<uint8_t> greedy(ready.size(), 0), picked(ready.size(), 0);
+        std::vector<uint32_t> picks(ready.size(), 0);
         try {
-            engine_.decode(items, logits_.data());
+            if (engine_.decode_pick) {
+                for (size_t i = 0; i < ready.size(); ++i) {
+                    const SamplerConfig& c = ready[i]->sampler.config();
+                    // the pick replaces the sample only where the request's next step samples (no prompt tokens left)
+                    greedy[i] = c.top_k && *c.top_k == 1 && !c.top_p && ready[i]->processed + 1 == ready[i]->ids.size();
+                }
+                engine_.decode_pick(items, greedy.data(), logits_.data(), picks.data(), picked.data());
+            } else {
+                engine_.decode(items, logits_.data());
+            }
         } catch (const std::exception& e) {
             fail_all(ready, std::string("batched decode forward failed: ") + e.what(), rep);   // server.rs:680-685
             return;
@@ -249,7 +267,7 @@ private:
                 active_.push_back(std::move(r));
                 continue;
             }
-            sample_and_route(std::move(r), logits_.data() + i * (size_t)engine_.vocab, rep);
+            sample_and_route(std::move(r), logits_.data() + i * (size_t)engine_.vocab, rep, picked[i] ? &picks[i] : nullptr);
         }
     }
 
