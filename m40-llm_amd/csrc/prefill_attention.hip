@@ -11,9 +11,11 @@
 // five times the rate of the f32 matrix instruction for the same product at f32-level accuracy:
 //   scores  S[query][key] = sum_d Q[query][d] K[key][d]   A = Q (two f16 parts, in registers for the whole kernel),
 //           B = K tile (two f16 planes in LDS)
-//   output  O[query][d]  += sum_key P[query][key] V[key][d]   A = softmax weights (two f16 planes through a small LDS
-//           tile per wave, which turns the accumulator layout into the A-operand layout), B = V tile, stored
-//           transposed [d][key] so that eight consecutive keys are one 16-byte read
+//   output  O[query][d]  += sum_key P[query][key] V[key][d]
+// Both are formed transposed (S^T = K Q^T, O^T = V^T P^T) with the tile's keys ordered along the second product's k
+// dimension the way the first product's accumulators hold them, so the softmax weights go from one matrix instruction
+// into the next inside the lane (no LDS round trip), and maximum, sum and rescaling factor are one value per lane.
+// V is stored transposed [d][key slot] so that a lane's eight key slots are one 16-byte read.
 // with a running maximum per query (the rows of a lane's accumulators are the same four queries in both products,
 // so the rescaling needs no exchange).  The result is the same softmax as the reference's three passes
 // (p = exp(s - max) / sum), within f32 rounding.  Operands beyond the f16 range (|x| > 65504) are not supported by the
@@ -39,13 +41,6 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ m40_float4 mfma32(half8 a, half8 b, m40_float4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
-__device__ __forceinline__ float row_max16(float x) {     // over the 16 lanes of a row group
-    x = fmaxf(x, m40_dpp_f<M40_DPP_XOR1>(x));
-    x = fmaxf(x, m40_dpp_f<M40_DPP_XOR2>(x));
-    x = fmaxf(x, m40_dpp_f<M40_DPP_HALF_MIRROR>(x));
-    x = fmaxf(x, m40_dpp_f<M40_DPP_MIRROR>(x));
-    return x;
-}
 // x = hi + lo with both parts f16: exact to about 2^-22 relative for values inside the f16 range
 __device__ __forceinline__ void split(float x, _Float16* hi, _Float16* lo) {
     const _Float16 h = static_cast<_Float16>(x);
@@ -60,6 +55,14 @@ struct PrefillArgs {
     const uint32_t* q_offsets; const uint32_t* kv_offsets; const uint32_t* q_lens; const uint32_t* kv_lens;
     uint32_t q_heads, kv_heads;
 };
+
+// Order of a tile's 32 keys along the k dimension of the P . V product: k-slot 8 g + i holds key 4 g + i (i < 4) or
+// key 16 + 4 g + (i - 4): exactly the eight keys whose scores lane group g holds after the two score products, so the
+// weights go from the score accumulators into the next product's operand without leaving the lane.
+__device__ __forceinline__ int key_of_slot(int slot) {
+    const int g = slot >> 3, i = slot & 7;
+    return i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4);
+}
 
 // First padded tile of sequence b in the packed planes: every sequence starts on a tile boundary of its own, so a
 // sequence gets one tile of slack (rows_before / 32 rounded down, plus b).
@@ -92,9 +95,9 @@ __global__ __launch_bounds__(kThreads) void prefill_pack_kv_kernel(PrefillArgs p
     }
     __syncthreads();
     for (int e = threadIdx.x; e < kKTile * HD; e += kThreads) {
-        const int d = e / kKTile, key_in = e % kKTile;
+        const int d = e / kKTile, slot = e % kKTile;
         _Float16 a, c;
-        split(vt[key_in][d], &a, &c);
+        split(vt[key_of_slot(slot)][d], &a, &c);
         vh[e] = a;
         vl[e] = c;
     }
@@ -106,10 +109,8 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     constexpr int DT = HD / 16;            // 16-column output tiles
     constexpr int KSTR = HD + 8;           // LDS halves per K row: 16-byte fragment reads of 16 keys hit 64 distinct banks
     constexpr int VSTR = kKTile + 8;       // LDS halves per row of the transposed V tile [column][key]
-    constexpr int PSTR = kKTile + 8;       // LDS halves per row of a wave's weight tile
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][kKTile * KSTR];   // [hi, lo][key][d]
     __shared__ __attribute__((aligned(16))) _Float16 v_lds[2][HD * VSTR];       // [hi, lo][d][key]
-    __shared__ __attribute__((aligned(16))) _Float16 p_lds[kWaves][2][16 * PSTR];
 
     const uint32_t b = blockIdx.z, h = blockIdx.y;
     const uint32_t q_len = p.q_lens[b], kv_len = p.kv_lens[b];
@@ -144,13 +145,9 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             }
         }
     }
-    // queries of this lane's accumulator rows: 4 g + r; their last visible key
-    uint32_t row_end[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const uint32_t q = wq0 + 4u * g + r;
-        row_end[r] = shift + (q < q_len ? q : q_len - 1);
-    }
+    // this lane's query (all its scores, weights and accumulators belong to it) and its last visible key
+    const uint32_t row_end = shift + my_q;
+    const uint32_t wave_first_end = shift + (wq0 < q_len ? wq0 : q_len - 1);          // last key the wave's first query sees
     const uint32_t wave_end = shift + (wq0 + 15u < q_len ? wq0 + 15u : q_len - 1);    // last key any query of the wave sees
 
     // ---- K / V tile loads: 16-byte pieces of the packed f16 planes (prefill_pack_kv_kernel), straight into LDS
@@ -186,14 +183,15 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     };
     issue(0);
 
-    float m_run[4], l_run[4];             // running maximum of the row (equal in its 16 lanes); this lane's share of the sum
-    m40_float4 O[DT];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) { m_run[r] = -INFINITY; l_run[r] = 0.0f; }
+    // Products are formed transposed, S^T = K Q^T and O^T = V^T P^T, so that a lane (query j, group g) ends up with the
+    // scores of ONE query for keys 4 g .. 4 g + 3 of both 16-key blocks, which are the k-slots 8 g .. 8 g + 7 of the
+    // second product (key_of_slot): the weights never pass through LDS, and the running maximum, the sum and the
+    // rescaling factor are one value per lane.
+    float m_run = -INFINITY, l_run = 0.0f;   // maximum over the query's keys so far (equal in its four lanes); this lane's share of the sum
+    m40_float4 O[DT];                        // O^T[16 d + 4 g + r][query j]
 #pragma unroll
     for (int d = 0; d < DT; ++d) O[d] = m40_float4{0.f, 0.f, 0.f, 0.f};
-    _Float16* my_ph = p_lds[wave][0];
-    _Float16* my_pl = p_lds[wave][1];
+    const float scale_log2 = inv_sqrt * 1.4426950408889634f;     // scores in units of log2: weights are exp2(x - max)
 
     for (uint32_t tile = 0; tile < n_tiles; ++tile) {
         __syncthreads();                  // the previous tile has been read by every wave
@@ -203,8 +201,8 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         const uint32_t key0 = tile * kKTile;
         if (!wave_live || key0 > wave_end) continue;              // nothing of this tile is visible to the wave
 
-        // scores of the two 16-key halves: lane (key j, g) gets rows 4 g + r.  q . k = qh kh + ql kh + qh kl
-        // (the ql kl term is below 2^-22 of |q| |k|)
+        // S^T of the two 16-key blocks: lane (query j, g) gets keys 4 g + r.  k . q = kh qh + kh ql + kl qh
+        // (the kl ql term is below 2^-22 of |q| |k|)
         m40_float4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -213,76 +211,71 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             const half8 k0l = *reinterpret_cast<const half8*>(&k_lds[1][j * KSTR + off]);
             const half8 k1h = *reinterpret_cast<const half8*>(&k_lds[0][(16 + j) * KSTR + off]);
             const half8 k1l = *reinterpret_cast<const half8*>(&k_lds[1][(16 + j) * KSTR + off]);
-            s0 = mfma32(qh[s], k0h, s0);
-            s1 = mfma32(qh[s], k1h, s1);
-            s0 = mfma32(ql[s], k0h, s0);
-            s1 = mfma32(ql[s], k1h, s1);
-            s0 = mfma32(qh[s], k0l, s0);
-            s1 = mfma32(qh[s], k1l, s1);
+            s0 = mfma32(k0h, qh[s], s0);
+            s1 = mfma32(k1h, qh[s], s1);
+            s0 = mfma32(k0h, ql[s], s0);
+            s1 = mfma32(k1h, ql[s], s1);
+            s0 = mfma32(k0l, qh[s], s0);
+            s1 = mfma32(k1l, qh[s], s1);
         }
-        float f[4], psum[4];
-        bool moved = false;
+        float x[8];
+        const bool whole = key0 + (uint32_t)kKTile - 1u <= wave_first_end;      // every key of the tile visible to every query
+        float mx = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const bool a0 = key0 + (uint32_t)j <= row_end[r], a1 = key0 + 16u + (uint32_t)j <= row_end[r];
-            const float x0 = a0 ? s0[r] * inv_sqrt : -INFINITY, x1 = a1 ? s1[r] * inv_sqrt : -INFINITY;
-            const float n = fmaxf(m_run[r], row_max16(fmaxf(x0, x1)));
-            const float p0 = a0 ? __expf(x0 - n) : 0.0f;                 // a masked key weighs nothing
-            const float p1 = a1 ? __expf(x1 - n) : 0.0f;
-            moved = moved || m_run[r] != n;
-            f[r] = m_run[r];                                             // the old maximum, turned into a factor below
-            m_run[r] = n;
-            psum[r] = p0 + p1;
-            _Float16 a, c;
-            split(p0, &a, &c);
-            my_ph[(4 * g + r) * PSTR + j] = a;
-            my_pl[(4 * g + r) * PSTR + j] = c;
-            split(p1, &a, &c);
-            my_ph[(4 * g + r) * PSTR + 16 + j] = a;
-            my_pl[(4 * g + r) * PSTR + 16 + j] = c;
+            const bool a0 = whole || key0 + 4u * g + r <= row_end, a1 = whole || key0 + 16u + 4u * g + r <= row_end;
+            x[r] = a0 ? s0[r] * scale_log2 : -INFINITY;
+            x[4 + r] = a1 ? s1[r] * scale_log2 : -INFINITY;
+            mx = fmaxf(mx, fmaxf(x[r], x[4 + r]));
         }
-        if (__any(moved)) {               // sums and accumulators are only rescaled when some row's maximum rose
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float n = fmaxf(m_run, mx);
+        const bool moved = n != m_run;
+        half8 ph, pl;
+        float psum = 0.0f;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                // no maximum yet: the old state weighs nothing
-                f[r] = f[r] == -INFINITY ? 0.0f : __expf(f[r] - m_run[r]);
-                l_run[r] *= f[r];
-            }
+        for (int i = 0; i < 8; ++i) {
+            const float pv = __builtin_amdgcn_exp2f(x[i] - n);               // a masked key: exp2(-inf) = 0
+            psum += pv;
+            _Float16 a, c;
+            split(pv, &a, &c);
+            ph[i] = a;
+            pl[i] = c;
+        }
+        if (__any(moved)) {               // sum and accumulators are only rescaled when some query's maximum rose
+            // no maximum yet: the old state weighs nothing
+            const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - n);
+            l_run *= f;
 #pragma unroll
             for (int d = 0; d < DT; ++d)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) O[d][r] *= f[r];
+                for (int r = 0; r < 4; ++r) O[d][r] *= f;
         }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) l_run[r] += psum[r];
-        __builtin_amdgcn_wave_barrier();
-        // O += P . V over the tile's 32 keys in one k-step: A = P[query j][key 8 g .. + 7], B = V^T[column 16 d + j][key 8 g .. + 7];
-        // p v = ph vh + pl vh + ph vl
-        const half8 ph = *reinterpret_cast<const half8*>(&my_ph[j * PSTR + 8 * g]);
-        const half8 pl = *reinterpret_cast<const half8*>(&my_pl[j * PSTR + 8 * g]);
-        __builtin_amdgcn_wave_barrier();
+        m_run = n;
+        l_run += psum;
+        // O^T += V^T . P^T over the tile's 32 keys in one k-step: A = V^T[column 16 d + j][k-slots 8 g .. + 7],
+        // B = this lane's eight weights;  v p = vh ph + vh pl + vl ph
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
             const half8 vh = *reinterpret_cast<const half8*>(&v_lds[0][(16 * d + j) * VSTR + 8 * g]);
             const half8 vl = *reinterpret_cast<const half8*>(&v_lds[1][(16 * d + j) * VSTR + 8 * g]);
-            O[d] = mfma32(ph, vh, O[d]);
-            O[d] = mfma32(pl, vh, O[d]);
-            O[d] = mfma32(ph, vl, O[d]);
+            O[d] = mfma32(vh, ph, O[d]);
+            O[d] = mfma32(vh, pl, O[d]);
+            O[d] = mfma32(vl, ph, O[d]);
         }
     }
 
-    // ---- out = O / sum
+    // ---- out = O / sum: this lane holds columns 16 d + 4 g .. + 3 of its query
     if (!wave_live) return;
+    float l = l_run + __shfl_xor(l_run, 16);
+    l += __shfl_xor(l, 32);
+    const float denom = l > 0.0f ? l : 1.0f;
+    if (wq0 + (uint32_t)j < q_len) {
+        float* op = p.Out + ((size_t)(p.q_offsets[b] + wq0 + j) * p.q_heads + h) * HD + 4 * g;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const uint32_t q = wq0 + 4u * g + r;
-        const float l = m40_sum16(l_run[r]);
-        const float denom = l > 0.0f ? l : 1.0f;
-        if (q < q_len) {
-            float* op = p.Out + ((size_t)(p.q_offsets[b] + q) * p.q_heads + h) * HD + j;
-#pragma unroll
-            for (int d = 0; d < DT; ++d) op[16 * d] = O[d][r] / denom;
-        }
+        for (int d = 0; d < DT; ++d)
+            *reinterpret_cast<float4*>(op + 16 * d) = make_float4(O[d][0] / denom, O[d][1] / denom, O[d][2] / denom, O[d][3] / denom);
     }
 }
 
@@ -304,7 +297,7 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
         max_q = ql > max_q ? ql : max_q;
         max_kv = kl > max_kv ? kl : max_kv;
     }
-    if (!m40_aligned16(q) || !m40_aligned16(k) || !m40_aligned16(v)) return -4;
+    if (!m40_aligned16(q) || !m40_aligned16(k) || !m40_aligned16(v) || !m40_aligned16(out)) return -4;
     PrefillArgs a{};
     a.Q = static_cast<const float*>(q); a.K = static_cast<const float*>(k); a.V = static_cast<const float*>(v);
     a.Out = static_cast<float*>(out);
