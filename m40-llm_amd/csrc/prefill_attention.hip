@@ -32,7 +32,9 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kQTile = 16 * kWaves;      // queries per workgroup
-constexpr int kKTile = 32;               // keys per LDS tile = the K depth of one matrix instruction of the P . V product
+// keys per LDS tile (KT below): one or two k-steps of the P . V product; 64 where two planes of K and V^T fit the
+// static LDS limit (head_dim 64), 32 otherwise
+constexpr int key_tile_of(int hd) { return hd == 64 ? 64 : 32; }
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -60,19 +62,20 @@ struct PrefillArgs {
 // key 16 + 4 g + (i - 4): exactly the eight keys whose scores lane group g holds after the two score products, so the
 // weights go from the score accumulators into the next product's operand without leaving the lane.
 __device__ __forceinline__ int key_of_slot(int slot) {
-    const int g = slot >> 3, i = slot & 7;
-    return i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4);
+    const int base = slot & ~31, g = (slot & 31) >> 3, i = slot & 7;      // every 32 slots: one k-step over 32 keys
+    return base + (i < 4 ? 4 * g + i : 16 + 4 * g + (i - 4));
 }
 
 // First padded tile of sequence b in the packed planes: every sequence starts on a tile boundary of its own, so a
 // sequence gets one tile of slack (rows_before / 32 rounded down, plus b).
-__device__ __forceinline__ uint32_t first_tile_of(uint32_t kv_offset, uint32_t b) { return kv_offset / kKTile + b; }
+__device__ __forceinline__ uint32_t first_tile_of(uint32_t kv_offset, uint32_t b, uint32_t key_tile) { return kv_offset / key_tile + b; }
 
 // K and V of one 32-key tile and kv head -> two f16 planes each, V transposed, in the order the attention kernel copies
 // them to LDS.  Done once per call so that the 64-query workgroups (and the q heads of a group) do not each repeat the
 // split.  Keys past the sequence end are written as zeros (they are masked anyway).
 template <int HD>
 __global__ __launch_bounds__(kThreads) void prefill_pack_kv_kernel(PrefillArgs p) {
+    constexpr int kKTile = key_tile_of(HD);
     __shared__ float vt[kKTile][HD + 1];
     const uint32_t b = blockIdx.z, kvh = blockIdx.y, tile = blockIdx.x;
     const uint32_t kv_len = p.kv_lens[b];
@@ -80,7 +83,7 @@ __global__ __launch_bounds__(kThreads) void prefill_pack_kv_kernel(PrefillArgs p
     const float* Kb = p.K + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
     const float* Vb = p.V + ((size_t)p.kv_offsets[b] * p.kv_heads + kvh) * HD;
     const size_t row_stride = (size_t)p.kv_heads * HD;
-    _Float16* out = const_cast<_Float16*>(p.planes) + ((size_t)(first_tile_of(p.kv_offsets[b], b) + tile) * p.kv_heads + kvh) * (4 * kKTile * HD);
+    _Float16* out = const_cast<_Float16*>(p.planes) + ((size_t)(first_tile_of(p.kv_offsets[b], b, kKTile) + tile) * p.kv_heads + kvh) * (4 * kKTile * HD);
     _Float16* kh = out, *kl = out + kKTile * HD, *vh = out + 2 * kKTile * HD, *vl = out + 3 * kKTile * HD;
     for (int e = threadIdx.x; e < kKTile * HD; e += kThreads) {
         const int key_in = e / HD, d = e % HD;
@@ -105,6 +108,8 @@ __global__ __launch_bounds__(kThreads) void prefill_pack_kv_kernel(PrefillArgs p
 
 template <int HD>
 __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
+    constexpr int kKTile = key_tile_of(HD);
+    constexpr int KB = kKTile / 16;        // 16-key score blocks of a tile
     constexpr int KS = HD / 32;            // matrix-instruction k-steps of a score tile
     constexpr int DT = HD / 16;            // 16-column output tiles
     constexpr int KSTR = HD + 8;           // LDS halves per K row: 16-byte fragment reads of 16 keys hit 64 distinct banks
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
 
     // ---- K / V tile loads: 16-byte pieces of the packed f16 planes (prefill_pack_kv_kernel), straight into LDS
     constexpr int PIECES = kKTile * HD / 8 / kThreads;           // per plane and thread: 1 (HD 64) or 2 (HD 128)
-    const _Float16* tile_base = p.planes + ((size_t)first_tile_of(p.kv_offsets[b], b) * p.kv_heads + kvh) * (4 * kKTile * HD);
+    const _Float16* tile_base = p.planes + ((size_t)first_tile_of(p.kv_offsets[b], b, kKTile) * p.kv_heads + kvh) * (4 * kKTile * HD);
     const size_t tile_stride = (size_t)p.kv_heads * (4 * kKTile * HD);
     uint4 kreg[2][PIECES], vreg[2][PIECES];
     auto issue = [&](uint32_t tile) {
@@ -201,47 +206,48 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         const uint32_t key0 = tile * kKTile;
         if (!wave_live || key0 > wave_end) continue;              // nothing of this tile is visible to the wave
 
-        // S^T of the two 16-key blocks: lane (query j, g) gets keys 4 g + r.  k . q = kh qh + kh ql + kl qh
+        // S^T of the tile's 16-key blocks: lane (query j, g) gets keys 16 kb + 4 g + r.  k . q = kh qh + kh ql + kl qh
         // (the kl ql term is below 2^-22 of |q| |k|)
-        m40_float4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+        m40_float4 sc[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) sc[kb] = m40_float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             const int off = 32 * s + 8 * g;
-            const half8 k0h = *reinterpret_cast<const half8*>(&k_lds[0][j * KSTR + off]);
-            const half8 k0l = *reinterpret_cast<const half8*>(&k_lds[1][j * KSTR + off]);
-            const half8 k1h = *reinterpret_cast<const half8*>(&k_lds[0][(16 + j) * KSTR + off]);
-            const half8 k1l = *reinterpret_cast<const half8*>(&k_lds[1][(16 + j) * KSTR + off]);
-            s0 = mfma32(k0h, qh[s], s0);
-            s1 = mfma32(k1h, qh[s], s1);
-            s0 = mfma32(k0h, ql[s], s0);
-            s1 = mfma32(k1h, ql[s], s1);
-            s0 = mfma32(k0l, qh[s], s0);
-            s1 = mfma32(k1l, qh[s], s1);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const half8 kh = *reinterpret_cast<const half8*>(&k_lds[0][(16 * kb + j) * KSTR + off]);
+                const half8 kl = *reinterpret_cast<const half8*>(&k_lds[1][(16 * kb + j) * KSTR + off]);
+                sc[kb] = mfma32(kh, qh[s], sc[kb]);
+                sc[kb] = mfma32(kh, ql[s], sc[kb]);
+                sc[kb] = mfma32(kl, qh[s], sc[kb]);
+            }
         }
-        float x[8];
+        float x[4 * KB];
         const bool whole = key0 + (uint32_t)kKTile - 1u <= wave_first_end;      // every key of the tile visible to every query
         float mx = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const bool a0 = whole || key0 + 4u * g + r <= row_end, a1 = whole || key0 + 16u + 4u * g + r <= row_end;
-            x[r] = a0 ? s0[r] * scale_log2 : -INFINITY;
-            x[4 + r] = a1 ? s1[r] * scale_log2 : -INFINITY;
-            mx = fmaxf(mx, fmaxf(x[r], x[4 + r]));
-        }
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool visible = whole || key0 + 16u * kb + 4u * g + r <= row_end;
+                x[4 * kb + r] = visible ? sc[kb][r] * scale_log2 : -INFINITY;
+                mx = fmaxf(mx, x[4 * kb + r]);
+            }
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float n = fmaxf(m_run, mx);
         const bool moved = n != m_run;
-        half8 ph, pl;
+        half8 ph[KB / 2], pl[KB / 2];       // k-step t: slots 8 g + i = blocks 2 t (i < 4) and 2 t + 1 (i >= 4)
         float psum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < 4 * KB; ++i) {
             const float pv = __builtin_amdgcn_exp2f(x[i] - n);               // a masked key: exp2(-inf) = 0
             psum += pv;
             _Float16 a, c;
             split(pv, &a, &c);
-            ph[i] = a;
-            pl[i] = c;
+            ph[i >> 3][i & 7] = a;
+            pl[i >> 3][i & 7] = c;
         }
         if (__any(moved)) {               // sum and accumulators are only rescaled when some query's maximum rose
             // no maximum yet: the old state weighs nothing
@@ -254,15 +260,18 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         }
         m_run = n;
         l_run += psum;
-        // O^T += V^T . P^T over the tile's 32 keys in one k-step: A = V^T[column 16 d + j][k-slots 8 g .. + 7],
-        // B = this lane's eight weights;  v p = vh ph + vh pl + vl ph
+        // O^T += V^T . P^T, 32 keys per k-step: A = V^T[column 16 d + j][k-slots 32 t + 8 g .. + 7], B = this lane's
+        // eight weights of the step;  v p = vh ph + vh pl + vl ph
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
-            const half8 vh = *reinterpret_cast<const half8*>(&v_lds[0][(16 * d + j) * VSTR + 8 * g]);
-            const half8 vl = *reinterpret_cast<const half8*>(&v_lds[1][(16 * d + j) * VSTR + 8 * g]);
-            O[d] = mfma32(vh, ph, O[d]);
-            O[d] = mfma32(vh, pl, O[d]);
-            O[d] = mfma32(vl, ph, O[d]);
+#pragma unroll
+            for (int t = 0; t < KB / 2; ++t) {
+                const half8 vh = *reinterpret_cast<const half8*>(&v_lds[0][(16 * d + j) * VSTR + 32 * t + 8 * g]);
+                const half8 vl = *reinterpret_cast<const half8*>(&v_lds[1][(16 * d + j) * VSTR + 32 * t + 8 * g]);
+                O[d] = mfma32(vh, ph[t], O[d]);
+                O[d] = mfma32(vh, pl[t], O[d]);
+                O[d] = mfma32(vl, ph[t], O[d]);
+            }
         }
     }
 
@@ -313,6 +322,7 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
         if (offs[i] < end_prev) return -8;
         end_prev = (uint64_t)offs[i] + host[batch + i];
     }
+    const uint32_t kKTile = (uint32_t)key_tile_of((int)head_dim);
     const uint64_t plane_tiles = (offs[batch - 1] / kKTile + (batch - 1)) + (host[2 * (size_t)batch - 1] + kKTile - 1) / kKTile;
     const size_t need = (size_t)plane_tiles * kv_heads * 4 * kKTile * head_dim * sizeof(_Float16);
     M40StreamScratch& sc = ctx->scratch[0];
