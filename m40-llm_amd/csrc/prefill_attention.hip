@@ -117,9 +117,15 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][kKTile * KSTR];   // [hi, lo][key][d]
     __shared__ __attribute__((aligned(16))) _Float16 v_lds[2][HD * VSTR];       // [hi, lo][d][key]
 
-    const uint32_t b = blockIdx.z, h = blockIdx.y;
+    // Workgroups are dispatched in index order, x fastest: x = q head, y = query tile from the end of the sequence,
+    // z = sequence (ordering the tiles of all sequences together by key count measured slower: the sequences' keys
+    // then compete for the caches).
+    // The tiles with the most keys (the longest workgroups) of every head start first and the short ones fill the
+    // tail; with the head as the slow index the last heads' long tiles started near the end of the kernel and the
+    // chip ran at a third of its occupancy.  Neighbouring workgroups are the q heads of one kv group on the same keys.
+    const uint32_t b = blockIdx.z, h = blockIdx.x;
     const uint32_t q_len = p.q_lens[b], kv_len = p.kv_lens[b];
-    const uint32_t q0 = (gridDim.x - 1u - blockIdx.x) * kQTile;   // late query tiles see the most keys: they start first
+    const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * kQTile;
     if (q0 >= q_len || q_len > kv_len) return;
     const uint32_t kvh = h / (p.q_heads / p.kv_heads);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -341,7 +347,7 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
     a.plane_tiles = (uint32_t)plane_tiles;
     (void)hipGetLastError();
     const dim3 pack_grid((max_kv + kKTile - 1) / kKTile, kv_heads, batch);
-    const dim3 grid((max_q + kQTile - 1) / kQTile, q_heads, batch);
+    const dim3 grid(q_heads, (max_q + kQTile - 1) / kQTile, batch);
     if (head_dim == 64) {
         prefill_pack_kv_kernel<64><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
         prefill_attn_kernel<64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
