@@ -63,14 +63,19 @@ __global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __re
 
 __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(const _Float16* __restrict__ A_hi,
                                                                               const _Float16* __restrict__ A_lo,
-                                                                              TiledMats mats, int M, int K) {
+                                                                              TiledMats mats, int M, int K, int k_splits) {
     extern __shared__ __align__(16) _Float16 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tiles_n = mats.tile_start[mats.n];
     // Workgroups are dealt to the eight dies in turn.  Renumbered so that each die owns a contiguous band of tile
     // rows: its L2 then holds one eighth of A (and streams B) instead of every die reading all of A.
     const int per_die = (int)gridDim.x / 8;
-    const int logical = (int)blockIdx.x < per_die * 8 ? ((int)blockIdx.x % 8) * per_die + (int)blockIdx.x / 8 : (int)blockIdx.x;
+    int logical = (int)blockIdx.x < per_die * 8 ? ((int)blockIdx.x % 8) * per_die + (int)blockIdx.x / 8 : (int)blockIdx.x;
+    // K split (few tiles, long K): split s of a tile walks its share of the K steps and writes its partial sums to
+    // plane s of the output buffer (a reduction launch adds the planes in order)
+    const int tiles_all = (int)gridDim.x / k_splits;
+    const int split = logical / tiles_all;
+    logical -= split * tiles_all;
     const int tile_m = logical / tiles_n;
     int tile_n = logical % tiles_n;
     int mat = 0;
@@ -93,10 +98,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
         a_off[i] = (size_t)ar * K + lchunk * 8;
         b_off[i] = (size_t)bc * K + lchunk * 8;
     }
-    const int steps = K / kBK;
+    const int steps_all = K / kBK, per_split = (steps_all + k_splits - 1) / k_splits;
+    const int step0 = split * per_split;
+    const int steps = step0 + per_split <= steps_all ? per_split : steps_all - step0;     // >= 1 by the host's choice of k_splits
 
     auto issue = [&](StepRegs& r, int step) {
-        const size_t k = (size_t)step * kBK;
+        const size_t k = (size_t)(step0 + step) * kBK;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             r.ah[i] = *reinterpret_cast<const uint4*>(A_hi + a_off[i] + k);
@@ -184,10 +191,23 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
                 const int col = n0 + wn * 64 + nt * 16 + out_col;
-                if (col < N) C[(size_t)row * N + col] = acc[mt][nt][r];
+                if (col < N) C[((size_t)split * M + row) * N + col] = acc[mt][nt][r];
             }
         }
     }
+}
+
+// out[i] = planes[0][i] + planes[1][i] + ... in that order (n4 float4 per plane)
+__global__ __launch_bounds__(256) void add_k_planes_kernel(const float4* __restrict__ planes, float4* __restrict__ out, size_t n4,
+                                                           int k_splits) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    float4 a = planes[i];
+    for (int s = 1; s < k_splits; ++s) {
+        const float4 b = planes[(size_t)s * n4 + i];
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    out[i] = a;
 }
 
 }  // namespace
@@ -217,9 +237,27 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
     const long long tiles_m = (M + kBM - 1) / kBM;
     if (tiles_m * tiles_n > 0x7fffffffll) return -2;
     constexpr size_t lds_bytes = 2 * kBufHalves * sizeof(_Float16);   // 49152
-    // two f16 planes of A in the stream's packing buffer, grown on demand (never while the stream is being captured)
+    // two f16 planes of A (and the partial sums of a K split) in the stream's packing buffer, grown on demand (never while
+    // the stream is being captured)
     M40StreamScratch& sc = ctx->scratch[stream_kind];
-    const size_t need = (size_t)M * K * 4;
+    // Few tiles and many K steps (short prompts, the down projection): split K so that the chip is covered and a
+    // workgroup's chain of dependent steps is shorter; partial sums go to planes behind the packed activations and are
+    // added in a fixed order by a second launch (every N a multiple of 4 for its float4 accesses).
+    const int steps = K / kBK;
+    int k_splits = 1;
+    const long long tiles = tiles_m * tiles_n;
+    bool n4_ok = true;
+    size_t out_floats = 0;
+    for (int i = 0; i < n_mats; ++i) {
+        n4_ok = n4_ok && N[i] % 4 == 0 && m40_aligned16(C[i]);
+        out_floats += (size_t)M * N[i];
+    }
+    if (n4_ok && tiles <= 128) {   // above that a split only adds a partial-sum pass (measured at 176 tiles)
+        k_splits = (int)(512 / tiles);
+        if (k_splits > 4) k_splits = 4;
+        while (k_splits > 1 && (steps / k_splits < 16 || (steps + k_splits - 1) / k_splits * (k_splits - 1) >= steps)) --k_splits;
+    }
+    const size_t need = (size_t)M * K * 4 + (k_splits > 1 ? (size_t)k_splits * out_floats * 4 : 0);
     if (sc.tiled_pack_bytes < need) {
         hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone) return 1;
@@ -239,7 +277,23 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
     _Float16* lo = hi + (size_t)M * K;
     const size_t total8 = (size_t)M * K / 8;
     pack_hilo_planes_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(A, hi, lo, total8);
-    gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles_m * tiles_n), kThreads, lds_bytes, stream>>>(hi, lo, mats, M, K);
+    float* partial = reinterpret_cast<float*>(static_cast<char*>(sc.tiled_pack) + (size_t)M * K * 4);
+    TiledMats launch = mats;
+    if (k_splits > 1) {
+        size_t at = 0;
+        for (int i = 0; i < n_mats; ++i) {
+            launch.C[i] = partial + at;
+            at += (size_t)k_splits * M * N[i];
+        }
+    }
+    gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles * k_splits), kThreads, lds_bytes, stream>>>(hi, lo, launch, M, K, k_splits);
+    if (k_splits > 1) {
+        for (int i = 0; i < n_mats; ++i) {
+            const size_t n4 = (size_t)M * N[i] / 4;
+            add_k_planes_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, stream>>>(reinterpret_cast<const float4*>(launch.C[i]),
+                                                                                  reinterpret_cast<float4*>(C[i]), n4, k_splits);
+        }
+    }
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
