@@ -128,6 +128,7 @@ def _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, S=None, seed=0, sca
     (32, 8, 128, 4096, 512, 64, 64),   # BASELINE config 5 geometry at 4K context
     (16, 4, 64, 2100, 1024, 32, 8),    # the reference's default window / block / top
     (6, 2, 128, 777, 100, 48, 5),      # ragged everything, partial last block
+    (32, 8, 128, 32768, 512, 64, 64),  # BASELINE config 5 at its full context: 504 old blocks per kv head
 ])
 def test_block_select_indices_exact_and_output(dev, orc, qh, kvh, hd, L, W, bs, top):
     r = _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top)

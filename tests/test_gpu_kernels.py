@@ -336,6 +336,36 @@ def test_q80_gemm_and_ffn_vs_oracle(dev, orc, M):
     close(out.download(np.float32, (M, d_model)), want, 1e-3, 1e-4 * max(np.abs(want).max(), 1.0))
 
 
+@pytest.fixture(scope="module")
+def q80_ffn_full_size():
+    """q8_0 gate / up / down of BASELINE config 4 (hidden 4096, FFN 14336): int8 uniform in [-127, 127], f16 scales
+    U(0.001, 0.01), built once for the rows-per-call cases below."""
+    rng = np.random.default_rng(404)
+    def qmat(n, k):
+        blob = np.empty((n, k // 32, 34), dtype=np.uint8)
+        blob[:, :, :2] = rng.uniform(0.001, 0.01, size=(n, k // 32)).astype(np.float16).view(np.uint8).reshape(n, k // 32, 2)
+        blob[:, :, 2:] = rng.integers(-127, 128, size=(n, k // 32, 32)).astype(np.int8).view(np.uint8)
+        return blob
+    return qmat(14336, 4096), qmat(14336, 4096), qmat(4096, 14336)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_q80_ffn_full_size_vs_oracle(dev, orc, q80_ffn_full_size, M):
+    """The fused q8_0 FFN at the full BASELINE config 4 size, batch sizes 1, 4 and 16, against the oracle's sequential
+    f32 sums: 1e-3 relative / 1e-4 absolute on outputs scaled to a unit row maximum."""
+    wg, wu, wd = q80_ffn_full_size
+    d_model, ffn = 4096, 14336
+    x = np.random.default_rng(40 + M).standard_normal((M, d_model)).astype(np.float32)
+    dx, dwg, dwu, dwd = dev.up(x), dev.up(wg), dev.up(wu), dev.up(wd)
+    scratch, out = dev.zeros(2 * M * ffn * 4), dev.zeros(M * d_model * 4)
+    dev.call("m40llm_ext_ffn_swiglu_q80_f32_async", dx.ptr, dwg.ptr, dwu.ptr, dwd.ptr, scratch.ptr, out.ptr, M, d_model, ffn)
+    dev.sync()
+    orc.set_threads(8)
+    want = orc.ffn_swiglu_q80(x, wg, wu, wd, M, d_model, ffn)
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    close(out.download(np.float32, (M, d_model)) / scale, want / scale, 1e-3, 1e-4)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 1000, 768), (8, 4096, 2048), (9, 520, 1280), (16, 2048, 4096),
                                    (20, 333, 256), (2, 64, 96), (1, 1000, 4096), (2, 777, 8192), (1, 513, 14336),
                                    (2, 260, 11008), (1, 40, 16384), (2, 3, 64)])
