@@ -548,6 +548,95 @@ __global__ __launch_bounds__(1024) void greedy_batch_kernel(GreedyBatchArgs a) {
         a.x_out[(size_t)row * a.d_model + i] = m40_h2f(a.table[(size_t)tok * a.d_model + i]);
 }
 
+// The same step in two launches for wide rows: kGreedyParts workgroups per row each reduce a contiguous range of the
+// logits to (maximum, runner-up, first index of the maximum); one workgroup per row then merges the parts -- ties go
+// to the lower index in both stages, so the pick equals the one-launch kernel's -- and does the bookkeeping.
+constexpr uint32_t kGreedyParts = 32;
+__global__ __launch_bounds__(256) void greedy_batch_part_kernel(GreedyBatchArgs a, float* part) {
+    __shared__ float sa[4], sb[4];
+    __shared__ uint32_t si[4];
+    const uint32_t row = blockIdx.y, pt = blockIdx.x;
+    const float4* lg4 = reinterpret_cast<const float4*>(a.logits + (size_t)row * a.n);
+    const uint32_t n4 = a.n >> 2;
+    const uint32_t per = (n4 + kGreedyParts - 1) / kGreedyParts;
+    const uint32_t beg = pt * per, end = beg + per < n4 ? beg + per : n4;
+    float va = -INFINITY, vb = -INFINITY;
+    uint32_t ia = 0xffffffffu;
+    auto offer = [&](float oa, float ob, uint32_t oi) {
+        if (oa > va || (oa == va && oi < ia)) { vb = fmaxf(va, ob); va = oa; ia = oi; }
+        else vb = fmaxf(vb, oa);
+    };
+    for (uint32_t base = beg; base < end; base += 8u * 256u) {
+        float4 v[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8u; ++u) {
+            const uint32_t i = base + u * 256u + threadIdx.x;
+            v[u] = lg4[i < n4 ? i : n4 - 1u];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8u; ++u) {
+            const uint32_t i = base + u * 256u + threadIdx.x;
+            if (i < end) {
+                offer(v[u].x, -INFINITY, 4u * i); offer(v[u].y, -INFINITY, 4u * i + 1u);
+                offer(v[u].z, -INFINITY, 4u * i + 2u); offer(v[u].w, -INFINITY, 4u * i + 3u);
+            }
+        }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float oa = __shfl_xor(va, o, 64), ob = __shfl_xor(vb, o, 64);
+        const uint32_t oi = __shfl_xor(ia, o, 64);
+        offer(oa, ob, oi);
+    }
+    const uint32_t wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63u) == 0u) { sa[wave] = va; sb[wave] = vb; si[wave] = ia; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < 4u; ++w) offer(sa[w], sb[w], si[w]);
+        float* dst = part + ((size_t)row * kGreedyParts + pt) * 4;
+        dst[0] = va; dst[1] = vb; dst[2] = __uint_as_float(ia);
+    }
+}
+__global__ __launch_bounds__(256) void greedy_batch_merge_kernel(GreedyBatchArgs a, const float* part) {
+    __shared__ uint32_t s_tok;
+    const uint32_t row = blockIdx.x;
+    if (threadIdx.x < 64u) {
+        static_assert(kGreedyParts <= 64, "one lane per part");
+        const float* src = part + ((size_t)row * kGreedyParts + (threadIdx.x < kGreedyParts ? threadIdx.x : 0u)) * 4;
+        const float pa = src[0], pb = src[1];
+        const uint32_t pi = __float_as_uint(src[2]);
+        const uint32_t step = a.state[2 + row], cap = a.state[1], len = a.lens[row];
+        const bool live = threadIdx.x < kGreedyParts;
+        float va = live ? pa : -INFINITY, vb = live ? pb : -INFINITY;
+        uint32_t ia = live ? pi : 0xffffffffu;
+        auto offer = [&](float oa, float ob, uint32_t oi) {
+            if (oa > va || (oa == va && oi < ia)) { vb = fmaxf(va, ob); va = oa; ia = oi; }
+            else vb = fmaxf(vb, oa);
+        };
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float oa = __shfl_xor(va, o, 64), ob = __shfl_xor(vb, o, 64);
+            const uint32_t oi = __shfl_xor(ia, o, 64);
+            offer(oa, ob, oi);
+        }
+        if (threadIdx.x == 0) {
+            uint32_t tok = ia == 0xffffffffu ? 0u : ia;
+            if (tok >= a.n) tok = a.n - 1;
+            if (step < cap) {
+                a.ids[(size_t)row * cap + step] = tok;
+                a.gaps[(size_t)row * cap + step] = va - vb;
+            }
+            a.state[2 + row] = step + 1u;
+            a.lens[row] = len + 1u;
+            s_tok = tok;
+        }
+    }
+    __syncthreads();
+    const uint32_t tok = s_tok;
+    for (uint32_t i = threadIdx.x; i < a.d_model; i += 256u)
+        a.x_out[(size_t)row * a.d_model + i] = m40_h2f(a.table[(size_t)tok * a.d_model + i]);
+}
+
 int pick_slices(int ntiles, int KT, int num_cus) {
     const long long groups = (ntiles + kWavesPerGroup - 1) / kWavesPerGroup;
     int s = 1;
@@ -787,7 +876,18 @@ int m40llm_ext_batched_greedy_step_async(M40llmCudaContext* ctx, const void* d_l
     a.logits = static_cast<const float*>(d_logits_f32); a.n = n; a.state = state_dev; a.lens = seq_lens_dev;
     a.ids = ids_dev; a.gaps = gaps_dev; a.table = static_cast<const uint16_t*>(d_table_f16); a.d_model = d_model;
     a.x_out = static_cast<float*>(d_x_out_f32);
-    greedy_batch_kernel<<<rows, 1024, 0, ctx->decode_stream>>>(a);
+    // Wide rows: parts in the block-select scratch of the decode stream (work on a stream is ordered, and the merge
+    // launch consumes them before anything else on the stream can write there).
+    M40StreamScratch& scr = ctx->scratch[1];
+    const size_t part_bytes = (size_t)rows * kGreedyParts * 4 * sizeof(float);
+    if (n >= 16384u && (n & 3u) == 0u && (reinterpret_cast<uintptr_t>(d_logits_f32) & 15u) == 0u && scr.select &&
+        part_bytes <= scr.select_bytes) {
+        float* part = static_cast<float*>(scr.select);
+        greedy_batch_part_kernel<<<dim3(kGreedyParts, rows), 256, 0, ctx->decode_stream>>>(a, part);
+        greedy_batch_merge_kernel<<<rows, 256, 0, ctx->decode_stream>>>(a, part);
+    } else {
+        greedy_batch_kernel<<<rows, 1024, 0, ctx->decode_stream>>>(a);
+    }
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -379,3 +379,38 @@ def test_batched_greedy_step_and_lm_head(dev, orc):
         assert gaps[r, 1] == srt[-1] - srt[-2]
         assert np.array_equal(xo[r], table[tok].view(np.float16).astype(np.float32))
     assert ids[4, 1] == 100 and gaps[4, 1] == 0.0
+
+
+@pytest.mark.parametrize("V", [151936, 16388, 32000])
+def test_batched_greedy_step_wide_rows(dev, orc, V):
+    """Rows of 16384 logits and more are reduced by several workgroups per row and merged by a second launch: the pick
+    is the first index of the maximum (ties inside one part and across parts), the gap is top-1 minus top-2."""
+    rng = np.random.default_rng(V)
+    rows, D, cap = 5, 64, 2
+    lg = rng.standard_normal((rows, V)).astype(np.float32)
+    top = float(lg.max()) + 1.0
+    lg[0, V - 1] = top                                       # last element of the last part
+    lg[1, 7] = lg[1, V // 2 + 3] = lg[1, V - 5] = top        # tie across parts: index 7 wins, gap 0
+    lg[2, 4001] = lg[2, 4002] = top                          # tie inside one part
+    lg[3, :] = -np.inf; lg[3, V // 3] = -1e30                # a single finite value
+    table = f16bits(rng.standard_normal((V, D)))
+    logits, dT = dev.up(lg), dev.up(table)
+    state = np.zeros(2 + rows, dtype=np.uint32); state[1] = cap
+    lens = np.arange(3, 3 + rows, dtype=np.uint32)
+    dstate, dlens = dev.up(state), dev.up(lens)
+    dids, dgaps, xout = dev.zeros(rows * cap * 4), dev.zeros(rows * cap * 4), dev.zeros(rows * D * 4)
+    for step in range(2):                                    # the second call reuses the scratch of the first
+        dev.call("m40llm_ext_batched_greedy_step_async", logits.ptr, rows, V, dstate.ptr, dlens.ptr, dids.ptr, dgaps.ptr,
+                 dT.ptr, D, xout.ptr)
+    dev.sync()
+    ids = dids.download(np.uint32, (rows, cap)); gaps = dgaps.download(np.float32, (rows, cap))
+    xo = xout.download(np.float32, (rows, D))
+    assert np.array_equal(dlens.download(np.uint32, (rows,)), lens + 2)
+    assert np.array_equal(dstate.download(np.uint32, state.shape)[2:], np.full(rows, 2))
+    for r in range(rows):
+        tok = orc.sample_greedy(lg[r])
+        assert ids[r, 0] == ids[r, 1] == tok == int(np.argmax(lg[r]))
+        srt = np.sort(lg[r])
+        assert gaps[r, 0] == gaps[r, 1] == srt[-1] - srt[-2]
+        assert np.array_equal(xo[r], table[tok].view(np.float16).astype(np.float32))
+    assert ids[1, 0] == 7 and gaps[1, 0] == 0.0 and ids[2, 0] == 4001 and ids[3, 0] == V // 3 and gaps[3, 0] == np.inf
