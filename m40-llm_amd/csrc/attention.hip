@@ -186,23 +186,40 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     __shared__ float s_num[NCG][HD];
     const uint32_t qh = blockIdx.x, b = blockIdx.y;
     const uint32_t d = threadIdx.x % HD, cg = threadIdx.x / HD;
+    // The lane's first kPre chunk partials are requested together with the row's length and id, before either is
+    // known (one memory round trip instead of a chain of three); partials of chunks past the row's end are stale
+    // values inside the buffer and are never used.  The chunks are folded in the same ascending order either way.
+    constexpr uint32_t kPre = 8;
+    const float* w = p.ws + (((size_t)b * p.q_heads + qh) * p.nchunks) * (HD + 2);
+    float pm[kPre], pl[kPre], pv[kPre];
+#pragma unroll
+    for (uint32_t u = 0; u < kPre; ++u) {
+        const uint32_t ch = cg + u * NCG;
+        const float* wc = w + (size_t)(ch < p.nchunks ? ch : 0u) * (HD + 2);
+        pm[u] = wc[0]; pl[u] = wc[1]; pv[u] = wc[2 + d];
+    }
     const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
+    const uint32_t sid = (p.max_batch != 0 && p.seq_ids_dev) ? p.seq_ids_dev[b] : 0u;
     if (len == 0 || len > p.max_seq_len) return;
-    if (p.max_batch != 0 && p.seq_ids_dev && p.seq_ids_dev[b] >= p.max_batch) return;
+    if (p.max_batch != 0 && p.seq_ids_dev && sid >= p.max_batch) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
     const uint32_t n = (len - t0 + p.chunk - 1) / p.chunk;
-    const float* w = p.ws + (((size_t)b * p.q_heads + qh) * p.nchunks) * (HD + 2);
     float m = -INFINITY, num = 0.0f, den = 0.0f;
-#pragma unroll 4
-    for (uint32_t ch = cg; ch < n; ch += NCG) {
-        const float* wc = w + (size_t)ch * (HD + 2);
-        const float mc = wc[0], lc = wc[1], vc = wc[2 + d];
+    auto fold = [&](float mc, float lc, float vc) {
         const float nm = fmaxf(m, mc);
         const float fa = m == -INFINITY ? 0.0f : expf(m - nm);
         const float fb = mc == -INFINITY ? 0.0f : expf(mc - nm);
         num = fmaf(num, fa, vc * fb);
         den = fmaf(den, fa, lc * fb);
         m = nm;
+    };
+#pragma unroll
+    for (uint32_t u = 0; u < kPre; ++u)
+        if (cg + u * NCG < n) fold(pm[u], pl[u], pv[u]);
+#pragma unroll 4
+    for (uint32_t ch = cg + kPre * NCG; ch < n; ch += NCG) {
+        const float* wc = w + (size_t)ch * (HD + 2);
+        fold(wc[0], wc[1], wc[2 + d]);
     }
     s_num[cg][d] = num;
     if (d == 0) { s_m[cg] = m; s_den[cg] = den; }
