@@ -342,7 +342,7 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
  * writes the top-1 minus top-2 gap to out_gap_dev (may be NULL).  Decode stream. */
 int m40llm_ext_argmax_f32_async(M40llmCudaContext* ctx, const void* d_logits_f32, uint32_t rows,
                                 size_t n, uint32_t* out_idx_dev, float* out_gap_dev);
-/* Bandwidth yardstick (no counterpart in the reference): reads `bytes` (16-byte aligned start) of device memory
+/* DIAGNOSTIC, not part of the decode path.  Bandwidth yardstick (no counterpart in the reference): reads `bytes` (16-byte aligned start) of device memory
  * once, `workgroups` (<= 65536) workgroups of 256 threads each owning a contiguous range, and xors every 32-bit word
  * read into d_out_u32[0 .. 2047] (word = workgroup index modulo 2048; not cleared by the call).  One launch on the
  * decode stream; the benchmarks time it beside the kernels it bounds. */
@@ -405,6 +405,18 @@ int m40llm_ext_attention_last_token_f32_gqa_position_dev_async(M40llmCudaContext
                                                                uint32_t q_heads, const uint32_t* position_dev,
                                                                uint32_t max_len_hint, void* out_dev_f32);
 /* embedding row of the token id stored at token_dev (f16 table [vocab][d_model]) -> f32 */
+/* No counterpart in the reference.  m40llm_attention_last_token_f32_gqa_async for callers that cannot allocate:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same argument checks, kernels
+ * and results as that entry point, but the chunk partials of rows longer than 512 tokens go into a fixed 2 MiB
+ * device array that is part of the library's code object (one copy per GPU, resolved once per device when a context
+ * is created), and the call allocates nothing.  Returns -9 when the partials of this (q_heads, head_dim, seq_len) do
+ * not fit 2 MiB: q_heads * chunks * (head_dim + 2) * 4 bytes, chunks = ceil(seq_len / chunk) with the chunk length
+ * the allocating entry point uses.  Every call on one GPU shares that array: calls that overlap on one GPU (other
+ * contexts, or the other stream) race; calls on the decode stream of one context are ordered and safe. */
+int m40llm_ext_attention_last_token_f32_gqa_static_scratch_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                                 uint32_t seq_id, const void* q_dev_f32,
+                                                                 uint32_t q_heads, uint32_t seq_len,
+                                                                 void* out_dev_f32);
 int m40llm_ext_embed_token_dev_async(M40llmCudaContext* ctx, const void* d_table_f16, const uint32_t* token_dev,
                                      uint32_t vocab, uint32_t d_model, void* d_out_f32);
 /* device-side greedy step over logits[n] (scanned directly, or through the per-workgroup candidates in

@@ -13,6 +13,33 @@
 // batched :1740-1823 and :4694-4832.
 #include "attention_params.hpp"
 
+#include <mutex>
+
+// Fixed chunk-partial buffer of m40llm_ext_attention_last_token_f32_gqa_static_scratch_async: device memory that
+// exists from the moment the code object is loaded, so that entry point never allocates.  Every GPU the library
+// runs on holds its own copy (at its own address) until the process ends.  In host code the array's name is a
+// stand-in, not a device address: host code only ever uses the pointers that hipGetSymbolAddress returned
+// (g_static_scratch_ptr), one per device.
+constexpr size_t kStaticScratchBytes = 2u << 20;   // 2 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kStaticScratchMaxDevices = 64;
+static float* g_static_scratch_ptr[kStaticScratchMaxDevices];
+static std::mutex g_static_scratch_mutex;
+
+int m40_attention_static_scratch_init(int device_id) {
+    if (device_id < 0 || device_id >= kStaticScratchMaxDevices) return -2;
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    if (g_static_scratch_ptr[device_id]) return 0;
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+        (void)hipGetLastError();
+        return -4;
+    }
+    g_static_scratch_ptr[device_id] = static_cast<float*>(ptr);
+    return 0;
+}
+
 namespace {
 
 constexpr int kAttnThreads = 512;
@@ -292,10 +319,9 @@ void launch_g(hipStream_t stream, const AttnParams& p, uint32_t batch, int S) {
 
 // Chooses rows per lane group (S), q heads per workgroup (G) and the chunking for a span of `span` tokens.
 template <int HD>
-int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, AttnParams& p, uint32_t batch,
-              uint32_t group, uint32_t span) {
+int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, float* partial, size_t partial_bytes, bool fixed_chunking,
+              AttnParams& p, uint32_t batch, uint32_t group, uint32_t span) {
     constexpr uint32_t kRowsPerStep = kWaves * (64 / (HD / 8));   // token rows one workgroup covers per S
-    M40StreamScratch& scr = ctx->scratch[stream_kind];
     if (span > 512 && m40_aligned16(p.Q)) {
         // long rows: matrix-core kernel (it reads q with 16-byte loads).  Chunks are a multiple of 128 tokens (one
         // 32-token tile per wave and pass) sized for about one workgroup per CU -- measured best at 32 K tokens (256
@@ -310,10 +336,11 @@ int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, 
         for (;;) {
             p.chunk = (uint32_t)chunk;
             p.nchunks = (span + p.chunk - 1) / p.chunk;
-            if (p.nchunks == 1 || (size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float) <= scr.attn_partial_bytes) break;
+            if (p.nchunks == 1 || (size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float) <= partial_bytes) break;
+            if (fixed_chunking) return -9;   // the caller wants this chunking or none (fixed-size partial buffer)
             chunk *= 2;
         }
-        p.ws = static_cast<float*>(scr.attn_partial);
+        p.ws = partial;
         m40_launch_attn_mfma(stream, p, HD, batch);
         if (p.nchunks > 1) {
             dim3 grid(p.q_heads, batch);
@@ -340,18 +367,18 @@ int launch_hd(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, 
     }
     p.chunk = kRowsPerStep * (uint32_t)S;
     p.nchunks = (span + p.chunk - 1) / p.chunk;
-    M40StreamScratch& sc = ctx->scratch[stream_kind];
     if (p.nchunks > 1) {
         const size_t need = (size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float);
-        if (need > sc.attn_partial_bytes) {
+        if (need > partial_bytes) {
+            if (fixed_chunking) return -9;
             if (S == 8) return -7;
             S = 8;
             p.chunk = kRowsPerStep * 8u;
             p.nchunks = (span + p.chunk - 1) / p.chunk;
-            if ((size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float) > sc.attn_partial_bytes) return -7;
+            if ((size_t)batch * p.q_heads * p.nchunks * (HD + 2) * sizeof(float) > partial_bytes) return -7;
         }
     }
-    p.ws = static_cast<float*>(sc.attn_partial);
+    p.ws = partial;
     switch (G) {
         case 4: launch_g<HD, 4>(stream, p, batch, S); break;
         case 2: launch_g<HD, 2>(stream, p, batch, S); break;
@@ -383,8 +410,12 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
     if (span == 0) span = 1;
 
     if ((a.head_dim == 64 || a.head_dim == 128) && m40_aligned16(a.Q) && m40_aligned16(a.K) && m40_aligned16(a.V)) {
-        const int rc = a.head_dim == 64 ? launch_hd<64>(ctx, stream, stream_kind, p, a.batch, group, span)
-                                        : launch_hd<128>(ctx, stream, stream_kind, p, a.batch, group, span);
+        M40StreamScratch& scr = ctx->scratch[stream_kind];
+        float* partial = a.partial_override ? a.partial_override : static_cast<float*>(scr.attn_partial);
+        const size_t partial_bytes = a.partial_override ? a.partial_override_bytes : scr.attn_partial_bytes;
+        const bool fixed = a.partial_override != nullptr;
+        const int rc = a.head_dim == 64 ? launch_hd<64>(ctx, stream, partial, partial_bytes, fixed, p, a.batch, group, span)
+                                        : launch_hd<128>(ctx, stream, partial, partial_bytes, fixed, p, a.batch, group, span);
         if (rc != 0) return rc;
     } else {
         p.chunk = span; p.nchunks = 1;
@@ -443,6 +474,38 @@ int m40llm_attention_last_token_f32_gqa_async(M40llmCudaContext* ctx, const M40l
     a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
     a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = seq_len;
     a.max_len_hint = seq_len;
+    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+}
+
+// m40llm_attention_last_token_f32_gqa_async for callers that cannot allocate (HIP graph capture, serving loops and
+// harnesses that forbid hipMalloc): same checks, kernels, chunking and results, but the chunk partials of a long
+// row go into this device's copy of the fixed 2 MiB array above instead of the context's arena.  Calls nothing that
+// allocates.  -9: the partials of this (q_heads, head_dim, seq_len) do not fit the fixed buffer.  All calls on one
+// GPU share that buffer (every partial a call reads it has written itself, so nothing needs clearing between
+// calls); two calls that overlap on one GPU -- from different contexts or streams -- race.
+int m40llm_ext_attention_last_token_f32_gqa_static_scratch_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
+                                                                 uint32_t seq_id, const void* q_dev_f32,
+                                                                 uint32_t q_heads, uint32_t seq_len,
+                                                                 void* out_dev_f32) {
+    if (!ctx || !kv || !q_dev_f32 || !out_dev_f32) return -1;
+    if (seq_id >= kv->max_batch_size) return -2;
+    if (seq_len == 0 || seq_len > kv->max_seq_len) return -3;
+    if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -6;
+    if (!kv->d_k || !kv->d_v) return -4;
+    if (ctx->device_id < 0 || ctx->device_id >= kStaticScratchMaxDevices) return -4;
+    float* ptr = g_static_scratch_ptr[ctx->device_id];
+    if (!ptr) {
+        // a context made before this translation unit could resolve the symbol: resolve it now, on the context's device
+        if (m40_ensure_device(ctx) != 0 || m40_attention_static_scratch_init(ctx->device_id) != 0) return -4;
+        ptr = g_static_scratch_ptr[ctx->device_id];
+    }
+    M40AttnArgs a{};
+    a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
+    a.head_dim = kv->head_dim; a.q_heads = q_heads; a.Q = static_cast<const float*>(q_dev_f32);
+    a.Out = static_cast<float*>(out_dev_f32); a.batch = 1; a.seq_id = seq_id; a.seq_len = seq_len;
+    a.max_len_hint = seq_len;
+    a.partial_override = ptr;
+    a.partial_override_bytes = kStaticScratchBytes;
     return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
 }
 

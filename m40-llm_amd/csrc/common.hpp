@@ -163,7 +163,14 @@ struct M40AttnArgs {
     uint32_t window;                // 0 = whole sequence, else only the last `window` tokens
     uint32_t len_bias;              // added to lengths read from seq_lens_dev
     uint32_t max_batch;             // 0, or the bound that device-side sequence ids are checked against
+    // chunk partials go here instead of into the context's per-stream arena (null = the arena); with an override
+    // the chunking is the one the arena would get, and a call whose partials do not fit is refused with -9
+    float* partial_override;
+    size_t partial_override_bytes;
 };
+// attention.hip: resolves this device's copy of the fixed partial buffer of
+// m40llm_ext_attention_last_token_f32_gqa_static_scratch_async (the device must be current); 0 or a negative code
+int m40_attention_static_scratch_init(int device_id);
 int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind,
                                const M40AttnArgs& a);
 

@@ -124,6 +124,10 @@ M40llmCudaContext* m40llm_create_context(int device_id) {
         m40llm_destroy_context(ctx);
         return nullptr;
     }
+    if (m40_attention_static_scratch_init(selected) != 0) {
+        m40llm_destroy_context(ctx);
+        return nullptr;
+    }
     hipDeviceProp_t prop;
     ctx->num_cus = 256;
     if (hipGetDeviceProperties(&prop, selected) == hipSuccess && prop.multiProcessorCount > 0) {
