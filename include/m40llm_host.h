@@ -148,6 +148,12 @@ int m40host_model_decode_timed(M40HostModel* model, uint32_t sequence_id, const 
 int m40host_model_decode_batch_timed(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
                                      const uint32_t* first_tokens, uint32_t rows, uint32_t warmup, uint32_t steps,
                                      uint32_t* ids_out, double* elapsed_ms);
+/* 1 when the last decode_timed / decode_batch_timed call measured the host-sampled path: a device-side greedy pick
+ * had a top-1 / top-2 logit gap under the tie guard, so warm-up and timed steps were redone through the host sampler
+ * (as m40host_model_decode_greedy / decode_batch_greedy do); 0 when the device path was measured */
+int m40host_model_last_timed_host_fallback(M40HostModel* model);
+/* top-1 / top-2 logit gap under which a device-side greedy pick is not trusted (default 1e-6) */
+int m40host_model_set_tie_guard(M40HostModel* model, float guard);
 /* one batched step: hidden_host [rows][d_model] and logits_host [rows][vocab] may be NULL */
 int m40host_model_forward_batched(M40HostModel* model, const uint32_t* sequence_ids, const uint32_t* kv_lens,
                                   const uint32_t* token_ids, uint32_t rows, float* hidden_host, float* logits_host);

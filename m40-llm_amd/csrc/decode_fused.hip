@@ -136,7 +136,7 @@ struct QkvArgs {
     uint32_t* seq_map_entry;
     const uint32_t* position_dev;
     const float* rope_table;   // pair frequencies of (head_dim, rope_base), or null: the kernel evaluates the power
-    float4* rope_cs;           // with rope_table: {position bits, cos, sin, scale bits} per pair, kept from launch to launch
+    float4* rope_cs;           // with rope_table: {position bits, cos, sin, tag of (position, scale)} per pair, kept from launch to launch
     uint32_t position, max_seq_len;
     uint32_t d_model, q_heads, kv_heads, head_dim, rope_layout, norm_dtype;
     float eps, rope_base, rope_scale;
@@ -194,15 +194,18 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
         cs[q] = make_float2(1.0f, 0.0f);
         if (which[q] != 2) {
             // The angle depends on the position only: all layers of a step share it.  An entry is 16 bytes, stored and
-            // loaded whole, and carries its own position and scale, so a reader takes it only when it is this step's.
-            const bool hit = p.rope_cs && __float_as_uint(kept[q].x) == position && __float_as_uint(kept[q].w) == __float_as_uint(p.rope_scale);
+            // loaded whole; its first word is the position and its last word a tag of (position, scale), so a reader
+            // takes cos / sin (the words between them) only when both ends are this step's -- also if a launch that
+            // writes the entry (the step's first layer) overlaps its readers and the 16 bytes were not seen as one.
+            const uint32_t tag = position ^ __float_as_uint(p.rope_scale) ^ 0x9e3779b9u;
+            const bool hit = p.rope_cs && __float_as_uint(kept[q].x) == position && __float_as_uint(kept[q].w) == tag;
             if (hit) {
                 cs[q] = make_float2(kept[q].y, kept[q].z);
             } else {
                 if (!p.rope_table) inv_freq[q] = m40_rope_inv_freq(off[q], p.head_dim, p.rope_base);
                 cs[q] = m40_rope_cos_sin_freq(position, inv_freq[q], p.rope_scale);
                 if (p.rope_cs && which[q] == 0 && local[q] < half && lane == 0)      // the waves of q head 0 keep it
-                    p.rope_cs[off[q]] = make_float4(__uint_as_float(position), cs[q].x, cs[q].y, p.rope_scale);
+                    p.rope_cs[off[q]] = make_float4(__uint_as_float(position), cs[q].x, cs[q].y, __uint_as_float(tag));
             }
         }
     }

@@ -367,6 +367,12 @@ int m40host_model_decode_batch_timed(M40HostModel* m, const uint32_t* seq_ids, c
         },
         -100);
 }
+int m40host_model_last_timed_host_fallback(M40HostModel* m) { return m && m->m->last_timed_host_fallback() ? 1 : 0; }
+int m40host_model_set_tie_guard(M40HostModel* m, float guard) {
+    if (!m) return -1;
+    m->m->set_tie_guard(guard);
+    return 0;
+}
 int m40host_model_forward_batched(M40HostModel* m, const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* tokens,
                                   uint32_t rows, float* hidden_host, float* logits_host) {
     return guarded(

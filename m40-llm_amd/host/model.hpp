@@ -86,6 +86,7 @@ private:
 // Named f32 scratch buffers sized by row count (src/infer/workspace.rs:60-126).
 struct ForwardWorkspace {
     uint32_t rows = 0;
+    uint32_t generation = 0;   // bumped whenever the buffers are reallocated: captured graphs hold their addresses
     DeviceBuf xn, q, k, v, ctx_out, y_attn, x1, x1n, gate, up, hid, y_mlp, scratch_a, scratch_b, norm_hidden, logits;
     DeviceBuf argmax_idx, argmax_gap, positions;
     void ensure(M40llmCudaContext* c, const ModelConfig& m, uint32_t want_rows) {
@@ -99,6 +100,7 @@ struct ForwardWorkspace {
         logits = DeviceBuf(c, R * (size_t)m.vocab * 4);
         argmax_idx = DeviceBuf(c, R * 4); argmax_gap = DeviceBuf(c, R * 4); positions = DeviceBuf(c, R * 4 * 2);
         rows = want_rows;
+        ++generation;
     }
 };
 
@@ -162,6 +164,16 @@ public:
     uint32_t kv_slot(uint32_t seq, uint32_t layer) const {
         if (seq >= cfg_.max_sequences) throw std::out_of_range("sequence id out of range");   // kv.rs:92-107
         return seq * cfg_.n_layers + layer;
+    }
+
+    // Grows the activation buffers.  A captured graph has the old buffers' addresses baked in, so both graphs are
+    // dropped (after the streams have drained: the old buffers may still be in use) before anything is reallocated.
+    void ensure_workspace(uint32_t rows) {
+        if (rows <= ws_.rows) return;
+        if (ws_.rows != 0) sync_all();
+        drop_graph();
+        drop_batch_graph();
+        ws_.ensure(ctx_, cfg_, rows);
     }
 
     // ---- single sequence ---------------------------------------------------------------------
@@ -247,7 +259,7 @@ public:
     // All layers for one token; returns the device pointer that holds the final hidden state.
     const float* forward_token(uint32_t seq, uint32_t pos, uint32_t token_id) {
         if (pos >= cfg_.max_seq_len) throw std::out_of_range("position beyond max_seq_len");
-        ws_.ensure(ctx_, cfg_, 1);
+        ensure_workspace(1);
         float* a = ws_.scratch_a.f32();
         float* b = ws_.scratch_b.f32();
         const bool fused = mode_ >= 1 && fused_available();
@@ -267,6 +279,9 @@ public:
     // ---- device-driven greedy loop (modes 1 and 2) ---------------------------------------------
     // state = {position of the last processed token, step, token, capacity, ids[cap], gaps[cap]}
     static constexpr float kGreedyTieGuard = 1e-6f;
+    // the guard in force; tests raise it to drive the host-sampled fallback on purpose
+    void set_tie_guard(float g) { tie_guard_ = g; }
+    float tie_guard() const { return tie_guard_; }
     void ensure_state(uint32_t capacity) {
         if (capacity <= state_cap_) return;
         state_ = DeviceBuf(ctx_, (size_t)(4 + 2 * capacity) * 4);
@@ -315,7 +330,8 @@ public:
             uint32_t n = steps - done;
             if (hint < cfg_.max_seq_len && pos + n > hint) n = hint - pos;
             if (mode_ >= 2) {
-                if (!graph_ || graph_seq_ != seq || graph_hint_ != hint || graph_hidden_ != hidden) {
+                if (!graph_ || graph_seq_ != seq || graph_hint_ != hint || graph_hidden_ != hidden ||
+                    graph_ws_generation_ != ws_.generation) {
                     drop_graph();
                     M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
                     M40H_TRY(m40llm_cuda_graph_begin_capture(ctx_, M40LLM_STREAM_DECODE));
@@ -326,7 +342,7 @@ public:
                         throw;
                     }
                     M40H_TRY(m40llm_cuda_graph_end_capture(ctx_, M40LLM_STREAM_DECODE, &graph_));
-                    graph_seq_ = seq; graph_hint_ = hint; graph_hidden_ = hidden;
+                    graph_seq_ = seq; graph_hint_ = hint; graph_hidden_ = hidden; graph_ws_generation_ = ws_.generation;
                 }
                 for (uint32_t i = 0; i < n; ++i) M40H_TRY(m40llm_cuda_graph_launch(ctx_, graph_, M40LLM_STREAM_DECODE));
             } else {
@@ -344,7 +360,7 @@ public:
         if (n_prompt == 0) throw std::invalid_argument("decode needs at least one prompt token");
         const uint32_t total = warmup + steps;
         if (start_pos + n_prompt + total > cfg_.max_seq_len) throw std::out_of_range("decode would exceed max_seq_len");
-        ws_.ensure(ctx_, cfg_, 1);
+        ensure_workspace(1);
         ensure_state(total);
         uint32_t pos = start_pos;
         const float* h = nullptr;
@@ -372,7 +388,7 @@ public:
             float gap;
             std::memcpy(&gap, &st[4 + state_cap_ + g], 4);
             if (gaps_out) gaps_out[g] = gap;
-            if (!(gap >= kGreedyTieGuard)) ok = false;
+            if (!(gap >= tie_guard_)) ok = false;
         }
         return ok;
     }
@@ -495,7 +511,7 @@ public:
     const float* forward_batched(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* token_ids, uint32_t rows) {
         if (rows == 0) throw std::invalid_argument("empty batch");
         if (kvcfg_.is_enabled()) throw std::invalid_argument("batched decode requires the dense KV cache");
-        ws_.ensure(ctx_, cfg_, rows);
+        ensure_workspace(rows);
         const uint32_t D = cfg_.d_model, KV = cfg_.kv_heads * cfg_.head_dim, F = cfg_.ffn;
         const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
         float* a = ws_.scratch_a.f32();
@@ -640,7 +656,7 @@ public:
         }
         for (uint32_t r0 = 0; r0 < rows; r0 += 16) {
             const uint32_t n = rows - r0 < 16 ? rows - r0 : 16;
-            ws_.ensure(ctx_, cfg_, n);
+            ensure_workspace(n);
             std::vector<uint32_t> table((size_t)cfg_.n_layers * n + 2 * n);   // slots per layer, then lengths, then tokens
             uint32_t longest = 0;
             for (uint32_t l = 0; l < cfg_.n_layers; ++l)
@@ -683,7 +699,7 @@ public:
                 M40H_TRY(m40llm_memcpy_d2h(ctx_, gap.data(), ws_.argmax_gap.ptr(), (size_t)n * 4));
             }
             for (uint32_t r = 0; r < n; ++r) {
-                if (any_greedy && greedy[r0 + r] && gap[r] >= kGreedyTieGuard) {
+                if (any_greedy && greedy[r0 + r] && gap[r] >= tie_guard_) {
                     picks[r0 + r] = idx[r];
                     picked[r0 + r] = 1;
                 } else {
@@ -704,7 +720,7 @@ public:
             if (seq_ids[r] >= cfg_.max_sequences) throw std::out_of_range("sequence id out of range");
             max_len = kv_lens[r] > max_len ? kv_lens[r] : max_len;
         }
-        ws_.ensure(ctx_, cfg_, rows);
+        ensure_workspace(rows);
         // device state: slot ids per layer, lengths, per-row step counters, picks and gaps
         std::vector<uint32_t> slots((size_t)cfg_.n_layers * rows);
         for (uint32_t l = 0; l < cfg_.n_layers; ++l)
@@ -731,7 +747,7 @@ public:
                 uint32_t n = n_steps - done;
                 if (hint < cfg_.max_seq_len && longest + n > hint) n = hint - longest;
                 if (mode_ >= 2) {
-                    if (!bgraph_ || bgraph_rows_ != rows || bgraph_hint_ != hint) {
+                    if (!bgraph_ || bgraph_rows_ != rows || bgraph_hint_ != hint || bgraph_ws_generation_ != ws_.generation) {
                         drop_batch_graph();
                         M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_DECODE));
                         M40H_TRY(m40llm_cuda_graph_begin_capture(ctx_, M40LLM_STREAM_DECODE));
@@ -742,7 +758,7 @@ public:
                             throw;
                         }
                         M40H_TRY(m40llm_cuda_graph_end_capture(ctx_, M40LLM_STREAM_DECODE, &bgraph_));
-                        bgraph_rows_ = rows; bgraph_hint_ = hint;
+                        bgraph_rows_ = rows; bgraph_hint_ = hint; bgraph_ws_generation_ = ws_.generation;
                     }
                     for (uint32_t i = 0; i < n; ++i) M40H_TRY(m40llm_cuda_graph_launch(ctx_, bgraph_, M40LLM_STREAM_DECODE));
                 } else {
@@ -765,7 +781,7 @@ public:
         bool ok = true;
         for (size_t i = 0; i < gaps.size(); ++i) {
             if (gaps_out) gaps_out[i] = gaps[i];
-            if (!(gaps[i] >= kGreedyTieGuard)) ok = false;
+            if (!(gaps[i] >= tie_guard_)) ok = false;
         }
         return ok;
     }
@@ -805,8 +821,11 @@ public:
                       uint32_t* ids_out, double* elapsed_ms) {
         if (n_prompt == 0) throw std::invalid_argument("decode_timed needs a prompt");
         if (mode_ >= 1 && fused_available()) {
+            last_timed_host_fallback_ = false;
             if (decode_greedy_device(seq, prompt, n_prompt, warmup, steps, 0, ids_out, nullptr, elapsed_ms)) return;
-            throw std::runtime_error("near-tie in a greedy pick on the device path; rerun in mode 0");
+            // a device pick was a near tie: the whole run (warm-up and timed steps) is redone through the host sampler,
+            // which rewrites the same cache rows; last_timed_host_fallback() tells the caller which path was timed
+            last_timed_host_fallback_ = true;
         }
         std::vector<float> logits(cfg_.vocab);
         Sampler sampler = greedy_sampler(42);
@@ -834,8 +853,9 @@ public:
     void decode_batch_timed(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens, uint32_t rows,
                             uint32_t warmup, uint32_t steps, uint32_t* ids_out, double* elapsed_ms) {
         if (mode_ >= 1 && batched_fused_available(rows)) {
+            last_timed_host_fallback_ = false;
             if (decode_batch_device(seq_ids, kv_lens, first_tokens, rows, warmup, steps, ids_out, nullptr, elapsed_ms)) return;
-            throw std::runtime_error("near-tie in a greedy pick on the device path; rerun in mode 0");
+            last_timed_host_fallback_ = true;   // as in decode_timed: redo everything on the host-sampled path
         }
         std::vector<uint32_t> lens(kv_lens, kv_lens + rows), toks(first_tokens, first_tokens + rows);
         std::vector<float> logits((size_t)rows * cfg_.vocab);
@@ -859,6 +879,10 @@ public:
         const auto t1 = std::chrono::steady_clock::now();
         if (elapsed_ms) *elapsed_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
     }
+
+    // true when the last decode_timed / decode_batch_timed call measured the host-sampled path because a device-side
+    // greedy pick was a near tie
+    bool last_timed_host_fallback() const { return last_timed_host_fallback_; }
 
     void sync_all() {
         M40H_TRY(m40llm_stream_synchronize(ctx_, M40LLM_STREAM_PREFILL));
@@ -923,6 +947,8 @@ private:
     ForwardWorkspace ws_;
     PrefillWorkspace pws_;
     uint32_t mode_ = 0;
+    bool last_timed_host_fallback_ = false;
+    float tie_guard_ = kGreedyTieGuard;
     DeviceBuf state_;
     DeviceBuf top2_;
     static constexpr uint32_t kTop2Capacity = 1u << 16;
@@ -931,9 +957,9 @@ private:
     DeviceBuf tick_table_;
     size_t tick_table_cap_ = 0;
     M40llmCudaGraphExec* bgraph_ = nullptr;
-    uint32_t bgraph_rows_ = 0, bgraph_hint_ = 0;
+    uint32_t bgraph_rows_ = 0, bgraph_hint_ = 0, bgraph_ws_generation_ = 0;
     M40llmCudaGraphExec* graph_ = nullptr;
-    uint32_t graph_seq_ = 0, graph_hint_ = 0;
+    uint32_t graph_seq_ = 0, graph_hint_ = 0, graph_ws_generation_ = 0;
     float* graph_hidden_ = nullptr;
 };
 

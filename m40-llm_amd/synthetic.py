@@ -198,6 +198,12 @@ class DeviceModel:
                                                    ids.ctypes.data_as(C.c_void_p), C.byref(ms)), "m40host_model_decode_timed")
         return ids, ms.value
 
+    def last_timed_host_fallback(self):
+        return bool(self.H.m40host_model_last_timed_host_fallback(self.h))
+
+    def set_tie_guard(self, guard):
+        self._ok(self.H.m40host_model_set_tie_guard(self.h, C.c_float(guard)), "m40host_model_set_tie_guard")
+
     def decode_batch_timed(self, seq_ids, kv_lens, first_tokens, warmup, steps):
         s = np.ascontiguousarray(seq_ids, dtype=np.uint32); l = np.ascontiguousarray(kv_lens, dtype=np.uint32)
         t = np.ascontiguousarray(first_tokens, dtype=np.uint32)
