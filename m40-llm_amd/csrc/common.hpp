@@ -53,6 +53,7 @@ struct M40llmCudaContext {
     struct { float base; uint32_t head_dim; uint32_t ready; } rope_slots[2][4];
 };
 constexpr int kM40HostStagingWords = 2048;
+constexpr uint32_t kM40OldStoreSlackRows = 64;
 constexpr int kM40RopeSlots = 4;
 constexpr int kM40RopeTableLen = 256;
 // Table of a (head_dim, base) for kernels launched on `stream` (of kind stream_kind), or nullptr (head_dim too large,
@@ -68,9 +69,12 @@ struct M40llmKVCache {
     // compressed storage
     uint16_t* d_recent_k;          // ring [seq][W][kvh][hd], slot = pos % W
     uint16_t* d_recent_v;
-    uint16_t* d_fp16_old_k;        // [seq][max_seq_len][kvh][hd], index = pos - W
-    uint8_t* d_q4_old_v;           // [seq][max_seq_len][kvh][hd/2]
-    float* d_q4_old_v_scale;       // [seq][max_seq_len][kvh]
+    // old store, head-major so that the tokens of a block are one contiguous run per kv head (the handle is
+    // opaque; debug read-backs answer in the reference's [seq][token][kvh] order).  Each array is followed by
+    // kM40OldStoreSlackRows zeroed rows: the attention reads whole passes of rows and ignores those past a block.
+    uint16_t* d_fp16_old_k;        // [seq][kvh][max_seq_len][hd], token index = absolute position
+    uint8_t* d_q4_old_v;           // [seq][kvh][max_seq_len][hd/2]
+    float* d_q4_old_v_scale;       // [seq][kvh][max_seq_len]
     uint32_t max_seq_len;
     uint32_t max_batch_size;
     uint32_t num_heads;            // kv heads

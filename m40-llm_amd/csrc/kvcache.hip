@@ -156,7 +156,9 @@ __global__ __launch_bounds__(64) void compressed_append_kernel(
 
     if (evict && position >= recent_window) {
         const uint32_t old_pos = position - recent_window;
-        const size_t old_base = ((size_t)seq_id * max_seq_len + old_pos) * ept + (size_t)head * HD;
+        // the old store is head-major, [sequence][kv head][token][...]: the tokens of a block are one contiguous run
+        const size_t old_row = ((size_t)seq_id * num_heads + head) * max_seq_len + old_pos;
+        const size_t old_base = old_row * HD;
         float v0 = 0.0f, v1 = 0.0f;
         if (active) {
             old_k[old_base + d0] = recent_k[ring_base + d0];
@@ -166,11 +168,8 @@ __global__ __launch_bounds__(64) void compressed_append_kernel(
         }
         const float max_v = m40_max64(fmaxf(fabsf(v0), fabsf(v1)));
         const float scale = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
-        if (lane == 0) q4_scale[((size_t)seq_id * max_seq_len + old_pos) * num_heads + head] = scale;
-        if (active) {
-            q4_v[((size_t)seq_id * max_seq_len + old_pos) * num_heads * PAIRS + (size_t)head * PAIRS + lane] =
-                m40_pack_q4_pair(v0, v1, scale);
-        }
+        if (lane == 0) q4_scale[old_row] = scale;
+        if (active) q4_v[old_row * PAIRS + lane] = m40_pack_q4_pair(v0, v1, scale);
     }
     __syncthreads();
     if (active) {
@@ -203,7 +202,8 @@ __global__ __launch_bounds__(64) void compressed_bulk_fill_kernel(
     const size_t src = (size_t)t * ept + (size_t)head * HD;
     if (t < old_len) {
         if (!has_old) return;
-        const size_t old_base = ((size_t)seq_id * max_seq_len + t) * ept + (size_t)head * HD;
+        const size_t old_row = ((size_t)seq_id * num_heads + head) * max_seq_len + t;
+        const size_t old_base = old_row * HD;
         float v0 = 0.0f, v1 = 0.0f;
         if (active) {
             old_k[old_base + d0] = k_rows[src + d0];
@@ -213,11 +213,8 @@ __global__ __launch_bounds__(64) void compressed_bulk_fill_kernel(
         }
         const float max_v = m40_max64(fmaxf(fabsf(v0), fabsf(v1)));
         const float scale = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
-        if (lane == 0) q4_scale[((size_t)seq_id * max_seq_len + t) * num_heads + head] = scale;
-        if (active) {
-            q4_v[((size_t)seq_id * max_seq_len + t) * num_heads * PAIRS + (size_t)head * PAIRS + lane] =
-                m40_pack_q4_pair(v0, v1, scale);
-        }
+        if (lane == 0) q4_scale[old_row] = scale;
+        if (active) q4_v[old_row * PAIRS + lane] = m40_pack_q4_pair(v0, v1, scale);
     } else {
         const size_t ring_base = ((size_t)seq_id * recent_window + (t % recent_window)) * ept + (size_t)head * HD;
         if (active) {
@@ -334,9 +331,10 @@ M40llmKVCache* m40llm_kvcache_create_compressed(M40llmCudaContext* ctx, uint32_t
         (void)hipMemset(kv->d_seq_map, 0, seq_map_size);
     }
     if (ok && exact_old_backing == 2u) {
-        const size_t old_k_bytes = kv_elems(kv) * sizeof(uint16_t);
-        const size_t q4_bytes = (size_t)max_seq_len * max_batch_size * num_heads * (head_dim / 2u);
-        const size_t scale_bytes = (size_t)max_seq_len * max_batch_size * num_heads * sizeof(float);
+        // kM40OldStoreSlackRows zeroed rows behind each array (see M40llmKVCache)
+        const size_t old_k_bytes = (kv_elems(kv) + (size_t)kM40OldStoreSlackRows * head_dim) * sizeof(uint16_t);
+        const size_t q4_bytes = ((size_t)max_seq_len * max_batch_size * num_heads + kM40OldStoreSlackRows) * (head_dim / 2u);
+        const size_t scale_bytes = ((size_t)max_seq_len * max_batch_size * num_heads + kM40OldStoreSlackRows) * sizeof(float);
         ok = hipMalloc(reinterpret_cast<void**>(&kv->d_fp16_old_k), old_k_bytes ? old_k_bytes : 2) == hipSuccess &&
              hipMalloc(reinterpret_cast<void**>(&kv->d_q4_old_v), q4_bytes ? q4_bytes : 1) == hipSuccess &&
              hipMalloc(reinterpret_cast<void**>(&kv->d_q4_old_v_scale), scale_bytes ? scale_bytes : 4) == hipSuccess;
@@ -624,12 +622,12 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
                                       size_t offset, size_t bytes, void* out_host) {
     if (!ctx || !kv || !out_host) return -1;
     const void* src = nullptr;
-    size_t total = 0;
+    size_t total = 0, item = 0;     // item: bytes of one (token, kv head) entry of a head-major array, else 0
     const size_t ept = (size_t)kv->num_heads * kv->head_dim;
     switch (which) {
-        case 0: src = kv->d_fp16_old_k; total = kv_elems(kv) * 2; break;
-        case 1: src = kv->d_q4_old_v; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * (kv->head_dim / 2u); break;
-        case 2: src = kv->d_q4_old_v_scale; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * 4; break;
+        case 0: src = kv->d_fp16_old_k; total = kv_elems(kv) * 2; item = (size_t)kv->head_dim * 2; break;
+        case 1: src = kv->d_q4_old_v; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * (kv->head_dim / 2u); item = kv->head_dim / 2u; break;
+        case 2: src = kv->d_q4_old_v_scale; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * 4; item = 4; break;
         case 3: src = kv->d_recent_k; total = (size_t)kv->max_batch_size * kv->recent_window * ept * 2; break;
         case 4: src = kv->d_recent_v; total = (size_t)kv->max_batch_size * kv->recent_window * ept * 2; break;
         case 5: src = kv->d_seq_map; total = (size_t)kv->max_batch_size * 4; break;
@@ -638,7 +636,20 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
     if (!src) return -3;
     if (offset > total || bytes > total - offset) return -4;
     if (hipStreamSynchronize(ctx->decode_stream) != hipSuccess) return -5;
-    if (hipMemcpy(out_host, static_cast<const char*>(src) + offset, bytes, hipMemcpyDeviceToHost) != hipSuccess) return -5;
+    if (item == 0) {
+        if (hipMemcpy(out_host, static_cast<const char*>(src) + offset, bytes, hipMemcpyDeviceToHost) != hipSuccess) return -5;
+        return 0;
+    }
+    // The old store lives head-major on the device ([sequence][kv head][token][...]); the answer is given in the
+    // reference's order, [sequence][token][kv head][...] (cuda/kernels.cu:5435-5543), whatever the device layout.
+    std::vector<char> raw(total), ordered(total);
+    if (hipMemcpy(raw.data(), src, total, hipMemcpyDeviceToHost) != hipSuccess) return -5;
+    const size_t S = kv->max_seq_len, H = kv->num_heads;
+    for (size_t b = 0; b < kv->max_batch_size; ++b)
+        for (size_t h = 0; h < H; ++h)
+            for (size_t t = 0; t < S; ++t)
+                std::memcpy(ordered.data() + ((b * S + t) * H + h) * item, raw.data() + ((b * H + h) * S + t) * item, item);
+    std::memcpy(out_host, ordered.data() + offset, bytes);
     return 0;
 }
 
@@ -710,7 +721,10 @@ int m40llm_kvcache_debug_select_old_blocks(M40llmCudaContext* ctx, const M40llmK
     if (fp16_old) src = kv->d_fp16_old_k;
     else if (!kv->compressed && kv->d_k) src = kv->d_k;
     else return -8;  // summary-backed ranking of the lossy modes is not part of this build
-    std::vector<uint16_t> kh((size_t)old_len * ept);
+    // rows of kv head 0: the fp16 old store is head-major (one contiguous [token][hd] plane per head), the dense
+    // cache token-major
+    const size_t row = fp16_old ? (size_t)hd : ept;
+    std::vector<uint16_t> kh((size_t)old_len * row);
     if (hipMemcpy(kh.data(), src + (size_t)seq_id * kv->max_seq_len * ept, kh.size() * 2,
                   hipMemcpyDeviceToHost) != hipSuccess)
         return -12;
@@ -722,7 +736,7 @@ int m40llm_kvcache_debug_select_old_blocks(M40llmCudaContext* ctx, const M40llmK
         float score = 0.0f;
         if (fp16_old) {
             for (uint32_t pos = start; pos < end; ++pos)
-                for (uint32_t d = 0; d < hd; ++d) score += q[d] * host_h2f(kh[(size_t)pos * ept + d]);
+                for (uint32_t d = 0; d < hd; ++d) score += q[d] * host_h2f(kh[(size_t)pos * row + d]);
             score /= (float)(end - start);
         } else {
             std::vector<float> mean_k(hd, 0.0f);

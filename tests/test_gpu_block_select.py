@@ -65,7 +65,7 @@ def test_compressed_append_evict_bit_exact(dev, orc, hd):
             c2.append(0, p, k, v, 1e4, 1.0, layout)
         g, w = _read_state(kv2, 0), _oracle_state(c2, 0)
         assert np.array_equal(g["recent_v"], w["recent_v"]) and g["seq_map"] == w["seq_map"]
-        close(g["recent_k"].view(np.float16).astype(np.float32), w["recent_k"].view(np.float16).astype(np.float32), 2e-3, 2e-3)
+        close(g["recent_k"].view(np.float16).astype(np.float32), w["recent_k"].view(np.float16).astype(np.float32))
     dk, dv = dev.up(k), dev.up(v)
     dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv.h, 2, dk.ptr, dv.ptr, 0, 0, 1e4, 1.0, 0, expect=-3)
     dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv.h, 0, dk.ptr, dv.ptr, S, 0, 1e4, 1.0, 0, expect=-5)
@@ -115,7 +115,9 @@ def _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, S=None, seed=0, sca
     dev.call("m40llm_ext_block_select_read_selection", kv.h, 0, dq.ptr, qh, L, W, bs, top,
              sel.ctypes.data, cnt.ctypes.data, ssc.ctypes.data)
     orc.set_threads(8)
-    rc, want, wsel, wcnt = c.attention(0, q, qh, L, top, score_order=2)
+    # score order 0 = the reference kernel's own order (cuda/kernels.cu:2893-2912: per dimension over the block's
+    # tokens, then the 128-slot halving tree), which the HIP kernel reproduces bit for bit
+    rc, want, wsel, wcnt = c.attention(0, q, qh, L, top, score_order=0)
     assert rc == 0
     return dict(got=got, want=want, sel=sel, cnt=cnt, ssc=ssc, wsel=wsel, wcnt=wcnt, c=c, q=q, kv=kv, k16=k16, v16=v16)
 
@@ -133,21 +135,62 @@ def _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, S=None, seed=0, sca
 def test_block_select_indices_exact_and_output(dev, orc, qh, kvh, hd, L, W, bs, top):
     r = _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top)
     assert np.array_equal(r["cnt"], r["wcnt"])
-    assert np.array_equal(r["sel"], r["wsel"])            # block ids bit-exact, in rank order
-    close(r["got"], r["want"], 2e-3, 2e-4)                # q4-V path tolerance of the reference: 2e-3
-    # scores of the selected blocks are the oracle's bits (same summation order)
+    assert np.array_equal(r["sel"], r["wsel"])            # block ids bit-exact vs the reference order, in rank order
+    close(r["got"], r["want"])                            # 1e-3 relative / 1e-4 absolute
+    # scores of the selected blocks carry the reference order's bits, and the ids are its own top-k
     c, q = r["c"], r["q"]
-    for h in range(qh):
-        s2 = c.block_scores(0, q[h], h // (qh // kvh), L, 2, W, bs)
-        n = int(r["cnt"][h])
-        assert np.array_equal(r["ssc"][h, :n], s2[r["sel"][h, :n]])
-    # report how far the selection is from flipping under the other summation orders
-    flips = 0
+    tight = []
     for h in range(qh):
         s0 = c.block_scores(0, q[h], h // (qh // kvh), L, 0, W, bs)
+        n = int(r["cnt"][h])
+        assert np.array_equal(r["ssc"][h, :n], s0[r["sel"][h, :n]])
         b0, _ = orc.select_top_blocks(s0, top)
-        flips += int(not np.array_equal(b0, r["sel"][h, :len(b0)]))
-    print(f"[block-select] heads whose ranking differs under the device-kernel summation order: {flips}/{qh}")
+        assert np.array_equal(b0, r["sel"][h, :len(b0)])
+        # how close the cut is in exact arithmetic: gap between the last listed and the first unlisted block
+        s64 = np.sort(c.block_scores(0, q[h], h // (qh // kvh), L, 1, W, bs))[::-1]
+        if len(s64) > n > 0:
+            tight.append((float(s64[n - 1] - s64[n]) / max(abs(float(s64[0])), 1e-30), h))
+    if tight:
+        g, h = min(tight)
+        print(f"[block-select L={L}] smallest float64 cut gap (relative to the top score): {g:.3e} at head {h}; "
+              f"heads under 1e-6: {[hh for gg, hh in tight if gg < 1e-6]}")
+
+
+def test_block_select_multi_slot_batch4_32k_vs_oracle(dev, orc):
+    """BASELINE config 5 at batch 4: 32 q / 8 kv heads, hd 128, context 32768, 64-token blocks, top 64 + 512 recent,
+    four slots with different seeds through the multi-slot entry point; outputs vs the oracle per slot, block ids exact."""
+    qh, kvh, hd, L, W, bs, top, nseq = 32, 8, 128, 32768, 512, 64, 64, 4
+    kv = m40.KVCache(dev.ctx, L, nseq, kvh, hd, dict(recent_window=W, block_size=bs, top_blocks=top))
+    q = np.zeros((nseq, qh, hd), dtype=np.float32)
+    caches = []
+    for sq in range(nseq):
+        rng = np.random.default_rng(100 + sq)
+        k16 = f16bits(rng.standard_normal((L, kvh, hd), dtype=np.float32)); v16 = f16bits(rng.standard_normal((L, kvh, hd), dtype=np.float32))
+        q[sq] = rng.standard_normal((qh, hd)).astype(np.float32)
+        dk, dv = dev.up(k16), dev.up(v16)
+        dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, sq, dk.ptr, dv.ptr, L)
+        dk.free(); dv.free()
+        c = orc.CompressedKV(L, 1, kvh, hd, W, bs)
+        c.bulk_fill(0, k16, v16)
+        caches.append(c)
+    order = np.array([2, 0, 3, 1], dtype=np.uint32)
+    lens = np.full(nseq, L, dtype=np.uint32)
+    dq = dev.up(np.ascontiguousarray(q[order]))
+    out = dev.zeros(q.nbytes)
+    dev.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, nseq, order.ctypes.data_as(C.c_void_p),
+             lens.ctypes.data_as(C.c_void_p), dq.ptr, qh, W, bs, top, out.ptr)
+    dev.sync()
+    got = out.download(np.float32, (nseq, qh * hd))
+    orc.set_threads(16)
+    for i, sq in enumerate(order):
+        rc, want, wsel, wcnt = caches[sq].attention(0, q[sq], qh, L, top, score_order=0)
+        assert rc == 0
+        close(got[i], want)
+        sel = np.zeros((qh, 64), dtype=np.uint32); cnt = np.zeros(qh, dtype=np.uint32)
+        dev.call("m40llm_ext_block_select_read_selection", kv.h, int(sq), dq.ptr + i * qh * hd * 4, qh, L, W, bs, top,
+                 sel.ctypes.data, cnt.ctypes.data, None)
+        assert np.array_equal(cnt, wcnt) and np.array_equal(sel, wsel), int(sq)
+    kv.destroy()
 
 
 def test_block_select_all_blocks_equals_dense(dev, orc):
@@ -172,7 +215,7 @@ def test_block_select_all_blocks_equals_dense(dev, orc):
         kvhh = h // (qh // kvh)
         s = (k[:, kvhh] @ q[h]) * 0.125
         p = np.exp(s - s.max()); p /= p.sum()
-        close(r["got"][h * hd:(h + 1) * hd], p @ vq[:, kvhh], 2e-3, 2e-4)
+        close(r["got"][h * hd:(h + 1) * hd], p @ vq[:, kvhh])
 
 
 def test_block_select_ties_and_degenerate_scores(dev, orc):
@@ -190,7 +233,7 @@ def test_block_select_ties_and_degenerate_scores(dev, orc):
     dev.call("m40llm_ext_block_select_read_selection", kv.h, 0, dq.ptr, qh, L, W, bs, top, sel.ctypes.data, cnt.ctypes.data, None)
     assert list(cnt) == [3] * qh and all(list(sel[h, :3]) == [0, 1, 2] for h in range(qh))
     c = orc.CompressedKV(L, 1, kvh, hd, W, bs); c.bulk_fill(0, k16, v16)
-    _, _, wsel, _ = c.attention(0, q, qh, L, top, score_order=2)
+    _, _, wsel, _ = c.attention(0, q, qh, L, top, score_order=0)
     assert np.array_equal(sel, wsel)
 
 
@@ -227,7 +270,7 @@ def test_dense_backed_block_select(dev, orc, hd):
     dev.sync()
     Kc = np.zeros((1, S, kvh, hd), dtype=np.uint16); Vc = np.zeros_like(Kc)
     Kc[0, :L] = k16; Vc[0, :L] = v16
-    rc, want, wsel, wcnt = orc.dense_block_select(Kc, Vc, S, kvh, hd, 0, q, qh, L, W, bs, top, 2)
+    rc, want, wsel, wcnt = orc.dense_block_select(Kc, Vc, S, kvh, hd, 0, q, qh, L, W, bs, top, 0)
     assert rc == 0
     close(out.download(np.float32, (qh * hd,)), want)
     sel = np.zeros((qh, 64), dtype=np.uint32); cnt = np.zeros(qh, dtype=np.uint32)

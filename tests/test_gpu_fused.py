@@ -79,7 +79,7 @@ def test_norm_qkv_rope_append_equals_call_sequence(dev, orc, qh, kvh, hd, d_mode
         close(q_f, q_o[0])
         k_o = orc.gemm("f32xf16_gguf", xn, wk, 1, kvh * hd, K) + (bk if bias else 0)
         k_o = orc.rope(k_o.astype(np.float32), kvh, hd, position, base, 1.0, layout)
-        close(kf.view(np.float16).astype(np.float32), k_o[0], 2e-3, 1e-3)   # f16 storage rounding
+        close(kf.view(np.float16).astype(np.float32), k_o[0])   # f16 storage rounding: half a step, 2^-11 relative
         kv_f.destroy(); kv_u.destroy()
 
 
@@ -332,9 +332,9 @@ def test_batched_norm_qkv_rope_append_vs_oracle(dev, orc, qh, kvh, hd, layout, b
         close(got_q[r] / sq, want_q / sq)
         gk, gv = kv.read_token(seq, pos)
         sk = np.abs(want_k).max()
-        close(gk.view(np.float16).astype(np.float32) / sk, want_k / sk, 2e-3, 1e-3)       # f16 storage
+        close(gk.view(np.float16).astype(np.float32) / sk, want_k / sk)       # f16 storage: half a step
         sv = np.abs(v[r]).max()
-        close(gv.view(np.float16).astype(np.float32) / sv, v[r] / sv, 2e-3, 1e-3)
+        close(gv.view(np.float16).astype(np.float32) / sv, v[r] / sv)
         # nothing but the row's own position was written
         if pos + 1 < S:
             ok, _ = kv.read_token(seq, pos + 1)
