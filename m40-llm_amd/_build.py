@@ -20,8 +20,11 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 HIP_SOURCES = ["context.hip", "elementwise.hip", "gemm.hip", "kvcache.hip", "attention.hip", "block_select.hip",
-               "decode_fused.hip", "skinny_mfma.hip", "attention_mfma.hip", "rows_gemv.hip", "rows_mfma.hip", "prefill_attention.hip", "gemm_tiled.hip"]
+               "decode_fused.hip", "skinny_mfma.hip", "attention_mfma.hip", "rows_gemv.hip", "rows_mfma.hip", "prefill_attention.hip", "gemm_tiled.hip", "q80_i8.hip"]
 CPP_SOURCES = ["unavailable.cpp"]
+# per-file additions: matrix-instruction results straight into vector registers (the default form writes them to
+# accumulation registers and copies every element out again)
+HIP_FILE_FLAGS = {}
 
 
 def _run(cmd):
@@ -41,7 +44,7 @@ def build_native(verbose: bool = False) -> str:
         if not os.path.exists(path):
             continue
         obj = os.path.join(OBJDIR, src + ".o")
-        jobs.append(([HIPCC, *HIP_FLAGS, "-c", path, "-o", obj], obj))
+        jobs.append(([HIPCC, *HIP_FLAGS, *HIP_FILE_FLAGS.get(src, []), "-c", path, "-o", obj], obj))
     for src in CPP_SOURCES:
         obj = os.path.join(OBJDIR, src + ".o")
         jobs.append((["g++", "-O2", "-std=c++17", "-fPIC", "-c", os.path.join(CSRC, src), "-o", obj], obj))

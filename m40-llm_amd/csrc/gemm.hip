@@ -582,6 +582,8 @@ static int launch_q80(M40llmCudaContext* ctx, hipStream_t stream, uint32_t strea
                       float* C, int M, int N, int K) {
     if (m40_aligned16(B) && m40_aligned16(A) && q80_gemv_supported(M, N, K))
         return launch_q80_gemv(stream, A, nullptr, B, C, nullptr, nullptr, M, N, K);
+    if (m40_aligned16(B) && m40_aligned16(A) && m40_q80_i8_supported(ctx, stream_kind, M, N, K))
+        return m40_launch_q80_i8(ctx, stream, stream_kind, A, B, C, M, N, K);
     if (m40_aligned16(B) && m40_aligned16(A) && m40_skinny_supported(ctx, stream_kind, M, N, K, 1))
         return m40_launch_skinny(ctx, stream, stream_kind, 1, A, nullptr, B, C, nullptr, nullptr, M, N, K);
     (void)hipGetLastError();
@@ -748,6 +750,11 @@ int m40llm_ext_ffn_swiglu_q80_f32_async(M40llmCudaContext* ctx, const void* d_x_
         int rc = launch_q80_gemv(ctx->decode_stream, x, nullptr, wg, gate, wu, up, M, ffn, d_model);
         if (rc != 0) return rc;
         return launch_q80_gemv(ctx->decode_stream, gate, up, wd, out, nullptr, nullptr, M, d_model, ffn);
+    }
+    if (aligned && m40_q80_i8_supported(ctx, 1, M, ffn, d_model) && m40_q80_i8_supported(ctx, 1, M, d_model, ffn)) {
+        // digit planes of x, gate / up / SwiGLU / digit planes of the hidden row, down projection: three launches
+        const int rc = m40_launch_q80_i8_ffn(ctx, ctx->decode_stream, 1, x, wg, wu, wd, out, M, d_model, ffn);
+        if (rc == 0) return 0;
     }
     if (aligned &&
         m40_skinny_supported(ctx, 1, M, ffn, d_model, 1) &&
