@@ -78,7 +78,27 @@ def measure_dominant_kernel(pkg, ctx, dm, cfg, reps, mode):
     ctx.record(e1, 1)
     ms = ctx.elapsed_ms(e0, e1)
     ctx.event_destroy(e0); ctx.event_destroy(e1)
-    return dict(kernel=name, shape=shape, launches=n, avg_us=ms * 1e3 / n, bytes=bytes_per_launch)
+    out = dict(kernel=name, shape=shape, launches=n, avg_us=ms * 1e3 / n, bytes=bytes_per_launch, in_token_us=None)
+    if mode >= 1:
+        # The same kernel as it runs inside a token: behind the O-projection launch it depends on and before the down
+        # projection, one event pair per launch (back-to-back launches of one kernel overlap their ramps; these do not).
+        h = ctx.alloc(D * 4); x1 = ctx.alloc(D * 4)
+        pairs = [(ctx.event(), ctx.event()) for _ in range(L)]
+        for rep in range(2):                      # the first pass warms up
+            for l in range(L):
+                ly = dm.layers[l]
+                lib.m40llm_ext_gemv_residual_f32xf16_async(ctx.h, x.ptr, ly.wo, x.ptr, x1.ptr, D, D)
+                ctx.record(pairs[l][0], 1)
+                lib.m40llm_ext_fused_norm_gate_up_swiglu_async(ctx.h, x1.ptr, ly.ffn_norm, 1, cfg["rms_eps"], ly.wgate, ly.wup,
+                                                               y.ptr, F, D)
+                ctx.record(pairs[l][1], 1)
+                lib.m40llm_ext_gemv_residual_f32xf16_async(ctx.h, y.ptr, ly.wdown, x1.ptr, h.ptr, D, F)
+            ctx.sync(1)
+        out["in_token_us"] = sum(ctx.elapsed_ms(a, b) for a, b in pairs) * 1e3 / L
+        for a, b in pairs:
+            ctx.event_destroy(a); ctx.event_destroy(b)
+        h.free(); x1.free()
+    return out
 
 
 def measured_traffic(kernel):
@@ -93,6 +113,24 @@ def measured_traffic(kernel):
         return None
 
 
+def host_cpu():
+    """CPU model string and the cores this process may run on."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return model, usable
+
+
 def cpu_baseline(cfg, W, steps, threads):
     """The CPU oracle (a scalar port of the reference's semantics) timed on this host: `steps` greedy decode
     tokens from an empty KV cache.  At this size a token is bound by the 2.07 GB of weights, not by context."""
@@ -105,7 +143,29 @@ def cpu_baseline(cfg, W, steps, threads):
     dt = time.perf_counter() - t0
     return dict(value=steps / dt, unit="tok/s", cores=threads, kind="port",
                 sample=f"{steps} greedy decode tokens of the same model from an empty KV cache, oracle/oracle.c "
-                       f"(gcc -O2, {threads} thread{'s' if threads > 1 else ''})")
+                       f"(gcc -O2{' -fopenmp' if threads > 1 else ''}, {threads} thread{'s' if threads > 1 else ''})")
+
+
+def cpu_baseline_b8(b8_state, threads, steps=1):
+    """The batch-8 half on the CPU: the same Qwen2.5-3B-shaped model, the same eight pre-filled contexts, `steps` greedy
+    steps of every sequence with the oracle (sequences one after the other, OpenMP inside each product)."""
+    from oracle import pyoracle as orc
+    cfg, W, lens, k16, v16, first = b8_state
+    orc.set_threads(threads)
+    B, L = len(lens), cfg["n_layers"]
+    om = orc.Model(dict(cfg, qkv_bias=True), W)
+    om.alloc_kv(int(lens.max()) + steps + 2, B)
+    Ko, Vo = om.kv_views()
+    for s in range(B):
+        for l in range(L):
+            Ko[s * L + l, :lens[s]] = k16[:lens[s]]; Vo[s * L + l, :lens[s]] = v16[:lens[s]]
+    t0 = time.perf_counter()
+    for s in range(B):
+        om.decode_greedy(s, [int(first[s])], steps, start_pos=int(lens[s]))
+    dt = time.perf_counter() - t0
+    return dict(value=B * steps / dt, unit="tok/s", cores=threads, kind="port",
+                sample=f"{steps} greedy step(s) of the 8 sequences of config.b8 (contexts U[256,4096]), oracle/oracle.c "
+                       f"(gcc -O2 -fopenmp, {threads} threads)")
 
 
 def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
@@ -122,8 +182,9 @@ def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
     dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=4096 + warmup + steps + 8, max_sequences=B)
     dm.set_mode(2)
     f16 = lambda a: np.ascontiguousarray(a.astype(np.float16).view(np.uint16))
-    dk = ctx.to_device(f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)))
-    dv = ctx.to_device(f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)))
+    k16h = f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32))
+    v16h = f16(rng.standard_normal((4096, cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32))
+    dk, dv = ctx.to_device(k16h), ctx.to_device(v16h)
     for s in range(B):
         for l in range(cfg["n_layers"]):
             slot = dm.H.m40host_model_kv_slot(dm.h, s, l)
@@ -135,13 +196,16 @@ def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
     KV = cfg["kv_heads"] * cfg["head_dim"]
     wbytes = L * 2 * (D * (D + 2 * KV) + D * D + 3 * D * F) + 2 * V * D
     kvbytes = int(lens.sum() + B * (warmup + steps / 2)) * L * KV * 2 * 2
+    fallback = dm.last_timed_host_fallback()
     dm.close()
     dk.free(); dv.free()
     ms_step = ms / steps
-    return {"workload": "Qwen2.5-3B-shaped random-init decode (BASELINE configs[2]), batch 8, contexts U[256,4096], "
-                        "row-batched greedy, fused + graph", "tok_s": B * steps / (ms / 1e3), "ms_per_step": ms_step,
-            "steps": steps, "warmup": warmup, "algorithmic_bytes_per_step": int(wbytes + kvbytes),
-            "whole_step_hbm_frac": (wbytes + kvbytes) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    rec = {"workload": "Qwen2.5-3B-shaped random-init decode (BASELINE configs[2]), batch 8, contexts U[256,4096], "
+                       "row-batched greedy, fused + graph", "tok_s": B * steps / (ms / 1e3), "ms_per_step": ms_step,
+           "steps": steps, "warmup": warmup, "algorithmic_bytes_per_step": int(wbytes + kvbytes),
+           "whole_step_hbm_frac": (wbytes + kvbytes) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "host_sampler_fallback": fallback}
+    return rec, (cfg, W, lens, k16h, v16h, first)
 
 
 def plain_read_yardstick(pkg, ctx, nbytes):
@@ -244,22 +308,44 @@ def main():
                    "algorithmic_bytes_per_token": token_bytes, "setup_s": round(setup_s, 1),
                    "first_generated_ids": [int(i) for i in ids[n_prompt:n_prompt + 8]]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(dom["kernel"]), "kernel": dom["kernel"],
-                     "shape": dom["shape"],
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic(dom["kernel"]),
+                     # not a quantity of this run: read from the committed counter summary of an earlier profiled run
+                     "traffic_source": "profiles/decode_b1_tinyllama_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                                       "collected beforehand with the same command under the profiler)",
+                     "kernel": dom["kernel"], "shape": dom["shape"],
+                     # avg_launch_us: launches of this kernel back to back (their ramps overlap); in_token_avg_us: the same
+                     # kernel between the launches that surround it in a token, one event pair per launch
                      "avg_launch_us": dom["avg_us"], "launches_timed": dom["launches"],
+                     "in_token_avg_us": dom["in_token_us"],
+                     "in_token_frac": (dom["bytes"] / (dom["in_token_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS) if dom["in_token_us"] else None,
                      "algorithmic_bytes_per_launch": dom["bytes"],
                      # a kernel that only reads the same number of bytes, one launch, fastest of five grid sizes
                      "plain_read_us": yard["us"], "plain_read_workgroups": yard["workgroups"],
                      "frac_of_plain_read": yard["us"] / dom["avg_us"]},
     }
+    out["config"]["host_sampler_fallback"] = dm.last_timed_host_fallback()
     dm.close()
+    b8_state = None
     if not args.no_b8 and not args.layers:
         try:
-            out["config"]["b8"] = measure_b8(pkg, syn, ctx)
+            out["config"]["b8"], b8_state = measure_b8(pkg, syn, ctx)
         except Exception as e:     # the batch-1 line must still be printed
             out["config"]["b8"] = {"error": repr(e)}
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, W, args.cpu_steps, 1)
+        model, usable = host_cpu()
+        threads = max(1, min(usable, 16))       # the GPU box gives one GPU's share of its cores: 16
+        base = cpu_baseline(cfg, W, args.cpu_steps, 1)
+        base["cpu_model"] = model
+        base["usable_cores"] = usable
+        variants = []
+        try:
+            variants.append(dict(cpu_baseline(cfg, W, 2 * args.cpu_steps, threads), workload="batch 1 (the headline workload), OpenMP"))
+            if b8_state is not None:
+                variants.append(dict(cpu_baseline_b8(b8_state, threads), workload="batch 8 (config.b8), OpenMP"))
+        except Exception as e:
+            variants.append({"error": repr(e)})
+        base["variants"] = variants
+        out["cpu_baseline"] = base
     print(json.dumps(out))
 
 

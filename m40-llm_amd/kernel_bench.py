@@ -438,10 +438,21 @@ def main():
     ap.add_argument("--only", default="read,attn,gemv,gemm8,q80,bsel,decode8,prefill,gguf,pfwd,gemmN,sched")
     ap.add_argument("--json", default=None)
     ap.add_argument("--decode-mode", type=int, default=2, help="host path of the decode8 case: 0 reference sequence, 1 fused, 2 fused + graph")
+    ap.add_argument("--decode-steps", type=int, default=32, help="timed steps of the decode8 case")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="first copy 256 MiB device-to-device three times through the library: a transfer of known size "
+                         "against which rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings of the other kernels are scaled")
     args = ap.parse_args()
     which = set(args.only.split(","))
     b = Bench()
     print(b.lib.m40llm_ext_build_info().decode() if hasattr(b.lib, "m40llm_ext_build_info") else "")
+    if args.traffic_probe:
+        n = 256 << 20
+        src, dst = b.ctx.alloc(n), b.ctx.alloc(n)
+        for _ in range(3):
+            b.call("m40llm_memcpy_d2d_async", dst.ptr, src.ptr, n, 1)
+        b.ctx.sync(1)
+        src.free(); dst.free()
     if "read" in which:
         bench_read_probe(b)
     if "attn" in which:
@@ -455,7 +466,7 @@ def main():
     if "bsel" in which:
         bench_block_select(b)
     if "decode8" in which:
-        bench_decode_batch(b, mode=args.decode_mode)
+        bench_decode_batch(b, steps=args.decode_steps, mode=args.decode_mode)
     if "prefill" in which:
         bench_prefill(b)
     if "gguf" in which:
