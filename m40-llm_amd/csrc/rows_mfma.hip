@@ -4,10 +4,18 @@
 // The split-K kernel of skinny_mfma.hip converts a step of activations per barrier and needs a second launch to add
 // its slices.  Here the workgroups are persistent: each converts the eight rows once into f16 hi + lo MFMA fragments
 // for the whole of K (64 KB of LDS, per-row power-of-two scale, RMSNorm weights folded in), then walks its share of
-// the column tiles.  A tile's K range is split over the four waves (16 MFMA steps each), so a wave requests a whole
-// tile quarter -- sixteen 16-byte loads per lane -- at once and keeps two tiles in flight; the waves' partial sums
-// meet in LDS in wave order and the first wave writes the result (residual, bias or SwiGLU applied), so nothing is
-// left for a second launch and no result depends on timing.
+// the column tiles.  A tile's K range is split over the eight waves (8 MFMA steps each), so a wave requests its whole
+// share of a tile -- eight 16-byte loads per lane -- at once and keeps two tiles in flight; the waves' partial sums
+// meet in LDS in wave order and every result element is written once (residual, bias or SwiGLU applied), so nothing
+// is left for a second launch and no result depends on timing.
+//
+// Start-up, measured with timestamps inside the kernel on the batch-8 step: the activation rows and norm weights are
+// requested before any index arithmetic and ahead of the weight tiles (loads return in issue order; behind 64 KB of
+// weights per CU the rows arrived 3 us later), one batch of loads whatever the norm weights' type (a branch around
+// loads costs a full wait at its join), and the fragment layout in LDS is swizzled so that the conversion pass, whose
+// lanes hold one row at consecutive chunks, does not pile onto four banks.  What remains is the memory system: a CU
+// holds about one tile of outstanding requests, the first tile arrives about 4 us after it is requested with all 256
+// CUs asking at once, and from there tiles arrive at the HBM rate (2.3-2.7 us per 64 KB and CU = 6.2-7.3 TB/s).
 //
 // SwiGLU form: a tile is eight gate columns and the eight up columns of the same index, so that gate and up of an
 // output element come out of one MFMA accumulator tile, eight lanes apart.
@@ -20,15 +28,25 @@
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
 constexpr int kRows = 8;
 constexpr int kK = 2048;                      // the one K this kernel is built for
-constexpr int kSteps = kK / 32 / kWaves;      // MFMA k-steps per wave and tile: 16
 constexpr int kFragBytes = (kK / 32) * 64 * 16;   // 64 KB: [k-step][lane] 16-byte A-operand entries
-constexpr int kStageRow = kK / kWaves * 2 + 16;   // LDS bytes per column of a wave's weight tile quarter: 1 KB + 16 (spreads the columns over the banks)
-constexpr int kStageBytes = 16 * kStageRow;       // per wave
-constexpr int kDynamicLds = kFragBytes + kWaves * kStageBytes;
+
+// Per wave count (4 or 8 waves share a tile's K range):
+template <int WAVES>
+struct Shape {
+    static constexpr int kThreads = 64 * WAVES;
+    static constexpr int kSteps = kK / 32 / WAVES;          // MFMA k-steps per wave and tile
+    static constexpr int kRunLanes = kK / WAVES * 2 / 16;   // lanes that cover a column's share of K with 16 bytes each
+    static constexpr int kColsPerLoad = 64 / kRunLanes;     // columns one load instruction of a wave covers
+    static constexpr int kLoads = 16 / kColsPerLoad;        // load instructions per wave and tile
+    static constexpr int kStageRow = kK / WAVES * 2 + 16;   // LDS bytes per column of a wave's share: +16 spreads the columns over the banks
+    static constexpr int kStageBytes = 16 * kStageRow;      // per wave
+    static constexpr int kDynamicLds = kFragBytes + WAVES * kStageBytes;
+    static constexpr int kRowThreads = kThreads / kRows;    // threads that convert one activation row
+    static constexpr int kChunks = kK / 8 / kRowThreads;    // 8-element chunks per thread
+    static_assert(kRunLanes <= 64 && kRowThreads <= 64, "a column run and an activation row stay inside a wave");
+};
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -38,6 +56,12 @@ __device__ __forceinline__ m40_float4 mfma16x16x32(const uint4& a, const uint4& 
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(m40_half8, a),
                                                   __builtin_bit_cast(m40_half8, b), c, 0, 0, 0);
 }
+
+// Where entry e of the A-operand fragments ([k-step][lane], 16 bytes each) lives in LDS.  The row index (low four bits)
+// is xor-ed with the four bits above it: a k-step's 64 entries stay one contiguous, merely permuted kilobyte for the
+// operand reads, while the conversion pass -- whose lanes hold the same row at consecutive chunks, entries 16 and 64
+// apart -- spreads over all banks instead of hitting four of them.
+__device__ __forceinline__ int frag_slot(int e) { return e ^ ((e >> 4) & 15); }
 
 struct RowsMfmaArgs {
     const float* x;            // [rows][K]
@@ -82,39 +106,78 @@ __device__ __forceinline__ int qkv_col(const RowsMfmaArgs& p, const QkvTile& t, 
 }
 
 // MODE 0: out = x W^T; 1: SwiGLU of gate and up; 2: Q/K/V with bias, RoPE and cache append
-template <int MODE>
-__global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) {
+template <int MODE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p) {
+    using S = Shape<WAVES>;
+    constexpr int kWaves = WAVES, kSteps = S::kSteps, kLoads = S::kLoads, kStageRow = S::kStageRow,
+                  kStageBytes = S::kStageBytes, kRunLanes = S::kRunLanes, kColsPerLoad = S::kColsPerLoad,
+                  kRowThreads = S::kRowThreads, kChunks = S::kChunks;
     constexpr bool SWIGLU = MODE == 1;
     constexpr bool QKV = MODE == 2;
     extern __shared__ __attribute__((aligned(16))) uint8_t frag_bytes[];
     uint4* a_frag = reinterpret_cast<uint4*>(frag_bytes);
-    uint8_t* stage = frag_bytes + kFragBytes + (threadIdx.x >> 6) * kStageBytes;     // this wave's weight tile quarter
+    uint8_t* stage = frag_bytes + kFragBytes + (threadIdx.x >> 6) * kStageBytes;     // this wave's share of the weight tile
     __shared__ float red_s[2][kWaves][4][64];      // the waves' tile sums, two tiles deep
     __shared__ float row_scale_s[kRows];           // undoes the row's power-of-two scale, times the RMSNorm factor
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int j = lane & 15, g = lane >> 4;
-    const int u_begin = (int)((long long)blockIdx.x * p.units / gridDim.x);
-    const int u_end = (int)((long long)(blockIdx.x + 1) * p.units / gridDim.x);
-    const int n_units = u_end - u_begin;
+    // The activation rows and the norm weights are requested before anything else is computed: they head the longest
+    // dependent chain of the kernel (rows -> scale -> fragments -> first matrix instruction).
+    const int row = tid / kRowThreads, l = tid % kRowThreads;
+    const bool live = row < p.rows;
+    const float* xr = p.x + (size_t)(live ? row : 0) * kK;
+    float v[kChunks][8];
+    float sq = 0.0f;            // sum of squares of the raw row (RMSNorm only)
+#pragma unroll
+    for (int c = 0; c < kChunks; ++c) {
+        const float4 a = reinterpret_cast<const float4*>(xr)[2 * (l + kRowThreads * c)];
+        const float4 b = reinterpret_cast<const float4*>(xr)[2 * (l + kRowThreads * c) + 1];
+        v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
+        v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
+    }
+    // Everything the prologue needs goes out first, the weight tiles behind it: loads return in issue order, so the
+    // rows and the norm weights (cache hits or a short fetch) are not kept waiting behind 64 KB of weights per
+    // workgroup, and both tiles are on their way while the rows are converted.
+    const bool norm16 = p.norm_w && p.norm_dtype == 0u;
+    uint4 wraw[2 * kChunks];
+    {
+        // one unconditional batch of loads whatever the weights are (a branch around loads costs a full wait at
+        // its join): f32 weights are 32 bytes per chunk; f16 weights 16 bytes, requested twice; without a norm the
+        // row itself is read again and ignored
+        const uint4* wp = p.norm_w ? static_cast<const uint4*>(p.norm_w) : reinterpret_cast<const uint4*>(xr);
+        const int mul = norm16 ? 1 : 2, second = norm16 ? 0 : 1;
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c) {
+            wraw[2 * c] = wp[mul * (l + kRowThreads * c)];
+            wraw[2 * c + 1] = wp[mul * (l + kRowThreads * c) + second];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // consecutive, nearly equal runs of tiles (a finer split of the last tile was measured and gains nothing: the
+    // launch is bound by the memory system, and the workgroups still running share what the finished ones leave)
+    const int u_begin = (int)((uint32_t)blockIdx.x * (uint32_t)p.units / gridDim.x);          // units < 2^20, workgroups <= 2^10
+    const int n_units = (int)(((uint32_t)blockIdx.x + 1u) * (uint32_t)p.units / gridDim.x) - u_begin;
 
-    // Weight loads are whole 1 KB runs: instruction i of a wave reads the wave's K quarter of column i of the tile,
-    // 16 bytes per lane.  (Reading the MFMA operand layout straight from memory -- 16 columns x 64 bytes per
+    // Weight loads are whole runs: an instruction of a wave reads the wave's share of K of one column (four waves) or
+    // two columns (eight) of the tile, 16 bytes per lane.  (Reading the MFMA operand layout straight from memory -- 16 columns x 64 bytes per
     // instruction, 4 KB apart -- streams a third slower: measured 26.5 us against 18.2 us for these 90 MB.)  The
     // operand layout is produced by a pass through the wave's own LDS tile.
     // No load under a branch: a tile past the workgroup's range re-reads the first 16 bytes of its first tile.
-    uint4 b0[kSteps], b1[kSteps];
-    auto issue = [&](uint4 (&b)[kSteps], int local) {
+    uint4 b0[kLoads], b1[kLoads];
+    const int run_lane = lane % kRunLanes, run_col = lane / kRunLanes;
+    auto issue = [&](uint4 (&b)[kLoads], int local) {
         const bool live = local < n_units;
         const int unit = u_begin + (live ? local : 0);
-        const int lane_off = live ? 8 * lane : 0;
+        const int lane_off = live ? 8 * run_lane : 0;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int li = 0; li < kLoads; ++li) {
+            const int i = li * kColsPerLoad + run_col;      // column of the tile (i & 8 is the same for the whole instruction)
             int col;
             const uint16_t* W = p.W0;
             if (SWIGLU) {
                 col = 8 * unit + (i & 7);
-                if (i & 8) W = p.W1;
+                if (li * kColsPerLoad & 8) W = p.W1;
                 col = col < p.N ? col : p.N - 1;
             } else if (QKV) {
                 const QkvTile t = qkv_tile(p, unit);
@@ -124,9 +187,12 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
                 col = 16 * unit + i;
                 col = col < p.N ? col : p.N - 1;
             }
-            b[i] = *reinterpret_cast<const uint4*>(W + (size_t)col * kK + wave * (kK / kWaves) + lane_off);
+            b[li] = *reinterpret_cast<const uint4*>(W + (size_t)col * kK + wave * (kK / kWaves) + lane_off);
         }
     };
+    issue(b0, 0);
+    if (!QKV) issue(b1, 1);            // the Q/K/V form has one tile per workgroup
+    __builtin_amdgcn_sched_barrier(0);
     // the tile element this thread writes (see `finish`)
     constexpr int kTileCols = SWIGLU ? 8 : 16;      // output columns of a tile
     const int n_out = kTileCols * p.rows;
@@ -163,47 +229,26 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
     if (QKV) first_ops = qkv_operands(u_begin);
 
     // ---- the eight rows -> f16 hi + lo fragments, once -------------------------------------------------------
-    // Thread (row = tid / 32, l = tid % 32) owns the 8-element chunks l, l + 32, ... of its row, so a row lives in
-    // one half-wave and its maximum and sum of squares need no LDS.
+    // Thread (row = tid / kRowThreads, l = tid % kRowThreads) owns the 8-element chunks l, l + kRowThreads, ... of its
+    // row, so a row lives in one wave (or half-wave) and its maximum and sum of squares need no LDS.
     {
-        const int row = tid >> 5, l = tid & 31;
-        const bool live = row < p.rows;
-        const float* xr = p.x + (size_t)(live ? row : 0) * kK;
-        float v[8][8];
-        float sq = 0.0f;            // sum of squares of the raw row (RMSNorm only)
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const float4 a = reinterpret_cast<const float4*>(xr)[2 * (l + 32 * c)];
-            const float4 b = reinterpret_cast<const float4*>(xr)[2 * (l + 32 * c) + 1];
-            v[c][0] = a.x; v[c][1] = a.y; v[c][2] = a.z; v[c][3] = a.w;
-            v[c][4] = b.x; v[c][5] = b.y; v[c][6] = b.z; v[c][7] = b.w;
-        }
-        issue(b0, 0);       // behind the rows (returns are in order: the rows, cache-resident, are not kept waiting)
-        // norm weights: every load of a branch goes out before its first use (one round trip, not one per chunk)
-        if (p.norm_w && p.norm_dtype == 0u) {
-            uint4 wq[8];
-#pragma unroll
-            for (int c = 0; c < 8; ++c) wq[c] = reinterpret_cast<const uint4*>(p.norm_w)[l + 32 * c];
+        if (norm16) {
             float sq0 = 0.0f;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
+            for (int c = 0; c < kChunks; ++c) {
                 float w[8];
-                m40_unpack8(wq[c], w);
+                m40_unpack8(wraw[2 * c], w);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) { sq0 = fmaf(v[c][e], v[c][e], sq0); v[c][e] *= w[e]; }
             }
             sq = sq0;
         } else if (p.norm_w) {
-            float4 wa[8], wb[8];
-#pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                wa[c] = reinterpret_cast<const float4*>(p.norm_w)[2 * (l + 32 * c)];
-                wb[c] = reinterpret_cast<const float4*>(p.norm_w)[2 * (l + 32 * c) + 1];
-            }
             float sq0 = 0.0f;
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
-                const float w[8] = {wa[c].x, wa[c].y, wa[c].z, wa[c].w, wb[c].x, wb[c].y, wb[c].z, wb[c].w};
+            for (int c = 0; c < kChunks; ++c) {
+                const uint4 a = wraw[2 * c], b = wraw[2 * c + 1];
+                const float w[8] = {__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z), __uint_as_float(a.w),
+                                    __uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w)};
 #pragma unroll
                 for (int e = 0; e < 8; ++e) { sq0 = fmaf(v[c][e], v[c][e], sq0); v[c][e] *= w[e]; }
             }
@@ -211,14 +256,14 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
         }
         float mx = 0.0f;
 #pragma unroll
-        for (int c = 0; c < 8; ++c)
+        for (int c = 0; c < kChunks; ++c)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 if (!live) v[c][e] = 0.0f;
                 mx = fmaxf(mx, fabsf(v[c][e]));
             }
 #pragma unroll
-        for (int o = 1; o < 32; o <<= 1) {
+        for (int o = 1; o < kRowThreads; o <<= 1) {
             sq += __shfl_xor(sq, o, 64);
             mx = fmaxf(mx, __shfl_xor(mx, o, 64));
         }
@@ -232,7 +277,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
             inv_scale = ldexpf(1.0f, -ex);
         }
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
+        for (int c = 0; c < kChunks; ++c) {
             uint32_t hi[4], lo[4];
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
@@ -242,23 +287,23 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
                 hi[e / 2] = __builtin_bit_cast(uint32_t, h2);
                 lo[e / 2] = __builtin_bit_cast(uint32_t, l2);
             }
-            const int chunk = l + 32 * c;                              // k = 8 chunk .. +7
+            const int chunk = l + kRowThreads * c;                              // k = 8 chunk .. +7
             const int entry = (chunk >> 2) * 64 + (chunk & 3) * 16 + row;   // A operand: lane = 16 (k / 8 % 4) + row
-            a_frag[entry] = make_uint4(hi[0], hi[1], hi[2], hi[3]);          // rows 0..7: hi parts
-            a_frag[entry + 8] = make_uint4(lo[0], lo[1], lo[2], lo[3]);      // rows 8..15: lo parts
+            a_frag[frag_slot(entry)] = make_uint4(hi[0], hi[1], hi[2], hi[3]);          // rows 0..7: hi parts
+            a_frag[frag_slot(entry + 8)] = make_uint4(lo[0], lo[1], lo[2], lo[3]);      // rows 8..15: lo parts
         }
         if (l == 0) row_scale_s[row] = scale * (p.norm_w ? rsqrtf(sq / (float)kK + p.eps) : 1.0f);
     }
     if (QKV && first_ops.which != 2) first_cs = m40_rope_cos_sin_freq(first_ops.position, first_ops.inv_freq, p.rope_scale);
-    if (!QKV) issue(b1, 1);            // the Q/K/V form has one tile per workgroup
     __syncthreads();
 
     // ---- tiles -------------------------------------------------------------------------------------------------
     // tile quarter: registers -> LDS (column-major as loaded) -> MFMA B operand (lane (j, g): 16 bytes of column j)
-    auto to_lds = [&](const uint4 (&b)[kSteps]) {
+    auto to_lds = [&](const uint4 (&b)[kLoads]) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i)      // built from the elements: a whole-struct copy would keep the array in scratch memory
-            *reinterpret_cast<u32x4*>(stage + i * kStageRow + 16 * lane) = u32x4{b[i].x, b[i].y, b[i].z, b[i].w};
+        for (int li = 0; li < kLoads; ++li)      // built from the elements: a whole-struct copy would keep the array in scratch memory
+            *reinterpret_cast<u32x4*>(stage + (li * kColsPerLoad + run_col) * kStageRow + 16 * run_lane) =
+                u32x4{b[li].x, b[li].y, b[li].z, b[li].w};
         __builtin_amdgcn_wave_barrier();
     };
     auto compute = [&](int parity) {
@@ -266,7 +311,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
 #pragma unroll
         for (int i = 0; i < kSteps; ++i) {
             const uint4 bw = *reinterpret_cast<const uint4*>(stage + j * kStageRow + 64 * i + 16 * g);
-            acc = mfma16x16x32(a_frag[(kSteps * wave + i) * 64 + lane], bw, acc);
+            acc = mfma16x16x32(a_frag[frag_slot((kSteps * wave + i) * 64 + lane)], bw, acc);
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -279,7 +324,10 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
     // the tile's live elements, so every thread stores exactly once (some twice the same value to the same address):
     // no store sits under a branch, and the waits of the loop stay exact.
     auto tile_sum = [&](int parity, int ln) {
-        return ((red_s[parity][0][e_r][ln] + red_s[parity][1][e_r][ln]) + red_s[parity][2][e_r][ln]) + red_s[parity][3][e_r][ln];
+        float t = red_s[parity][0][e_r][ln];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) t += red_s[parity][w][e_r][ln];
+        return t;
     };
     auto finish = [&](int local, int parity) {
         const int unit = u_begin + local;
@@ -315,7 +363,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
         p.out[(size_t)e_row * p.N + col] = v;
     };
     // One tile from register set b; PREFETCH: tile local + 2 exists and is requested into the same set.
-    auto tile = [&](uint4 (&b)[kSteps], auto prefetch_c, int local, int parity) {
+    auto tile = [&](uint4 (&b)[kLoads], auto prefetch_c, int local, int parity) {
         to_lds(b);
         if (decltype(prefetch_c)::value) issue(b, local + 2);
         compute(parity);
@@ -346,15 +394,22 @@ __global__ __launch_bounds__(kThreads, 1) void rows_mfma_kernel(RowsMfmaArgs p) 
     }
 }
 
+template <int MODE, int WAVES>
+int launch_w(M40llmCudaContext* ctx, hipStream_t stream, const RowsMfmaArgs& a) {
+    using S = Shape<WAVES>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rows_mfma_kernel<MODE, WAVES>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, S::kDynamicLds);
+    if (attr != hipSuccess) return -7;
+    int grid = ctx->num_cus;           // one workgroup per CU: most of its LDS
+    if (grid > a.units) grid = a.units;
+    rows_mfma_kernel<MODE, WAVES><<<grid, S::kThreads, S::kDynamicLds, stream>>>(a);
+    return hipGetLastError() == hipSuccess ? 0 : -7;
+}
 template <int MODE>
 int launch(M40llmCudaContext* ctx, hipStream_t stream, const RowsMfmaArgs& a) {
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rows_mfma_kernel<MODE>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDynamicLds);
-    if (attr != hipSuccess) return -7;
-    int grid = ctx->num_cus;           // one workgroup per CU: 138 KB of LDS each
-    if (grid > a.units) grid = a.units;
-    rows_mfma_kernel<MODE><<<grid, kThreads, kDynamicLds, stream>>>(a);
-    return hipGetLastError() == hipSuccess ? 0 : -7;
+    // eight waves: the conversion pass is spread over twice the lanes and twice as many requests are in flight per CU
+    // as with four (batch-8 step at the Qwen2.5-3B shape: 2.58 -> 2.55 ms)
+    return launch_w<MODE, 8>(ctx, stream, a);
 }
 
 }  // namespace
