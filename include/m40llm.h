@@ -14,7 +14,8 @@
  *   - stream_kind: 0 = prefill stream, 1 = decode stream, anything else is an error
  *     (cuda/kernels.cu:287-292);
  *   - rope_layout: 0 = adjacent pairs (2i,2i+1), 1 = NeoX split half (i,i+hd/2);
- *   - weight_dtype: 0 = f16, 1 = f32;  exact_old_backing: 0 dense, 1 q8, 2 fp16-K/q4-V;
+ *   - weight_dtype: 0 = f16, 1 = f32;  exact_old_backing: 0 dense, 1 q8, 2 fp16-K/q4-V,
+ *     3 (extension, M40LLM_EXT_OLD_BACKING_FP16_K_Q4G32_V) fp16-K with V 4-bit in groups of 32;
  *   - `_async` = enqueue on the decode stream and return; the GEMMs and
  *     f16_to_f32 / q80_to_f32 run on the prefill stream and block until done.
  *   - calls on one context are serialised by the caller (the reference holds a
@@ -150,8 +151,16 @@ int m40llm_swiglu_f32_async(M40llmCudaContext* ctx, const void* d_gate, const vo
 /* ---- KV cache (cuda/kernels.cu:5304-5543, 5793-6379) ---------------------------- */
 M40llmKVCache* m40llm_kvcache_create(M40llmCudaContext* ctx, uint32_t max_seq_len,
                                      uint32_t max_batch_size, uint32_t num_heads, uint32_t head_dim);
-/* Only exact_old_backing 0 (ring only) and 2 (fp16-K/q4-V) allocate usable
- * storage here; backing 1 (q8) returns NULL. */
+/* Only exact_old_backing 0 (ring only), 2 (fp16-K/q4-V) and 3 allocate usable
+ * storage here; backing 1 (q8) returns NULL.
+ * Backing 3 has no counterpart in the reference: it is backing 2 with the old V rows held 4-bit in groups of 32
+ * dimensions under an f16 scale and an f16 minimum (the V format the compressed-attention benchmark configuration
+ * names; 80 bytes per token and head at head_dim 128 against 68).  Per group: d = f16((max - min) / 15),
+ * m = f16(min), q = d > 0 ? clamp(lrintf((v - m) / d), 0, 15) : 0, value = fmaf(q, d, m).  Appends, evictions, the
+ * block-select attention entry points and the debug read-backs take such a cache like a backing-2 cache;
+ * m40llm_ext_kvcache_debug_read_raw(which = 2) returns head_dim / 32 words (bits of d | bits of m << 16) per token
+ * and head instead of one f32 scale. */
+#define M40LLM_EXT_OLD_BACKING_FP16_K_Q4G32_V 3u
 M40llmKVCache* m40llm_kvcache_create_compressed(M40llmCudaContext* ctx, uint32_t max_seq_len,
                                                 uint32_t max_batch_size, uint32_t num_heads,
                                                 uint32_t head_dim, uint32_t recent_window,

@@ -34,7 +34,8 @@ struct BsParams {
     const uint16_t* new_k;     // ring [W][kvh][hd] of this sequence, or dense K of this sequence
     const uint16_t* dense_v;   // ring V (compressed) or dense V of this sequence
     const uint8_t* q4_v;       // [kvh][max_seq_len][hd/2] of this sequence (compressed only)
-    const float* q4_scale;     // [kvh][max_seq_len]
+    const float* q4_scale;     // [kvh][max_seq_len]; v_format 1: u32 [kvh][max_seq_len][hd/32], scale | min << 16
+    uint32_t v_format;
     const float* Q;            // [q_heads][hd]
     float* Out;
     float* scores;             // [q_heads][nblk]
@@ -277,14 +278,16 @@ struct BsWaveState {
 };
 
 // Token rows of one pass of a wave (at most kPass tokens) as they arrive from memory.
-template <int HD, bool QUANT>
+// VF (with QUANT): old V format, 0 the reference's q4 with one f32 scale per token and head, 1 groups of 32 with an f16
+// scale and an f16 minimum.
+template <int HD, bool QUANT, int VF = 0>
 struct BsRows {
     static constexpr int kPass = QUANT ? kBsPassQuant : kBsPassF16;
     static constexpr int S = kPass / (64 / (HD / 8));
     uint4 kw[S];
     uint4 vw[QUANT ? 1 : S];
     uint32_t qw[QUANT ? S : 1];
-    float qs[QUANT ? S : 1];
+    float qs[QUANT ? S : 1];         // VF 1: the bits of the group's scale | min << 16
     uint32_t t_begin, t_end;
 };
 
@@ -295,24 +298,28 @@ struct BsRows {
 //   t_end are read as they lie (the next tokens, the next head, or the zeroed slack rows the cache allocates behind
 //   its old store) and carry no weight.
 //   Otherwise: f16 K and V rows of the ring or of a dense cache; rows past the end repeat the last one.
-template <int HD, bool QUANT>
+template <int HD, bool QUANT, int VF>
 __device__ __forceinline__ void bs_issue(const BsParams& p, uint32_t kvh, uint32_t t_begin, uint32_t t_end,
-                                         BsRows<HD, QUANT>& r) {
-    constexpr int LPT = HD / 8, TPW = 64 / LPT, S = BsRows<HD, QUANT>::S;
+                                         BsRows<HD, QUANT, VF>& r) {
+    constexpr int LPT = HD / 8, TPW = 64 / LPT, S = BsRows<HD, QUANT, VF>::S;
     const int lane = threadIdx.x & 63;
     const int c = lane % LPT, tg = lane / LPT;
     r.t_begin = t_begin; r.t_end = t_end;
     if (QUANT) {
         const char* kbase = reinterpret_cast<const char*>(p.old_k + (size_t)kvh * p.old_head_stride);
         const char* vbase = reinterpret_cast<const char*>(p.q4_v + (size_t)kvh * p.max_seq_len * (HD / 2));
-        const char* sbase = reinterpret_cast<const char*>(p.q4_scale + (size_t)kvh * p.max_seq_len);
+        // bytes of scale data per row: one f32, or one word per group of 32 dimensions (a lane's eight dimensions 8c..8c+7
+        // lie in group c / 4)
+        constexpr int SB = VF == 1 ? (HD / 32) * 4 : 4;
+        const char* sbase = reinterpret_cast<const char*>(p.q4_scale) + (size_t)kvh * p.max_seq_len * SB;
         const uint32_t row = t_begin + (uint32_t)tg;
-        const uint32_t koff = row * (HD * 2) + 16 * c, voff = row * (HD / 2) + 4 * c, soff = row * 4;
+        const uint32_t koff = row * (HD * 2) + 16 * c, voff = row * (HD / 2) + 4 * c;
+        const uint32_t soff = row * SB + (VF == 1 ? 4 * (c / 4) : 0);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             r.kw[s] = *reinterpret_cast<const uint4*>(kbase + koff + s * (TPW * HD * 2));
             r.qw[s] = *reinterpret_cast<const uint32_t*>(vbase + voff + s * (TPW * HD / 2));
-            r.qs[s] = *reinterpret_cast<const float*>(sbase + soff + s * (TPW * 4));
+            r.qs[s] = *reinterpret_cast<const float*>(sbase + soff + s * (TPW * SB));
         }
     } else {
         const uint32_t row_bytes = p.kv_heads * HD * 2;
@@ -348,9 +355,9 @@ __device__ __forceinline__ uint32_t bs_f2h_pair(float a, float b) {
 }
 
 // Softmax terms of the rows of one pass, joined to the wave's running state.
-template <int HD, bool QUANT>
-__device__ __forceinline__ void bs_consume(const float (&q)[8], const BsRows<HD, QUANT>& r, BsWaveState& st) {
-    constexpr int LPT = HD / 8, TPW = 64 / LPT, S = BsRows<HD, QUANT>::S;
+template <int HD, bool QUANT, int VF>
+__device__ __forceinline__ void bs_consume(const float (&q)[8], const BsRows<HD, QUANT, VF>& r, BsWaveState& st) {
+    constexpr int LPT = HD / 8, TPW = 64 / LPT, S = BsRows<HD, QUANT, VF>::S;
     const int lane = threadIdx.x & 63;
     const int c = lane % LPT, tg = lane / LPT;
     const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
@@ -379,7 +386,17 @@ __device__ __forceinline__ void bs_consume(const float (&q)[8], const BsRows<HD,
     for (int s = 0; s < S; ++s) {
         const float e = __expf(sc[s] - m_new);        // rows past the end: exp(-inf) = 0
         if (c == 0) st.l += e;
-        if (QUANT) {
+        if (QUANT && VF == 1) {
+            // value = fmaf(nibble, scale, min), scale and min f16 (one rounding; no pass through f16)
+            const uint32_t dm = __float_as_uint(r.qs[s]);
+            const float d = m40_h2f((uint16_t)(dm & 0xffffu)), mn = m40_h2f((uint16_t)(dm >> 16));
+            const uint32_t even = r.qw[s] & 0x0f0f0f0fu, odd = (r.qw[s] >> 4) & 0x0f0f0f0fu;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                st.acc[2 * k] = fmaf(e, fmaf((float)((even >> (8 * k)) & 0xffu), d, mn), st.acc[2 * k]);
+                st.acc[2 * k + 1] = fmaf(e, fmaf((float)((odd >> (8 * k)) & 0xffu), d, mn), st.acc[2 * k + 1]);
+            }
+        } else if (QUANT) {
             // value = nibble * scale rounded to f32, then through f16 (cuda/kernels.cu:3078-3084).  The eight nibbles
             // become bytes biased by 8 (two's complement n -> (n ^ 8) - 8), a byte converts in one instruction, and
             // byte * scale - 8 * scale in one fused operation is the product nibble * scale rounded once.
@@ -405,14 +422,14 @@ __device__ __forceinline__ void bs_consume(const float (&q)[8], const BsRows<HD,
 
 // Tokens [t_begin, t_end) for one wave, kPass tokens per pass (one pass for a block of at most 64 old tokens, and
 // for a wave's share of a chunk of the recent window).
-template <int HD, bool QUANT>
+template <int HD, bool QUANT, int VF = 0>
 __device__ __forceinline__ void bs_wave_attend(const BsParams& p, uint32_t kvh, const float (&q)[8], uint32_t t_begin,
                                                uint32_t t_end, BsWaveState& st) {
-    constexpr uint32_t kPass = BsRows<HD, QUANT>::kPass;
+    constexpr uint32_t kPass = BsRows<HD, QUANT, VF>::kPass;
     for (uint32_t t0 = t_begin; t0 < t_end; t0 += kPass) {
-        BsRows<HD, QUANT> rows;
-        bs_issue<HD, QUANT>(p, kvh, t0, t0 + kPass < t_end ? t0 + kPass : t_end, rows);
-        bs_consume<HD, QUANT>(q, rows, st);
+        BsRows<HD, QUANT, VF> rows;
+        bs_issue<HD, QUANT, VF>(p, kvh, t0, t0 + kPass < t_end ? t0 + kPass : t_end, rows);
+        bs_consume<HD, QUANT, VF>(q, rows, st);
     }
 }
 
@@ -460,7 +477,8 @@ __global__ __launch_bounds__(kBsThreads, 3) void bs_attend_kernel(BsMulti multi)
             b0 = blk * p.block_size;
             b1 = b0 + p.block_size < p.old_len ? b0 + p.block_size : p.old_len;
         }
-        if (p.compressed) bs_wave_attend<HD, true>(p, kvh, q, b0, b1, st);
+        if (p.compressed && p.v_format) bs_wave_attend<HD, true, 1>(p, kvh, q, b0, b1, st);
+        else if (p.compressed) bs_wave_attend<HD, true, 0>(p, kvh, q, b0, b1, st);
         else bs_wave_attend<HD, false>(p, kvh, q, b0, b1, st);
     }
 
@@ -585,7 +603,8 @@ int prepare(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id, co
         p->new_k = kv->d_recent_k + (size_t)seq_id * kv->recent_window * ept;
         p->dense_v = kv->d_recent_v + (size_t)seq_id * kv->recent_window * ept;
         p->q4_v = kv->d_q4_old_v + (size_t)seq_id * kv->max_seq_len * kvh * (hd / 2u);
-        p->q4_scale = kv->d_q4_old_v_scale + (size_t)seq_id * kv->max_seq_len * kvh;
+        p->q4_scale = kv->d_q4_old_v_scale + (size_t)seq_id * kv->max_seq_len * kvh * (kv->v_format ? hd / 32u : 1u);
+        p->v_format = kv->v_format;
     } else {
         p->old_k = kv->d_k + (size_t)seq_id * kv->max_seq_len * ept;
         p->old_tok_stride = (uint32_t)ept;

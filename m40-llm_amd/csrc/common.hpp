@@ -74,7 +74,7 @@ struct M40llmKVCache {
     // kM40OldStoreSlackRows zeroed rows: the attention reads whole passes of rows and ignores those past a block.
     uint16_t* d_fp16_old_k;        // [seq][kvh][max_seq_len][hd], token index = absolute position
     uint8_t* d_q4_old_v;           // [seq][kvh][max_seq_len][hd/2]
-    float* d_q4_old_v_scale;       // [seq][kvh][max_seq_len]
+    float* d_q4_old_v_scale;       // [seq][kvh][max_seq_len]; with v_format 1: u32 [seq][kvh][max_seq_len][hd/32]
     uint32_t max_seq_len;
     uint32_t max_batch_size;
     uint32_t num_heads;            // kv heads
@@ -87,6 +87,7 @@ struct M40llmKVCache {
     uint32_t representatives;
     uint32_t representative_policy;
     uint32_t fp16_k_q4_v_old_backing;
+    uint32_t v_format;             // old V: 0 the reference's q4 (f32 scale per token and head), 1 groups of 32 with f16 scale + f16 min
     int device_id;
 };
 
@@ -320,5 +321,25 @@ __device__ __forceinline__ uint8_t m40_pack_q4_pair(float a, float b, float scal
     qa = qa < -7 ? -7 : (qa > 7 ? 7 : qa);
     qb = qb < -7 ? -7 : (qb > 7 ? 7 : qb);
     return (uint8_t)((qa & 0x0f) | ((qb & 0x0f) << 4));
+}
+
+// 4-bit V in groups of 32 under an f16 scale and an f16 minimum (old-store format 1; no counterpart in the reference).
+// The lane holds dimensions 2 lane, 2 lane + 1 of a head; a group is 16 consecutive lanes.  Returns the packed byte
+// and, in *dm, the group's word: bits of d = f16((max - min) / 15) | bits of m = f16(min) << 16.
+__device__ __forceinline__ uint8_t m40_pack_q4g32_pair(float a, float b, uint32_t* dm) {
+    float mn = fminf(a, b), mx = fmaxf(a, b);
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+        mn = fminf(mn, __shfl_xor(mn, o, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    }
+    const uint16_t db = m40_f2h((mx - mn) / 15.0f), mb = m40_f2h(mn);
+    const float d = m40_h2f(db), m = m40_h2f(mb);
+    *dm = (uint32_t)db | ((uint32_t)mb << 16);
+    int qa = d > 0.0f ? (int)lrintf((a - m) / d) : 0;
+    int qb = d > 0.0f ? (int)lrintf((b - m) / d) : 0;
+    qa = qa < 0 ? 0 : (qa > 15 ? 15 : qa);
+    qb = qb < 0 ? 0 : (qb > 15 ? 15 : qb);
+    return (uint8_t)(qa | (qb << 4));
 }
 #endif  // __HIPCC__

@@ -46,15 +46,15 @@ __device__ __forceinline__ void stage_load(const float* __restrict__ x, const vo
     }
 #pragma unroll
     for (int u = 0; u < kStageBatch; ++u) r.x[u] = reinterpret_cast<const float4*>(x)[idx[u]];
-    if (w_dtype == 0u) {
+    // One unconditional batch whatever the weights' type: a branch around loads makes the compiler wait for every
+    // load in flight at its join (the rows above).  f32: 16 bytes per index as two halves; f16: 8 bytes, asked for twice.
+    const char* wb = static_cast<const char*>(w);
+    const int stride = w_dtype == 0u ? 8 : 16, hi_off = w_dtype == 0u ? 0 : 8;
 #pragma unroll
-        for (int u = 0; u < kStageBatch; ++u) {
-            const uint2 h = reinterpret_cast<const uint2*>(w)[idx[u]];
-            r.w[u].x = h.x; r.w[u].y = h.y; r.w[u].z = 0u; r.w[u].w = 0u;
-        }
-    } else {
-#pragma unroll
-        for (int u = 0; u < kStageBatch; ++u) r.w[u] = reinterpret_cast<const uint4*>(w)[idx[u]];
+    for (int u = 0; u < kStageBatch; ++u) {
+        const uint2 lo = *reinterpret_cast<const uint2*>(wb + (size_t)idx[u] * stride);
+        const uint2 hi = *reinterpret_cast<const uint2*>(wb + (size_t)idx[u] * stride + hi_off);
+        r.w[u].x = lo.x; r.w[u].y = lo.y; r.w[u].z = hi.x; r.w[u].w = hi.y;
     }
 }
 
@@ -150,6 +150,11 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
     __shared__ float wave_sums[kWavesPerBlock];
     const int K = (int)p.d_model;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // x and the norm weights are requested before anything else is computed, then (below) the position and the pair's
+    // rotation entry, then the GEMV weights; the norm prologue runs while the weights stream in
+    StageRegs xr;
+    stage_load(p.x, p.norm_w, p.norm_dtype, K, 0, xr);
+    __builtin_amdgcn_sched_barrier(0);
     const uint32_t half = p.head_dim / 2u;
     const uint32_t q_pairs = p.q_heads * half, kv_pairs = p.kv_heads * half;
     const uint32_t pair0 = (blockIdx.x * kWavesPerBlock + wave) * PAIRS;
@@ -173,20 +178,22 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
         bp[2 * q] = reinterpret_cast<const uint4*>(W + i0[q] * (size_t)K);
         bp[2 * q + 1] = reinterpret_cast<const uint4*>(W + i1[q] * (size_t)K);
     }
-    // x and the norm weights are requested first, then the GEMV weights; the norm prologue runs while those stream in
-    StageRegs xr;
-    stage_load(p.x, p.norm_w, p.norm_dtype, K, 0, xr);
-    // position and pair frequencies are requested with x, ahead of the weights
-    const uint32_t position = p.position_dev ? *p.position_dev : p.position;
+    // position and pair frequencies are requested with x, ahead of the weights.  Unconditionally: a load under a branch
+    // costs a wait for everything in flight at the branch's join, which here held the weight requests back until x, the
+    // norm weights and the position had arrived.  An absent input reads the first bytes of Wq and is ignored.
+    const uint32_t position_loaded = *(p.position_dev ? p.position_dev : reinterpret_cast<const uint32_t*>(p.wq));
     float inv_freq[PAIRS];
     float4 kept[PAIRS];        // the pair's rotation as left by an earlier launch (the step's first layer)
 #pragma unroll
     for (int q = 0; q < PAIRS; ++q) {
-        inv_freq[q] = p.rope_table ? p.rope_table[off[q]] : 0.0f;
-        kept[q] = p.rope_cs ? p.rope_cs[off[q]] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        inv_freq[q] = *(p.rope_table ? p.rope_table + off[q] : reinterpret_cast<const float*>(p.wq));
+        kept[q] = *(p.rope_cs ? p.rope_cs + off[q] : reinterpret_cast<const float4*>(p.wq));
     }
+    const uint32_t position = p.position_dev ? position_loaded : p.position;
+    __builtin_amdgcn_sched_barrier(0);
     GemvRegs<2 * PAIRS> regs;
     gemv_prefetch<2 * PAIRS>(bp, 0, K >> 3, lane, regs);
+    __builtin_amdgcn_sched_barrier(0);
     // the rotation angle does not depend on the data: evaluated while the weights are in flight
     float2 cs[PAIRS];
 #pragma unroll
@@ -202,7 +209,7 @@ __global__ __launch_bounds__(kThreads) void norm_qkv_rope_append_kernel(QkvArgs 
             if (hit) {
                 cs[q] = make_float2(kept[q].y, kept[q].z);
             } else {
-                if (!p.rope_table) inv_freq[q] = m40_rope_inv_freq(off[q], p.head_dim, p.rope_base);
+                if (!p.rope_table) inv_freq[q] = m40_rope_inv_freq(off[q], p.head_dim, p.rope_base);      // replaces the ignored bytes
                 cs[q] = m40_rope_cos_sin_freq(position, inv_freq[q], p.rope_scale);
                 if (p.rope_cs && which[q] == 0 && local[q] < half && lane == 0)      // the waves of q head 0 keep it
                     p.rope_cs[off[q]] = make_float4(__uint_as_float(position), cs[q].x, cs[q].y, __uint_as_float(tag));

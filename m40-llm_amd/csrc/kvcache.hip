@@ -139,7 +139,7 @@ __global__ __launch_bounds__(kThreads) void prefill_rope_append_kernel(
 // overwritten into registers and, when position >= W, evicts it to old index position-W
 // (K copied, V quantised to 4 bits with one f32 scale per token-head).  Phase 2, after a
 // barrier, writes the rotated K and the cast V into the ring.
-template <int HD>
+template <int HD, bool G32>
 __global__ __launch_bounds__(64) void compressed_append_kernel(
     const float* __restrict__ k_in, const float* __restrict__ v_in, uint16_t* __restrict__ recent_k,
     uint16_t* __restrict__ recent_v, uint16_t* __restrict__ old_k, uint8_t* __restrict__ q4_v,
@@ -166,10 +166,19 @@ __global__ __launch_bounds__(64) void compressed_append_kernel(
             v0 = m40_h2f(recent_v[ring_base + d0]);
             v1 = m40_h2f(recent_v[ring_base + d0 + 1]);
         }
-        const float max_v = m40_max64(fmaxf(fabsf(v0), fabsf(v1)));
-        const float scale = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
-        if (lane == 0) q4_scale[old_row] = scale;
-        if (active) q4_v[old_row * PAIRS + lane] = m40_pack_q4_pair(v0, v1, scale);
+        if (G32) {
+            // groups of 32 dimensions = 16 lanes; lanes past the head (head_dim 64) form groups of their own, unused
+            uint32_t dm;
+            const uint8_t byte = m40_pack_q4g32_pair(v0, v1, &dm);
+            if (active && (lane & 15u) == 0u)
+                reinterpret_cast<uint32_t*>(q4_scale)[old_row * (HD / 32) + lane / 16u] = dm;
+            if (active) q4_v[old_row * PAIRS + lane] = byte;
+        } else {
+            const float max_v = m40_max64(fmaxf(fabsf(v0), fabsf(v1)));
+            const float scale = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
+            if (lane == 0) q4_scale[old_row] = scale;
+            if (active) q4_v[old_row * PAIRS + lane] = m40_pack_q4_pair(v0, v1, scale);
+        }
     }
     __syncthreads();
     if (active) {
@@ -187,7 +196,7 @@ __global__ __launch_bounds__(64) void compressed_append_kernel(
 }
 
 // Bulk fill of a compressed cache from f16 rows: grid (token, kv head), one wave each.
-template <int HD>
+template <int HD, bool G32>
 __global__ __launch_bounds__(64) void compressed_bulk_fill_kernel(
     const uint16_t* __restrict__ k_rows, const uint16_t* __restrict__ v_rows, uint16_t* __restrict__ recent_k,
     uint16_t* __restrict__ recent_v, uint16_t* __restrict__ old_k, uint8_t* __restrict__ q4_v,
@@ -211,10 +220,19 @@ __global__ __launch_bounds__(64) void compressed_bulk_fill_kernel(
             v0 = m40_h2f(v_rows[src + d0]);
             v1 = m40_h2f(v_rows[src + d0 + 1]);
         }
-        const float max_v = m40_max64(fmaxf(fabsf(v0), fabsf(v1)));
-        const float scale = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
-        if (lane == 0) q4_scale[old_row] = scale;
-        if (active) q4_v[old_row * PAIRS + lane] = m40_pack_q4_pair(v0, v1, scale);
+        if (G32) {
+            // groups of 32 dimensions = 16 lanes; lanes past the head (head_dim 64) form groups of their own, unused
+            uint32_t dm;
+            const uint8_t byte = m40_pack_q4g32_pair(v0, v1, &dm);
+            if (active && (lane & 15u) == 0u)
+                reinterpret_cast<uint32_t*>(q4_scale)[old_row * (HD / 32) + lane / 16u] = dm;
+            if (active) q4_v[old_row * PAIRS + lane] = byte;
+        } else {
+            const float max_v = m40_max64(fmaxf(fabsf(v0), fabsf(v1)));
+            const float scale = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
+            if (lane == 0) q4_scale[old_row] = scale;
+            if (active) q4_v[old_row * PAIRS + lane] = m40_pack_q4_pair(v0, v1, scale);
+        }
     } else {
         const size_t ring_base = ((size_t)seq_id * recent_window + (t % recent_window)) * ept + (size_t)head * HD;
         if (active) {
@@ -300,8 +318,10 @@ M40llmKVCache* m40llm_kvcache_create_compressed(M40llmCudaContext* ctx, uint32_t
                                                 uint32_t exact_old_backing) {
     if (!ctx || recent_window == 0 || block_size == 0) return nullptr;
     if (m40_ensure_device(ctx) != 0) return nullptr;
-    if (exact_old_backing == 1u) return nullptr;  // q8 backing is not part of this build
-    if (exact_old_backing == 2u && head_dim != 64 && head_dim != 128) return nullptr;  // kernels.cu:5371
+    if (exact_old_backing == 1u || exact_old_backing > 3u) return nullptr;  // q8 backing is not part of this build
+    // backing 3 (no counterpart in the reference): backing 2 with old V in groups of 32 under an f16 scale and minimum
+    const bool old_store = exact_old_backing == 2u || exact_old_backing == 3u;
+    if (old_store && head_dim != 64 && head_dim != 128) return nullptr;  // kernels.cu:5371
     M40llmKVCache* kv = new (std::nothrow) M40llmKVCache();
     if (!kv) return nullptr;
     std::memset(kv, 0, sizeof(*kv));
@@ -330,11 +350,12 @@ M40llmKVCache* m40llm_kvcache_create_compressed(M40llmCudaContext* ctx, uint32_t
         (void)hipMemset(kv->d_recent_v, 0, recent_bytes);
         (void)hipMemset(kv->d_seq_map, 0, seq_map_size);
     }
-    if (ok && exact_old_backing == 2u) {
+    if (ok && old_store) {
         // kM40OldStoreSlackRows zeroed rows behind each array (see M40llmKVCache)
         const size_t old_k_bytes = (kv_elems(kv) + (size_t)kM40OldStoreSlackRows * head_dim) * sizeof(uint16_t);
         const size_t q4_bytes = ((size_t)max_seq_len * max_batch_size * num_heads + kM40OldStoreSlackRows) * (head_dim / 2u);
-        const size_t scale_bytes = ((size_t)max_seq_len * max_batch_size * num_heads + kM40OldStoreSlackRows) * sizeof(float);
+        const size_t scale_bytes = ((size_t)max_seq_len * max_batch_size * num_heads + kM40OldStoreSlackRows) *
+                                   (exact_old_backing == 3u ? (head_dim / 32u) * sizeof(uint32_t) : sizeof(float));
         ok = hipMalloc(reinterpret_cast<void**>(&kv->d_fp16_old_k), old_k_bytes ? old_k_bytes : 2) == hipSuccess &&
              hipMalloc(reinterpret_cast<void**>(&kv->d_q4_old_v), q4_bytes ? q4_bytes : 1) == hipSuccess &&
              hipMalloc(reinterpret_cast<void**>(&kv->d_q4_old_v_scale), scale_bytes ? scale_bytes : 4) == hipSuccess;
@@ -343,6 +364,7 @@ M40llmKVCache* m40llm_kvcache_create_compressed(M40llmCudaContext* ctx, uint32_t
             (void)hipMemset(kv->d_q4_old_v, 0, q4_bytes);
             (void)hipMemset(kv->d_q4_old_v_scale, 0, scale_bytes);
             kv->fp16_k_q4_v_old_backing = 1;
+            kv->v_format = exact_old_backing == 3u ? 1u : 0u;
         }
     }
     if (!ok) {
@@ -380,7 +402,8 @@ int m40llm_kvcache_reset(M40llmCudaContext* ctx, M40llmKVCache* kv) {
                                  (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * (kv->head_dim / 2u), s);
         if (kv->d_q4_old_v_scale)
             (void)hipMemsetAsync(kv->d_q4_old_v_scale, 0,
-                                 (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * sizeof(float), s);
+                                 (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads *
+                                     (kv->v_format ? (kv->head_dim / 32u) * sizeof(uint32_t) : sizeof(float)), s);
     }
     return hipStreamSynchronize(s) == hipSuccess ? 0 : -4;
 }
@@ -484,16 +507,16 @@ int m40llm_kvcache_append_token_f32_rope_k_compressed_at_layout_async(
     if (position >= kv->max_seq_len) return -5;
     (void)hipGetLastError();
     const uint32_t evict = kv->fp16_k_q4_v_old_backing ? 1u : 0u;
+    auto launch = [&](auto kernel) {
+        kernel<<<kv->num_heads, 64, 0, ctx->decode_stream>>>(
+            static_cast<const float*>(k_dev_f32), static_cast<const float*>(v_dev_f32), kv->d_recent_k,
+            kv->d_recent_v, kv->d_fp16_old_k, kv->d_q4_old_v, kv->d_q4_old_v_scale, kv->d_seq_map, seq_id,
+            kv->max_seq_len, kv->recent_window, kv->num_heads, position, freq_base, freq_scale, rope_layout, evict);
+    };
     if (kv->head_dim == 64) {
-        compressed_append_kernel<64><<<kv->num_heads, 64, 0, ctx->decode_stream>>>(
-            static_cast<const float*>(k_dev_f32), static_cast<const float*>(v_dev_f32), kv->d_recent_k,
-            kv->d_recent_v, kv->d_fp16_old_k, kv->d_q4_old_v, kv->d_q4_old_v_scale, kv->d_seq_map, seq_id,
-            kv->max_seq_len, kv->recent_window, kv->num_heads, position, freq_base, freq_scale, rope_layout, evict);
+        if (kv->v_format) launch(compressed_append_kernel<64, true>); else launch(compressed_append_kernel<64, false>);
     } else {
-        compressed_append_kernel<128><<<kv->num_heads, 64, 0, ctx->decode_stream>>>(
-            static_cast<const float*>(k_dev_f32), static_cast<const float*>(v_dev_f32), kv->d_recent_k,
-            kv->d_recent_v, kv->d_fp16_old_k, kv->d_q4_old_v, kv->d_q4_old_v_scale, kv->d_seq_map, seq_id,
-            kv->max_seq_len, kv->recent_window, kv->num_heads, position, freq_base, freq_scale, rope_layout, evict);
+        if (kv->v_format) launch(compressed_append_kernel<128, true>); else launch(compressed_append_kernel<128, false>);
     }
     return hipGetLastError() == hipSuccess ? 0 : -6;
 }
@@ -627,7 +650,9 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
     switch (which) {
         case 0: src = kv->d_fp16_old_k; total = kv_elems(kv) * 2; item = (size_t)kv->head_dim * 2; break;
         case 1: src = kv->d_q4_old_v; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * (kv->head_dim / 2u); item = kv->head_dim / 2u; break;
-        case 2: src = kv->d_q4_old_v_scale; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * 4; item = 4; break;
+        case 2:      // f32 scale per (token, kv head); with groups of 32: head_dim / 32 words of scale | min << 16
+            item = kv->v_format ? (size_t)(kv->head_dim / 32u) * 4 : 4;
+            src = kv->d_q4_old_v_scale; total = (size_t)kv->max_seq_len * kv->max_batch_size * kv->num_heads * item; break;
         case 3: src = kv->d_recent_k; total = (size_t)kv->max_batch_size * kv->recent_window * ept * 2; break;
         case 4: src = kv->d_recent_v; total = (size_t)kv->max_batch_size * kv->recent_window * ept * 2; break;
         case 5: src = kv->d_seq_map; total = (size_t)kv->max_batch_size * 4; break;
@@ -671,16 +696,16 @@ int m40llm_ext_kvcache_bulk_fill_f16(M40llmCudaContext* ctx, M40llmKVCache* kv, 
         if (kv->head_dim != 64 && kv->head_dim != 128) return -5;
         dim3 grid(seq_len, kv->num_heads);
         const uint32_t has_old = kv->fp16_k_q4_v_old_backing ? 1u : 0u;
+        auto launch = [&](auto kernel) {
+            kernel<<<grid, 64, 0, s>>>(
+                static_cast<const uint16_t*>(k_dev_f16), static_cast<const uint16_t*>(v_dev_f16), kv->d_recent_k,
+                kv->d_recent_v, kv->d_fp16_old_k, kv->d_q4_old_v, kv->d_q4_old_v_scale, kv->d_seq_map, seq_id,
+                kv->max_seq_len, kv->recent_window, kv->num_heads, seq_len, has_old);
+        };
         if (kv->head_dim == 64) {
-            compressed_bulk_fill_kernel<64><<<grid, 64, 0, s>>>(
-                static_cast<const uint16_t*>(k_dev_f16), static_cast<const uint16_t*>(v_dev_f16), kv->d_recent_k,
-                kv->d_recent_v, kv->d_fp16_old_k, kv->d_q4_old_v, kv->d_q4_old_v_scale, kv->d_seq_map, seq_id,
-                kv->max_seq_len, kv->recent_window, kv->num_heads, seq_len, has_old);
+            if (kv->v_format) launch(compressed_bulk_fill_kernel<64, true>); else launch(compressed_bulk_fill_kernel<64, false>);
         } else {
-            compressed_bulk_fill_kernel<128><<<grid, 64, 0, s>>>(
-                static_cast<const uint16_t*>(k_dev_f16), static_cast<const uint16_t*>(v_dev_f16), kv->d_recent_k,
-                kv->d_recent_v, kv->d_fp16_old_k, kv->d_q4_old_v, kv->d_q4_old_v_scale, kv->d_seq_map, seq_id,
-                kv->max_seq_len, kv->recent_window, kv->num_heads, seq_len, has_old);
+            if (kv->v_format) launch(compressed_bulk_fill_kernel<128, true>); else launch(compressed_bulk_fill_kernel<128, false>);
         }
     }
     if (hipGetLastError() != hipSuccess) return -6;

@@ -361,38 +361,42 @@ def bench_q80(b: Bench):
 
 
 def bench_block_select(b: Bench):
-    rng = np.random.default_rng(3)
+    import ctypes as C
     qh, kvh, hd, L, bs, top, W = 32, 8, 128, 32768, 64, 64, 512
     nseq = 4
-    kv = m40.KVCache(b.ctx, L, nseq, kvh, hd, compressed=dict(recent_window=W, block_size=bs, top_blocks=top))
-    for s in range(nseq):
-        k = f16(rng.standard_normal((L, kvh, hd))); v = f16(rng.standard_normal((L, kvh, hd)))
-        dk, dv = b.ctx.to_device(k), b.ctx.to_device(v)
-        b.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, s, dk.ptr, dv.ptr, L)
-        dk.free(); dv.free()
-    q = b.ctx.to_device(rng.standard_normal(qh * hd).astype(np.float32))
-    out = b.ctx.alloc(qh * hd * 4)
     old = L - W
-    score = old * kvh * hd * 2
-    attend = qh * (top * bs * hd * 2 + W * hd * 2 + top * bs * (hd // 2 + 4) + W * hd * 2)
-    algo = score + attend
-    name = "m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async"
-    b.time("block_select fp16-K/q4-V, B=1", f"qh32 kvh8 hd128 L32768 bs64 top64 W512", algo,
-           lambda i: b.call(name, kv.h, i, q.ptr, qh, L, W, bs, top, out.ptr), nseq)
-
-    def four(i):
+    # old V: the reference's q4 (one f32 scale per token and head) and the groups-of-32 scale + min format (backing 3)
+    for backing, label, vbytes in ((2, "fp16-K/q4-V", hd // 2 + 4), (3, "fp16-K/q4-V groups of 32", hd // 2 + 4 * (hd // 32))):
+        rng = np.random.default_rng(3)
+        kv = m40.KVCache(b.ctx, L, nseq, kvh, hd, compressed=dict(recent_window=W, block_size=bs, top_blocks=top,
+                                                                  exact_old_backing=backing))
         for s in range(nseq):
-            b.call(name, kv.h, s, q.ptr, qh, L, W, bs, top, out.ptr)
-    b.time("block_select fp16-K/q4-V, B=4", "4 slots per step, one call per slot", 4 * algo, four, 1, reps=16, warm=2)
-    q4 = b.ctx.to_device(rng.standard_normal((nseq, qh * hd)).astype(np.float32))
-    out4 = b.ctx.alloc(nseq * qh * hd * 4)
-    ids_h = np.arange(nseq, dtype=np.uint32); lens_h = np.full(nseq, L, dtype=np.uint32)
-    import ctypes as C
-    b.time("block_select fp16-K/q4-V, B=4", "4 slots per step, multi-slot call", 4 * algo,
-           lambda i: b.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, nseq,
-                            ids_h.ctypes.data_as(C.c_void_p), lens_h.ctypes.data_as(C.c_void_p), q4.ptr, qh, W, bs, top, out4.ptr),
-           1, reps=16, warm=2)
-    kv.destroy()
+            k = f16(rng.standard_normal((L, kvh, hd))); v = f16(rng.standard_normal((L, kvh, hd)))
+            dk, dv = b.ctx.to_device(k), b.ctx.to_device(v)
+            b.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, s, dk.ptr, dv.ptr, L)
+            dk.free(); dv.free()
+        q = b.ctx.to_device(rng.standard_normal(qh * hd).astype(np.float32))
+        out = b.ctx.alloc(qh * hd * 4)
+        score = old * kvh * hd * 2
+        attend = qh * (top * bs * hd * 2 + W * hd * 2 + top * bs * vbytes + W * hd * 2)
+        algo = score + attend
+        name = "m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async"
+        b.time(f"block_select {label}, B=1", f"qh32 kvh8 hd128 L32768 bs64 top64 W512", algo,
+               lambda i: b.call(name, kv.h, i, q.ptr, qh, L, W, bs, top, out.ptr), nseq)
+
+        def four(i):
+            for s in range(nseq):
+                b.call(name, kv.h, s, q.ptr, qh, L, W, bs, top, out.ptr)
+        if backing == 2:
+            b.time(f"block_select {label}, B=4", "4 slots per step, one call per slot", 4 * algo, four, 1, reps=16, warm=2)
+        q4 = b.ctx.to_device(rng.standard_normal((nseq, qh * hd)).astype(np.float32))
+        out4 = b.ctx.alloc(nseq * qh * hd * 4)
+        ids_h = np.arange(nseq, dtype=np.uint32); lens_h = np.full(nseq, L, dtype=np.uint32)
+        b.time(f"block_select {label}, B=4", "4 slots per step, multi-slot call", 4 * algo,
+               lambda i: b.call("m40llm_ext_attention_block_select_fp16_k_q4_v_multi_async", kv.h, nseq,
+                                ids_h.ctypes.data_as(C.c_void_p), lens_h.ctypes.data_as(C.c_void_p), q4.ptr, qh, W, bs, top, out4.ptr),
+               1, reps=16, warm=2)
+        kv.destroy()
 
 
 def bench_decode_batch(b: Bench, steps=32, warmup=4, mode=2):

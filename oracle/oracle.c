@@ -482,7 +482,11 @@ int orc_attention_prefill_gqa_varlen(const float* q, const float* k, const float
 /* ------------------------------------------------------------------------ */
 orc_ckv* orc_ckv_create(uint32_t max_seq_len, uint32_t max_batch, uint32_t kv_heads,
                         uint32_t head_dim, uint32_t recent_window, uint32_t block_size) {
-    if (recent_window == 0 || block_size == 0) return NULL;
+    return orc_ckv_create_fmt(max_seq_len, max_batch, kv_heads, head_dim, recent_window, block_size, 0u);
+}
+orc_ckv* orc_ckv_create_fmt(uint32_t max_seq_len, uint32_t max_batch, uint32_t kv_heads,
+                            uint32_t head_dim, uint32_t recent_window, uint32_t block_size, uint32_t v_format) {
+    if (recent_window == 0 || block_size == 0 || v_format > 1u) return NULL;
     if (head_dim != 64 && head_dim != 128) return NULL;
     orc_ckv* c = (orc_ckv*)calloc(1, sizeof(orc_ckv));
     c->max_seq_len = max_seq_len;
@@ -497,13 +501,15 @@ orc_ckv* orc_ckv_create(uint32_t max_seq_len, uint32_t max_batch, uint32_t kv_he
     c->old_k = (uint16_t*)calloc((size_t)max_batch * max_seq_len * ept, 2);
     c->q4_v = (uint8_t*)calloc((size_t)max_batch * max_seq_len * kv_heads * (head_dim / 2), 1);
     c->q4_scale = (float*)calloc((size_t)max_batch * max_seq_len * kv_heads, 4);
+    c->v_format = v_format;
+    c->q4_dm = v_format ? (uint32_t*)calloc((size_t)max_batch * max_seq_len * kv_heads * (head_dim / 32), 4) : NULL;
     c->seq_map = (uint32_t*)calloc(max_batch, 4);
     return c;
 }
 void orc_ckv_destroy(orc_ckv* c) {
     if (!c) return;
     free(c->recent_k); free(c->recent_v); free(c->old_k);
-    free(c->q4_v); free(c->q4_scale); free(c->seq_map);
+    free(c->q4_v); free(c->q4_scale); free(c->q4_dm); free(c->seq_map);
     free(c);
 }
 size_t orc_ckv_bytes_old_k(const orc_ckv* c) {
@@ -513,6 +519,7 @@ size_t orc_ckv_bytes_q4_v(const orc_ckv* c) {
     return (size_t)c->max_batch * c->max_seq_len * c->kv_heads * (c->head_dim / 2);
 }
 size_t orc_ckv_bytes_q4_scale(const orc_ckv* c) {
+    if (c->v_format) return (size_t)c->max_batch * c->max_seq_len * c->kv_heads * (c->head_dim / 32) * 4;
     return (size_t)c->max_batch * c->max_seq_len * c->kv_heads * 4;
 }
 
@@ -542,6 +549,38 @@ float orc_q4_unpack(uint8_t packed, uint32_t lane, float scale) {
     return (float)sv * scale;
 }
 
+/* 4-bit V in groups of 32 with an f16 scale and an f16 minimum (the V format BASELINE's compressed-attention
+ * configuration names; the reference has no such format, so this definition is the contract):
+ *   per group: mn, mx = smallest and largest value; d = f16((mx - mn) / 15), m = f16(mn), both then read back as f32;
+ *   q = d > 0 ? clamp(lrintf((v - m) / d), 0, 15) : 0;  byte = q_even | q_odd << 4;  word = bits(d) | bits(m) << 16;
+ *   value = fmaf((float)q, d, m)  (one rounding, no pass through f16). */
+void orc_q4g32_quantize_row(const uint16_t* v_f16, uint32_t head_dim, uint8_t* packed, uint32_t* dm) {
+    for (uint32_t g = 0; g < head_dim / 32u; ++g) {
+        float mn = orc_f16_to_f32(v_f16[32 * g]), mx = mn;
+        for (uint32_t i = 1; i < 32u; ++i) {
+            const float v = orc_f16_to_f32(v_f16[32 * g + i]);
+            mn = fminf(mn, v); mx = fmaxf(mx, v);
+        }
+        const uint16_t db = orc_f32_to_f16((mx - mn) / 15.0f), mb = orc_f32_to_f16(mn);
+        const float d = orc_f16_to_f32(db), m = orc_f16_to_f32(mb);
+        dm[g] = (uint32_t)db | ((uint32_t)mb << 16);
+        for (uint32_t pair = 0; pair < 16u; ++pair) {
+            long q[2];
+            for (int e = 0; e < 2; ++e) {
+                const float v = orc_f16_to_f32(v_f16[32 * g + 2 * pair + e]);
+                q[e] = d > 0.0f ? lrintf((v - m) / d) : 0;
+                if (q[e] < 0) q[e] = 0;
+                if (q[e] > 15) q[e] = 15;
+            }
+            packed[16 * g + pair] = (uint8_t)((int)q[0] | ((int)q[1] << 4));
+        }
+    }
+}
+float orc_q4g32_unpack(uint8_t packed, uint32_t lane, uint32_t dm) {
+    const uint8_t nib = lane == 0u ? (packed & 0x0f) : ((packed >> 4) & 0x0f);
+    return fmaf((float)nib, orc_f16_to_f32((uint16_t)(dm & 0xffffu)), orc_f16_to_f32((uint16_t)(dm >> 16)));
+}
+
 /* m40llm_kvcache_append_token_f32_rope_k_compressed_at_layout_async,
  * cuda/kernels.cu:6108-6250: evict ring slot pos%W to old index pos-W first,
  * then overwrite the ring slot; seq_map[seq] = pos+1.  Error codes as there. */
@@ -564,7 +603,11 @@ int orc_ckv_append_rope_k_at(orc_ckv* c, uint32_t seq, uint32_t position,
             uint8_t* qv = c->q4_v + ((size_t)seq * c->max_seq_len + old_pos) * kvh * (hd / 2) +
                           (size_t)h * (hd / 2);
             float* sc = c->q4_scale + ((size_t)seq * c->max_seq_len + old_pos) * kvh + h;
-            orc_q4_quantize_row(rv + (size_t)h * hd, hd, qv, sc);
+            if (c->v_format)
+                orc_q4g32_quantize_row(rv + (size_t)h * hd, hd, qv,
+                                       c->q4_dm + (((size_t)seq * c->max_seq_len + old_pos) * kvh + h) * (hd / 32));
+            else
+                orc_q4_quantize_row(rv + (size_t)h * hd, hd, qv, sc);
         }
     }
     rope_k_to_f16(k_f32, rk, kvh, hd, position, freq_base, freq_scale, layout);
@@ -713,6 +756,9 @@ static float src_v(const kv_src* s, uint32_t t, uint32_t kvh, uint32_t d) {
             const size_t q4_base = ((size_t)s->seq * s->max_seq_len + t) * s->kv_heads * (s->head_dim / 2) +
                                    (size_t)kvh * (s->head_dim / 2);
             const size_t sc_idx = ((size_t)s->seq * s->max_seq_len + t) * s->kv_heads + kvh;
+            if (s->c->v_format)
+                return orc_q4g32_unpack(s->c->q4_v[q4_base + d / 2u], d & 1u,
+                                        s->c->q4_dm[sc_idx * (s->head_dim / 32) + d / 32u]);
             const float v = orc_q4_unpack(s->c->q4_v[q4_base + d / 2u], d & 1u, s->c->q4_scale[sc_idx]);
             return orc_f16_to_f32(orc_f32_to_f16(v)); /* rounded through f16, kernels.cu:3085-3086 */
         }

@@ -91,10 +91,18 @@ typedef struct orc_ckv {
     uint8_t*  q4_v;       /* [batch][max_seq_len][kvh][hd/2]                    */
     float*    q4_scale;   /* [batch][max_seq_len][kvh]                          */
     uint32_t* seq_map;    /* [batch]                                             */
+    uint32_t  v_format;   /* 0: reference q4 (one f32 scale per token and head); 1: groups of 32 with f16 scale + f16 min */
+    uint32_t* q4_dm;      /* v_format 1: [batch][max_seq_len][kvh][hd/32], scale bits | min bits << 16 */
 } orc_ckv;
 
 orc_ckv* orc_ckv_create(uint32_t max_seq_len, uint32_t max_batch, uint32_t kv_heads,
                         uint32_t head_dim, uint32_t recent_window, uint32_t block_size);
+/* the same cache with old V held 4-bit in groups of 32 under an f16 scale and an f16 minimum (no counterpart in the
+ * reference: the benchmark configuration's V format, defined by orc_q4g32_quantize_row / orc_q4g32_unpack) */
+orc_ckv* orc_ckv_create_fmt(uint32_t max_seq_len, uint32_t max_batch, uint32_t kv_heads,
+                            uint32_t head_dim, uint32_t recent_window, uint32_t block_size, uint32_t v_format);
+void     orc_q4g32_quantize_row(const uint16_t* v_f16, uint32_t head_dim, uint8_t* packed, uint32_t* dm);
+float    orc_q4g32_unpack(uint8_t packed, uint32_t lane, uint32_t dm);
 void     orc_ckv_destroy(orc_ckv* c);
 size_t   orc_ckv_bytes_old_k(const orc_ckv* c);
 size_t   orc_ckv_bytes_q4_v(const orc_ckv* c);

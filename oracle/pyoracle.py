@@ -51,7 +51,7 @@ class OrcCkv(C.Structure):
         ("max_seq_len", u32), ("max_batch", u32), ("kv_heads", u32), ("head_dim", u32),
         ("recent_window", u32), ("block_size", u32),
         ("recent_k", vp), ("recent_v", vp), ("old_k", vp), ("q4_v", vp), ("q4_scale", vp),
-        ("seq_map", vp),
+        ("seq_map", vp), ("v_format", u32), ("q4_dm", vp),
     ]
 
 
@@ -103,6 +103,9 @@ def lib() -> C.CDLL:
     sig("orc_ckv_bytes_old_k", sz, C.POINTER(OrcCkv))
     sig("orc_ckv_bytes_q4_v", sz, C.POINTER(OrcCkv))
     sig("orc_ckv_bytes_q4_scale", sz, C.POINTER(OrcCkv))
+    sig("orc_ckv_create_fmt", C.POINTER(OrcCkv), u32, u32, u32, u32, u32, u32, u32)
+    sig("orc_q4g32_quantize_row", None, vp, u32, vp, vp)
+    sig("orc_q4g32_unpack", f32, C.c_uint8, u32, u32)
     sig("orc_q4_quantize_row", None, vp, u32, vp, vp)
     sig("orc_q4_unpack", f32, C.c_uint8, u32, f32)
     sig("orc_ckv_append_rope_k_at", C.c_int, C.POINTER(OrcCkv), u32, u32, vp, vp, f32, f32, u32)
@@ -256,9 +259,11 @@ def attention_batched(K, V, max_seq_len, kv_heads, head_dim, seq_ids, seq_lens, 
 class CompressedKV:
     """fp16-K / q4-V compressed cache model (one object = all sequences)."""
 
-    def __init__(self, max_seq_len, max_batch, kv_heads, head_dim, recent_window, block_size):
-        self.p = lib().orc_ckv_create(max_seq_len, max_batch, kv_heads, head_dim, recent_window, block_size)
+    def __init__(self, max_seq_len, max_batch, kv_heads, head_dim, recent_window, block_size, v_format=0):
+        """v_format 0: the reference's q4 V (one f32 scale per token and head); 1: groups of 32, f16 scale + f16 min."""
+        self.p = lib().orc_ckv_create_fmt(max_seq_len, max_batch, kv_heads, head_dim, recent_window, block_size, v_format)
         assert self.p, "orc_ckv_create failed"
+        self.v_format = v_format
         self.max_seq_len, self.max_batch = max_seq_len, max_batch
         self.kv_heads, self.head_dim = kv_heads, head_dim
         self.recent_window, self.block_size = recent_window, block_size
@@ -295,6 +300,10 @@ class CompressedKV:
         return self._view("q4_scale", np.float32, (self.max_batch, self.max_seq_len, self.kv_heads))
 
     @property
+    def q4_dm(self):
+        return self._view("q4_dm", np.uint32, (self.max_batch, self.max_seq_len, self.kv_heads, self.head_dim // 32))
+
+    @property
     def seq_map(self):
         return self._view("seq_map", np.uint32, (self.max_batch,))
 
@@ -316,12 +325,17 @@ class CompressedKV:
             self.old_k[seq, :old_len] = k_f16_bits[:old_len]
             packed = np.empty(self.head_dim // 2, dtype=np.uint8)
             sc = np.empty(1, dtype=np.float32)
+            dm = np.empty(self.head_dim // 32, dtype=np.uint32)
             for t in range(old_len):
                 for h in range(self.kv_heads):
                     row = np.ascontiguousarray(v_f16_bits[t, h])
-                    lib().orc_q4_quantize_row(ptr(row), self.head_dim, ptr(packed), ptr(sc))
+                    if self.v_format:
+                        lib().orc_q4g32_quantize_row(ptr(row), self.head_dim, ptr(packed), ptr(dm))
+                        self.q4_dm[seq, t, h] = dm
+                    else:
+                        lib().orc_q4_quantize_row(ptr(row), self.head_dim, ptr(packed), ptr(sc))
+                        self.q4_scale[seq, t, h] = sc[0]
                     self.q4_v[seq, t, h] = packed
-                    self.q4_scale[seq, t, h] = sc[0]
         for t in range(old_len, L):
             self.recent_k[seq, t % W] = k_f16_bits[t]
             self.recent_v[seq, t % W] = v_f16_bits[t]

@@ -73,6 +73,67 @@ def test_compressed_append_evict_bit_exact(dev, orc, hd):
     dev.call("m40llm_kvcache_append_token_f32_rope_k_compressed_at_layout_async", dense.h, 0, dk.ptr, dv.ptr, 0, 1e4, 1.0, 0, expect=-2)
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+def test_group32_v_format_append_evict_and_bulk_fill_bit_exact(dev, orc, hd):
+    """Old-store format 3 (V 4-bit in groups of 32 under an f16 scale and an f16 minimum): evictions and bulk fill write
+    the oracle's bytes -- nibbles, scale | min words, K rows -- including constant groups (scale 0) and a zero row."""
+    rng = np.random.default_rng(300 + hd)
+    kvh, W, bs, L, S = 2, 4, 4, 13, 16
+    G = hd // 32
+    fmt = dict(recent_window=W, block_size=bs, top_blocks=3, exact_old_backing=3)
+    kv = m40.KVCache(dev.ctx, S, 2, kvh, hd, fmt)
+    c = orc.CompressedKV(S, 2, kvh, hd, W, bs, v_format=1)
+    for p in range(L):
+        k = rng.standard_normal(kvh * hd).astype(np.float32); v = (3.0 * rng.standard_normal(kvh * hd)).astype(np.float32)
+        if p == 2:
+            v[:hd] = 0.0                       # all-zero row: scale 0, every nibble 0, value = min = 0
+        if p == 3:
+            v[32:64] = 1.25                    # one constant group
+        if p == 4:
+            v[:32] = np.linspace(-2.0, 1.75, 32)   # a group on an exact grid
+        dk, dv = dev.up(k), dev.up(v)
+        dev.call("m40llm_kvcache_append_token_f32_rope_k_at_layout_async", kv.h, 1, dk.ptr, dv.ptr, p, 0, 1e4, 0.0, 0)
+        assert c.append(1, p, k, v, 1e4, 0.0, 0) == 0
+
+    def state(cache):
+        B = cache.max_batch
+        return dict(old_k=cache.read_raw(0, np.uint16, (B, S, kvh, hd)), q4_v=cache.read_raw(1, np.uint8, (B, S, kvh, hd // 2)),
+                    q4_dm=cache.read_raw(2, np.uint32, (B, S, kvh, G)), recent_v=cache.read_raw(4, np.uint16, (B, W, kvh, hd)),
+                    seq_map=cache.read_raw(5, np.uint32, (B,)))
+    got = state(kv)
+    assert np.array_equal(got["old_k"][1], c.old_k[1]) and np.array_equal(got["q4_v"][1], c.q4_v[1])
+    assert np.array_equal(got["q4_dm"][1], c.q4_dm[1]) and np.array_equal(got["recent_v"][1], c.recent_v[1])
+    assert got["seq_map"][1] == L and not got["q4_v"][0].any() and not got["q4_dm"][0].any()
+    # bytes per (token, kv head): hd / 2 nibble bytes + 4 per group = 80 at head_dim 128 (68 in the reference's format)
+    assert hd // 2 + 4 * G == (80 if hd == 128 else 40)
+    # bulk fill = the same rows appended in order = the oracle's bulk fill
+    L2 = 11
+    k16 = f16bits(rng.standard_normal((L2, kvh, hd))); v16 = f16bits(2.0 * rng.standard_normal((L2, kvh, hd)))
+    a = m40.KVCache(dev.ctx, S, 1, kvh, hd, fmt)
+    dk, dv = dev.up(k16), dev.up(v16)
+    dev.call("m40llm_ext_kvcache_bulk_fill_f16", a.h, 0, dk.ptr, dv.ptr, L2)
+    c2 = orc.CompressedKV(S, 1, kvh, hd, W, bs, v_format=1); c2.bulk_fill(0, k16, v16)
+    ga = state(a)
+    assert np.array_equal(ga["old_k"][0], c2.old_k[0]) and np.array_equal(ga["q4_v"][0], c2.q4_v[0])
+    assert np.array_equal(ga["q4_dm"][0], c2.q4_dm[0]) and np.array_equal(ga["recent_v"][0], c2.recent_v[0])
+    dev.call("m40llm_kvcache_reset", a.h)
+    assert not state(a)["q4_dm"].any()
+
+
+@pytest.mark.parametrize("qh,kvh,hd,L,W,bs,top", [
+    (4, 2, 128, 16, 4, 4, 3),
+    (8, 2, 64, 300, 32, 16, 4),
+    (6, 2, 128, 777, 100, 48, 5),
+    (32, 8, 128, 4096, 512, 64, 64),
+    (32, 8, 128, 32768, 512, 64, 64),      # BASELINE config 5 as written: V in groups of 32 with scale and minimum
+])
+def test_block_select_group32_v_format_vs_oracle(dev, orc, qh, kvh, hd, L, W, bs, top):
+    r = _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, seed=7, backing=3)
+    assert np.array_equal(r["cnt"], r["wcnt"])
+    assert np.array_equal(r["sel"], r["wsel"])            # the selection reads K only: same ids as the reference order
+    close(r["got"], r["want"])                            # 1e-3 relative / 1e-4 absolute
+
+
 def test_bulk_fill_equals_ordered_appends(dev, orc):
     rng = np.random.default_rng(2)
     kvh, hd, W, bs, S = 2, 64, 8, 4, 64
@@ -96,15 +157,15 @@ def test_bulk_fill_equals_ordered_appends(dev, orc):
             assert np.array_equal(ga[name], wo[name]), (L, name)
 
 
-def _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, S=None, seed=0, scale_k=1.0):
+def _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, S=None, seed=0, scale_k=1.0, backing=2):
     rng = np.random.default_rng(seed)
     S = S or L
     k16 = f16bits(rng.standard_normal((L, kvh, hd)) * scale_k); v16 = f16bits(rng.standard_normal((L, kvh, hd)))
     q = rng.standard_normal((qh, hd)).astype(np.float32)
-    kv = m40.KVCache(dev.ctx, S, 1, kvh, hd, dict(recent_window=W, block_size=bs, top_blocks=top))
+    kv = m40.KVCache(dev.ctx, S, 1, kvh, hd, dict(recent_window=W, block_size=bs, top_blocks=top, exact_old_backing=backing))
     dk, dv = dev.up(k16), dev.up(v16)
     dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, 0, dk.ptr, dv.ptr, L)
-    c = orc.CompressedKV(S, 1, kvh, hd, W, bs)
+    c = orc.CompressedKV(S, 1, kvh, hd, W, bs, v_format=1 if backing == 3 else 0)
     c.bulk_fill(0, k16, v16)
     dq, out = dev.up(q), dev.zeros(qh * hd * 4)
     dev.call("m40llm_attention_last_token_f32_gqa_block_select_exact_fp16_k_q4_v_old_direct_async",

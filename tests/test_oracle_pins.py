@@ -430,6 +430,109 @@ def test_block_select_all_blocks_equals_dense_and_partial_fixture(orc):
     assert c.attention(0, q, qh, L, 65)[0] == -6 and c.attention(0, q, qh, L, 0)[0] == -6
 
 
+# ---- old V in groups of 32 with an f16 scale and an f16 minimum (the benchmark configuration's V format; the reference
+# has none, so the definition in oracle.c is the contract and these are its pins)
+def _brute_q4g32(v_f16):
+    """float64 / numpy restatement: per group d = f16((max - min) / 15), m = f16(min), q = rint((v - m) / d) in 0..15."""
+    v = v_f16.astype(np.float32).reshape(-1, 32)
+    mn, mx = v.min(axis=1), v.max(axis=1)
+    d16 = ((mx - mn) / np.float32(15)).astype(np.float16); m16 = mn.astype(np.float16)
+    d, m = d16.astype(np.float32), m16.astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(d[:, None] > 0, np.clip(np.rint(((v - m[:, None]) / d[:, None]).astype(np.float32)), 0, 15), 0).astype(np.uint8)
+    q = q.reshape(-1)
+    packed = (q[0::2] | (q[1::2] << 4)).astype(np.uint8)
+    dm = d16.view(np.uint16).astype(np.uint32) | (m16.view(np.uint16).astype(np.uint32) << 16)
+    return packed, dm, q, d, m
+
+
+def _q4g32(orc, v_f16):
+    hd = v_f16.size
+    packed = np.zeros(hd // 2, dtype=np.uint8); dm = np.zeros(hd // 32, dtype=np.uint32)
+    orc.lib().orc_q4g32_quantize_row(orc.ptr(np.ascontiguousarray(v_f16.view(np.uint16))), hd, orc.ptr(packed), orc.ptr(dm))
+    deq = np.array([orc.lib().orc_q4g32_unpack(int(packed[i // 2]), i & 1, int(dm[i // 32])) for i in range(hd)], dtype=np.float32)
+    return packed, dm, deq
+
+
+def test_q4_group32_closed_forms(orc):
+    hd = 128
+    # (1) values on an exact grid min + k * step (min, step and 15 * step exact in f16): the round trip is exact, the
+    # nibble is k, even dimensions sit in the low nibble, the word is bits(step) | bits(min) << 16
+    ks = np.tile(np.array([0, 15, 3, 12, 7, 8, 1, 14, 5, 10, 2, 13, 6, 9, 4, 11] * 2), hd // 32)
+    v = (np.float32(-2.0) + np.float32(0.25) * ks).astype(np.float16)
+    packed, dm, deq = _q4g32(orc, v)
+    assert np.array_equal(deq, v.astype(np.float32))
+    assert np.array_equal(packed, (ks[0::2] | (ks[1::2] << 4)).astype(np.uint8))
+    want_dm = int(np.float16(0.25).view(np.uint16)) | (int(np.float16(-2.0).view(np.uint16)) << 16)
+    assert all(int(w) == want_dm for w in dm)
+    # (2) a constant group: scale 0, every nibble 0, every value the constant itself; an all-zero row likewise
+    v = np.full(hd, np.float16(1.25)); v[32:64] = np.float16(-0.375); v[64:] = 0
+    packed, dm, deq = _q4g32(orc, v)
+    assert not packed.any() and np.array_equal(deq, v.astype(np.float32))
+    assert [int(w) & 0xffff for w in dm] == [0, 0, 0, 0]
+    # (3) the two ends of a group map to nibbles 0 and 15, and every value is within half a step (plus the rounding
+    # of the stored minimum and scale) of what went in
+    rng = np.random.default_rng(23)
+    for trial in range(40):
+        v = (rng.standard_normal(hd) * rng.uniform(0.01, 30.0)).astype(np.float16)
+        packed, dm, deq = _q4g32(orc, v)
+        wp, wdm, q, d, m = _brute_q4g32(v)
+        assert np.array_equal(packed, wp) and np.array_equal(dm, wdm)            # independent restatement, same bytes
+        vf = v.astype(np.float32).reshape(-1, 32); qg = q.reshape(-1, 32)
+        for g in range(hd // 32):
+            assert qg[g, vf[g].argmin()] == 0 and qg[g, vf[g].argmax()] >= 14
+            bound = 0.5 * d[g] * (1 + 2.0 ** -9) + abs(m[g] - vf[g].min()) + 15 * abs(d[g] - (vf[g].max() - vf[g].min()) / 15) + 1e-7
+            assert np.abs(deq.reshape(-1, 32)[g] - vf[g]).max() <= bound
+        # value = fmaf(q, d, m): one rounding of the exact q * d + m
+        exact = q.astype(np.float64) * np.repeat(d, 32).astype(np.float64) + np.repeat(m, 32).astype(np.float64)
+        assert np.array_equal(deq, exact.astype(np.float32))
+
+
+def test_compressed_cache_group32_bytes_appends_and_attention(orc):
+    rng = np.random.default_rng(29)
+    qh, kvh, hd, L, W, bs = 4, 2, 128, 24, 4, 4
+    c = orc.CompressedKV(32, 1, kvh, hd, W, bs, v_format=1)
+    # 16 B of scale | min words per (token, head) beside 64 B of nibbles: 80 B against the reference format's 68
+    assert c.bytes() == (32 * kvh * hd * 2, 32 * kvh * hd // 2, 32 * kvh * (hd // 32) * 4)
+    k = rng.standard_normal((L, kvh, hd)).astype(np.float16)
+    v = (2.0 * rng.standard_normal((L, kvh, hd))).astype(np.float16)
+    for p in range(L):
+        assert c.append(0, p, k[p].astype(np.float32).reshape(-1), v[p].astype(np.float32).reshape(-1), 1e4, 0.0, 0) == 0
+    for t in range(L - W):
+        for h in range(kvh):
+            wp, wdm, _, _, _ = _brute_q4g32(v[t, h])
+            assert np.array_equal(c.q4_v[0, t, h], wp) and np.array_equal(c.q4_dm[0, t, h], wdm)
+    c2 = orc.CompressedKV(32, 1, kvh, hd, W, bs, v_format=1)
+    c2.bulk_fill(0, k.view(np.uint16), v.view(np.uint16))
+    for name in ("old_k", "q4_v", "q4_dm", "recent_k", "recent_v", "seq_map"):
+        assert np.array_equal(getattr(c, name), getattr(c2, name)), name
+    # attention over everything (top >= old blocks) = float64 softmax over the dequantised V
+    q = rng.standard_normal((qh, hd)).astype(np.float32)
+    rc, out, sel, cnt = c.attention(0, q, qh, L, 64, score_order=0)
+    assert rc == 0 and list(cnt) == [5] * qh
+    vq = v.astype(np.float64).copy()
+    for t in range(L - W):
+        for h in range(kvh):
+            _, _, qn, d, m = _brute_q4g32(v[t, h])
+            vq[t, h] = (qn.astype(np.float64) * np.repeat(d, 32) + np.repeat(m, 32)).astype(np.float32)
+    for h in range(qh):
+        kvhh = h // (qh // kvh)
+        s = (k[:, kvhh].astype(np.float64) @ q[h].astype(np.float64)) * 0.08838834764831845
+        p = np.exp(s - s.max()); p /= p.sum()
+        assert np.allclose(out[h * hd:(h + 1) * hd], p @ vq[:, kvhh], rtol=1e-4, atol=1e-5)
+    # V rows that the format holds exactly: the compressed cache and a dense f16 cache give the same attention
+    vg = (np.float32(-1.0) + np.float32(0.125) * rng.integers(0, 16, size=(L, kvh, hd))).astype(np.float16)
+    vg[:, :, 0::32] = np.float16(-1.0); vg[:, :, 1::32] = np.float16(0.875)          # every group spans the whole grid
+    c3 = orc.CompressedKV(32, 1, kvh, hd, W, bs, v_format=1)
+    c3.bulk_fill(0, k.view(np.uint16), vg.view(np.uint16))
+    rc, out3, sel3, _ = c3.attention(0, q, qh, L, 3, score_order=0)
+    K = np.zeros((1, 32, kvh, hd), dtype=np.uint16); V = np.zeros_like(K)
+    K[0, :L] = k.view(np.uint16); V[0, :L] = vg.view(np.uint16)
+    rc2, outd, seld, _ = orc.dense_block_select(K, V, 32, kvh, hd, 0, q, qh, L, W, bs, 3, score_order=0)
+    assert rc == 0 and rc2 == 0 and np.array_equal(sel3, seld)
+    assert np.allclose(out3, outd, rtol=1e-6, atol=1e-7)
+
+
 def test_dense_backed_block_select_matches_dense_when_all_selected(orc):
     # property of tests/attention_parity_cuda_grid.rs:182-486
     rng = np.random.default_rng(37)
