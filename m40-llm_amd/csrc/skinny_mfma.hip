@@ -132,21 +132,28 @@ __global__ __launch_bounds__(kThreads, 2) void skinny_mfma_kernel(SkinnyArgs p) 
         return x;
     };
 
-    float fa[EPT], fb[EPT];    // this thread's activations of a step (and their SwiGLU partner or norm weights)
+    float fa[EPT];             // this thread's activations of a step
+    uint4 fbraw[EPT / 4];      // and their SwiGLU partner or norm weights, as loaded: f32 values, or (f16 norm weights)
+                               // the eight weights of elements 8j..8j+7 in entries 2j and 2j+1 alike
     constexpr int NW = FMT == 0 ? 8 : 5;
     uint4 rb[2][NW];           // weights of two steps in flight.  f16: eight 16-byte loads; q8_0: five tile pieces
+    // One batch of 16-byte loads whatever the second operand is: a branch around loads makes the compiler wait for
+    // every load in flight at its join -- here that was a full wait right behind each step's barrier, which drained the
+    // weight requests of the next two steps.  f16 norm weights are 16 bytes per eight elements, requested twice.
     auto issue_a = [&](int kt) {
         load_f32(a_ptr + (size_t)kt * kTileK, fa);
-        if (norm16) {
+        const char* src = norm16 ? reinterpret_cast<const char*>(nw16 + (size_t)kt * kTileK)
+                                 : reinterpret_cast<const char*>(b_ptr + (size_t)kt * kTileK);
 #pragma unroll
-            for (int e = 0; e < EPT; e += 4) {
-                const uint2 w = *reinterpret_cast<const uint2*>(nw16 + (size_t)kt * kTileK + e);
-                fb[e / 2] = __uint_as_float(w.x); fb[e / 2 + 1] = __uint_as_float(w.y);   // raw f16 pairs
-            }
-        } else {
-            load_f32(b_ptr + (size_t)kt * kTileK, fb);
-        }
+        for (int i = 0; i < EPT / 4; ++i)
+            fbraw[i] = *reinterpret_cast<const uint4*>(src + (norm16 ? 16 * (i / 2) : 16 * i));
     };
+    auto fb_word = [&](int i, int w) -> uint32_t {
+        const uint4 v = fbraw[i];
+        return w == 0 ? v.x : (w == 1 ? v.y : (w == 2 ? v.z : v.w));
+    };
+    auto fb_f32 = [&](int e) { return __uint_as_float(fb_word(e / 4, e % 4)); };
+    auto fb_f16 = [&](int e) { return m40_h2f((uint16_t)((fb_word(2 * (e / 8), (e % 8) / 2) >> (16 * (e & 1))) & 0xffffu)); };
     // Plain loads, not streaming ones: a lane's 16 bytes are a quarter of a 64-byte run of its column, and the rest
     // of each 128-byte line is asked for by the next instruction -- with the streaming hint the line is fetched again
     // (measured: +4.7 % on the batch-8 step with plain loads).
@@ -199,9 +206,9 @@ __global__ __launch_bounds__(kThreads, 2) void skinny_mfma_kernel(SkinnyArgs p) 
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
             float v = fa[e];
-            if (p.up) v = v / (1.0f + expf(-v)) * fb[e];
-            else if (norm16) v = v * rms * m40_h2f((uint16_t)((__float_as_uint(fb[e / 2]) >> (16 * (e & 1))) & 0xffffu));
-            else if (p.norm_w) v = v * rms * fb[e];
+            if (p.up) v = v / (1.0f + expf(-v)) * fb_f32(e);
+            else if (norm16) v = v * rms * fb_f16(e);
+            else if (p.norm_w) v = v * rms * fb_f32(e);
             if (!a_live) v = 0.0f;
             x[e] = v;
             mx = fmaxf(mx, fabsf(v));
