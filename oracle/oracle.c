@@ -549,7 +549,7 @@ float orc_q4_unpack(uint8_t packed, uint32_t lane, float scale) {
     return (float)sv * scale;
 }
 
-/* 4-bit V in groups of 32 with an f16 scale and an f16 minimum (the V format BASELINE's compressed-attention
+/* 4-bit V in groups of 32 with an f16 scale and an f16 minimum (the V format the compressed-attention benchmark
  * configuration names; the reference has no such format, so this definition is the contract):
  *   per group: mn, mx = smallest and largest value; d = f16((mx - mn) / 15), m = f16(mn), both then read back as f32;
  *   q = d > 0 ? clamp(lrintf((v - m) / d), 0, 15) : 0;  byte = q_even | q_odd << 4;  word = bits(d) | bits(m) << 16;
