@@ -152,7 +152,7 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
 bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
 int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);
-// q8_0 weights on the int8 matrix instruction (q80_i8.hip): 3 <= M <= 16 rows, K a multiple of 32; A 8-byte aligned
+// q8_0 weights on the int8 matrix instruction (q80_i8.hip): 2 <= M <= 16 rows, K a multiple of 256; A and W 16-byte aligned
 bool m40_q80_i8_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K);
 int m40_launch_q80_i8(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint8_t* W,
                       float* C, int M, int N, int K);

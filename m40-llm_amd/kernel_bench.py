@@ -342,7 +342,7 @@ def bench_q80(b: Bench):
     nset = 6
     sets = [(b.ctx.to_device(gate), b.ctx.to_device(up), b.ctx.to_device(down)) for _ in range(nset)]
     wbytes = gate.nbytes + up.nbytes + down.nbytes
-    for M in (1, 2, 4, 16):
+    for M in (1, 2, 4, 8, 16):
         x = b.ctx.to_device(rng.standard_normal((M, d_model)).astype(np.float32))
         scratch = b.ctx.alloc(2 * M * ffn * 4)
         out = b.ctx.alloc(M * d_model * 4)
@@ -350,7 +350,7 @@ def bench_q80(b: Bench):
         b.time("ffn_swiglu_q80", f"M={M} d_model 4096 ffn 14336", algo,
                lambda i: b.call("m40llm_ext_ffn_swiglu_q80_f32_async", x.ptr, sets[i][0].ptr, sets[i][1].ptr, sets[i][2].ptr,
                                 scratch.ptr, out.ptr, M, d_model, ffn), nset)
-    for M in (1, 2, 4, 16):
+    for M in (1, 2, 4, 8, 16):
         a = b.ctx.to_device(rng.standard_normal((M, d_model)).astype(np.float32))
         c = b.ctx.alloc(M * ffn * 4)
         b.time(f"gemm_f32xq80_gguf M={M}", "N=14336 K=4096", gate.nbytes,

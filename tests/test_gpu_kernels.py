@@ -350,10 +350,11 @@ def q80_ffn_full_size():
     return qmat(14336, 4096), qmat(14336, 4096), qmat(4096, 14336)
 
 
-@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 16])
 def test_q80_ffn_full_size_vs_oracle(dev, orc, q80_ffn_full_size, M):
-    """The fused q8_0 FFN at the full BASELINE config 4 size, batch sizes 1, 4 and 16, against the oracle's sequential
-    f32 sums: 1e-3 relative / 1e-4 absolute on outputs scaled to a unit row maximum."""
+    """The fused q8_0 FFN at the full BASELINE config 4 size, batch sizes 1, 2, 4, 7 and 16, against the oracle's sequential
+    f32 sums: 1e-3 relative / 1e-4 absolute on outputs scaled to a unit row maximum (7 and 16 rows: the two paddings of
+    the three-plane int8 form)."""
     wg, wu, wd = q80_ffn_full_size
     d_model, ffn = 4096, 14336
     x = np.random.default_rng(40 + M).standard_normal((M, d_model)).astype(np.float32)
@@ -369,9 +370,11 @@ def test_q80_ffn_full_size_vs_oracle(dev, orc, q80_ffn_full_size, M):
 
 @pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 1000, 768), (8, 4096, 2048), (9, 520, 1280), (16, 2048, 4096),
                                    (20, 333, 256), (2, 64, 96), (1, 1000, 4096), (2, 777, 8192), (1, 513, 14336),
-                                   (2, 260, 11008), (1, 40, 16384), (2, 3, 64)])
+                                   (2, 260, 11008), (1, 40, 16384), (2, 3, 64), (8, 6200, 512), (12, 24600, 256),
+                                   (5, 8192, 1024), (4, 12300, 512)])
 def test_q80_gemm_shapes_vs_oracle(dev, orc, M, N, K):
-    """MFMA path (3 rows and more, K % 256 == 0; column tails, split K, more than 16 rows), the register-resident
+    """MFMA path (3 rows and more, K % 256 == 0; column tails, split K, more than 16 rows; 5 rows and more with 6144
+    columns and more: two column tiles per wave, split K and, from ~24 500 columns, whole K), the register-resident
     GEMV of one and two rows (K % 64 == 0, one, two and four K-parts per column) and the simple path (K = 96)."""
     rng = np.random.default_rng(M * 7919 + N + K)
     d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
