@@ -282,7 +282,8 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_ker
                 const i32x4 r3 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2, B, z, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float sum = fmaf((float)(r1[r] * 128 + r2[r]), 128.0f, (float)r3[r]);
+                    // |r1|, |r2|, |r3| <= 32 * 64 * 127 < 2^18: the recombination fits 32 bits exactly
+                    const float sum = (float)((r1[r] * 128 + r2[r]) * 128 + r3[r]);
                     acc[t][r] = fmaf(sa[r] * dw, sum, acc[t][r]);
                 }
             }
@@ -440,7 +441,7 @@ static void launch_gemm0(hipStream_t stream, const Q80I8Args& a) {
     }
     // three-plane form: two column tiles per wave where the grid still covers the chip with them (measured at 16
     // rows: N = 14336, K = 4096 34.4 -> 22.8 us); else, with K long enough, eight waves share a tile's K (N = 4096,
-    // K = 14336: 24.4 -> 23.5 us)
+    // K = 14336: 24.4 -> 23.5 us; two tiles per wave there would leave 128 workgroups: 31.5 us)
     const int pairs = (tiles + 1) / 2;
     if (whole_k) {
         if ((pairs + 3) / 4 >= 192) q80i8_gemm_kernel<0, 1, false, 2><<<(pairs + 3) / 4, 256, 0, stream>>>(a);
