@@ -408,7 +408,8 @@ int m40llm_ext_fused_norm_gemv_f32xf16_async(M40llmCudaContext* ctx, const void*
                                              uint32_t norm_weight_dtype, float eps, const void* d_w_f16,
                                              void* d_out_f32, int N, int K, void* d_block_top2,
                                              uint32_t top2_capacity, uint32_t* out_n_blocks);
-/* attention with the length taken from the device: seq_len = *position_dev + 1 <= max_len_hint */
+/* attention with the length taken from the device: seq_len = *position_dev + 1 <= max_len_hint (the launch is sized
+ * for max_len_hint tokens: with a longer sequence nothing is written) */
 int m40llm_ext_attention_last_token_f32_gqa_position_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
                                                                uint32_t seq_id, const void* q_dev_f32,
                                                                uint32_t q_heads, const uint32_t* position_dev,
@@ -446,7 +447,8 @@ int m40llm_ext_batched_norm_qkv_rope_append_async(
     const void* d_wk_f16, const void* d_wv_f16, const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32,
     uint32_t d_model, uint32_t q_heads, float freq_base, float freq_scale, uint32_t rope_layout, void* d_q_out_f32);
 /*   attention of every row over seq_lens_dev[row] + len_bias tokens (no host-side validation: rows with an id or
- *   length out of range are skipped); max_len_hint >= every row's length */
+ *   length out of range are skipped); max_len_hint >= every row's length: the launch is sized for it, and a row
+ *   that is longer is skipped like one out of range */
 int m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
                                                                    const uint32_t* seq_ids_dev,
                                                                    const uint32_t* seq_lens_dev, uint32_t len_bias,

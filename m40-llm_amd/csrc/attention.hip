@@ -61,6 +61,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_partial_kernel(AttnParam
     if (len == 0 || len > p.max_seq_len) return;
     if (p.max_batch != 0 && seq_id >= p.max_batch) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    if (len - t0 > p.span_limit) return;      // longer than the launch was sized for: the row is skipped
     const uint32_t cbeg = t0 + blockIdx.y * p.chunk;
     if (cbeg >= len) return;
     const uint32_t cend = cbeg + p.chunk < len ? cbeg + p.chunk : len;
@@ -230,6 +231,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(AttnParams p) {
     if (len == 0 || len > p.max_seq_len) return;
     if (p.max_batch != 0 && p.seq_ids_dev && sid >= p.max_batch) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    if (len - t0 > p.span_limit) return;      // longer than the launch was sized for: the row is skipped
     const uint32_t n = (len - t0 + p.chunk - 1) / p.chunk;
     float m = -INFINITY, num = 0.0f, den = 0.0f;
     auto fold = [&](float mc, float lc, float vc) {
@@ -277,6 +279,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p, uint32_t
     const uint32_t len = p.seq_lens_dev ? p.seq_lens_dev[b] + p.len_bias : p.seq_len;
     if (len == 0 || len > p.max_seq_len) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    if (len - t0 > p.span_limit) return;      // longer than the launch was sized for: the row is skipped
     const uint32_t kvh = qh / (p.q_heads / p.kv_heads);
     const size_t ept = (size_t)p.kv_heads * head_dim;
     const float inv_sqrt = m40_inv_sqrt_head_dim(head_dim);
@@ -408,6 +411,7 @@ int m40_launch_dense_attention(M40llmCudaContext* ctx, hipStream_t stream, uint3
     uint32_t span = a.max_len_hint;
     if (a.window != 0 && span > a.window) span = a.window;
     if (span == 0) span = 1;
+    p.span_limit = span;
 
     if ((a.head_dim == 64 || a.head_dim == 128) && m40_aligned16(a.Q) && m40_aligned16(a.K) && m40_aligned16(a.V)) {
         M40StreamScratch& scr = ctx->scratch[stream_kind];

@@ -51,6 +51,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_mfma_kernel(AttnParams p) {
     if (len == 0 || len > p.max_seq_len) return;
     if (p.max_batch != 0 && seq_id >= p.max_batch) return;
     const uint32_t t0 = (p.window != 0 && len > p.window) ? len - p.window : 0;
+    if (len - t0 > p.span_limit) return;      // longer than the launch was sized for: the row is skipped
     const uint32_t cbeg = t0 + blockIdx.y * p.chunk;
     if (cbeg >= len) return;
     const uint32_t cend = cbeg + p.chunk < len ? cbeg + p.chunk : len;

@@ -17,6 +17,8 @@ struct AttnParams {
     uint32_t subgroups;           // q-head subgroups per kv head
     uint32_t len_bias;            // added to a device-side length (position -> length)
     uint32_t max_batch;           // device-side sequence ids at or above this are skipped (0 = not checked)
+    uint32_t span_limit;          // tokens a row may attend (the length bound the grid and chunking were sized for): rows
+                                  // whose device-side length asks for more are skipped
 };
 
 // attention_mfma.hip: chunks of `p.chunk` tokens (a multiple of 128), G <= 8 q heads per workgroup

@@ -552,6 +552,49 @@ def test_attention_batched_head128_qwen_shape(dev, orc):
     close(out.download(np.float32, q.shape), orc.attention_batched(Kc, Vc, maxL, kvh, hd, ids, lens, q, qh))
 
 
+def test_attention_device_lengths_and_skipped_rows(dev, orc):
+    """The entry points that read lengths (and ids) on the device: rows inside the bound equal the oracle; a row whose
+    length exceeds max_len_hint, a zero-length row and a row with an id outside the cache are skipped (their output rows
+    keep what was there), for the chunked (hint > 512) and the single-chunk launch shapes."""
+    rng = np.random.default_rng(21)
+    qh, kvh, hd, S, maxL = 8, 2, 128, 6, 1536
+    kv = m40.KVCache(dev.ctx, maxL, S, kvh, hd)
+    Kc = f16bits(rng.standard_normal((S, maxL, kvh, hd))); Vc = f16bits(rng.standard_normal((S, maxL, kvh, hd)))
+    for s_ in range(S):
+        dev.fill_dense(kv, s_, Kc[s_], Vc[s_])
+    for hint, lens in ((1024, [300, 700, 1200, 0, 1024, 50]), (400, [300, 399, 401, 17, 400, 1])):
+        lens = np.asarray(lens, dtype=np.uint32)
+        ids = np.asarray([3, 0, 1, 2, 5, 9], dtype=np.uint32)          # id 9 does not exist
+        B = len(lens)
+        q = rng.standard_normal((B, qh * hd)).astype(np.float32)
+        sentinel = np.full(q.shape, 7.25, dtype=np.float32)
+        dq, out, dids, dlens = dev.up(q), dev.up(sentinel), dev.up(ids), dev.up(lens)
+        dev.call("m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async", kv.h, dids.ptr, dlens.ptr, 0, B, hint,
+                 dq.ptr, qh, out.ptr)
+        dev.sync()
+        got = out.download(np.float32, q.shape)
+        live = [b for b in range(B) if 0 < lens[b] <= hint and ids[b] < S]
+        assert 3 <= len(live) < B
+        want = orc.attention_batched(Kc, Vc, maxL, kvh, hd, ids[live], lens[live], q[live], qh)
+        close(got[live], want)
+        for b in range(B):
+            if b not in live:
+                assert np.array_equal(got[b], sentinel[b]), b
+    # single sequence, length = *position_dev + 1
+    q = rng.standard_normal((1, qh * hd)).astype(np.float32)
+    for pos, hint, skipped in ((699, 1024, False), (699, 700, False), (700, 700, True), (99, 128, False), (128, 128, True)):
+        sentinel = np.full(q.shape, -3.5, dtype=np.float32)
+        dq, out, dpos = dev.up(q), dev.up(sentinel), dev.up(np.asarray([pos], dtype=np.uint32))
+        dev.call("m40llm_ext_attention_last_token_f32_gqa_position_dev_async", kv.h, 4, dq.ptr, qh, dpos.ptr, hint, out.ptr)
+        dev.sync()
+        got = out.download(np.float32, q.shape)
+        if skipped:
+            assert np.array_equal(got, sentinel)
+        else:
+            close(got, orc.attention_batched(Kc, Vc, maxL, kvh, hd, np.asarray([4], np.uint32), np.asarray([pos + 1], np.uint32), q, qh))
+    dev.call("m40llm_ext_attention_last_token_f32_gqa_position_dev_async", kv.h, 4, dq.ptr, qh, dpos.ptr, maxL + 1, out.ptr, expect=-3)
+
+
 def test_argmax_extension(dev, orc):
     rng = np.random.default_rng(9)
     rows, n = 8, 151936
