@@ -142,7 +142,7 @@ __device__ __forceinline__ void q80i8_unrolled(std::integer_sequence<int, I...>,
 // WAVES / KSPLIT column groups per workgroup, wave = group * KSPLIT + K part.
 template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4>
 __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_kernel(Q80I8Args p) {
-    static_assert(T == 1 || (T == 2 && !STACK), "two column tiles per wave exist in the three-plane form only");
+    static_assert(T == 1 || T == 2, "one or two column tiles per wave");
     constexpr int kWaves = WAVES;  // (stacked form, eight waves splitting K, measured for the down projection: 21.4 against 20.5 us)
     constexpr int kThreads = 64 * kWaves;
     constexpr int kGroups = kWaves / KSPLIT;
@@ -204,7 +204,8 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_ker
     const uint32_t e_off = (uint32_t)(12 * 1024 + (lane & 3) * 64 + g * 16);
     constexpr int kStepBytes = STACK ? kStackStepBytes : kPlaneStepBytes;
     constexpr int kPlanes = STACK ? 4 : 12;
-    constexpr int D = STACK ? 4 : 2;          // steps in flight (the three-plane form has no registers for more)
+    constexpr int D = STACK ? (T == 1 ? 4 : 2) : 2;   // steps in flight (two 32-column steps are as many bytes as four of 16
+                                                 // columns; the three-plane form has no registers for more)
 
     WPiece wr[D][kWLoads];
     Q80I8Acts<STACK> acts[D];
@@ -258,12 +259,16 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_ker
         const i32x4 z = {0, 0, 0, 0};
         auto half = [](const uint4& two) { return __builtin_bit_cast(long, (b & 1) ? make_uint2(two.z, two.w) : make_uint2(two.x, two.y)); };
         if constexpr (STACK) {
-            const float dw = w[0].dw;
-            const i32x4 rr = __builtin_amdgcn_mfma_i32_16x16x32_i8(half(act.pl[b >> 1]), w[0].B, z, 0, 0, 0);
+            float sa[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float sa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, act.sv), 4 * b + r));
-                acc[0][r] = fmaf(sa * dw, (float)rr[r], acc[0][r]);
+            for (int r = 0; r < 4; ++r)
+                sa[r] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, act.sv), 4 * b + r));
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const float dw = w[t].dw;
+                const i32x4 rr = __builtin_amdgcn_mfma_i32_16x16x32_i8(half(act.pl[b >> 1]), w[t].B, z, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][r] = fmaf(sa[r] * dw, (float)rr[r], acc[t][r]);
             }
         } else {
             const long a0 = half(act.pl[(b >> 1) * 3]), a1 = half(act.pl[(b >> 1) * 3 + 1]), a2 = half(act.pl[(b >> 1) * 3 + 2]);
@@ -308,7 +313,7 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_ker
             issue_w(wr[i], s0 + i);
             __builtin_amdgcn_sched_barrier(0);
         }
-        auto step = [&](auto set_c, int s) {
+        auto step = [&](auto set_c, int s) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
             // weights of this step -> the wave's LDS tile (waits for them and for everything older: this step's
             // activations; the younger steps stay in flight)
@@ -340,28 +345,25 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_ker
             issue_w(wr[SET], s + D);
             __builtin_amdgcn_sched_barrier(0);
         };
-        using std::integral_constant;
+        // whole turns of the ring, then the steps that are left (each in its own register set)
         int s = s0;
-        for (; s + D <= s1; s += D) {
-            step(integral_constant<int, 0>(), s);
-            step(integral_constant<int, 1>(), s + 1);
-            if (D == 4) {
-                step(integral_constant<int, D - 2>(), s + 2);
-                step(integral_constant<int, D - 1>(), s + 3);
-            }
-        }
-        if (s < s1) step(integral_constant<int, 0>(), s);
-        if (D == 4 && s + 1 < s1) step(integral_constant<int, 1>(), s + 1);
-        if (D == 4 && s + 2 < s1) step(integral_constant<int, D - 2>(), s + 2);
+        for (; s + D <= s1; s += D)
+            q80i8_unrolled(std::make_integer_sequence<int, D>(),
+                           [&](auto set_c) __attribute__((always_inline)) { step(set_c, s + decltype(set_c)::value); });
+        q80i8_unrolled(std::make_integer_sequence<int, D - 1>(), [&](auto set_c) __attribute__((always_inline)) {
+            if (s + decltype(set_c)::value < s1) step(set_c, s + decltype(set_c)::value);
+        });
     }
 
     if (STACK) {
         // lane (j, g) holds digit g of rows r: the three sums meet in the lanes g = 0
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float d2 = __shfl(acc[0][r], j + 16, 64), d3 = __shfl(acc[0][r], j + 32, 64);
-            acc[0][r] = g == 0 ? fmaf(acc[0][r], 16384.0f, fmaf(d2, 128.0f, d3)) : 0.0f;
-        }
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float d2 = __shfl(acc[t][r], j + 16, 64), d3 = __shfl(acc[t][r], j + 32, 64);
+                acc[t][r] = g == 0 ? fmaf(acc[t][r], 16384.0f, fmaf(d2, 128.0f, d3)) : 0.0f;
+            }
     }
     // lane (j, g) holds rows 4g + r of columns 16 t + j
     if (KSPLIT > 1) {
@@ -435,6 +437,7 @@ static void launch_gemm0(hipStream_t stream, const Q80I8Args& a) {
     // (stacked form, N = 14336, K = 4096: 224 workgroups walking the whole K 16.6 us, 896 splitting it 23.7 us)
     const bool whole_k = tiles >= (a.MP == 0 ? 768 : 1024) || nsteps < 4;
     if (a.MP == 0) {
+        // (N = 14336 as 448 workgroups of two tiles splitting K: 17.5 us against 16.7 us for the 224 walking the whole K)
         if (whole_k) q80i8_gemm_kernel<0, 1, true><<<(tiles + 3) / 4, 256, 0, stream>>>(a);
         else q80i8_gemm_kernel<0, 4, true><<<tiles, 256, 0, stream>>>(a);
         return;
@@ -482,7 +485,10 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     q80i8_pack_kernel<<<d_model >> 5, 256, 0, stream>>>(x, M, MP, d_model, xp);
     Q80I8Args a{};
     a.pack = xp; a.W0 = wg; a.W1 = wu; a.out_pack = hp; a.M = M; a.MP = MP; a.N = ffn; a.K = d_model;
-    if (MP == 0) q80i8_gemm_kernel<1, 1, true><<<ffn / 32, 256, 0, stream>>>(a);
+    // two column tiles per wave where 192 workgroups and more remain: every activation plane fetched is used twice
+    // (stacked form, FFN 14336: 52.9 -> 49.2 us; with three 32-column steps in flight instead of two 50.1 us)
+    if (MP == 0 && ffn % 64 == 0 && ffn / 64 >= 192) q80i8_gemm_kernel<1, 1, true, 2><<<ffn / 64, 256, 0, stream>>>(a);
+    else if (MP == 0) q80i8_gemm_kernel<1, 1, true><<<ffn / 32, 256, 0, stream>>>(a);
     // (a workgroup of two column groups x two K halves, two waves per SIMD instead of one: measured, 64.5 -> 66 us)
     else if (ffn % 64 == 0 && ffn / 64 >= 192) q80i8_gemm_kernel<1, 1, false, 2><<<ffn / 64, 256, 0, stream>>>(a);
     else q80i8_gemm_kernel<1, 1, false><<<ffn / 32, 256, 0, stream>>>(a);
