@@ -368,6 +368,30 @@ def test_q80_ffn_full_size_vs_oracle(dev, orc, q80_ffn_full_size, M):
     close(out.download(np.float32, (M, d_model)) / scale, want / scale, 1e-3, 1e-4)
 
 
+@pytest.mark.parametrize("M,d_model", [(3, 1024), (4, 768), (2, 2048)])
+def test_q80_ffn_wide_hidden_short_k_vs_oracle(dev, orc, M, d_model):
+    """A wide FFN (12288 hidden columns: the launch shape whose workgroups pack the activation rows themselves) over a
+    short K, where some of the packing passes have no block to pack; 768 = 3 steps, 1024 = 4, 2048 = 8."""
+    rng = np.random.default_rng(500 + M)
+    ffn = 12288
+    def qmat(n, k):
+        blob = np.empty((n, k // 32, 34), dtype=np.uint8)
+        blob[:, :, :2] = rng.uniform(0.001, 0.01, size=(n, k // 32)).astype(np.float16).view(np.uint8).reshape(n, k // 32, 2)
+        blob[:, :, 2:] = rng.integers(-127, 128, size=(n, k // 32, 32)).astype(np.int8).view(np.uint8)
+        return blob
+    wg, wu, wd = qmat(ffn, d_model), qmat(ffn, d_model), qmat(d_model, ffn)
+    x = rng.standard_normal((M, d_model)).astype(np.float32)
+    x[M - 1] *= 1e-3
+    dx, dwg, dwu, dwd = dev.up(x), dev.up(wg), dev.up(wu), dev.up(wd)
+    scratch, out = dev.zeros(2 * M * ffn * 4), dev.zeros(M * d_model * 4)
+    dev.call("m40llm_ext_ffn_swiglu_q80_f32_async", dx.ptr, dwg.ptr, dwu.ptr, dwd.ptr, scratch.ptr, out.ptr, M, d_model, ffn)
+    dev.sync()
+    orc.set_threads(8)
+    want = orc.ffn_swiglu_q80(x, wg, wu, wd, M, d_model, ffn)
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    close(out.download(np.float32, (M, d_model)) / scale, want / scale, 1e-3, 1e-4)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 1000, 768), (8, 4096, 2048), (9, 520, 1280), (16, 2048, 4096),
                                    (20, 333, 256), (2, 64, 96), (1, 1000, 4096), (2, 777, 8192), (1, 513, 14336),
                                    (2, 260, 11008), (1, 40, 16384), (2, 3, 64), (8, 6200, 512), (12, 24600, 256),
