@@ -141,7 +141,7 @@ __device__ __forceinline__ void q80i8_unrolled(std::integer_sequence<int, I...>,
 // weights (FFN at 16 rows: 91 -> 75 us with that alone).
 // WAVES / KSPLIT column groups per workgroup, wave = group * KSPLIT + K part.
 template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4>
-__global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void q80i8_gemm_kernel(Q80I8Args p) {
+__global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) {
     static_assert(T == 1 || T == 2, "one or two column tiles per wave");
     constexpr int kWaves = WAVES;  // (stacked form, eight waves splitting K, measured for the down projection: 21.4 against 20.5 us)
     constexpr int kThreads = 64 * kWaves;
