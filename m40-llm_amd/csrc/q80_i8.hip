@@ -97,6 +97,8 @@ struct Q80I8Args {
     const uint8_t* W1;         // MODE 1: up
     float* C;                  // MODE 0: [M][N]
     uint8_t* out_pack;         // MODE 1: packed SwiGLU output (the A operand of the down projection)
+    float* zero;               // MODE 1: cleared by the launch (zero_count floats), or null: the result of a down projection
+    int zero_count;            //         whose two K halves are added into it
     int M, MP, N, K;
 };
 
@@ -140,8 +142,12 @@ __device__ __forceinline__ void q80i8_unrolled(std::integer_sequence<int, I...>,
 // weight tile, and fetching them once per 32 columns instead of once per 16 halves the loads a CU issues beside its
 // weights (FFN at 16 rows: 91 -> 75 us with that alone).
 // WAVES / KSPLIT column groups per workgroup, wave = group * KSPLIT + K part.
-template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4>
+// KHALVES = 2 (MODE 0): two workgroups share a column group, each walks half of K and ADDS its sums into C, which the
+// launch before has cleared: 0 + a + b is the same f32 in either order, so the result does not depend on timing.  A
+// workgroup then needs only half of the activation planes, and twice as many workgroups can own two tiles each.
+template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1>
 __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) {
+    static_assert(KHALVES == 1 || (KHALVES == 2 && MODE == 0), "halves of K are added into a cleared result");
     static_assert(T == 1 || T == 2, "one or two column tiles per wave");
     constexpr int kWaves = WAVES;  // (stacked form, eight waves splitting K, measured for the down projection: 21.4 against 20.5 us)
     constexpr int kThreads = 64 * kWaves;
@@ -168,13 +174,17 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
     const size_t col_stride = (size_t)(p.K >> 5) * 34;
     int n0, s0, s1;
     if (MODE == 0) {
-        n0 = (blockIdx.x * kGroups + group) * kCols;
+        n0 = ((blockIdx.x / KHALVES) * kGroups + group) * kCols;
         if (n0 >= p.N) n0 = (p.N - 1) / kCols * kCols;        // surplus waves repeat the last tile (no early exit: barriers)
     } else {
         n0 = (blockIdx.x * kGroups + group) * 8 * T;
     }
-    s0 = (int)(((long long)kpart * nsteps_all) / KSPLIT);
-    s1 = (int)(((long long)(kpart + 1) * nsteps_all) / KSPLIT);
+    {
+        // the workgroup's share of K (a half, or all of it), split over the K parts of a column group
+        const int kparts = KSPLIT * KHALVES, part = (int)(blockIdx.x % KHALVES) * KSPLIT + kpart;
+        s0 = (int)(((long long)part * nsteps_all) / kparts);
+        s1 = (int)(((long long)(part + 1) * nsteps_all) / kparts);
+    }
     // ---- weight pieces of this lane: piece q of the step tile (17 pieces per column), q = lane + 64 i
     // (MODE 1: B columns 16 t + 0..7 are gate columns n0 + 8 t + 0..7, 16 t + 8..15 the same columns of up; the up
     // matrix is addressed from the gate matrix's base: both lie in one address space)
@@ -385,15 +395,20 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
         }
     }
     if constexpr (MODE == 0) {
-        const bool tile_live = kpart == 0 && (blockIdx.x * kGroups + group) * kCols < p.N;
+        const bool tile_live = kpart == 0 && ((blockIdx.x / KHALVES) * kGroups + group) * kCols < p.N;
 #pragma unroll
         for (int t = 0; t < T; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = 4 * g + r, n = n0 + 16 * t + j;
-                if (tile_live && m < p.M && n < p.N) p.C[(size_t)m * p.N + n] = acc[t][r];
+                if (tile_live && m < p.M && n < p.N) {
+                    if (KHALVES == 1) p.C[(size_t)m * p.N + n] = acc[t][r];
+                    else atomicAdd(&p.C[(size_t)m * p.N + n], acc[t][r]);
+                }
             }
     } else {
+        if (p.zero)
+            for (int i = (int)blockIdx.x * kThreads + tid; i < p.zero_count; i += (int)gridDim.x * kThreads) p.zero[i] = 0.0f;
         // SwiGLU of gate (lanes j < 8) and up (j >= 8, eight lanes on), then the digit pack of the workgroup's blocks
         constexpr int kHidden = kGroups * 8 * T, kHStride = kHidden + 1;
         __shared__ float hbuf[16 * kHStride];          // [16 rows][hidden columns of the workgroup]
@@ -485,6 +500,13 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     q80i8_pack_kernel<<<d_model >> 5, 256, 0, stream>>>(x, M, MP, d_model, xp);
     Q80I8Args a{};
     a.pack = xp; a.W0 = wg; a.W1 = wu; a.out_pack = hp; a.M = M; a.MP = MP; a.N = ffn; a.K = d_model;
+    // down projection as column-tile pairs x two halves of K, added into a result the gate + up launch clears
+    const bool out_apart = reinterpret_cast<const char*>(out) + (size_t)M * d_model * 4 <= reinterpret_cast<const char*>(x) ||
+                           reinterpret_cast<const char*>(x) + (size_t)M * d_model * 4 <= reinterpret_cast<const char*>(out);
+    // (FFN 14336 -> 4096: 49.6 -> 48.1 us at four rows, 64.2 -> 61.0 us at sixteen; with eight waves per workgroup 63.1 us)
+    const int down_pairs = (d_model + 31) / 32;
+    const bool halves = out_apart && 2 * down_pairs >= 192 && 2 * down_pairs <= 1024 && ffn / (32 * kStepBlocks) >= 32;
+    if (halves) { a.zero = out; a.zero_count = M * d_model; }
     // two column tiles per wave where 192 workgroups and more remain: every activation plane fetched is used twice
     // (stacked form, FFN 14336: 52.9 -> 49.2 us; with three 32-column steps in flight instead of two 50.1 us)
     if (MP == 0 && ffn % 64 == 0 && ffn / 64 >= 192) q80i8_gemm_kernel<1, 1, true, 2><<<ffn / 64, 256, 0, stream>>>(a);
@@ -494,6 +516,12 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     else q80i8_gemm_kernel<1, 1, false><<<ffn / 32, 256, 0, stream>>>(a);
     Q80I8Args b{};
     b.pack = hp; b.W0 = wd; b.C = out; b.M = M; b.MP = MP; b.N = d_model; b.K = ffn;
-    launch_gemm0(stream, b);
+    if (halves) {
+        const int pairs = (d_model + 31) / 32;
+        if (MP == 0) q80i8_gemm_kernel<0, 4, true, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(b);
+        else q80i8_gemm_kernel<0, 4, false, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(b);
+    } else {
+        launch_gemm0(stream, b);
+    }
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }

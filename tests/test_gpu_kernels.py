@@ -365,7 +365,17 @@ def test_q80_ffn_full_size_vs_oracle(dev, orc, q80_ffn_full_size, M):
     orc.set_threads(8)
     want = orc.ffn_swiglu_q80(x, wg, wu, wd, M, d_model, ffn)
     scale = np.abs(want).max(axis=1, keepdims=True)
-    close(out.download(np.float32, (M, d_model)) / scale, want / scale, 1e-3, 1e-4)
+    got = out.download(np.float32, (M, d_model))
+    close(got / scale, want / scale, 1e-3, 1e-4)
+    # twice the same call: the same bits (the down projection adds two halves of K into a cleared result: 0 + a + b)
+    dev.call("m40llm_ext_ffn_swiglu_q80_f32_async", dx.ptr, dwg.ptr, dwu.ptr, dwd.ptr, scratch.ptr, out.ptr, M, d_model, ffn)
+    dev.sync()
+    assert np.array_equal(out.download(np.float32, (M, d_model)), got)
+    if M in (4, 16):
+        # result written over the input rows
+        dev.call("m40llm_ext_ffn_swiglu_q80_f32_async", dx.ptr, dwg.ptr, dwu.ptr, dwd.ptr, scratch.ptr, dx.ptr, M, d_model, ffn)
+        dev.sync()
+        close(dx.download(np.float32, (M, d_model)) / scale, want / scale, 1e-3, 1e-4)
 
 
 @pytest.mark.parametrize("M,d_model", [(3, 1024), (4, 768), (2, 2048)])
