@@ -83,11 +83,15 @@ __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int p
     if (pair == 0) reinterpret_cast<float*>(step + 12 * 1024)[b * 16 + m] = ldexpf(1.0f, ex - 20);
 }
 
-// grid = K / 32 blocks, 256 threads: thread (row tid / 16, pair tid % 16)
-__global__ __launch_bounds__(256) void q80i8_pack_kernel(const float* __restrict__ A, int M, int MP, int K, uint8_t* pack) {
+// grid = K / 32 blocks, 256 threads: thread (row tid / 16, pair tid % 16).  zero (may be null): zero_count floats the
+// launch clears on the side (the result of a product whose two K halves are added into it).
+__global__ __launch_bounds__(256) void q80i8_pack_kernel(const float* __restrict__ A, int M, int MP, int K, uint8_t* pack,
+                                                         float* zero, int zero_count) {
     const int blk = blockIdx.x, m = threadIdx.x >> 4, pair = threadIdx.x & 15;
     float2 v = make_float2(0.0f, 0.0f);
     if (m < M) v = *reinterpret_cast<const float2*>(A + (size_t)m * K + 32 * blk + 2 * pair);
+    if (zero)
+        for (int i = blk * 256 + (int)threadIdx.x; i < zero_count; i += (int)gridDim.x * 256) zero[i] = 0.0f;
     q80i8_pack_pair(v.x, v.y, m, pair, MP, pack, blk);
 }
 
@@ -478,9 +482,20 @@ int m40_launch_q80_i8(M40llmCudaContext* ctx, hipStream_t stream, uint32_t strea
     (void)hipGetLastError();
     uint8_t* pack = static_cast<uint8_t*>(ctx->scratch[stream_kind].gemm_pack);
     const int MP = rows_padded(M);
-    q80i8_pack_kernel<<<K >> 5, 256, 0, stream>>>(A, M, MP, K, pack);
     Q80I8Args a{};
     a.pack = pack; a.W0 = W; a.C = C; a.M = M; a.MP = MP; a.N = N; a.K = K;
+    // few column tiles and a long K: tile pairs x two halves of K, added into a result the pack launch clears
+    // (N = 4096, K = 14336: 17.5 -> 15.5 us at four rows, 23.7 -> 21.0 us at sixteen, pack launch aside)
+    const char *c0 = reinterpret_cast<const char*>(C), *a0 = reinterpret_cast<const char*>(A);
+    const bool apart = c0 + (size_t)M * N * 4 <= a0 || a0 + (size_t)M * K * 4 <= c0;
+    const int pairs = (N + 31) / 32;
+    if (apart && 2 * pairs >= 192 && 2 * pairs <= 1024 && K / (32 * kStepBlocks) >= 32) {
+        q80i8_pack_kernel<<<K >> 5, 256, 0, stream>>>(A, M, MP, K, pack, C, M * N);
+        if (MP == 0) q80i8_gemm_kernel<0, 4, true, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(a);
+        else q80i8_gemm_kernel<0, 4, false, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(a);
+        return hipGetLastError() == hipSuccess ? 0 : -2;
+    }
+    q80i8_pack_kernel<<<K >> 5, 256, 0, stream>>>(A, M, MP, K, pack, nullptr, 0);
     launch_gemm0(stream, a);
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
@@ -497,7 +512,7 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     uint8_t* xp = static_cast<uint8_t*>(ctx->scratch[stream_kind].gemm_pack);
     uint8_t* hp = xp + x_bytes;
     const int MP = rows_padded(M);
-    q80i8_pack_kernel<<<d_model >> 5, 256, 0, stream>>>(x, M, MP, d_model, xp);
+    q80i8_pack_kernel<<<d_model >> 5, 256, 0, stream>>>(x, M, MP, d_model, xp, nullptr, 0);
     Q80I8Args a{};
     a.pack = xp; a.W0 = wg; a.W1 = wu; a.out_pack = hp; a.M = M; a.MP = MP; a.N = ffn; a.K = d_model;
     // down projection as column-tile pairs x two halves of K, added into a result the gate + up launch clears

@@ -405,10 +405,11 @@ def test_q80_ffn_wide_hidden_short_k_vs_oracle(dev, orc, M, d_model):
 @pytest.mark.parametrize("M,N,K", [(1, 300, 512), (3, 1000, 768), (8, 4096, 2048), (9, 520, 1280), (16, 2048, 4096),
                                    (20, 333, 256), (2, 64, 96), (1, 1000, 4096), (2, 777, 8192), (1, 513, 14336),
                                    (2, 260, 11008), (1, 40, 16384), (2, 3, 64), (8, 6200, 512), (12, 24600, 256),
-                                   (5, 8192, 1024), (4, 12300, 512)])
+                                   (5, 8192, 1024), (4, 12300, 512), (6, 3100, 8192), (3, 4096, 8192)])
 def test_q80_gemm_shapes_vs_oracle(dev, orc, M, N, K):
     """MFMA path (3 rows and more, K % 256 == 0; column tails, split K, more than 16 rows; 5 rows and more with 6144
-    columns and more: two column tiles per wave, split K and, from ~24 500 columns, whole K), the register-resident
+    columns and more: two column tiles per wave, split K and, from ~24 500 columns, whole K; ~3100 to 16 000 columns with
+    K of 8192 and more: tile pairs x two halves of K added into a cleared result), the register-resident
     GEMV of one and two rows (K % 64 == 0, one, two and four K-parts per column) and the simple path (K = 96)."""
     rng = np.random.default_rng(M * 7919 + N + K)
     d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
