@@ -34,6 +34,23 @@ constexpr int kStackStepBytes = 4 * 1024 + kStepBlocks * 4 * 4;        // 4224
 constexpr int kPlaneStepBytes = 12 * 1024 + kStepBlocks * 16 * 4;      // 12800
 __host__ __device__ constexpr int q80i8_step_bytes(int MP) { return MP == 0 ? kStackStepBytes : kPlaneStepBytes; }
 
+// Digits of one element under its block's scale: n = rint(v * 2^(20 - ex)), |n| <= 2^20, cut into balanced base-128
+// digits n = (d1 * 128 + d2) * 128 + d3 with d2, d3 in [-64, 63] and |d1| <= 64 (exact integer arithmetic, one rounding).
+__device__ __forceinline__ void q80i8_digits(float v, float inv, int& d1, int& d2, int& d3) {
+    const float s = fminf(fmaxf(v * inv, -1048576.0f), 1048576.0f);
+    const int n = (int)rintf(s);
+    d3 = (n << 25) >> 25;
+    const int n1 = (n - d3) >> 7;
+    d2 = (n1 << 25) >> 25;
+    d1 = (n1 - d2) >> 7;
+}
+// the low bytes of four values as one word
+__device__ __forceinline__ uint32_t q80i8_bytes4(int a, int b, int c, int d) {
+    const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+    const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
 // Digits of two neighbouring elements of one row of one block.  The 16 threads of a row (lanes pair = 0..15 of an
 // aligned group of 16) hold the row's 32 values; digits go to dst in A-operand order, the exponent to dst's tail.
 __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int pair, int MP, uint8_t* pack, int blk) {
@@ -43,20 +60,11 @@ __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int p
     int ex = 0;
     if (mx > 0.0f && mx < INFINITY) (void)frexpf(mx, &ex);        // mx = f * 2^ex, f in [0.5, 1)
     ex = ex < -100 ? -100 : (ex > 100 ? 100 : ex);
-    const float inv = ldexpf(1.0f, 6 - ex);                        // |a| * inv < 64
+    const float inv = ldexpf(1.0f, 20 - ex);                       // |a| * inv < 2^20
     const float v[2] = {v0, v1};
     int d[3][2];
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-        float s = (mx < INFINITY ? v[e] : 0.0f) * inv;
-        s = fminf(fmaxf(s, -64.0f), 64.0f);
-        const float d1 = rintf(s);
-        const float r1 = (s - d1) * 128.0f;                        // exact: |s - d1| <= 0.5
-        const float d2 = rintf(r1);
-        const float r2 = (r1 - d2) * 128.0f;
-        const float d3 = rintf(r2);
-        d[0][e] = (int)d1; d[1][e] = (int)d2; d[2][e] = (int)d3;
-    }
+    for (int e = 0; e < 2; ++e) q80i8_digits(mx < INFINITY ? v[e] : 0.0f, inv, d[0][e], d[1][e], d[2][e]);
     const int k = 2 * pair, kg = k >> 3, kb = k & 7;
     // value = 2^(ex - 20) * ((d1 * 128 + d2) * 128 + d3)
     const int b = blk % kStepBlocks;
@@ -95,12 +103,40 @@ __global__ __launch_bounds__(256) void q80i8_pack_kernel(const float* __restrict
     q80i8_pack_pair(v.x, v.y, m, pair, MP, pack, blk);
 }
 
+// Stacked digits of eight consecutive elements (k group kg of block blk) of row m < 4, written into the step planes
+// at `planes` (LDS).  The four threads of a (block, row) are four neighbouring lanes; the arithmetic of q80i8_pack_pair.
+__device__ __forceinline__ void q80i8_pack8_stacked(const float4& lo, const float4& hi, int m, int kg, int blk, bool store,
+                                                    uint8_t* planes) {
+    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    float mx = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
+    mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+    int ex = 0;
+    if (mx > 0.0f && mx < INFINITY) (void)frexpf(mx, &ex);
+    ex = ex < -100 ? -100 : (ex > 100 ? 100 : ex);
+    const float inv = mx < INFINITY ? ldexpf(1.0f, 20 - ex) : 0.0f;
+    int d[3][8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q80i8_digits(mx < INFINITY ? v[e] : 0.0f, inv, d[0][e], d[1][e], d[2][e]);
+    if (!store) return;
+    uint8_t* step = planes + (size_t)(blk / kStepBlocks) * kStackStepBytes;
+    const int b = blk % kStepBlocks;
+#pragma unroll
+    for (int dg = 0; dg < 3; ++dg)
+        *reinterpret_cast<uint2*>(step + (b >> 1) * 1024 + (kg * 16 + dg * 4 + m) * 16 + (b & 1) * 8) =
+            make_uint2(q80i8_bytes4(d[dg][0], d[dg][1], d[dg][2], d[dg][3]), q80i8_bytes4(d[dg][4], d[dg][5], d[dg][6], d[dg][7]));
+    if (kg == 0) reinterpret_cast<float*>(step + 4 * 1024)[b * 4 + m] = ldexpf(1.0f, ex - 20);
+}
+
 struct Q80I8Args {
     const uint8_t* pack;       // packed activations
     const uint8_t* W0;         // MODE 0: the matrix; MODE 1: gate
     const uint8_t* W1;         // MODE 1: up
     float* C;                  // MODE 0: [M][N]
     uint8_t* out_pack;         // MODE 1: packed SwiGLU output (the A operand of the down projection)
+    const float* x;            // SELF: the f32 rows [M][K], packed by every workgroup for itself
     float* zero;               // MODE 1: cleared by the launch (zero_count floats), or null: the result of a down projection
     int zero_count;            //         whose two K halves are added into it
     int M, MP, N, K;
@@ -149,8 +185,13 @@ __device__ __forceinline__ void q80i8_unrolled(std::integer_sequence<int, I...>,
 // KHALVES = 2 (MODE 0): two workgroups share a column group, each walks half of K and ADDS its sums into C, which the
 // launch before has cleared: 0 + a + b is the same f32 in either order, so the result does not depend on timing.  A
 // workgroup then needs only half of the activation planes, and twice as many workgroups can own two tiles each.
-template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1>
+// SELF (stacked gate + up only, K <= 4096): no pack launch -- every workgroup turns the f32 rows into the digit planes of
+// all steps itself, in LDS (4224 bytes per step, dynamic), behind its first weight requests, and the K loop reads its
+// activation operands from there.
+template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1, bool SELF = false>
 __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) {
+    static_assert(!SELF || (STACK && MODE == 1 && KSPLIT == 1 && WAVES == 4), "self-packing: the stacked gate + up launch");
+    extern __shared__ __attribute__((aligned(16))) uint8_t q80i8_planes[];    // SELF: [step][4224]
     static_assert(KHALVES == 1 || (KHALVES == 2 && MODE == 0), "halves of K are added into a cleared result");
     static_assert(T == 1 || T == 2, "one or two column tiles per wave");
     constexpr int kWaves = WAVES;  // (stacked form, eight waves splitting K, measured for the down projection: 21.4 against 20.5 us)
@@ -221,6 +262,21 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
     constexpr int D = STACK ? (T == 1 ? 4 : 2) : 2;   // steps in flight (two 32-column steps are as many bytes as four of 16
                                                  // columns; the three-plane form has no registers for more)
 
+    // SELF: the rows' elements of this thread, requested before the weights (loads return in issue order).  Thread ->
+    // (block 16 pass + tid / 16, row (tid / 4) % 4, k group tid % 4), eight passes for K <= 4096
+    constexpr int kSelfPasses = SELF ? 8 : 1;
+    float4 xr[kSelfPasses][2];
+    if constexpr (SELF) {
+        const int nblk = p.K >> 5, m = (tid >> 2) & 3, kg = tid & 3;
+#pragma unroll
+        for (int ps = 0; ps < kSelfPasses; ++ps) {
+            const int blk = ps * 16 + (tid >> 4);
+            const float* src = p.x + (size_t)(m < p.M ? m : 0) * p.K + 32 * (blk < nblk ? blk : 0) + 8 * kg;
+            xr[ps][0] = reinterpret_cast<const float4*>(src)[0];
+            xr[ps][1] = reinterpret_cast<const float4*>(src)[1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     WPiece wr[D][kWLoads];
     Q80I8Acts<STACK> acts[D];
     auto issue_w = [&](WPiece (&dst)[kWLoads], int step) {
@@ -320,15 +376,46 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
         // register set and refills it with step s + D, activations before weights.
 #pragma unroll
         for (int i = 0; i < D; ++i) {
-            issue_a(acts[i], s0 + i);
+            if constexpr (!SELF) issue_a(acts[i], s0 + i);
             // the order of these first requests must be the loop's own (waits count outstanding loads in issue order:
             // were the compiler free to interleave them, the loop's waits would have to assume the worst of both orders)
             __builtin_amdgcn_sched_barrier(0);
             issue_w(wr[i], s0 + i);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (SELF) {
+            // operand rows 12-15 of every plane are zero
+            for (int i = tid; i < nsteps_all * 4 * 4 * 4; i += kThreads) {
+                const int st = i >> 6, pl = (i >> 4) & 3, kgz = (i >> 2) & 3, row = 12 + (i & 3);
+                *reinterpret_cast<uint4*>(q80i8_planes + st * kStackStepBytes + pl * 1024 + (kgz * 16 + row) * 16) = make_uint4(0, 0, 0, 0);
+            }
+            const int nblk = p.K >> 5, m = (tid >> 2) & 3, kg = tid & 3;
+#pragma unroll
+            for (int ps = 0; ps < kSelfPasses; ++ps) {
+                const int blk = ps * 16 + (tid >> 4);
+                const bool row_live = m < p.M;
+                const float4 z4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                q80i8_pack8_stacked(row_live ? xr[ps][0] : z4, row_live ? xr[ps][1] : z4, m, kg, blk, blk < nblk, q80i8_planes);
+            }
+            __syncthreads();
+        }
+        // SELF: the planes of a step are read from LDS one step ahead of their use
+        Q80I8Acts<STACK> lds_next;
+        auto read_planes = [&](int s) {
+            const uint8_t* base = q80i8_planes + (s < s1 ? s : s1 - 1) * kStackStepBytes;
+#pragma unroll
+            for (int i = 0; i < kPlanes; ++i) lds_next.pl[i] = *reinterpret_cast<const uint4*>(base + a_off + 1024 * i);
+            lds_next.sv = *reinterpret_cast<const float*>(base + sv_off);
+        };
+        if constexpr (SELF) read_planes(s0);
         auto step = [&](auto set_c, int s) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
+            Q80I8Acts<STACK> from_lds;
+            if constexpr (SELF) {
+                from_lds = lds_next;
+                read_planes(s + 1);
+            }
+            const Q80I8Acts<STACK>& act_now = SELF ? from_lds : acts[SET];
             // weights of this step -> the wave's LDS tile (waits for them and for everything older: this step's
             // activations; the younger steps stay in flight)
 #pragma unroll
@@ -350,12 +437,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
                 WOperand w[T];
 #pragma unroll
                 for (int t = 0; t < T; ++t) w[t] = weight_operand(cur[t], b);
-                compute_block(acts[SET], b_c, w);
+                compute_block(act_now, b_c, w);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int t = 0; t < T; ++t) cur[t] = nxt[t];
             });
-            issue_a(acts[SET], s + D);
+            if constexpr (!SELF) issue_a(acts[SET], s + D);
             issue_w(wr[SET], s + D);
             __builtin_amdgcn_sched_barrier(0);
         };
@@ -512,9 +599,13 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     uint8_t* xp = static_cast<uint8_t*>(ctx->scratch[stream_kind].gemm_pack);
     uint8_t* hp = xp + x_bytes;
     const int MP = rows_padded(M);
-    q80i8_pack_kernel<<<d_model >> 5, 256, 0, stream>>>(x, M, MP, d_model, xp, nullptr, 0);
     Q80I8Args a{};
-    a.pack = xp; a.W0 = wg; a.W1 = wu; a.out_pack = hp; a.M = M; a.MP = MP; a.N = ffn; a.K = d_model;
+    a.pack = xp; a.W0 = wg; a.W1 = wu; a.out_pack = hp; a.x = x; a.M = M; a.MP = MP; a.N = ffn; a.K = d_model;
+    const bool two_tiles = ffn % 64 == 0 && ffn / 64 >= 192;
+    // stacked form, K <= 4096: no pack launch, the gate + up workgroups pack the rows themselves into LDS (FFN 14336 at
+    // four rows: 47.8 -> 46.9 us; with the earlier, twice as long digit arithmetic the launch lost what the pack launch cost)
+    const bool self_pack = MP == 0 && two_tiles && d_model <= 16 * 32 * kStepBlocks && m40_aligned16(x);
+    if (!self_pack) q80i8_pack_kernel<<<d_model >> 5, 256, 0, stream>>>(x, M, MP, d_model, xp, nullptr, 0);
     // down projection as column-tile pairs x two halves of K, added into a result the gate + up launch clears
     const bool out_apart = reinterpret_cast<const char*>(out) + (size_t)M * d_model * 4 <= reinterpret_cast<const char*>(x) ||
                            reinterpret_cast<const char*>(x) + (size_t)M * d_model * 4 <= reinterpret_cast<const char*>(out);
@@ -524,7 +615,13 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     if (halves) { a.zero = out; a.zero_count = M * d_model; }
     // two column tiles per wave where 192 workgroups and more remain: every activation plane fetched is used twice
     // (stacked form, FFN 14336: 52.9 -> 49.2 us; with three 32-column steps in flight instead of two 50.1 us)
-    if (MP == 0 && ffn % 64 == 0 && ffn / 64 >= 192) q80i8_gemm_kernel<1, 1, true, 2><<<ffn / 64, 256, 0, stream>>>(a);
+    if (self_pack) {
+        auto* kern = q80i8_gemm_kernel<1, 1, true, 2, 4, 1, true>;
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 16 * kStackStepBytes);
+        if (attr != hipSuccess) return -2;
+        kern<<<ffn / 64, 256, (size_t)(d_model / (32 * kStepBlocks)) * kStackStepBytes, stream>>>(a);
+    } else if (MP == 0 && two_tiles) q80i8_gemm_kernel<1, 1, true, 2><<<ffn / 64, 256, 0, stream>>>(a);
     else if (MP == 0) q80i8_gemm_kernel<1, 1, true><<<ffn / 32, 256, 0, stream>>>(a);
     // (a workgroup of two column groups x two K halves, two waves per SIMD instead of one: measured, 64.5 -> 66 us)
     else if (ffn % 64 == 0 && ffn / 64 >= 192) q80i8_gemm_kernel<1, 1, false, 2><<<ffn / 64, 256, 0, stream>>>(a);
