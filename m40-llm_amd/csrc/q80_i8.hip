@@ -188,7 +188,10 @@ __device__ __forceinline__ void q80i8_unrolled(std::integer_sequence<int, I...>,
 // SELF (stacked gate + up only, K <= 4096): no pack launch -- every workgroup turns the f32 rows into the digit planes of
 // all steps itself, in LDS (4224 bytes per step, dynamic), behind its first weight requests, and the K loop reads its
 // activation operands from there.
-template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1, bool SELF = false>
+// DEPTH: steps in flight per wave, 0 = the form's default.  What pays is about 70 KB of weight requests outstanding per
+// CU, not more (measured: 104 KB and 139 KB are slower, 35 KB too): a launch that puts two workgroups on a CU runs
+// with half the depth of one that puts one there.
+template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1, bool SELF = false, int DEPTH = 0>
 __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) {
     static_assert(!SELF || (STACK && MODE == 1 && KSPLIT == 1 && WAVES == 4), "self-packing: the stacked gate + up launch");
     extern __shared__ __attribute__((aligned(16))) uint8_t q80i8_planes[];    // SELF: [step][4224]
@@ -259,7 +262,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
     const uint32_t e_off = (uint32_t)(12 * 1024 + (lane & 3) * 64 + g * 16);
     constexpr int kStepBytes = STACK ? kStackStepBytes : kPlaneStepBytes;
     constexpr int kPlanes = STACK ? 4 : 12;
-    constexpr int D = STACK ? (T == 1 ? 4 : 2) : 2;   // steps in flight (two 32-column steps are as many bytes as four of 16
+    constexpr int D = DEPTH ? DEPTH : (STACK ? (T == 1 ? 4 : 2) : 2);   // steps in flight (two 32-column steps are as many bytes as four of 16
                                                  // columns; the three-plane form has no registers for more)
 
     // SELF: the rows' elements of this thread, requested before the weights (loads return in issue order).  Thread ->
@@ -556,7 +559,8 @@ static void launch_gemm0(hipStream_t stream, const Q80I8Args& a) {
         if ((pairs + 3) / 4 >= 192) q80i8_gemm_kernel<0, 1, false, 2><<<(pairs + 3) / 4, 256, 0, stream>>>(a);
         else q80i8_gemm_kernel<0, 1, false><<<(tiles + 3) / 4, 256, 0, stream>>>(a);
     } else {
-        if (pairs >= 192) q80i8_gemm_kernel<0, 4, false, 2><<<pairs, 256, 0, stream>>>(a);
+        if (pairs > 256) q80i8_gemm_kernel<0, 4, false, 2, 4, 1, false, 1><<<pairs, 256, 0, stream>>>(a);   // two workgroups per CU
+        else if (pairs >= 192) q80i8_gemm_kernel<0, 4, false, 2><<<pairs, 256, 0, stream>>>(a);
         else if (nsteps >= 16) q80i8_gemm_kernel<0, 8, false, 1, 8><<<tiles, 512, 0, stream>>>(a);
         else q80i8_gemm_kernel<0, 4, false><<<tiles, 256, 0, stream>>>(a);
     }
