@@ -453,6 +453,33 @@ def test_q80_gemv_random_shapes_vs_float64(dev):
         dA.free(); dW.free(); dC.free()
 
 
+def test_q80_int8_forms_seeded_shapes_vs_float64(dev):
+    """The int8 matrix-instruction forms over seeded shapes: 2 to 16 rows (stacked and three-plane form), column counts on
+    both sides of every launch-shape switch (whole K / split K / two tiles per wave / two halves of K added into a cleared
+    result) with ragged tails, K from one step (256) to 40; against float64 of the same operands."""
+    rng = np.random.default_rng(90210)
+    shapes = [(3, 17, 256), (16, 1, 512), (5, 6143, 256), (5, 6145, 512), (4, 12287, 256), (4, 12289, 512), (9, 3071, 8192),
+              (9, 3073, 8192), (2, 3073, 10240), (16, 16385, 256), (7, 8209, 1024), (13, 24577, 256), (4, 8193, 2048)]
+    for _ in range(10):
+        shapes.append((int(rng.integers(3, 17)), int(rng.integers(1, 9000)), 256 * int(rng.integers(1, 9))))
+    for M, N, K in shapes:
+        d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
+        qs = rng.integers(-127, 128, size=(N, K // 32, 32)).astype(np.int8)
+        W = np.empty((N, K // 32, 34), dtype=np.uint8)
+        W[:, :, :2] = d.view(np.uint8).reshape(N, K // 32, 2)
+        W[:, :, 2:] = qs.view(np.uint8)
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        A[M - 1] *= 1e-4
+        A[0, ::7] *= 50.0
+        dA, dW, dC = dev.up(A), dev.up(W), dev.up(np.full((M, N), 3.0, dtype=np.float32))
+        dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dA.ptr, dW.ptr, dC.ptr, M, N, K)
+        got = dC.download(np.float32, (M, N))
+        f64 = A.astype(np.float64) @ (d.astype(np.float64)[:, :, None] * qs.astype(np.float64)).reshape(N, K).T
+        scale = np.abs(f64).max(axis=1, keepdims=True)
+        close(got / scale, f64 / scale, 1e-4, 1e-5)
+        dA.free(); dW.free(); dC.free()
+
+
 # ------------------------------------------------------------------ dense attention
 def _attention_case(dev, orc, qh, kvh, hd, L, k, v, q, max_seq=None, seq=0, batch=1):
     max_seq = max_seq or L
