@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256) void gemm_f32xq80_kernel(const float* __restri
 constexpr int kQ80GemvThreads = 512;
 constexpr int kQ80GemvWaves = kQ80GemvThreads / 64;
 constexpr int kQ80GemvMaxCols = 32;   // columns per team of waves
-constexpr int kQ80GemvDepth = 4;      // columns in flight per wave
+constexpr int kQ80GemvDepth = 2;      // columns in flight per wave (N = 14336, K = 4096 at one row: 15.2 / 13.2 / 14.8 / 14.4 us with 1 / 2 / 3 / 4)
 constexpr int kQ80GemvChunk = 128;    // blocks of activations staged through LDS at a time (two float4 per thread)
 constexpr int kQ80GemvMaxChunks = 64 * kQ80GemvWaves / kQ80GemvChunk;
 static_assert(kQ80GemvChunk * 8 == 2 * kQ80GemvThreads, "two float4 per thread and chunk");
