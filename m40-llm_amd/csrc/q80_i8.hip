@@ -10,10 +10,14 @@
 //     a = 2^E * (d1 + d2 / 128 + d3 / 16384),   |d1| <= 64, |d2|, |d3| <= 64,   error <= 2^-20 of the block's largest,
 // each digit plane is one matrix instruction, the three exact i32 results are recombined once per block, and the
 // block's factor 2^E * d_w multiplies them in f32.  No weight is converted and no product is rounded before that.
+// Up to four rows the three planes of all rows are stacked into the 16 operand rows: one instruction per block.
 //
 // Launches: a small pack kernel turns the f32 rows into digit planes (laid out in the order the A operand is
-// loaded), then the product kernel; the FFN form packs its SwiGLU output itself (a workgroup's four waves produce
-// exactly one 32-column block of the hidden row), so gate / up / down take three launches in all.
+// loaded), then the product kernel; the FFN form packs its SwiGLU output itself (a workgroup produces whole
+// 32-column blocks of the hidden row), so gate / up / down take three launches in all -- two in the stacked form up
+// to K = 4096, whose gate + up workgroups also pack the input rows themselves.  Where a product has few columns and a
+// long K (the down projection), two workgroups share a column group, each adds its half of K into the result, and the
+// launch before (pack, or gate + up) has cleared it: two terms onto zero, the same bits in either order.
 #include "common.hpp"
 
 #include <type_traits>
