@@ -12,6 +12,15 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """The libraries are built in-tree beforehand and loaded as they are; only a tree with nothing built (a fresh clone)
+    builds them here, once."""
+    import importlib
+    pkg = importlib.import_module("m40-llm_amd")
+    if not (os.path.exists(pkg.NATIVE_LIB) and os.path.exists(pkg.HOST_LIB)):
+        pkg.build()
+
+
 def _has_gpu() -> bool:
     # /dev/kfd is the ROCm compute device node; probing it does not initialise HIP.
     return os.path.exists("/dev/kfd")
