@@ -258,6 +258,8 @@ def main():
     import torch
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     pkg = importlib.import_module("m40-llm_amd")
+    if not (os.path.exists(pkg.NATIVE_LIB) and os.path.exists(pkg.HOST_LIB)):
+        pkg.build()                      # nothing built in this tree: build once; otherwise load what is there
     syn = importlib.import_module("m40-llm_amd.synthetic")
 
     cfg = dict(syn.TINYLLAMA_1B)
