@@ -48,6 +48,9 @@ __device__ __forceinline__ void q80i8_digits(float v, float inv, int& d1, int& d
     d2 = (n1 << 25) >> 25;
     d1 = (n1 - d2) >> 7;
 }
+// |v|, or +inf for a NaN: a block that holds a non-finite element gets a NaN block scale, so that every output fed by it
+// is NaN (the f32 product of the reference, kernels.cu:5037-5052, would give +-inf or NaN there; never a finite value)
+__device__ __forceinline__ float q80i8_abs_or_inf(float v) { return fabsf(v) <= 3.402823466e+38f ? fabsf(v) : INFINITY; }
 // the low bytes of four values as one word
 __device__ __forceinline__ uint32_t q80i8_bytes4(int a, int b, int c, int d) {
     const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
@@ -58,9 +61,10 @@ __device__ __forceinline__ uint32_t q80i8_bytes4(int a, int b, int c, int d) {
 // Digits of two neighbouring elements of one row of one block.  The 16 threads of a row (lanes pair = 0..15 of an
 // aligned group of 16) hold the row's 32 values; digits go to dst in A-operand order, the exponent to dst's tail.
 __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int pair, int MP, uint8_t* pack, int blk) {
-    float mx = fmaxf(fabsf(v0), fabsf(v1));
+    float mx = fmaxf(q80i8_abs_or_inf(v0), q80i8_abs_or_inf(v1));
 #pragma unroll
     for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float block_scale_bad = __builtin_nanf("");
     int ex = 0;
     if (mx > 0.0f && mx < INFINITY) (void)frexpf(mx, &ex);        // mx = f * 2^ex, f in [0.5, 1)
     ex = ex < -100 ? -100 : (ex > 100 ? 100 : ex);
@@ -80,7 +84,7 @@ __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int p
                 const uint16_t two = (uint16_t)((d[dg][0] & 0xff) | ((d[dg][1] & 0xff) << 8));
                 *reinterpret_cast<uint16_t*>(step + (b >> 1) * 1024 + (kg * 16 + dg * 4 + m) * 16 + (b & 1) * 8 + kb) = two;
             }
-            if (pair == 0) reinterpret_cast<float*>(step + 64 * 64)[b * 4 + m] = ldexpf(1.0f, ex - 20);
+            if (pair == 0) reinterpret_cast<float*>(step + 64 * 64)[b * 4 + m] = mx < INFINITY ? ldexpf(1.0f, ex - 20) : block_scale_bad;
         } else if (m >= 12) {
             *reinterpret_cast<uint16_t*>(step + (b >> 1) * 1024 + (kg * 16 + m) * 16 + (b & 1) * 8 + kb) = 0;
         }
@@ -92,7 +96,7 @@ __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int p
         const uint16_t two = (uint16_t)((d[dg][0] & 0xff) | ((d[dg][1] & 0xff) << 8));
         *reinterpret_cast<uint16_t*>(step + ((b >> 1) * 3 + dg) * 1024 + (kg * 16 + m) * 16 + (b & 1) * 8 + kb) = two;
     }
-    if (pair == 0) reinterpret_cast<float*>(step + 12 * 1024)[b * 16 + m] = ldexpf(1.0f, ex - 20);
+    if (pair == 0) reinterpret_cast<float*>(step + 12 * 1024)[b * 16 + m] = mx < INFINITY ? ldexpf(1.0f, ex - 20) : block_scale_bad;
 }
 
 // grid = K / 32 blocks, 256 threads: thread (row tid / 16, pair tid % 16).  zero (may be null): zero_count floats the
@@ -114,7 +118,7 @@ __device__ __forceinline__ void q80i8_pack8_stacked(const float4& lo, const floa
     const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     float mx = 0.0f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, q80i8_abs_or_inf(v[e]));
     mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
     int ex = 0;
@@ -131,7 +135,7 @@ __device__ __forceinline__ void q80i8_pack8_stacked(const float4& lo, const floa
     for (int dg = 0; dg < 3; ++dg)
         *reinterpret_cast<uint2*>(step + (b >> 1) * 1024 + (kg * 16 + dg * 4 + m) * 16 + (b & 1) * 8) =
             make_uint2(q80i8_bytes4(d[dg][0], d[dg][1], d[dg][2], d[dg][3]), q80i8_bytes4(d[dg][4], d[dg][5], d[dg][6], d[dg][7]));
-    if (kg == 0) reinterpret_cast<float*>(step + 4 * 1024)[b * 4 + m] = ldexpf(1.0f, ex - 20);
+    if (kg == 0) reinterpret_cast<float*>(step + 4 * 1024)[b * 4 + m] = mx < INFINITY ? ldexpf(1.0f, ex - 20) : __builtin_nanf("");
 }
 
 struct Q80I8Args {
@@ -364,8 +368,11 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
                 const i32x4 r3 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a2, B, z, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    // |r1|, |r2|, |r3| <= 32 * 64 * 127 < 2^18: the recombination fits 32 bits exactly
-                    const float sum = (float)((r1[r] * 128 + r2[r]) * 128 + r3[r]);
+                    // |r1|, |r2|, |r3| <= 32 * 64 * 128 = 2^18 each.  The whole sum (r1 * 128 + r2) * 128 + r3 reaches 2^32 (a
+                    // block of like-signed activations against like-signed large quants) and would wrap in 32 bits: the
+                    // two low digits are joined as an integer (< 2^26), the leading one (exact as f32) is added by one
+                    // fused multiply-add -- two roundings of <= 2^-24 of the block sum in place of none
+                    const float sum = fmaf((float)r1[r], 16384.0f, (float)(r2[r] * 128 + r3[r]));
                     acc[t][r] = fmaf(sa[r] * dw, sum, acc[t][r]);
                 }
             }

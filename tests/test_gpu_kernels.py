@@ -480,6 +480,81 @@ def test_q80_int8_forms_seeded_shapes_vs_float64(dev):
         dA.free(); dW.free(); dC.free()
 
 
+def _q80_const_matrix(n, k, scale, pattern):
+    """q8_0 matrix whose column c holds the single quant pattern[c % len(pattern)] in every block (scale as f16)."""
+    W = np.empty((n, k // 32, 34), dtype=np.uint8)
+    W[:, :, :2] = np.full((n, k // 32), scale, dtype=np.float16).view(np.uint8).reshape(n, k // 32, 2)
+    q = np.array([pattern[c % len(pattern)] for c in range(n)], dtype=np.int8)
+    W[:, :, 2:] = np.broadcast_to(q.view(np.uint8)[:, None, None], (n, k // 32, 32))
+    dense = np.float64(np.float16(scale)) * np.broadcast_to(q.astype(np.float64)[:, None], (n, k))
+    return W, dense
+
+
+@pytest.mark.parametrize("M", [3, 5, 16])
+def test_q80_int8_like_signed_blocks_vs_float64(dev, M):
+    """Blocks whose activations all have one sign and one size against columns of one large quant (127 or -128): the
+    integer block sum of the three-digit form reaches 2^32 there (x = 0.9, 0.6, -1, 0.99 are the cases that wrapped a
+    32-bit recombination).  GEMM and fused FFN, stacked (3 rows) and three-plane form (5, 16 rows), against float64."""
+    K, N = 512, 96
+    W, dense = _q80_const_matrix(N, K, 0.0078125, [127, -128, 80, -127])
+    vals = [0.9, 0.6, -1.0, 0.99, 0.5, -0.9, 1.0, 0.75]
+    A = np.empty((M, K), dtype=np.float32)
+    for m in range(M):
+        A[m] = vals[m % len(vals)]
+    A[M - 1, 32:64] = -0.9                                  # one block of the other sign
+    dA, dW, dC = dev.up(A), dev.up(W), dev.zeros(M * N * 4)
+    dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dA.ptr, dW.ptr, dC.ptr, M, N, K)
+    got = dC.download(np.float32, (M, N))
+    f64 = A.astype(np.float64) @ dense.T
+    scale = np.abs(f64).max(axis=1, keepdims=True)
+    close(got / scale, f64 / scale, 1e-5, 1e-6)
+    # fused FFN: gate columns of both signs, up and down of one sign each; long K for the two-halves down projection too
+    for d_model, ffn in ((512, 1024), (3072, 8192)):
+        wg, g64 = _q80_const_matrix(ffn, d_model, 0.001, [127, -128, 64, -3])
+        wu, u64 = _q80_const_matrix(ffn, d_model, 0.002, [127, 127, -128, 90])
+        wd, d64 = _q80_const_matrix(d_model, ffn, 0.001, [127, -128])
+        x = np.ascontiguousarray(np.tile(A[:, :256], (1, d_model // 256))) * np.float32(0.125)
+        dx, dwg, dwu, dwd = dev.up(x), dev.up(wg), dev.up(wu), dev.up(wd)
+        scratch, out = dev.zeros(2 * M * ffn * 4), dev.zeros(M * d_model * 4)
+        dev.call("m40llm_ext_ffn_swiglu_q80_f32_async", dx.ptr, dwg.ptr, dwu.ptr, dwd.ptr, scratch.ptr, out.ptr, M, d_model, ffn)
+        dev.sync()
+        g = x.astype(np.float64) @ g64.T
+        h = g / (1.0 + np.exp(-g)) * (x.astype(np.float64) @ u64.T)
+        want = h @ d64.T
+        scale = np.abs(want).max(axis=1, keepdims=True)
+        close(out.download(np.float32, (M, d_model)) / scale, want / scale, 1e-4, 1e-5)
+        for b in (dx, dwg, dwu, dwd, scratch, out):
+            b.free()
+
+
+@pytest.mark.parametrize("M", [2, 4, 5, 16])
+def test_q80_non_finite_activations_stay_non_finite(dev, M):
+    """A NaN or an infinity in an activation row reaches every output of that row as a non-finite value on every q8_0
+    path (register GEMV at 2 rows, stacked int8 form at 4, three-plane form at 5 and 16), as the f32 product of the
+    reference does (kernels.cu:5037-5052); the other rows are unaffected."""
+    rng = np.random.default_rng(77 + M)
+    N, K = 160, 512
+    d = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16)
+    qs = rng.integers(-127, 128, size=(N, K // 32, 32)).astype(np.int8)
+    qs[qs == 0] = 1
+    W = np.empty((N, K // 32, 34), dtype=np.uint8)
+    W[:, :, :2] = d.view(np.uint8).reshape(N, K // 32, 2)
+    W[:, :, 2:] = qs.view(np.uint8)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    clean = A.copy()
+    A[0, 37] = np.nan
+    A[1, 300] = np.inf
+    dA, dW, dC = dev.up(A), dev.up(W), dev.zeros(M * N * 4)
+    dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dA.ptr, dW.ptr, dC.ptr, M, N, K)
+    got = dC.download(np.float32, (M, N))
+    assert not np.isfinite(got[0]).any() and not np.isfinite(got[1]).any()
+    assert np.isnan(got[0]).all()
+    if M > 2:
+        f64 = clean.astype(np.float64) @ (d.astype(np.float64)[:, :, None] * qs.astype(np.float64)).reshape(N, K).T
+        scale = np.abs(f64[2:]).max(axis=1, keepdims=True)
+        close(got[2:] / scale, f64[2:] / scale, 1e-4, 1e-5)
+
+
 # ------------------------------------------------------------------ dense attention
 def _attention_case(dev, orc, qh, kvh, hd, L, k, v, q, max_seq=None, seq=0, batch=1):
     max_seq = max_seq or L
