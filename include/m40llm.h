@@ -462,6 +462,19 @@ int m40llm_ext_batched_gemm_residual_f32xf16_async(M40llmCudaContext* ctx, const
 int m40llm_ext_batched_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
                                                  uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
                                                  const void* d_wup_f16, void* d_hid_f32, uint32_t rows, int ffn, int d_model);
+/*   the same, and clear_floats floats at d_clear_f32 are set to zero on the side (the result of a following
+ *   ..._onto_zero call; d_clear_f32 NULL: nothing is cleared) */
+int m40llm_ext_batched_norm_gate_up_swiglu_clear_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                                       uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
+                                                       const void* d_wup_f16, void* d_hid_f32, uint32_t rows, int ffn,
+                                                       int d_model, void* d_clear_f32, uint32_t clear_floats);
+/*   out[rows][N] = residual + a[rows][K] . W^T for an out that HOLDS ZEROS stored by an earlier call on the decode
+ *   stream (the ..._clear call above) and overlaps neither a nor residual: with rows <= 8, a long K and few columns (the
+ *   down projection) one launch whose workgroups add the two halves of K into out -- two terms onto zero, the same
+ *   bits in either order; any other shape falls to m40llm_ext_batched_gemm_residual_f32xf16_async, which overwrites */
+int m40llm_ext_batched_gemm_residual_onto_zero_f32xf16_async(M40llmCudaContext* ctx, const void* d_a_f32, const void* d_w_f16,
+                                                             const void* d_residual_f32, void* d_out_f32, uint32_t rows, int N,
+                                                             int K);
 /*   out[rows][N] = (RMSNorm(x) * w) . W^T  (output norm + lm_head) */
 int m40llm_ext_batched_norm_gemm_f32xf16_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
                                                uint32_t norm_weight_dtype, float eps, const void* d_w_f16, void* d_out_f32,

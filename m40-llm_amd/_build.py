@@ -20,7 +20,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 HIP_SOURCES = ["context.hip", "elementwise.hip", "gemm.hip", "kvcache.hip", "attention.hip", "block_select.hip",
-               "decode_fused.hip", "skinny_mfma.hip", "attention_mfma.hip", "rows_gemv.hip", "rows_mfma.hip", "prefill_attention.hip", "gemm_tiled.hip", "q80_i8.hip"]
+               "decode_fused.hip", "skinny_mfma.hip", "attention_mfma.hip", "rows_gemv.hip", "rows_mfma.hip", "rows_khalf_mfma.hip", "prefill_attention.hip", "gemm_tiled.hip", "q80_i8.hip"]
 CPP_SOURCES = ["unavailable.cpp"]
 # per-file additions: matrix-instruction results straight into vector registers (the default form writes them to
 # accumulation registers and copies every element out again)

@@ -133,7 +133,14 @@ int m40_rows_norm_qkv(M40llmCudaContext* ctx, hipStream_t stream, const M40llmKV
 float4* m40_rope_cs_cache(M40llmCudaContext* ctx, const float* table);
 bool m40_rows_mfma_supported(int rows, int K);
 int m40_rows_mfma_swiglu(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
-                         float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K);
+                         float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K,
+                         float* zero = nullptr, int zero_count = 0);
+// rows_khalf_mfma.hip: up to eight rows against [N][K] with a long K in one launch: tiles x two halves of K, each
+// workgroup adding its sums (the first half's with the residual) into a result that an earlier launch has cleared
+bool m40_rows_khalf_supported(const M40llmCudaContext* ctx, int rows, int N, int K);
+int m40_rows_khalf_residual(M40llmCudaContext* ctx, hipStream_t stream, const float* a, const uint16_t* W,
+                            const float* residual, float* out_zeroed, int rows, int N, int K);
+int m40_zero_f32(hipStream_t stream, float* dst, size_t n);
 int m40_rows_mfma_plain(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
                         float eps, const uint16_t* W, float* out, int rows, int N, int K);
 bool m40_rows_mfma_qkv_supported(int rows, int K, uint32_t head_dim);

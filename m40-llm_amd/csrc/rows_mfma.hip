@@ -72,6 +72,8 @@ struct RowsMfmaArgs {
     const uint16_t* W1;        // SwiGLU: the up matrix
     float* out;                // [rows][N]
     int rows, N, units;        // units: 16-column tiles (plain) or 8-column gate/up tiles (SwiGLU)
+    float* zero;               // not null: zero_count floats the launch clears on the side (the result of a following
+    int zero_count;            // product whose two K halves are added into it)
     // Q/K/V form: W0 / W1 / W2 are the three matrices; a tile is 16 columns of one head that hold eight whole rotation
     // pairs (split-half layout: eight columns and their partners half a head further on)
     const uint16_t* W2;
@@ -392,6 +394,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
             tile(b0, no, local, 0);
         }
     }
+    // behind everything else: nothing in this launch waits for these stores
+    if (p.zero)
+        for (int i = (int)blockIdx.x * S::kThreads + tid; i < p.zero_count; i += (int)gridDim.x * S::kThreads) p.zero[i] = 0.0f;
 }
 
 template <int MODE, int WAVES>
@@ -417,12 +422,14 @@ int launch(M40llmCudaContext* ctx, hipStream_t stream, const RowsMfmaArgs& a) {
 bool m40_rows_mfma_supported(int rows, int K) { return rows >= 1 && rows <= kRows && K == kK; }
 
 int m40_rows_mfma_swiglu(M40llmCudaContext* ctx, hipStream_t stream, const float* x, const void* norm_w, uint32_t norm_dtype,
-                         float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K) {
+                         float eps, const uint16_t* wgate, const uint16_t* wup, float* out, int rows, int ffn, int K,
+                         float* zero, int zero_count) {
     if (!m40_rows_mfma_supported(rows, K) || ffn <= 0) return -6;
     if (!m40_aligned16(x) || !m40_aligned16(wgate) || !m40_aligned16(wup) || (norm_w && !m40_aligned16(norm_w))) return -6;
     RowsMfmaArgs a{};
     a.x = x; a.norm_w = norm_w; a.norm_dtype = norm_dtype; a.eps = eps; a.W0 = wgate; a.W1 = wup; a.out = out;
     a.rows = rows; a.N = ffn; a.units = (ffn + 7) / 8;
+    a.zero = zero; a.zero_count = zero_count;
     return launch<1>(ctx, stream, a);
 }
 

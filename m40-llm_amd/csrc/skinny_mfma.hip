@@ -829,10 +829,41 @@ int m40llm_ext_batched_gemm_residual_f32xf16_async(M40llmCudaContext* ctx, const
     return hipGetLastError() == hipSuccess ? 0 : -7;
 }
 
+int m40llm_ext_batched_gemm_residual_onto_zero_f32xf16_async(M40llmCudaContext* ctx, const void* d_a_f32, const void* d_w_f16,
+                                                             const void* d_residual_f32, void* d_out_f32, uint32_t rows, int N,
+                                                             int K) {
+    if (!ctx || !d_a_f32 || !d_w_f16 || !d_out_f32) return -1;
+    if (N <= 0 || K <= 0) return -2;
+    const char* o = static_cast<const char*>(d_out_f32);
+    auto apart = [&](const void* q, size_t bytes) {
+        const char* c = static_cast<const char*>(q);
+        return !c || c + bytes <= o || o + (size_t)rows * N * 4 <= c;
+    };
+    if (m40_rows_khalf_supported(ctx, (int)rows, N, K) && m40_aligned16(d_a_f32) && m40_aligned16(d_w_f16) &&
+        apart(d_a_f32, (size_t)rows * K * 4) && apart(d_residual_f32, (size_t)rows * N * 4)) {
+        (void)hipGetLastError();
+        return m40_rows_khalf_residual(ctx, ctx->decode_stream, static_cast<const float*>(d_a_f32),
+                                       static_cast<const uint16_t*>(d_w_f16), static_cast<const float*>(d_residual_f32),
+                                       static_cast<float*>(d_out_f32), (int)rows, N, K);
+    }
+    // any other shape: the form that overwrites its result
+    return m40llm_ext_batched_gemm_residual_f32xf16_async(ctx, d_a_f32, d_w_f16, d_residual_f32, d_out_f32, rows, N, K);
+}
+
 int m40llm_ext_batched_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
                                                  uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
                                                  const void* d_wup_f16, void* d_hid_f32, uint32_t rows, int ffn, int d_model) {
+    return m40llm_ext_batched_norm_gate_up_swiglu_clear_async(ctx, d_x_f32, d_norm_w, norm_weight_dtype, eps, d_wgate_f16,
+                                                              d_wup_f16, d_hid_f32, rows, ffn, d_model, nullptr, 0);
+}
+
+int m40llm_ext_batched_norm_gate_up_swiglu_clear_async(M40llmCudaContext* ctx, const void* d_x_f32, const void* d_norm_w,
+                                                       uint32_t norm_weight_dtype, float eps, const void* d_wgate_f16,
+                                                       const void* d_wup_f16, void* d_hid_f32, uint32_t rows, int ffn,
+                                                       int d_model, void* d_clear_f32, uint32_t clear_floats) {
     if (!ctx || !d_x_f32 || !d_norm_w || !d_wgate_f16 || !d_wup_f16 || !d_hid_f32) return -1;
+    if (!d_clear_f32) clear_floats = 0;
+    if (clear_floats > (1u << 30)) return -2;
     if (ffn <= 0 || d_model <= 0) return -2;
     if (norm_weight_dtype > 1) return -4;
     if (!rows_ok(ctx, (int)rows, d_model) || !m40_aligned16(d_wgate_f16) || !m40_aligned16(d_wup_f16)) return -6;
@@ -841,7 +872,9 @@ int m40llm_ext_batched_norm_gate_up_swiglu_async(M40llmCudaContext* ctx, const v
     if (m40_rows_mfma_supported((int)rows, d_model) && m40_aligned16(d_x_f32) && m40_aligned16(d_norm_w))
         return m40_rows_mfma_swiglu(ctx, ctx->decode_stream, static_cast<const float*>(d_x_f32), d_norm_w, norm_weight_dtype,
                                     eps, static_cast<const uint16_t*>(d_wgate_f16), static_cast<const uint16_t*>(d_wup_f16),
-                                    static_cast<float*>(d_hid_f32), (int)rows, ffn, d_model);
+                                    static_cast<float*>(d_hid_f32), (int)rows, ffn, d_model,
+                                    clear_floats ? static_cast<float*>(d_clear_f32) : nullptr, (int)clear_floats);
+    if (clear_floats && m40_zero_f32(ctx->decode_stream, static_cast<float*>(d_clear_f32), clear_floats) != 0) return -7;
     PackSpec pk{static_cast<const float*>(d_x_f32), nullptr, d_norm_w, norm_weight_dtype, eps};
     const void* W[2] = {d_wgate_f16, d_wup_f16};
     const int Ns[2] = {ffn, ffn};

@@ -602,9 +602,13 @@ public:
         M40H_TRY(m40llm_ext_attention_last_token_f32_gqa_batched_lens_dev_async(ctx_, kv_, slots_dev, lens_dev, 1, rows, hint,
                                                                                 ws_.q.ptr(), cfg_.q_heads, ws_.ctx_out.ptr()));
         M40H_TRY(m40llm_ext_batched_gemm_residual_f32xf16_async(ctx_, ws_.ctx_out.ptr(), w.wo, d_x, ws_.x1.ptr(), rows, (int)D, (int)D));
-        M40H_TRY(m40llm_ext_batched_norm_gate_up_swiglu_async(ctx_, ws_.x1.ptr(), w.ffn_norm, cfg_.norm_weight_dtype, cfg_.rms_eps,
-                                                              w.wgate, w.wup, ws_.hid.ptr(), rows, (int)F, (int)D));
-        M40H_TRY(m40llm_ext_batched_gemm_residual_f32xf16_async(ctx_, ws_.hid.ptr(), w.wdown, ws_.x1.ptr(), d_out, rows, (int)D, (int)F));
+        // d_out is dead until the down projection writes it: the gate + up launch clears it on the side, and the down
+        // projection adds its two halves of K into it
+        M40H_TRY(m40llm_ext_batched_norm_gate_up_swiglu_clear_async(ctx_, ws_.x1.ptr(), w.ffn_norm, cfg_.norm_weight_dtype,
+                                                                    cfg_.rms_eps, w.wgate, w.wup, ws_.hid.ptr(), rows, (int)F,
+                                                                    (int)D, d_out, rows * D));
+        M40H_TRY(m40llm_ext_batched_gemm_residual_onto_zero_f32xf16_async(ctx_, ws_.hid.ptr(), w.wdown, ws_.x1.ptr(), d_out, rows,
+                                                                          (int)D, (int)F));
     }
     void enqueue_batched_step(uint32_t rows, uint32_t hint, float* hidden, float* other) {
         const uint32_t* slots = static_cast<const uint32_t*>(bslots_.ptr());

@@ -291,6 +291,47 @@ def test_batched_down_projection_k_chunks_vs_oracle(dev, orc, rows, N, K):
     close(got / sc, want / sc)
 
 
+@pytest.mark.parametrize("rows,N,K", [(8, 2048, 11008), (5, 2040, 5632), (1, 4096, 4096), (3, 1027, 4352), (6, 2048, 4128), (7, 8192, 14336),
+                                      (8, 512, 8192), (9, 2048, 11008), (4, 2048, 2048)])
+def test_batched_down_projection_onto_zero_vs_oracle(dev, orc, rows, N, K):
+    """Gate + up with the clear on the side (d_model 2048: the persistent kernel clears; otherwise a fill launch), then
+    the down projection whose two K halves are added into the cleared result (up to eight rows, K >= 4096, 64 to 512
+    column tiles; column tails, k-step counts that do not divide by the waves; other shapes fall to the overwriting
+    form), against the oracle; the same call twice gives the same bits."""
+    rng = np.random.default_rng(rows * 31 + K)
+    a = _rows_case(rng, rows, K)
+    w = f16bits(rng.standard_normal((N, K)) * 0.03)
+    res = rng.standard_normal((rows, N)).astype(np.float32)
+    da, dw, dres = dev.up(a), dev.up(w), dev.up(res)
+    out = dev.up(np.full((rows, N), 7.0, dtype=np.float32))
+    # the clear rides on a gate + up call (its own result is not used here)
+    D = 2048
+    x = _rows_case(rng, rows, D)
+    nw = np.ones(D, dtype=np.float32)
+    wg = f16bits(rng.standard_normal((64, D)) * 0.03)
+    dx, dnw, dwg, hid = dev.up(x), dev.up(nw), dev.up(wg), dev.zeros(rows * 64 * 4)
+    def run():
+        dev.call("m40llm_ext_batched_norm_gate_up_swiglu_clear_async", dx.ptr, dnw.ptr, 1, 1e-5, dwg.ptr, dwg.ptr, hid.ptr, rows,
+                 64, D, out.ptr, rows * N)
+        dev.call("m40llm_ext_batched_gemm_residual_onto_zero_f32xf16_async", da.ptr, dw.ptr, dres.ptr, out.ptr, rows, N, K)
+        dev.sync()
+        return out.download(np.float32, (rows, N))
+    got = run()
+    want = res + orc.gemm("f32xf16_gguf", a, w, rows, N, K)
+    sc = np.abs(want).max(axis=1, keepdims=True)
+    close(got / sc, want / sc)
+    f64 = res.astype(np.float64) + a.astype(np.float64) @ w.view(np.float16).astype(np.float64).T
+    close(got / sc, f64 / sc, 1e-5, 1e-6)
+    for _ in range(3):
+        assert np.array_equal(run(), got)
+    # no residual
+    dev.call("m40llm_ext_batched_norm_gate_up_swiglu_clear_async", dx.ptr, dnw.ptr, 1, 1e-5, dwg.ptr, dwg.ptr, hid.ptr, rows, 64, D,
+             out.ptr, rows * N)
+    dev.call("m40llm_ext_batched_gemm_residual_onto_zero_f32xf16_async", da.ptr, dw.ptr, None, out.ptr, rows, N, K)
+    dev.sync()
+    close(out.download(np.float32, (rows, N)) / sc, (f64 - res) / sc, 1e-5, 1e-6)
+
+
 @pytest.mark.parametrize("qh,kvh,hd,layout,bias,rows", [
     (8, 2, 64, 0, False, 5), (4, 2, 128, 1, True, 8), (4, 1, 128, 1, True, 12),
     # d_model 2048 with up to eight rows: the persistent matrix-core kernel (adjacent and split-half pairs, with and without bias)
