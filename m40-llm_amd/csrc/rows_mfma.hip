@@ -5,7 +5,8 @@
 // its slices.  Here the workgroups are persistent: each converts the eight rows once into f16 hi + lo MFMA fragments
 // for the whole of K (64 KB of LDS, per-row power-of-two scale, RMSNorm weights folded in), then walks its share of
 // the column tiles.  A tile's K range is split over the eight waves (8 MFMA steps each), so a wave requests its whole
-// share of a tile -- eight 16-byte loads per lane -- at once and keeps two tiles in flight; the waves' partial sums
+// share of a tile in eight 16-byte loads per lane, with at most one tile in flight (more outstanding requests per CU
+// make the launch slower, not faster: the first data then reaches some CUs late); the waves' partial sums
 // meet in LDS in wave order and every result element is written once (residual, bias or SwiGLU applied), so nothing
 // is left for a second launch and no result depends on timing.
 //
@@ -166,14 +167,17 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
     // instruction, 4 KB apart -- streams a third slower: measured 26.5 us against 18.2 us for these 90 MB.)  The
     // operand layout is produced by a pass through the wave's own LDS tile.
     // No load under a branch: a tile past the workgroup's range re-reads the first 16 bytes of its first tile.
-    uint4 b0[kLoads], b1[kLoads];
+    uint4 b0[kLoads];
+    constexpr int kEarlyLoads = kLoads * 5 / 8;       // (B=8 step at the Qwen2.5-3B shape, early part 0 / 2 / 3 / 4 / 5 / 6 / 8 of 8 loads:
+                                                      // 2.49 / 2.38 / 2.34 / 2.33 / 2.32 / 2.33 / 2.35 ms; two whole tiles in flight: 2.39 ms)
     const int run_lane = lane % kRunLanes, run_col = lane / kRunLanes;
-    auto issue = [&](uint4 (&b)[kLoads], int local) {
+    auto issue = [&](uint4 (&b)[kLoads], int local, int l_begin = 0, int l_end = 64) {
         const bool live = local < n_units;
         const int unit = u_begin + (live ? local : 0);
         const int lane_off = live ? 8 * run_lane : 0;
 #pragma unroll
         for (int li = 0; li < kLoads; ++li) {
+            if (li < l_begin || li >= l_end) continue;
             const int i = li * kColsPerLoad + run_col;      // column of the tile (i & 8 is the same for the whole instruction)
             int col;
             const uint16_t* W = p.W0;
@@ -193,7 +197,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
         }
     };
     issue(b0, 0);
-    if (!QKV) issue(b1, 1);            // the Q/K/V form has one tile per workgroup
     __builtin_amdgcn_sched_barrier(0);
     // the tile element this thread writes (see `finish`)
     constexpr int kTileCols = SWIGLU ? 8 : 16;      // output columns of a tile
@@ -364,13 +367,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
         }
         p.out[(size_t)e_row * p.N + col] = v;
     };
-    // One tile from register set b; PREFETCH: tile local + 2 exists and is requested into the same set.
+    // One tile from register set b; PREFETCH: tile local + 1 exists and is requested into the same set.
     auto tile = [&](uint4 (&b)[kLoads], auto prefetch_c, int local, int parity) {
         to_lds(b);
-        if (decltype(prefetch_c)::value) issue(b, local + 2);
+        // the next tile's requests go out in two parts, around this tile's arithmetic: at most one tile (64 KB per
+        // CU) is ever in flight, and for the length of the arithmetic only kEarlyLoads / kLoads of it
+        if (decltype(prefetch_c)::value) issue(b, local + 1, 0, kEarlyLoads);
         compute(parity);
         __syncthreads();
         finish(local, parity);
+        if (decltype(prefetch_c)::value) issue(b, local + 1, kEarlyLoads, kLoads);
     };
     if (QKV) {
         tile(b0, std::integral_constant<bool, false>{}, 0, 0);
@@ -378,21 +384,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
         const std::integral_constant<bool, true> yes;
         const std::integral_constant<bool, false> no;
         int local = 0;
-        for (; local + 3 < n_units; local += 2) {        // both tiles of a pair have a tile two ahead
-            tile(b0, yes, local, 0);
-            tile(b1, yes, local + 1, 1);
-        }
-        const int rem = n_units - local;                  // 1, 2 or 3
-        if (rem == 3) {
-            tile(b0, yes, local, 0);
-            tile(b1, no, local + 1, 1);
-            tile(b0, no, local + 2, 0);
-        } else if (rem == 2) {
-            tile(b0, no, local, 0);
-            tile(b1, no, local + 1, 1);
-        } else {
-            tile(b0, no, local, 0);
-        }
+        for (; local + 1 < n_units; ++local) tile(b0, yes, local, local & 1);
+        tile(b0, no, local, local & 1);
     }
     // behind everything else: nothing in this launch waits for these stores
     if (p.zero)
