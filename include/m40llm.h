@@ -421,8 +421,10 @@ int m40llm_ext_attention_last_token_f32_gqa_position_dev_async(M40llmCudaContext
  * device array that is part of the library's code object (one copy per GPU, resolved once per device when a context
  * is created), and the call allocates nothing.  Returns -9 when the partials of this (q_heads, head_dim, seq_len) do
  * not fit 2 MiB: q_heads * chunks * (head_dim + 2) * 4 bytes, chunks = ceil(seq_len / chunk) with the chunk length
- * the allocating entry point uses.  Every call on one GPU shares that array: calls that overlap on one GPU (other
- * contexts, or the other stream) race; calls on the decode stream of one context are ordered and safe. */
+ * the allocating entry point uses.  Every call on one GPU shares that array: calls on the decode stream of one context
+ * are ordered and safe; a call from another context while the last user's launches are still outstanding returns -10
+ * (busy) instead of racing.  Captured calls are not guarded (no event can be queried under capture): graph replays
+ * that overlap on one GPU race. */
 int m40llm_ext_attention_last_token_f32_gqa_static_scratch_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
                                                                  uint32_t seq_id, const void* q_dev_f32,
                                                                  uint32_t q_heads, uint32_t seq_len,

@@ -13,6 +13,7 @@
 // batched :1740-1823 and :4694-4832.
 #include "attention_params.hpp"
 
+#include <atomic>
 #include <mutex>
 
 // Fixed chunk-partial buffer of m40llm_ext_attention_last_token_f32_gqa_static_scratch_async: device memory that
@@ -24,19 +25,32 @@ constexpr size_t kStaticScratchBytes = 2u << 20;   // 2 MiB
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kStaticScratchMaxDevices = 64;
-static float* g_static_scratch_ptr[kStaticScratchMaxDevices];
+static std::atomic<float*> g_static_scratch_ptr[kStaticScratchMaxDevices];
 static std::mutex g_static_scratch_mutex;
+// Who used a device's array last, and an event behind that call's last launch: a call from another context while
+// that work is still outstanding is refused (-10) instead of racing.  The event is made with the pointer, at set-up.
+struct StaticScratchUse {
+    const M40llmCudaContext* owner;
+    hipEvent_t done;
+    bool have_event, recorded;
+};
+static StaticScratchUse g_static_scratch_use[kStaticScratchMaxDevices];
 
 int m40_attention_static_scratch_init(int device_id) {
     if (device_id < 0 || device_id >= kStaticScratchMaxDevices) return -2;
     std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
-    if (g_static_scratch_ptr[device_id]) return 0;
+    if (g_static_scratch_ptr[device_id].load(std::memory_order_acquire)) return 0;
     void* ptr = nullptr;
     if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
         (void)hipGetLastError();
         return -4;
     }
-    g_static_scratch_ptr[device_id] = static_cast<float*>(ptr);
+    StaticScratchUse& use = g_static_scratch_use[device_id];
+    if (!use.have_event) {
+        if (hipEventCreateWithFlags(&use.done, hipEventDisableTiming) == hipSuccess) use.have_event = true;
+        else (void)hipGetLastError();
+    }
+    g_static_scratch_ptr[device_id].store(static_cast<float*>(ptr), std::memory_order_release);
     return 0;
 }
 
@@ -486,7 +500,9 @@ int m40llm_attention_last_token_f32_gqa_async(M40llmCudaContext* ctx, const M40l
 // row go into this device's copy of the fixed 2 MiB array above instead of the context's arena.  Calls nothing that
 // allocates.  -9: the partials of this (q_heads, head_dim, seq_len) do not fit the fixed buffer.  All calls on one
 // GPU share that buffer (every partial a call reads it has written itself, so nothing needs clearing between
-// calls); two calls that overlap on one GPU -- from different contexts or streams -- race.
+// calls).  Calls of one context are ordered on its decode stream; a call from another context while the last user's
+// work is still outstanding returns -10 (busy) instead of racing.  Under stream capture no event can be queried, so
+// captured calls are not guarded: replays that overlap on one GPU race.
 int m40llm_ext_attention_last_token_f32_gqa_static_scratch_async(M40llmCudaContext* ctx, const M40llmKVCache* kv,
                                                                  uint32_t seq_id, const void* q_dev_f32,
                                                                  uint32_t q_heads, uint32_t seq_len,
@@ -497,11 +513,24 @@ int m40llm_ext_attention_last_token_f32_gqa_static_scratch_async(M40llmCudaConte
     if (q_heads == 0 || kv->num_heads == 0 || q_heads % kv->num_heads != 0) return -6;
     if (!kv->d_k || !kv->d_v) return -4;
     if (ctx->device_id < 0 || ctx->device_id >= kStaticScratchMaxDevices) return -4;
-    float* ptr = g_static_scratch_ptr[ctx->device_id];
+    float* ptr = g_static_scratch_ptr[ctx->device_id].load(std::memory_order_acquire);
     if (!ptr) {
         // a context made before this translation unit could resolve the symbol: resolve it now, on the context's device
         if (m40_ensure_device(ctx) != 0 || m40_attention_static_scratch_init(ctx->device_id) != 0) return -4;
-        ptr = g_static_scratch_ptr[ctx->device_id];
+        ptr = g_static_scratch_ptr[ctx->device_id].load(std::memory_order_acquire);
+    }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->decode_stream, &capture) != hipSuccess) { (void)hipGetLastError(); capture = hipStreamCaptureStatusNone; }
+    const bool guarded = capture == hipStreamCaptureStatusNone;
+    std::unique_lock<std::mutex> lock(g_static_scratch_mutex, std::defer_lock);
+    StaticScratchUse& use = g_static_scratch_use[ctx->device_id];
+    if (guarded) {
+        lock.lock();
+        if (use.owner && use.owner != ctx && use.have_event && use.recorded) {
+            const hipError_t q = hipEventQuery(use.done);
+            if (q == hipErrorNotReady) return -10;
+            if (q != hipSuccess) (void)hipGetLastError();
+        }
     }
     M40AttnArgs a{};
     a.K = kv->d_k; a.V = kv->d_v; a.max_seq_len = kv->max_seq_len; a.kv_heads = kv->num_heads;
@@ -510,7 +539,13 @@ int m40llm_ext_attention_last_token_f32_gqa_static_scratch_async(M40llmCudaConte
     a.max_len_hint = seq_len;
     a.partial_override = ptr;
     a.partial_override_bytes = kStaticScratchBytes;
-    return m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+    const int rc = m40_launch_dense_attention(ctx, ctx->decode_stream, 1, a);
+    if (guarded && rc == 0 && use.have_event) {
+        use.owner = ctx;
+        use.recorded = hipEventRecord(use.done, ctx->decode_stream) == hipSuccess;
+        if (!use.recorded) (void)hipGetLastError();
+    }
+    return rc;
 }
 
 int m40llm_attention_last_token_f32_gqa(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t seq_id,

@@ -667,14 +667,31 @@ int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCach
     }
     // The old store lives head-major on the device ([sequence][kv head][token][...]); the answer is given in the
     // reference's order, [sequence][token][kv head][...] (cuda/kernels.cu:5435-5543), whatever the device layout.
-    std::vector<char> raw(total), ordered(total);
-    if (hipMemcpy(raw.data(), src, total, hipMemcpyDeviceToHost) != hipSuccess) return -5;
+    // Only the (sequence, kv head) token runs that meet [offset, offset + bytes) are copied: one contiguous device
+    // run per sequence and head into a staging buffer of at most one head's tokens, then item by item into place.
+    if (bytes == 0) return 0;
     const size_t S = kv->max_seq_len, H = kv->num_heads;
-    for (size_t b = 0; b < kv->max_batch_size; ++b)
-        for (size_t h = 0; h < H; ++h)
-            for (size_t t = 0; t < S; ++t)
-                std::memcpy(ordered.data() + ((b * S + t) * H + h) * item, raw.data() + ((b * H + h) * S + t) * item, item);
-    std::memcpy(out_host, ordered.data() + offset, bytes);
+    const size_t row0 = offset / item / H, row1 = (offset + bytes - 1) / item / H;      // token rows b * S + t
+    char* out = static_cast<char*>(out_host);
+    try {
+        std::vector<char> run;
+        for (size_t b = row0 / S; b <= row1 / S; ++b) {
+            const size_t t_lo = b == row0 / S ? row0 % S : 0, t_hi = b == row1 / S ? row1 % S : S - 1;
+            run.resize((t_hi - t_lo + 1) * item);
+            for (size_t h = 0; h < H; ++h) {
+                if (hipMemcpy(run.data(), static_cast<const char*>(src) + ((b * H + h) * S + t_lo) * item, run.size(),
+                              hipMemcpyDeviceToHost) != hipSuccess)
+                    return -5;
+                for (size_t t = t_lo; t <= t_hi; ++t) {
+                    const size_t at = ((b * S + t) * H + h) * item;                     // in the reference's order
+                    const size_t lo = at > offset ? at : offset, hi = at + item < offset + bytes ? at + item : offset + bytes;
+                    if (lo < hi) std::memcpy(out + (lo - offset), run.data() + (t - t_lo) * item + (lo - at), hi - lo);
+                }
+            }
+        }
+    } catch (const std::bad_alloc&) {
+        return -6;
+    }
     return 0;
 }
 

@@ -824,8 +824,8 @@ public:
     void decode_timed(uint32_t seq, const uint32_t* prompt, uint32_t n_prompt, uint32_t warmup, uint32_t steps,
                       uint32_t* ids_out, double* elapsed_ms) {
         if (n_prompt == 0) throw std::invalid_argument("decode_timed needs a prompt");
+        last_timed_host_fallback_ = false;
         if (mode_ >= 1 && fused_available()) {
-            last_timed_host_fallback_ = false;
             if (decode_greedy_device(seq, prompt, n_prompt, warmup, steps, 0, ids_out, nullptr, elapsed_ms)) return;
             // a device pick was a near tie: the whole run (warm-up and timed steps) is redone through the host sampler,
             // which rewrites the same cache rows; last_timed_host_fallback() tells the caller which path was timed
@@ -856,8 +856,8 @@ public:
 
     void decode_batch_timed(const uint32_t* seq_ids, const uint32_t* kv_lens, const uint32_t* first_tokens, uint32_t rows,
                             uint32_t warmup, uint32_t steps, uint32_t* ids_out, double* elapsed_ms) {
+        last_timed_host_fallback_ = false;
         if (mode_ >= 1 && batched_fused_available(rows)) {
-            last_timed_host_fallback_ = false;
             if (decode_batch_device(seq_ids, kv_lens, first_tokens, rows, warmup, steps, ids_out, nullptr, elapsed_ms)) return;
             last_timed_host_fallback_ = true;   // as in decode_timed: redo everything on the host-sampled path
         }

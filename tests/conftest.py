@@ -41,3 +41,18 @@ def orc():
     pyoracle.build()
     pyoracle.lib()
     return pyoracle
+
+
+@pytest.fixture
+def heartbeat(request):
+    """A long test's sign of life: writes to the real terminal while output is captured, so that a run whose output is
+    watched for activity does not look hung during minutes of CPU-side checking."""
+    capman = request.config.pluginmanager.getplugin("capturemanager")
+
+    def beat(text="."):
+        if capman is None:
+            sys.stdout.write(text); sys.stdout.flush()
+            return
+        with capman.global_and_fixture_disabled():
+            sys.stdout.write(text); sys.stdout.flush()
+    return beat

@@ -217,11 +217,17 @@ def test_block_select_indices_exact_and_output(dev, orc, qh, kvh, hd, L, W, bs, 
               f"heads under 1e-6: {[hh for gg, hh in tight if gg < 1e-6]}")
 
 
-def test_block_select_multi_slot_batch4_32k_vs_oracle(dev, orc):
+@pytest.mark.parametrize("backing", [None, 3])
+def test_block_select_multi_slot_batch4_32k_vs_oracle(dev, orc, backing):
     """BASELINE config 5 at batch 4: 32 q / 8 kv heads, hd 128, context 32768, 64-token blocks, top 64 + 512 recent,
-    four slots with different seeds through the multi-slot entry point; outputs vs the oracle per slot, block ids exact."""
+    four slots with different seeds through the multi-slot entry point; outputs vs the oracle per slot, block ids exact.
+    backing None: the reference's q4 V (f32 scale per token and head); 3: V in groups of 32 with f16 scale and minimum,
+    the format the config names."""
     qh, kvh, hd, L, W, bs, top, nseq = 32, 8, 128, 32768, 512, 64, 64, 4
-    kv = m40.KVCache(dev.ctx, L, nseq, kvh, hd, dict(recent_window=W, block_size=bs, top_blocks=top))
+    fmt = dict(recent_window=W, block_size=bs, top_blocks=top)
+    if backing is not None:
+        fmt["exact_old_backing"] = backing
+    kv = m40.KVCache(dev.ctx, L, nseq, kvh, hd, fmt)
     q = np.zeros((nseq, qh, hd), dtype=np.float32)
     caches = []
     for sq in range(nseq):
@@ -231,7 +237,7 @@ def test_block_select_multi_slot_batch4_32k_vs_oracle(dev, orc):
         dk, dv = dev.up(k16), dev.up(v16)
         dev.call("m40llm_ext_kvcache_bulk_fill_f16", kv.h, sq, dk.ptr, dv.ptr, L)
         dk.free(); dv.free()
-        c = orc.CompressedKV(L, 1, kvh, hd, W, bs)
+        c = orc.CompressedKV(L, 1, kvh, hd, W, bs, v_format=1 if backing == 3 else 0)
         c.bulk_fill(0, k16, v16)
         caches.append(c)
     order = np.array([2, 0, 3, 1], dtype=np.uint32)

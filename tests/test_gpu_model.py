@@ -30,7 +30,7 @@ def _toy_cfg(layout, bias, hd=64):
                 rope_base=10000.0 if layout == 0 else 1e6, rope_scale=1.0, rope_layout=layout, qkv_bias=bias)
 
 
-def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0):
+def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0, beat=None):
     """orc_decode_greedy's loop (oracle/oracle.c) driven from here so that every pick's logits row is seen:
     returns ids (prompt + picks), the top-1 / top-2 gap and the largest |logit| of every pick."""
     pos = start_pos
@@ -46,6 +46,8 @@ def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0):
         ids.append(nxt)
         if g + 1 < n_gen:
             hidden = om.token_forward(seq, pos, nxt); pos += 1
+        if beat and g % 8 == 7:
+            beat()
     return np.array(ids, dtype=np.uint32), np.array(gaps), np.array(scale)
 
 
@@ -57,9 +59,12 @@ def _tie_bound(row_scale):
 
 
 def _assert_ids_equal_up_to_legitimate_tie(got, want, gaps, scale, label):
-    """got / want: generated ids only.  Equal everywhere, or equal up to the first divergence, which must be a pick
-    whose oracle gap is inside the tie bound (after it the two runs are different sequences)."""
+    """got / want: generated ids only.  Every pick equal -- unless the first divergence is one of the listed ties, picks
+    whose oracle top-2 gap is inside the tie bound (after it the two runs are different sequences).  The list of such
+    picks is printed; returns the number of equal picks."""
     n = len(want)
+    ties = [i for i in range(n) if gaps[i] <= _tie_bound(scale[i])]
+    print(f"[{label}] picks whose oracle gap is inside the tie bound: {ties if ties else 'none'}")
     diff = np.flatnonzero(np.asarray(got[:n]) != np.asarray(want))
     if diff.size == 0:
         print(f"[{label}] all {n} picks equal; smallest oracle gap {gaps.min():.3e} (tie bound there "
@@ -67,7 +72,7 @@ def _assert_ids_equal_up_to_legitimate_tie(got, want, gaps, scale, label):
         return n
     i = int(diff[0])
     print(f"[{label}] first divergence at pick {i} of {n}: oracle gap {gaps[i]:.3e}, tie bound {_tie_bound(scale[i]):.3e}")
-    assert gaps[i] <= _tie_bound(scale[i]), (label, i, got[i], want[i], gaps[i], _tie_bound(scale[i]))
+    assert i in ties, (label, i, got[i], want[i], gaps[i], _tie_bound(scale[i]))
     return i
 
 
@@ -308,7 +313,7 @@ def test_tinyllama_shape_graph_mode_greedy_ids(ctx, orc):
     dm.close()
 
 
-def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc):
+def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc, heartbeat):
     """BASELINE config 2 at full size (22 layers, 2.07 GB of f16 weights): 32 random prompt ids + 128 greedy tokens.
     (1) Teacher-forced along the oracle's own sequence, the fused kernels' logits of every one of the 128 picks stay
     within 1e-3 of the row's largest magnitude + 1e-4 of the oracle's, and pick the same token unless the oracle's
@@ -321,7 +326,7 @@ def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc):
     om = _oracle_model(orc, cfg, W, S, 1)
     orc.set_threads(16)
     prompt = np.random.default_rng(0).integers(0, cfg["vocab"], size=n_prompt).astype(np.uint32)
-    want, wgap, wscale = _oracle_greedy_with_logits(orc, om, 0, prompt, n_gen)
+    want, wgap, wscale = _oracle_greedy_with_logits(orc, om, 0, prompt, n_gen, beat=heartbeat)
     dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=1)
     # (1) teacher-forced, fused kernels (mode 1): position p holds want[p]; the logits after it pick want[p + 1]
     dm.set_mode(1)
@@ -331,6 +336,8 @@ def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc):
         need = p >= n_prompt - 1
         _, gl = dm.forward_token(0, p, int(want[p]), want_hidden=False, want_logits=need)
         wh = om2.token_forward(0, p, int(want[p]))
+        if p % 16 == 15:
+            heartbeat()
         if not need:
             continue
         wl = om2.logits(wh)
@@ -347,19 +354,20 @@ def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc):
     dm.set_mode(2)
     got, ggap = dm.decode_greedy(0, prompt, n_gen)
     assert np.array_equal(got[:n_prompt], want[:n_prompt])
-    same = _assert_ids_equal_up_to_legitimate_tie(got[n_prompt:], want[n_prompt:], wgap, wscale, "tinyllama-22L graph")
-    assert same >= 8
+    # all 128 picks equal, or equal up to a listed tie (asserted inside; the run on record has no divergence)
+    _assert_ids_equal_up_to_legitimate_tie(got[n_prompt:], want[n_prompt:], wgap, wscale, "tinyllama-22L graph")
     dm.close()
 
 
-def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc):
+def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
     """BASELINE config 3 at full depth: 36 layers (four distinct random layers repeated, every layer its own device
     copy, as the benchmark builds it), hidden 2048, 16 q / 2 kv heads, hd 128, FFN 11008, vocab 151936, biases, NeoX
-    RoPE theta 1e6; batch 8, contexts U[256, 4096] pre-filled N(0,1), 8 greedy steps on the fused graph path against
-    the oracle's per-sequence decode; then the same steps through the reference's row-batched call sequence."""
+    RoPE theta 1e6; batch 8, contexts U[256, 4096] pre-filled N(0,1), 64 greedy steps on the fused graph path.  The
+    oracle decodes the rows with the longest and the shortest context for all 64 steps and the other six rows for 8
+    (about a second of 16 threads per token); then 8 steps of all rows through the reference's row-batched call sequence."""
     cfg = dict(syn.QWEN25_3B)
     W = syn.make_weights(cfg, seed=0, unique_layers=4, tie_embeddings=True)
-    B, steps = 8, 8
+    B, steps, short_steps = 8, 64, 8
     S = 4096 + steps + 8
     L, KVH, HD = cfg["n_layers"], cfg["kv_heads"], cfg["head_dim"]
     rng = np.random.default_rng(0)
@@ -373,7 +381,9 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc):
         for l in range(L):           # every (sequence, layer) slot holds the first lens[s] rows of the same K / V
             Ko[s * L + l, :lens[s]] = k16[:lens[s]]; Vo[s * L + l, :lens[s]] = v16[:lens[s]]
     orc.set_threads(16)
-    want = [_oracle_greedy_with_logits(orc, om, s, [toks[s]], steps, start_pos=int(lens[s])) for s in range(B)]
+    deep = {int(np.argmax(lens)), int(np.argmin(lens))}
+    n_steps = [steps if s in deep else short_steps for s in range(B)]
+    want = [_oracle_greedy_with_logits(orc, om, s, [toks[s]], n_steps[s], start_pos=int(lens[s]), beat=heartbeat) for s in range(B)]
     dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=B)
     dk, dv = ctx.to_device(k16), ctx.to_device(v16)
     for mode in (2, 0):
@@ -383,12 +393,14 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc):
                 slot = dm.H.m40host_model_kv_slot(dm.h, s, l)
                 m40.check(ctx.lib.m40llm_ext_kvcache_bulk_fill_f16(ctx.h, dm.kv_handle(), slot, dk.ptr, dv.ptr, int(lens[s])),
                           "m40llm_ext_kvcache_bulk_fill_f16")
-        ids, gaps = dm.decode_batch_greedy(np.arange(B), lens, toks, steps)
+        run_steps = steps if mode == 2 else short_steps
+        ids, gaps = dm.decode_batch_greedy(np.arange(B), lens, toks, run_steps)
         for s in range(B):
             wid, wgap, wscale = want[s]
-            same = _assert_ids_equal_up_to_legitimate_tie(ids[s], wid[1:], wgap, wscale, f"qwen-36L B=8 mode {mode} row {s}")
-            assert same >= 1
-        print(f"[qwen-36L B=8 mode {mode}] min device top-2 gap over {B * steps} picks: {gaps.min():.3e}")
+            n = min(n_steps[s], run_steps)
+            _assert_ids_equal_up_to_legitimate_tie(ids[s][:n], wid[1:1 + n], wgap[:n], wscale[:n],
+                                                   f"qwen-36L B=8 mode {mode} row {s} ({n} steps, context {int(lens[s])})")
+        print(f"[qwen-36L B=8 mode {mode}] min device top-2 gap over {B * run_steps} picks: {gaps.min():.3e}")
     dk.free(); dv.free()
     dm.close()
 

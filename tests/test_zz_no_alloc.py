@@ -66,3 +66,34 @@ def test_static_scratch_argument_codes_and_size_limit(dev):
     dev.call(name, big.h, 0, dq.ptr, qh, L // 2, out.ptr)      # half the chunks fit
     dev.sync()
     big.destroy()
+
+
+def test_static_scratch_second_context_is_refused_while_busy(dev, orc):
+    """The fixed array is one per GPU: a call from another context while the last user's launches are still outstanding
+    returns -10 (busy) instead of racing; once that work has finished the call goes through and gives the arena path's
+    bits."""
+    qh, kvh, hd, L = 64, 8, 128, 60000
+    rng = np.random.default_rng(5)
+    k16 = f16bits(rng.standard_normal((L, kvh, hd), dtype=np.float32))
+    v16 = f16bits(rng.standard_normal((L, kvh, hd), dtype=np.float32))
+    name = "m40llm_ext_attention_last_token_f32_gqa_static_scratch_async"
+    other = Dev()
+    kv1, kv2 = m40.KVCache(dev.ctx, L, 1, kvh, hd), m40.KVCache(other.ctx, L, 1, kvh, hd)
+    dev.fill_dense(kv1, 0, k16, v16); other.fill_dense(kv2, 0, k16, v16)
+    q = rng.standard_normal(qh * hd).astype(np.float32)
+    dq1, dq2 = dev.up(q), other.up(q)
+    o1, o2, o3 = dev.zeros(qh * hd * 4), other.zeros(qh * hd * 4), other.zeros(qh * hd * 4)
+    dev.sync(); other.sync()
+    for _ in range(4):                      # a few launches in a row keep the first context's stream busy
+        dev.call(name, kv1.h, 0, dq1.ptr, qh, L, o1.ptr)
+    rc = getattr(other.lib, name)(other.h, kv2.h, 0, dq2.ptr, qh, L, o2.ptr)
+    assert rc in (0, -10), rc
+    dev.sync(); other.sync()
+    other.call(name, kv2.h, 0, dq2.ptr, qh, L, o2.ptr)
+    other.call("m40llm_attention_last_token_f32_gqa_async", kv2.h, 0, dq2.ptr, qh, L, o3.ptr)
+    other.sync()
+    got = o2.download(np.float32, (qh * hd,))
+    assert np.array_equal(got, o3.download(np.float32, (qh * hd,)))
+    assert np.array_equal(got, o1.download(np.float32, (qh * hd,)))
+    print(f"[static scratch] second context while busy returned {rc}")
+    kv1.destroy(); kv2.destroy()
