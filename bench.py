@@ -147,6 +147,17 @@ def measured_traffic(kernel):
         return None
 
 
+def trace_duration(kernel, key):
+    """Average start-to-end duration of a kernel inside the decoded tokens / steps of the committed rocprofv3 kernel
+    trace of this same command (profiles/kernel_trace_durations.json), or None."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "kernel_trace_durations.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel, {}).get(key)
+    except (OSError, ValueError):
+        return None
+
+
 def host_cpu():
     """CPU model string and the cores this process may run on."""
     model = "unknown"
@@ -254,6 +265,15 @@ def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
     yard = plain_read_yardstick(pkg, ctx, gate_up_bytes)
     for b in (xa, x1, hid, xo):
         b.free()
+    gate_up_traffic = None
+    try:
+        with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "kernel_counters.json")) as f:
+            gate_up_traffic = json.load(f)["decode_b8"]["rows_mfma_kernel<1, 8>@131072"]["hbm_bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        pass
+    gate_up_trace_us = trace_duration("rows_mfma_kernel<1, 8>", "in_step_avg_us")
+    gate_up_live_us = gate_up_us
+    gate_up_us = max(gate_up_live_us, gate_up_trace_us) if gate_up_trace_us else gate_up_live_us
     wbytes = L * 2 * (D * (D + 2 * KV) + D * D + 3 * D * F) + 2 * V * D
     kvbytes = int(lens.sum() + B * (warmup + steps / 2)) * L * KV * 2 * 2
     fallback = dm.last_timed_host_fallback()
@@ -269,11 +289,17 @@ def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
                         "algorithmic_bytes_per_launch": gate_up_bytes,
                         "achieved": gate_up_bytes / (gate_up_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                         "frac": gate_up_bytes / (gate_up_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                        # in_step_us: the launch inside the chain O projection -> gate/up -> down projection (chain with minus
-                        # chain without, per layer); back_to_back_us: launches of this kernel alone, one after the other
-                        "in_step_us": gate_up_us, "back_to_back_us": gate_up_b2b_us,
+                        # avg_launch_us (what achieved and frac follow from): the larger of in_chain_us -- live: the chain O
+                        # projection -> gate/up -> down projection over the layers, with minus without the kernel, per layer -- and
+                        # trace_in_step_us, the kernel's start-to-end time inside the steps of the committed rocprofv3 trace;
+                        # back_to_back_us: launches of this kernel alone, one after the other
+                        "avg_launch_us": gate_up_us, "in_chain_us": gate_up_live_us, "trace_in_step_us": gate_up_trace_us,
+                        "trace_source": "profiles/kernel_trace_durations.json", "back_to_back_us": gate_up_b2b_us,
                         "plain_read_us": yard["us"], "plain_read_workgroups": yard["workgroups"],
-                        "frac_of_plain_read": yard["us"] / gate_up_us, "traffic": None}}
+                        "frac_of_plain_read": yard["us"] / gate_up_us,
+                        # HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, scaled by a copy
+                        # of known size): not a quantity of this run
+                        "traffic": gate_up_traffic, "traffic_source": "profiles/kernel_counters.json (decode_b8)"}}
     return rec, (cfg, W, lens, k16h, v16h, first)
 
 
@@ -361,9 +387,14 @@ def main():
         ctx.sync(1)
         src.free(); dst.free()
     dom = measure_dominant_kernel(pkg, ctx, dm, cfg, args.kernel_reps, mode)
-    # the kernel's duration inside a token (in the chain of launches it depends on) where that was measured; launches of
-    # the kernel alone, back to back, overlap their ramps and read faster: kept beside it as back_to_back_*
-    dom_us = dom["in_chain_us"] or dom["avg_us"]
+    # The kernel's duration inside a token: live, from the chain of launches it depends on (chain with minus chain
+    # without); launches of the kernel alone, back to back, overlap their ramps and read faster (kept as back_to_back_*).
+    # The committed kernel trace of this command gives the kernel's own start-to-end time inside graph-replayed tokens;
+    # the chain difference can hide part of the kernel behind its neighbours, so the larger of the two is what achieved
+    # and frac are computed from.
+    trace_us = trace_duration(dom["kernel"], "in_token_avg_us")
+    live_us = dom["in_chain_us"] or dom["avg_us"]
+    dom_us = max(live_us, trace_us) if trace_us else live_us
     achieved = dom["bytes"] / (dom_us * 1e-6) / 1e9
     yard = plain_read_yardstick(pkg, ctx, dom["bytes"])
     token_bytes = algorithmic_bytes_per_token(cfg)
@@ -387,12 +418,15 @@ def main():
                      "traffic_source": "profiles/decode_b1_tinyllama_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                                        "collected beforehand with the same command under the profiler)",
                      "kernel": dom["kernel"], "shape": dom["shape"],
-                     # avg_launch_us: what achieved / frac are computed from: the kernel inside the chain of launches of a token
-                     # (O projection -> this kernel -> down projection over all layers between one pair of events, minus the
-                     # same chain without it, per layer).  back_to_back_us: launches of this kernel alone, one after the other
-                     # (their ramps overlap).  event_pair_us: one event pair around every launch inside that chain (includes
-                     # the wait for the launch before)
+                     # avg_launch_us: what achieved / frac are computed from: the larger of in_chain_us (live: the chain O
+                     # projection -> this kernel -> down projection over all layers between one pair of events, minus the same
+                     # chain without it, per layer) and trace_in_token_us (the kernel's start-to-end time inside the decoded
+                     # tokens of the committed rocprofv3 trace of this command).  back_to_back_us: launches of this kernel alone,
+                     # one after the other (their ramps overlap).  event_pair_us: one event pair around every launch inside
+                     # that chain (includes the wait for the launch before)
                      "avg_launch_us": dom_us, "launches_timed": dom["launches"],
+                     "in_chain_us": live_us, "trace_in_token_us": trace_us,
+                     "trace_source": "profiles/kernel_trace_durations.json (rocprofv3 --kernel-trace of this command, collected beforehand)",
                      "back_to_back_us": dom["avg_us"],
                      "back_to_back_frac": dom["bytes"] / (dom["avg_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
                      "event_pair_us": dom["in_token_us"],
