@@ -10,7 +10,9 @@
 //     a = 2^E * (d1 + d2 / 128 + d3 / 16384),   |d1| <= 64, |d2|, |d3| <= 64,   error <= 2^-20 of the block's largest,
 // each digit plane is one matrix instruction, the three exact i32 results are recombined once per block, and the
 // block's factor 2^E * d_w multiplies them in f32.  No weight is converted and no product is rounded before that.
-// Up to four rows the three planes of all rows are stacked into the 16 operand rows: one instruction per block.
+// Up to four rows the three planes of all rows are stacked into the 16 operand rows: one instruction per block.  Five to
+// eight rows take two operands per block -- digits 1 and 2 of the eight rows fill the sixteen rows of the first, digit 3
+// the low half of the second -- two instructions and two thirds of the plane bytes.
 //
 // Launches: a small pack kernel turns the f32 rows into digit planes (laid out in the order the A operand is
 // loaded), then the product kernel; the FFN form packs its SwiGLU output itself (a workgroup produces whole
@@ -33,10 +35,15 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 //   MP = 0, "stacked", for at most four rows: the operand row 4 d + m holds digit d of row m (rows 12-15 zero), so
 //   that a single matrix instruction multiplies all three digits: four planes [block pair][lane = 16 (k / 8) + operand
 //   row][block of the pair][8 bytes], then the scales [block][row < 4].
+//   MP = 8, "two operands", 5 to 8 rows: eight planes [block pair][operand][lane = 16 (k / 8) + operand row][block of
+//   the pair][8 bytes]; operand 0 holds digit 1 of row m in operand row m and digit 2 in operand row 8 + m, operand 1
+//   digit 3 in operand row m and zeros in rows 8-15: two matrix instructions per block instead of three, two thirds of
+//   the plane bytes.  Then the scales [block][operand row], rows 8-15 repeating rows 0-7.
 constexpr int kStepBlocks = 8;
 constexpr int kStackStepBytes = 4 * 1024 + kStepBlocks * 4 * 4;        // 4224
 constexpr int kPlaneStepBytes = 12 * 1024 + kStepBlocks * 16 * 4;      // 12800
-__host__ __device__ constexpr int q80i8_step_bytes(int MP) { return MP == 0 ? kStackStepBytes : kPlaneStepBytes; }
+constexpr int kTwoStepBytes = 8 * 1024 + kStepBlocks * 16 * 4;         // 8704
+__host__ __device__ constexpr int q80i8_step_bytes(int MP) { return MP == 0 ? kStackStepBytes : (MP == 8 ? kTwoStepBytes : kPlaneStepBytes); }
 
 // Digits of one element under its block's scale: n = rint(v * 2^(20 - ex)), |n| <= 2^20, cut into balanced base-128
 // digits n = (d1 * 128 + d2) * 128 + d3 with d2, d3 in [-64, 63] and |d1| <= 64 (exact integer arithmetic, one rounding).
@@ -87,6 +94,23 @@ __device__ __forceinline__ void q80i8_pack_pair(float v0, float v1, int m, int p
             if (pair == 0) reinterpret_cast<float*>(step + 64 * 64)[b * 4 + m] = mx < INFINITY ? ldexpf(1.0f, ex - 20) : block_scale_bad;
         } else if (m >= 12) {
             *reinterpret_cast<uint16_t*>(step + (b >> 1) * 1024 + (kg * 16 + m) * 16 + (b & 1) * 8 + kb) = 0;
+        }
+        return;
+    }
+    if (MP == 8) {
+        uint8_t* step = pack + (size_t)(blk / kStepBlocks) * kTwoStepBytes;
+        if (m < 8) {
+            // (operand, operand row): digit 1 -> (0, m), digit 2 -> (0, 8 + m), digit 3 -> (1, m), zeros -> (1, 8 + m)
+            const uint16_t two[4] = {(uint16_t)((d[0][0] & 0xff) | ((d[0][1] & 0xff) << 8)), (uint16_t)((d[1][0] & 0xff) | ((d[1][1] & 0xff) << 8)),
+                                     (uint16_t)((d[2][0] & 0xff) | ((d[2][1] & 0xff) << 8)), (uint16_t)0};
+#pragma unroll
+            for (int o = 0; o < 4; ++o)
+                *reinterpret_cast<uint16_t*>(step + ((b >> 1) * 2 + (o >> 1)) * 1024 + (kg * 16 + (o & 1) * 8 + m) * 16 + (b & 1) * 8 + kb) = two[o];
+            if (pair == 0) {
+                const float sc = mx < INFINITY ? ldexpf(1.0f, ex - 20) : block_scale_bad;
+                reinterpret_cast<float*>(step + 8 * 1024)[b * 16 + m] = sc;
+                reinterpret_cast<float*>(step + 8 * 1024)[b * 16 + 8 + m] = sc;
+            }
         }
         return;
     }
@@ -161,9 +185,9 @@ constexpr int kTileBytes = 16 * kColStride;
 // Activation operand of one step as loaded: the lane's 16 bytes of every plane, and its block scales.  Three-plane
 // form: e[h] = the scales of block 4 h + (lane & 3) for the lane's four output rows -- the four lanes of a quad hold the
 // four blocks, and the arithmetic fetches block b's from quad lane b & 3.  Stacked form: one scale per lane 0-31.
-template <bool STACK>
+template <bool STACK, bool TWO = false>
 struct Q80I8Acts {
-    uint4 pl[STACK ? 4 : 12];
+    uint4 pl[STACK ? 4 : (TWO ? 8 : 12)];
     float4 e[STACK ? 1 : 2];
     float sv;
 };
@@ -199,8 +223,12 @@ __device__ __forceinline__ void q80i8_unrolled(std::integer_sequence<int, I...>,
 // DEPTH: steps in flight per wave, 0 = the form's default.  What pays is about 70 KB of weight requests outstanding per
 // CU, not more (measured: 104 KB and 139 KB are slower, 35 KB too): a launch that puts two workgroups on a CU runs
 // with half the depth of one that puts one there.
-template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1, bool SELF = false, int DEPTH = 0>
+// TWO (not STACK): the two-operand form of 5 to 8 rows (digits 1 and 2 of the eight rows in one operand, digit 3 in the low
+// half of a second): two matrix instructions per block and tile.
+template <int MODE, int KSPLIT, bool STACK, int T = 1, int WAVES = 4, int KHALVES = 1, bool SELF = false, int DEPTH = 0,
+          bool TWO = false>
 __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) {
+    static_assert(!TWO || !STACK, "two operands: a form of the unstacked kernel");
     static_assert(!SELF || (STACK && MODE == 1 && KSPLIT == 1 && WAVES == 4), "self-packing: the stacked gate + up launch");
     extern __shared__ __attribute__((aligned(16))) uint8_t q80i8_planes[];    // SELF: [step][4224]
     static_assert(KHALVES == 1 || (KHALVES == 2 && MODE == 0), "halves of K are added into a cleared result");
@@ -267,9 +295,9 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
     // STACK: the 32 block scales of a step (8 blocks x 4 rows), one per lane 0-31, fetched with one load per step;
     // three planes: [block][row] f32, the lane takes rows 4 g .. 4 g + 3 of blocks (lane & 3) and 4 + (lane & 3)
     const uint32_t sv_off = (uint32_t)(4 * 1024 + (lane & 31) * 4);
-    const uint32_t e_off = (uint32_t)(12 * 1024 + (lane & 3) * 64 + g * 16);
-    constexpr int kStepBytes = STACK ? kStackStepBytes : kPlaneStepBytes;
-    constexpr int kPlanes = STACK ? 4 : 12;
+    const uint32_t e_off = (uint32_t)((TWO ? 8 : 12) * 1024 + (lane & 3) * 64 + g * 16);
+    constexpr int kStepBytes = STACK ? kStackStepBytes : (TWO ? kTwoStepBytes : kPlaneStepBytes);
+    constexpr int kPlanes = STACK ? 4 : (TWO ? 8 : 12);
     constexpr int D = DEPTH ? DEPTH : (STACK ? (T == 1 ? 4 : 2) : 2);   // steps in flight (two 32-column steps are as many bytes as four of 16
                                                  // columns; the three-plane form has no registers for more)
 
@@ -289,14 +317,14 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
         __builtin_amdgcn_sched_barrier(0);
     }
     WPiece wr[D][kWLoads];
-    Q80I8Acts<STACK> acts[D];
+    Q80I8Acts<STACK, TWO> acts[D];
     auto issue_w = [&](WPiece (&dst)[kWLoads], int step) {
         step = step < s1 ? step : s1 - 1;
         const uint8_t* base = w_base + (size_t)step * (34 * kStepBlocks);
 #pragma unroll
         for (int i = 0; i < kWLoads; ++i) dst[i] = *reinterpret_cast<const WPiece*>(base + w_off[i]);
     };
-    auto issue_a = [&](Q80I8Acts<STACK>& act, int step) {
+    auto issue_a = [&](Q80I8Acts<STACK, TWO>& act, int step) {
         step = step < s1 ? step : s1 - 1;
         const uint8_t* base = p.pack + (size_t)step * kStepBytes;                    // uniform
 #pragma unroll
@@ -335,7 +363,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
                                  : make_uint2(__builtin_amdgcn_alignbyte(r.w1, r.w0, 2), __builtin_amdgcn_alignbyte(r.w2, r.w1, 2));
         return WOperand{__builtin_bit_cast(long, bq), m40_h2f(r.d)};
     };
-    auto compute_block = [&](const Q80I8Acts<STACK>& act, auto b_c, const WOperand (&w)[T]) {
+    auto compute_block = [&](const Q80I8Acts<STACK, TWO>& act, auto b_c, const WOperand (&w)[T]) {
         constexpr int b = decltype(b_c)::value;
         const i32x4 z = {0, 0, 0, 0};
         auto half = [](const uint4& two) { return __builtin_bit_cast(long, (b & 1) ? make_uint2(two.z, two.w) : make_uint2(two.x, two.y)); };
@@ -351,6 +379,28 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[t][r] = fmaf(sa[r] * dw, (float)rr[r], acc[t][r]);
             }
+        } else if constexpr (TWO) {
+            const long a0 = half(act.pl[(b >> 1) * 2]), a1 = half(act.pl[(b >> 1) * 2 + 1]);
+            constexpr int kQuad = (b & 3) * 0x55;
+            const float4 eh = act.e[b >> 2];
+#define M40_FROM_QUAD(v) __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), kQuad, 0xf, 0xf, true))
+            const float sa[4] = {M40_FROM_QUAD(eh.x), M40_FROM_QUAD(eh.y), M40_FROM_QUAD(eh.z), M40_FROM_QUAD(eh.w)};
+#undef M40_FROM_QUAD
+            // operand rows 0-7 (lanes g < 2): digit 1 in the first product, digit 3 in the second; rows 8-15: digit 2, zero
+            const float wgt = g < 2 ? 16384.0f : 128.0f;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const long B = w[t].B;
+                const float dw = w[t].dw;
+                const i32x4 r1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a0, B, z, 0, 0, 0);
+                const i32x4 r2 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a1, B, z, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][r] = fmaf(sa[r] * dw, fmaf((float)r1[r], wgt, (float)r2[r]), acc[t][r]);
+            }
+#pragma unroll
+            for (int t = 0; t < T; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) asm volatile("" : "+v"(acc[t][r]));
         } else {
             const long a0 = half(act.pl[(b >> 1) * 3]), a1 = half(act.pl[(b >> 1) * 3 + 1]), a2 = half(act.pl[(b >> 1) * 3 + 2]);
             // the block's scales sit in quad lane b & 3
@@ -414,7 +464,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
             __syncthreads();
         }
         // SELF: the planes of a step are read from LDS one step ahead of their use
-        Q80I8Acts<STACK> lds_next;
+        Q80I8Acts<STACK, TWO> lds_next;
         auto read_planes = [&](int s) {
             const uint8_t* base = q80i8_planes + (s < s1 ? s : s1 - 1) * kStackStepBytes;
 #pragma unroll
@@ -424,12 +474,12 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
         if constexpr (SELF) read_planes(s0);
         auto step = [&](auto set_c, int s) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
-            Q80I8Acts<STACK> from_lds;
+            Q80I8Acts<STACK, TWO> from_lds;
             if constexpr (SELF) {
                 from_lds = lds_next;
                 read_planes(s + 1);
             }
-            const Q80I8Acts<STACK>& act_now = SELF ? from_lds : acts[SET];
+            const Q80I8Acts<STACK, TWO>& act_now = SELF ? from_lds : acts[SET];
             // weights of this step -> the wave's LDS tile (waits for them and for everything older: this step's
             // activations; the younger steps stay in flight)
 #pragma unroll
@@ -470,6 +520,13 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
         });
     }
 
+    if (TWO) {
+        // lanes g and g + 2 hold the (digit 1, digit 3) and the digit 2 part of rows 4 (g & 1) + r: both get the sum
+#pragma unroll
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[t][r] += __shfl_xor(acc[t][r], 32, 64);
+    }
     if (STACK) {
         // lane (j, g) holds digit g of rows r: the three sums meet in the lanes g = 0
 #pragma unroll
@@ -548,7 +605,14 @@ bool m40_q80_i8_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, in
     return pack_bytes(K) <= ctx->scratch[stream_kind].gemm_pack_bytes;
 }
 
-static int rows_padded(int M) { return M <= 4 ? 0 : 16; }   // 0: the stacked form
+static int rows_padded(int M) { return M <= 4 ? 0 : (M <= 8 ? 8 : 16); }   // 0: the stacked form, 8: two operands, 16: three planes
+
+// the unstacked kernel in its three-plane (MP 16) or two-operand (MP 8) form
+#define M40_Q80_UNSTACKED(MP, GRID, THREADS, ARGS, ...)                                                             \
+    do {                                                                                                            \
+        if ((MP) == 8) q80i8_gemm_kernel<__VA_ARGS__, true><<<(GRID), (THREADS), 0, stream>>>(ARGS);                \
+        else q80i8_gemm_kernel<__VA_ARGS__, false><<<(GRID), (THREADS), 0, stream>>>(ARGS);                         \
+    } while (0)
 
 static void launch_gemm0(hipStream_t stream, const Q80I8Args& a) {
     const int tiles = (a.N + 15) / 16;
@@ -567,13 +631,13 @@ static void launch_gemm0(hipStream_t stream, const Q80I8Args& a) {
     // K = 14336: 24.4 -> 23.5 us; two tiles per wave there would leave 128 workgroups: 31.5 us)
     const int pairs = (tiles + 1) / 2;
     if (whole_k) {
-        if ((pairs + 3) / 4 >= 192) q80i8_gemm_kernel<0, 1, false, 2><<<(pairs + 3) / 4, 256, 0, stream>>>(a);
-        else q80i8_gemm_kernel<0, 1, false><<<(tiles + 3) / 4, 256, 0, stream>>>(a);
+        if ((pairs + 3) / 4 >= 192) M40_Q80_UNSTACKED(a.MP, (pairs + 3) / 4, 256, a, 0, 1, false, 2, 4, 1, false, 0);
+        else M40_Q80_UNSTACKED(a.MP, (tiles + 3) / 4, 256, a, 0, 1, false, 1, 4, 1, false, 0);
     } else {
-        if (pairs > 256) q80i8_gemm_kernel<0, 4, false, 2, 4, 1, false, 1><<<pairs, 256, 0, stream>>>(a);   // two workgroups per CU
-        else if (pairs >= 192) q80i8_gemm_kernel<0, 4, false, 2><<<pairs, 256, 0, stream>>>(a);
-        else if (nsteps >= 16) q80i8_gemm_kernel<0, 8, false, 1, 8><<<tiles, 512, 0, stream>>>(a);
-        else q80i8_gemm_kernel<0, 4, false><<<tiles, 256, 0, stream>>>(a);
+        if (pairs > 256) M40_Q80_UNSTACKED(a.MP, pairs, 256, a, 0, 4, false, 2, 4, 1, false, 1);   // two workgroups per CU
+        else if (pairs >= 192) M40_Q80_UNSTACKED(a.MP, pairs, 256, a, 0, 4, false, 2, 4, 1, false, 0);
+        else if (nsteps >= 16) M40_Q80_UNSTACKED(a.MP, tiles, 512, a, 0, 8, false, 1, 8, 1, false, 0);
+        else M40_Q80_UNSTACKED(a.MP, tiles, 256, a, 0, 4, false, 1, 4, 1, false, 0);
     }
 }
 
@@ -594,7 +658,7 @@ int m40_launch_q80_i8(M40llmCudaContext* ctx, hipStream_t stream, uint32_t strea
     if (apart && 2 * pairs >= 192 && 2 * pairs <= 1024 && K / (32 * kStepBlocks) >= 32) {
         q80i8_pack_kernel<<<K >> 5, 256, 0, stream>>>(A, M, MP, K, pack, C, M * N);
         if (MP == 0) q80i8_gemm_kernel<0, 4, true, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(a);
-        else q80i8_gemm_kernel<0, 4, false, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(a);
+        else M40_Q80_UNSTACKED(MP, 2 * pairs, 256, a, 0, 4, false, 2, 4, 2, false, 0);
         return hipGetLastError() == hipSuccess ? 0 : -2;
     }
     q80i8_pack_kernel<<<K >> 5, 256, 0, stream>>>(A, M, MP, K, pack, nullptr, 0);
@@ -639,14 +703,14 @@ int m40_launch_q80_i8_ffn(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
     } else if (MP == 0 && two_tiles) q80i8_gemm_kernel<1, 1, true, 2><<<ffn / 64, 256, 0, stream>>>(a);
     else if (MP == 0) q80i8_gemm_kernel<1, 1, true><<<ffn / 32, 256, 0, stream>>>(a);
     // (a workgroup of two column groups x two K halves, two waves per SIMD instead of one: measured, 64.5 -> 66 us)
-    else if (ffn % 64 == 0 && ffn / 64 >= 192) q80i8_gemm_kernel<1, 1, false, 2><<<ffn / 64, 256, 0, stream>>>(a);
-    else q80i8_gemm_kernel<1, 1, false><<<ffn / 32, 256, 0, stream>>>(a);
+    else if (ffn % 64 == 0 && ffn / 64 >= 192) M40_Q80_UNSTACKED(MP, ffn / 64, 256, a, 1, 1, false, 2, 4, 1, false, 0);
+    else M40_Q80_UNSTACKED(MP, ffn / 32, 256, a, 1, 1, false, 1, 4, 1, false, 0);
     Q80I8Args b{};
     b.pack = hp; b.W0 = wd; b.C = out; b.M = M; b.MP = MP; b.N = d_model; b.K = ffn;
     if (halves) {
         const int pairs = (d_model + 31) / 32;
         if (MP == 0) q80i8_gemm_kernel<0, 4, true, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(b);
-        else q80i8_gemm_kernel<0, 4, false, 2, 4, 2><<<2 * pairs, 256, 0, stream>>>(b);
+        else M40_Q80_UNSTACKED(MP, 2 * pairs, 256, b, 0, 4, false, 2, 4, 2, false, 0);
     } else {
         launch_gemm0(stream, b);
     }
