@@ -9,11 +9,18 @@
 // precision.  The global loads of the next three steps are in flight (three rotating register sets) while a step
 // computes from one LDS buffer and the following step's data moves into the other: one barrier per step.
 //
+// Large grids (at least one 128 x 256 tile per CU) take a second kernel built the same way round a wider tile and the
+// direct global-to-LDS loads of gfx950 (gemm_tiled_wide_kernel, below): what bounded the 128 x 128 kernel was not
+// arithmetic but the issue of its memory instructions, all of them between the barrier and the first matrix instruction.
+//
 // The split is done once per call by a packing pass (A -> two f16 planes in a per-stream buffer that grows on
 // demand), so the 128 x 128 tiles along N do not each repeat it.  When the buffer cannot be grown (the stream is being
 // captured) the launch is declined and the caller falls back to the skinny kernels.  Several weight matrices that
 // share A (Q/K/V, gate/up) can be served by one packing pass and one launch.
 #include "common.hpp"
+
+#include <type_traits>
+#include <utility>
 
 namespace {
 
@@ -197,6 +204,189 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
     }
 }
 
+// ---- wide tile: 128 x 256 per workgroup of four waves (wave tile 64 x 128), one workgroup per CU ---------------------------
+//
+// Measured on the 128 x 128 kernel above with parts of it switched off (M 4096, N 2048, K 2048): arithmetic alone 46 us,
+// loads + LDS traffic + barriers alone 45 us, everything 87 us -- the two did not overlap.  A wave issues in order, and a
+// memory instruction holds the issue slot until its unit accepts it; with the four waves of a CU in step behind the
+// barrier, sixteen fragment reads, eight LDS writes and eight global loads each queue for ~500 cycles before the first
+// matrix instruction of the step can go.  Here:
+//  * every memory instruction of a step is issued under the step's matrix instructions, one per two of them
+//    (sched_group_barrier), so it waits for its unit while the matrix pipe works;
+//  * the fragments of step s + 1 are read from LDS during the arithmetic of step s (two fragment sets in registers);
+//  * global data goes straight into LDS (global_load_lds_dwordx4: no registers, no LDS write instruction, no wait
+//    before one), five 32 KB buffers deep -- a lane fetches the 16-byte chunk that belongs at its place in the swizzled
+//    row layout, so a wave's instruction fills one contiguous kilobyte; the workgroup waits only for the step after
+//    next (vmcnt) ahead of the barrier that publishes it;
+//  * the wave tile is 64 x 128: per matrix instruction two thirds of the fragment bytes of a 64 x 64 tile (the activation
+//    rows, read twice -- high and low part -- are the short side).
+// M 4096, N 2048, K 2048: 79 -> 60 us; N 11264: 479 -> 404 us; K 5632: 232 -> 173 us.  Under this load the part lowers
+// its clock (1.4-1.9 GHz measured inside the kernel, against 2.0-2.2 GHz in short or memory-bound launches), and a form
+// with fewer issue cycles (32 x 32 x 16 instructions: 1370 instead of 1500 cycles per step) ran at a lower clock
+// still and took the same time: what is left is energy per product, of which the exact hi + lo split is half.
+constexpr int kWideBN = 256;
+constexpr int kWideWM = 64, kWideWN = 128;                   // wave tile, waves 2 x 2
+constexpr int kWideMT = kWideWM / 16, kWideNT = kWideWN / 16;
+constexpr int kWidePlane = kBM * 64;                          // bytes of a 128-row operand block (32 k)
+constexpr int kWideBuf = 2 * kWidePlane + kWideBN * 64;      // A high, A low, B: 32 KB
+constexpr int kWideBufs = 5;
+constexpr int kWideLds = kWideBufs * kWideBuf;               // 160 KB: the whole LDS of a CU
+constexpr int kWideAL = kBM / 64, kWideBL = kWideBN / 64;    // 16-byte loads per thread: rows lrow + 64 i of a plane
+constexpr int kWideLoads = 2 * kWideAL + kWideBL;
+
+struct WideFrags { half8 hi[kWideMT], lo[kWideMT], b[kWideNT]; };
+
+template <int... I, class F>
+__device__ __forceinline__ void tiled_unrolled(std::integer_sequence<int, I...>, F&& f) { (f(std::integral_constant<int, I>{}), ...); }
+
+// s_waitcnt for vector-memory operations only: at most n of them may still be outstanding
+__device__ __forceinline__ constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
+
+__global__ __launch_bounds__(kThreads, 1) void gemm_tiled_wide_kernel(const _Float16* __restrict__ A_hi,
+                                                                      const _Float16* __restrict__ A_lo, TiledMats mats,
+                                                                      int M, int K) {
+    typedef __attribute__((address_space(3))) void* lds_dst_t;
+    typedef const __attribute__((address_space(1))) void* global_src_t;
+    extern __shared__ __align__(16) uint8_t wide_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tiles_n = mats.tile_start[mats.n];
+    // each die owns a contiguous band of tile rows, as above
+    const int per_die = (int)gridDim.x / 8;
+    const int logical = (int)blockIdx.x < per_die * 8 ? ((int)blockIdx.x % 8) * per_die + (int)blockIdx.x / 8 : (int)blockIdx.x;
+    const int tile_m = logical / tiles_n;
+    int tile_n = logical % tiles_n;
+    int mat = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMats; ++i)
+        if (i < mats.n && tile_n >= mats.tile_start[i]) mat = i;
+    tile_n -= mats.tile_start[mat];
+    const uint16_t* __restrict__ B = mats.B[mat];
+    float* __restrict__ C = mats.C[mat];
+    const int N = mats.N[mat];
+    const int m0 = tile_m * kBM, n0 = tile_n * kWideBN;
+    // loader: thread -> row lrow (+ 64 i) of a plane and the place tid % 4 in that row's 64 bytes, which holds chunk
+    // (tid % 4) ^ ((lrow / 4) % 4) of the row; the host guarantees that M * K and N * K fit 31 bits
+    const int lrow = tid >> 2, gchunk = (tid & 3) ^ ((lrow >> 2) & 3);
+    uint32_t a_off[kWideAL], b_off[kWideBL];     // in halves
+#pragma unroll
+    for (int i = 0; i < kWideAL; ++i) {
+        const int ar = m0 + lrow + 64 * i < M ? m0 + lrow + 64 * i : M - 1;     // clamped: computed, never stored
+        a_off[i] = (uint32_t)ar * (uint32_t)K + gchunk * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < kWideBL; ++i) {
+        const int bc = n0 + lrow + 64 * i < N ? n0 + lrow + 64 * i : N - 1;
+        b_off[i] = (uint32_t)bc * (uint32_t)K + gchunk * 8;
+    }
+    const int steps = K / kBK, last = steps - 1;
+    // one instruction of a wave fills rows 16 wave .. 16 wave + 15 (+ 64 i) of a plane: a contiguous kilobyte, lane by lane
+    auto issue = [&](int buf, int step) {
+        step = step < last ? step : last;          // past the end: the last step again (no branch around loads)
+        const _Float16* ah = A_hi + (size_t)step * kBK;
+        const _Float16* al = A_lo + (size_t)step * kBK;
+        const uint16_t* bb = B + (size_t)step * kBK;
+        uint8_t* dst = wide_lds + buf * kWideBuf + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < kWideAL; ++i) {
+            __builtin_amdgcn_global_load_lds((global_src_t)(ah + a_off[i]), (lds_dst_t)(dst + i * 4096), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_src_t)(al + a_off[i]), (lds_dst_t)(dst + kWidePlane + i * 4096), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < kWideBL; ++i)
+            __builtin_amdgcn_global_load_lds((global_src_t)(bb + b_off[i]), (lds_dst_t)(dst + 2 * kWidePlane + i * 4096), 16, 0, 0);
+    };
+    const int wm = wave >> 1, wn = wave & 1;
+    const int frag_row = lane & 15;
+    const int fr_off = frag_row * 64 + (((lane >> 4) ^ ((frag_row >> 2) & 3)) * 16);
+    auto read_frags = [&](WideFrags& f, int buf) {
+        const uint8_t* base = wide_lds + buf * kWideBuf + fr_off;
+        const uint8_t* a = base + wm * kWideWM * 64;
+        const uint8_t* b = base + 2 * kWidePlane + wn * kWideWN * 64;
+#pragma unroll
+        for (int mt = 0; mt < kWideMT; ++mt) {
+            f.hi[mt] = *reinterpret_cast<const half8*>(a + mt * 16 * 64);
+            f.lo[mt] = *reinterpret_cast<const half8*>(a + kWidePlane + mt * 16 * 64);
+        }
+#pragma unroll
+        for (int nt = 0; nt < kWideNT; ++nt) f.b[nt] = *reinterpret_cast<const half8*>(b + nt * 16 * 64);
+    };
+    floatx4 acc[kWideMT][kWideNT];
+#pragma unroll
+    for (int i = 0; i < kWideMT; ++i)
+#pragma unroll
+        for (int j = 0; j < kWideNT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // per accumulator the same order as the 128 x 128 kernel (step by step, high part then low part): the same bits
+    auto compute = [&](const WideFrags& f) {
+#pragma unroll
+        for (int mt = 0; mt < kWideMT; ++mt) {
+#pragma unroll
+            for (int nt = 0; nt < kWideNT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.hi[mt], f.b[nt], acc[mt][nt], 0, 0, 0);
+#pragma unroll
+            for (int nt = 0; nt < kWideNT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f.lo[mt], f.b[nt], acc[mt][nt], 0, 0, 0);
+        }
+    };
+
+    WideFrags f[2];
+    // steps 0 .. 4 requested, one per buffer; steps 0 and 1 awaited.  The barriers are bare s_barrier instructions with
+    // the vector-memory wait written out: __syncthreads() would wait for every outstanding load (its fence covers LDS).
+#pragma unroll
+    for (int i = 0; i < kWideBufs; ++i) issue(i, i);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(vmcnt_only((kWideBufs - 2) * kWideLoads));
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(f[0], 0);
+    // Before step s: the fragments of step s are requested into f[s % 2]; buffer (s + 1) % 5 is complete and visible;
+    // steps s + 2 .. s + 3 are in flight.  Step s refills the buffer of step s - 1 -- whose fragments every wave had in
+    // registers before the last barrier -- with step s + 4, and waits for step s + 2 ahead of its barrier.  (Step 0
+    // requests step 4 a second time: buffer 0 is still being read then.)
+    constexpr int kPeriod = 2 * kWideBufs;
+    auto step = [&](auto ph_c, int s) __attribute__((always_inline)) {
+        constexpr int ph = decltype(ph_c)::value;
+        read_frags(f[(ph + 1) & 1], (ph + 1) % kWideBufs);
+        issue((ph + kWideBufs - 1) % kWideBufs, s - 1 + kWideBufs);
+        compute(f[ph & 1]);
+        // issue order: two matrix instructions, one LDS read (16 times), then two matrix instructions, one load (8 times)
+#pragma unroll
+        for (int i = 0; i < 2 * kWideMT + kWideNT; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < kWideLoads; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(vmcnt_only((kWideBufs - 3) * kWideLoads));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    int s = 0;
+    for (; s + kPeriod <= steps; s += kPeriod)
+        tiled_unrolled(std::make_integer_sequence<int, kPeriod>(),
+                       [&](auto ph_c) __attribute__((always_inline)) { step(ph_c, s + decltype(ph_c)::value); });
+    tiled_unrolled(std::make_integer_sequence<int, kPeriod - 1>(), [&](auto ph_c) __attribute__((always_inline)) {
+        if (s + decltype(ph_c)::value < steps) step(ph_c, s + decltype(ph_c)::value);
+    });
+    __builtin_amdgcn_s_waitcnt(vmcnt_only(0));      // no write into LDS may be outstanding when the workgroup ends
+
+    const int out_col = lane & 15, out_row = (lane >> 4) * 4;
+#pragma unroll
+    for (int mt = 0; mt < kWideMT; ++mt) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = m0 + wm * kWideWM + mt * 16 + out_row + r;
+            if (row >= M) continue;
+#pragma unroll
+            for (int nt = 0; nt < kWideNT; ++nt) {
+                const int col = n0 + wn * kWideWN + nt * 16 + out_col;
+                if (col < N) C[(size_t)row * N + col] = acc[mt][nt][r];
+            }
+        }
+    }
+}
+
 // out[i] = planes[0][i] + planes[1][i] + ... in that order (n4 float4 per plane)
 __global__ __launch_bounds__(256) void add_k_planes_kernel(const float4* __restrict__ planes, float4* __restrict__ out, size_t n4,
                                                            int k_splits) {
@@ -286,7 +476,27 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
             at += (size_t)k_splits * M * N[i];
         }
     }
-    gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles * k_splits), kThreads, lds_bytes, stream>>>(hi, lo, launch, M, K, k_splits);
+    // the wide tile where it covers the CUs at least once (and element offsets fit the kernel's 32-bit arithmetic)
+    long long wide_tiles_n = 0;
+    TiledMats wide = mats;
+    bool wide_ok = k_splits == 1 && (long long)M * K < 0x7fffffffll;
+    for (int i = 0; i < n_mats; ++i) {
+        wide.tile_start[i] = (int)wide_tiles_n;
+        wide_tiles_n += (N[i] + kWideBN - 1) / kWideBN;
+        wide_ok = wide_ok && (long long)N[i] * K < 0x7fffffffll;
+    }
+    wide.tile_start[n_mats] = (int)wide_tiles_n;
+    if (wide_ok && tiles_m * wide_tiles_n >= ctx->num_cus) {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_wide_kernel),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds);
+        wide_ok = attr == hipSuccess;
+    } else {
+        wide_ok = false;
+    }
+    if (wide_ok)
+        gemm_tiled_wide_kernel<<<(unsigned)(tiles_m * wide_tiles_n), kThreads, kWideLds, stream>>>(hi, lo, wide, M, K);
+    else
+        gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles * k_splits), kThreads, lds_bytes, stream>>>(hi, lo, launch, M, K, k_splits);
     if (k_splits > 1) {
         for (int i = 0; i < n_mats; ++i) {
             const size_t n4 = (size_t)M * N[i] / 4;

@@ -220,6 +220,48 @@ def test_gemm_many_rows_vs_oracle(dev, orc, M, N, K):
     close(got[1:], want[1:])
 
 
+@pytest.mark.parametrize("M,N,K", [(2100, 4000, 96), (2100, 4000, 352), (4100, 2056, 2048)])
+def test_gemm_wide_tile_vs_float64_oracle_rows_and_narrow_kernel(dev, orc, M, N, K):
+    # Grids of at least one 128 x 256 tile per CU take the wide-tile kernel (direct global-to-LDS loads, five buffers):
+    # fewer K steps than buffers, one turn of its ten-step ring plus a remainder, and many turns; ragged in M and N.
+    # Per element within 1e-4 relative + 1e-5 absolute of the float64 product; the first rows also against the oracle's
+    # f32 x f16 product (cuda/kernels.cu:5037-5052); and bit for bit what the 128 x 128 kernel gives for the same rows
+    # (a call with 1000 rows is too small a grid for the wide tile and too large for a K split: both kernels add a step's
+    # high and low products in the same order)
+    rng = np.random.default_rng(M + N + K)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    A[1, :8] *= 1e-6
+    B = f16bits(rng.standard_normal((N, K)) * 0.05)
+    got = dev.gemm_gguf(A, B, M, N, K)
+    want = A.astype(np.float64) @ B.view(np.float16).astype(np.float64).T
+    close(got, want, 1e-4, 1e-5 * np.sqrt(K / 32.0))
+    close(got[:24], orc.gemm("f32xf16_gguf", A[:24], B, 24, N, K))
+    for r0 in (0, M - 1000):
+        narrow = dev.gemm_gguf(np.ascontiguousarray(A[r0:r0 + 1000]), B, 1000, N, K)
+        assert np.array_equal(narrow.view(np.uint32), got[r0:r0 + 1000].view(np.uint32)), r0
+    assert np.array_equal(dev.gemm_gguf(A, B, M, N, K).view(np.uint32), got.view(np.uint32))      # the same bits on a second call
+
+
+def test_gemm_wide_tile_multi_matrix_equals_separate_calls(dev):
+    # three matrices side by side in one wide-tile launch (8 + 2 + 1 tile columns x 32 tile rows): the same bits as one
+    # call per matrix, whichever kernel those calls take
+    M, K, Ns = 4096, 256, (2048, 264, 136)
+    rng = np.random.default_rng(11)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    Bs = [f16bits(rng.standard_normal((n, K)) * 0.05) for n in Ns]
+    dA, dB = dev.up(A), [dev.up(b) for b in Bs]
+    outs = [dev.zeros(M * n * 4) for n in Ns]
+    args = []
+    for i in range(3):
+        args += [dB[i].ptr, Ns[i], outs[i].ptr]
+    dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_multi_async", dA.ptr, M, K, 3, *args, 1)
+    dev.sync()
+    for i in range(3):
+        got = outs[i].download(np.float32, (M, Ns[i]))
+        assert np.array_equal(got.view(np.uint32), dev.gemm_gguf(A, Bs[i], M, Ns[i], K).view(np.uint32)), i
+        close(got, A.astype(np.float64) @ Bs[i].view(np.float16).astype(np.float64).T, 1e-4, 1e-5 * np.sqrt(K / 32.0))
+
+
 def test_gemm_known_answers(dev, orc):
     A = f16bits([[1, 2], [3, 4]]); B = f16bits([[5, 6], [7, 8]])
     dA, dB, dC = dev.up(A), dev.up(B), dev.zeros(16)
