@@ -3,7 +3,8 @@
 // beyond what the skinny kernels serve in one pass, where they would stream the weights once per 16 rows.
 //
 // Tiling: a workgroup of 4 waves owns a 128 x 128 tile of C and walks K in steps of 32.  Per step the 128 x 32 block
-// of A, split exactly into an f16 high part and an f16 low part (a = hi + lo up to 2^-22 relative), is written to
+// of A, split into an f16 high part and an f16 low part under a per-row power-of-two scale (a = scale (hi + lo) up to
+// 2^-22 relative; the scale multiplies the row of C at the end), is written to
 // LDS with the 128 x 32 block of B; each wave then computes its 64 x 64 quarter with
 // v_mfma_f32_16x16x32_f16, once with the high and once with the low part, so the products carry the f32 activations'
 // precision.  The global loads of the next three steps are in flight (three rotating register sets) while a step
@@ -48,28 +49,108 @@ struct StepRegs {   // one K step of one thread: rows lrow and lrow + 64, 16 byt
     uint4 ah[2], al[2], b[2];
 };
 
-// A [total] f32 -> hi [total] f16, lo [total] f16 (a = hi + lo up to 2^-22 relative); 8 elements per thread
-__global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __restrict__ A, _Float16* __restrict__ hi,
-                                                               _Float16* __restrict__ lo, size_t total8) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total8) return;
-    const float4 x0 = reinterpret_cast<const float4*>(A)[2 * i], x1 = reinterpret_cast<const float4*>(A)[2 * i + 1];
+// A [M][K] f32 -> hi, lo [M][K] f16 planes and one scale per row: a = scale * (hi + lo) up to 2^-22 relative.  The scale is
+// the power of two that brings the row's largest magnitude into [2^10, 2^11) -- any finite f32 row fits the f16 planes,
+// and small elements keep their low part out of the f16 subnormals.  The row stays in registers between the maximum and
+// the split (up to K = 16384; beyond that it is read a second time).  A row that holds an
+// infinity or a NaN is packed unscaled with those elements as they are (their low parts zero), so that its products come
+// out non-finite as the f32 arithmetic of the reference would give them (cuda/kernels.cu:5037-5052), never as a finite
+// value.
+constexpr int kPackChunks = 8;       // 8-element chunks a thread keeps in registers
+
+__device__ __forceinline__ float pack_abs_or_inf(float v) { return fabsf(v) <= 3.402823466e+38f ? fabsf(v) : INFINITY; }
+
+__device__ __forceinline__ void pack_split8(const float4& x0, const float4& x1, float inv_scale, half8& h, half8& l) {
     const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-    half8 h, l;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        // clamped to the f16 range: a value beyond +-65504 keeps its sign and loses precision instead of becoming an
-        // infinity (and its low part a NaN)
-        const float xc = fminf(fmaxf(x[j], -65504.0f), 65504.0f);
-        h[j] = static_cast<_Float16>(xc);
-        l[j] = static_cast<_Float16>(fminf(fmaxf(x[j] - static_cast<float>(h[j]), -65504.0f), 65504.0f));
+        const bool finite = fabsf(x[j]) <= 3.402823466e+38f;
+        // (a row with a non-finite element is not scaled: a finite neighbour beyond the f16 range then saturates, in a
+        // row whose products are non-finite wherever that element meets a non-zero weight)
+        const float xs = finite ? fminf(fmaxf(x[j] * inv_scale, -65504.0f), 65504.0f) : x[j];
+        h[j] = static_cast<_Float16>(xs);
+        l[j] = finite ? static_cast<_Float16>(xs - static_cast<float>(h[j])) : static_cast<_Float16>(0.0f);
     }
-    reinterpret_cast<half8*>(hi)[i] = h;
-    reinterpret_cast<half8*>(lo)[i] = l;
+}
+
+// ROW_THREADS = 64: a wave per row, four rows per workgroup, no barrier (K <= 4096 keeps the row in registers);
+// 256: a workgroup per row.
+template <int ROW_THREADS>
+__global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __restrict__ A, _Float16* __restrict__ hi,
+                                                               _Float16* __restrict__ lo, float* __restrict__ row_scale,
+                                                               int M, int K) {
+    __shared__ float wave_max[4];
+    constexpr int kRowsPerGroup = 256 / ROW_THREADS;
+    const int row = (int)blockIdx.x * kRowsPerGroup + (int)threadIdx.x / ROW_THREADS, tid = (int)threadIdx.x % ROW_THREADS;
+    if (ROW_THREADS == 64 && row >= M) return;          // whole waves: no barrier in this form
+    const float4* src = reinterpret_cast<const float4*>(A + (size_t)row * K);
+    const int chunks = K >> 3;                     // K is a multiple of 32
+    const bool in_regs = chunks <= kPackChunks * ROW_THREADS;
+    float4 x0[kPackChunks], x1[kPackChunks];
+    float mx = 0.0f;
+    if (in_regs) {
+#pragma unroll
+        for (int i = 0; i < kPackChunks; ++i) {
+            const int c = tid + ROW_THREADS * i;
+            if (c < chunks) { x0[i] = src[2 * c]; x1[i] = src[2 * c + 1]; }
+        }
+#pragma unroll
+        for (int i = 0; i < kPackChunks; ++i) {
+            if (tid + ROW_THREADS * i < chunks) {
+                mx = fmaxf(mx, fmaxf(fmaxf(pack_abs_or_inf(x0[i].x), pack_abs_or_inf(x0[i].y)), fmaxf(pack_abs_or_inf(x0[i].z), pack_abs_or_inf(x0[i].w))));
+                mx = fmaxf(mx, fmaxf(fmaxf(pack_abs_or_inf(x1[i].x), pack_abs_or_inf(x1[i].y)), fmaxf(pack_abs_or_inf(x1[i].z), pack_abs_or_inf(x1[i].w))));
+            }
+        }
+    } else {
+        for (int c = tid; c < chunks; c += ROW_THREADS) {
+            const float4 a = src[2 * c], b = src[2 * c + 1];
+            mx = fmaxf(mx, fmaxf(fmaxf(pack_abs_or_inf(a.x), pack_abs_or_inf(a.y)), fmaxf(pack_abs_or_inf(a.z), pack_abs_or_inf(a.w))));
+            mx = fmaxf(mx, fmaxf(fmaxf(pack_abs_or_inf(b.x), pack_abs_or_inf(b.y)), fmaxf(pack_abs_or_inf(b.z), pack_abs_or_inf(b.w))));
+        }
+    }
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if (ROW_THREADS == 256) {
+        if ((tid & 63) == 0) wave_max[tid >> 6] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    }
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (mx > 0.0f && mx < INFINITY) {
+        int ex;
+        (void)frexpf(mx, &ex);        // mx = f * 2^ex, f in [0.5, 1)
+        ex -= 11;
+        ex = ex < -100 ? -100 : (ex > 100 ? 100 : ex);
+        scale = ldexpf(1.0f, ex);
+        inv_scale = ldexpf(1.0f, -ex);
+    }
+    if (tid == 0) row_scale[row] = scale;
+    half8* hp = reinterpret_cast<half8*>(hi + (size_t)row * K);
+    half8* lp = reinterpret_cast<half8*>(lo + (size_t)row * K);
+    if (in_regs) {
+#pragma unroll
+        for (int i = 0; i < kPackChunks; ++i) {
+            const int c = tid + ROW_THREADS * i;
+            if (c < chunks) {
+                half8 h, l;
+                pack_split8(x0[i], x1[i], inv_scale, h, l);
+                hp[c] = h;
+                lp[c] = l;
+            }
+        }
+    } else {
+        for (int c = tid; c < chunks; c += ROW_THREADS) {
+            half8 h, l;
+            pack_split8(src[2 * c], src[2 * c + 1], inv_scale, h, l);
+            hp[c] = h;
+            lp[c] = l;
+        }
+    }
 }
 
 __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(const _Float16* __restrict__ A_hi,
                                                                               const _Float16* __restrict__ A_lo,
+                                                                              const float* __restrict__ row_scale,
                                                                               TiledMats mats, int M, int K, int k_splits) {
     extern __shared__ __align__(16) _Float16 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -139,6 +220,16 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
         for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int wm = wave >> 1, wn = wave & 1;
+    // the scales of the rows this lane will store, requested now: at the end they would be 16 dependent round trips
+    // (a load behind a store to memory it might alias waits for the store)
+    float sc_all[4][4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = m0 + wm * 64 + mt * 16 + (lane >> 4) * 4 + r;
+            sc_all[mt][r] = row_scale[row < M ? row : M - 1];
+        }
     const int frag_row = lane & 15, frag_k = ((lane >> 4) ^ ((frag_row >> 2) & 3)) * 8;   // swizzled chunk of this lane's k group
     auto compute = [&](int buf) {
         const _Float16* base = lds + buf * kBufHalves;
@@ -195,10 +286,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
         for (int r = 0; r < 4; ++r) {
             const int row = m0 + wm * 64 + mt * 16 + out_row + r;
             if (row >= M) continue;
+            const float sc = sc_all[mt][r];       // a power of two: partial sums of a K split scale exactly
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
                 const int col = n0 + wn * 64 + nt * 16 + out_col;
-                if (col < N) C[((size_t)split * M + row) * N + col] = acc[mt][nt][r];
+                if (col < N) C[((size_t)split * M + row) * N + col] = acc[mt][nt][r] * sc;
             }
         }
     }
@@ -243,7 +335,8 @@ __device__ __forceinline__ void tiled_unrolled(std::integer_sequence<int, I...>,
 __device__ __forceinline__ constexpr int vmcnt_only(int n) { return 0x0f70 | (n & 15) | ((n >> 4) << 14); }
 
 __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_wide_kernel(const _Float16* __restrict__ A_hi,
-                                                                      const _Float16* __restrict__ A_lo, TiledMats mats,
+                                                                      const _Float16* __restrict__ A_lo,
+                                                                      const float* __restrict__ row_scale, TiledMats mats,
                                                                       int M, int K) {
     typedef __attribute__((address_space(3))) void* lds_dst_t;
     typedef const __attribute__((address_space(1))) void* global_src_t;
@@ -296,6 +389,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_wide_kernel(const _Flo
             __builtin_amdgcn_global_load_lds((global_src_t)(bb + b_off[i]), (lds_dst_t)(dst + 2 * kWidePlane + i * 4096), 16, 0, 0);
     };
     const int wm = wave >> 1, wn = wave & 1;
+    float sc_all[kWideMT][4];          // the scales of the rows this lane will store, requested ahead of everything else
+#pragma unroll
+    for (int mt = 0; mt < kWideMT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = m0 + wm * kWideWM + mt * 16 + (lane >> 4) * 4 + r;
+            sc_all[mt][r] = row_scale[row < M ? row : M - 1];
+        }
     const int frag_row = lane & 15;
     const int fr_off = frag_row * 64 + (((lane >> 4) ^ ((frag_row >> 2) & 3)) * 16);
     auto read_frags = [&](WideFrags& f, int buf) {
@@ -378,10 +479,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_wide_kernel(const _Flo
         for (int r = 0; r < 4; ++r) {
             const int row = m0 + wm * kWideWM + mt * 16 + out_row + r;
             if (row >= M) continue;
+            const float sc = sc_all[mt][r];
 #pragma unroll
             for (int nt = 0; nt < kWideNT; ++nt) {
                 const int col = n0 + wn * kWideWN + nt * 16 + out_col;
-                if (col < N) C[(size_t)row * N + col] = acc[mt][nt][r];
+                if (col < N) C[(size_t)row * N + col] = acc[mt][nt][r] * sc;
             }
         }
     }
@@ -447,7 +549,8 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
         if (k_splits > 4) k_splits = 4;
         while (k_splits > 1 && (steps / k_splits < 16 || (steps + k_splits - 1) / k_splits * (k_splits - 1) >= steps)) --k_splits;
     }
-    const size_t need = (size_t)M * K * 4 + (k_splits > 1 ? (size_t)k_splits * out_floats * 4 : 0);
+    const size_t scale_bytes = ((size_t)M * 4 + 15) & ~(size_t)15;
+    const size_t need = (size_t)M * K * 4 + scale_bytes + (k_splits > 1 ? (size_t)k_splits * out_floats * 4 : 0);
     if (sc.tiled_pack_bytes < need) {
         hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone) return 1;
@@ -465,9 +568,12 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
     (void)hipGetLastError();
     _Float16* hi = static_cast<_Float16*>(sc.tiled_pack);
     _Float16* lo = hi + (size_t)M * K;
-    const size_t total8 = (size_t)M * K / 8;
-    pack_hilo_planes_kernel<<<(unsigned)((total8 + 255) / 256), 256, 0, stream>>>(A, hi, lo, total8);
-    float* partial = reinterpret_cast<float*>(static_cast<char*>(sc.tiled_pack) + (size_t)M * K * 4);
+    float* row_scale = reinterpret_cast<float*>(static_cast<char*>(sc.tiled_pack) + (size_t)M * K * 4);
+    if (K <= kPackChunks * 64 * 8)
+        pack_hilo_planes_kernel<64><<<(unsigned)((M + 3) / 4), 256, 0, stream>>>(A, hi, lo, row_scale, M, K);
+    else
+        pack_hilo_planes_kernel<256><<<(unsigned)M, 256, 0, stream>>>(A, hi, lo, row_scale, M, K);
+    float* partial = reinterpret_cast<float*>(static_cast<char*>(sc.tiled_pack) + (size_t)M * K * 4 + scale_bytes);
     TiledMats launch = mats;
     if (k_splits > 1) {
         size_t at = 0;
@@ -494,9 +600,9 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
         wide_ok = false;
     }
     if (wide_ok)
-        gemm_tiled_wide_kernel<<<(unsigned)(tiles_m * wide_tiles_n), kThreads, kWideLds, stream>>>(hi, lo, wide, M, K);
+        gemm_tiled_wide_kernel<<<(unsigned)(tiles_m * wide_tiles_n), kThreads, kWideLds, stream>>>(hi, lo, row_scale, wide, M, K);
     else
-        gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles * k_splits), kThreads, lds_bytes, stream>>>(hi, lo, launch, M, K, k_splits);
+        gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles * k_splits), kThreads, lds_bytes, stream>>>(hi, lo, row_scale, launch, M, K, k_splits);
     if (k_splits > 1) {
         for (int i = 0; i < n_mats; ++i) {
             const size_t n4 = (size_t)M * N[i] / 4;
