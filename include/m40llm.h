@@ -372,6 +372,31 @@ int m40llm_ext_prefill_rope_append_async(M40llmCudaContext* ctx, M40llmKVCache* 
                                          const uint32_t* q_lens_host, const uint32_t* start_pos_host, uint32_t q_heads,
                                          float freq_base, float freq_scale, uint32_t rope_layout, const void* d_bq_f32,
                                          const void* d_bk_f32, const void* d_bv_f32);
+/* The same launch on the stream `stream_kind` names (0 prefill, 1 decode), so that a prefill can keep all of its launches on
+ * one stream.  No counterpart in the reference (its per-token calls run on the decode stream). */
+int m40llm_ext_prefill_rope_append_on_stream_async(M40llmCudaContext* ctx, M40llmKVCache* kv, void* d_q_f32, void* d_k_f32,
+                                                   void* d_v_f32, uint32_t batch, const uint32_t* seq_slots_host,
+                                                   const uint32_t* q_lens_host, const uint32_t* start_pos_host,
+                                                   uint32_t q_heads, float freq_base, float freq_scale, uint32_t rope_layout,
+                                                   const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32,
+                                                   uint32_t stream_kind);
+/* Many-row projections of the packed prefill with the element-wise step before them and the residual add after them
+ * folded in (src/infer/forward.rs:2300-2345, 2440-2530 issue these as rms_norm / swiglu, the GEMMs and residual_add, one
+ * launch each).  The rows that enter the product are, by source_kind,
+ *   0: d_a_f32 [M][K] as it is;
+ *   1: what m40llm_rms_norm_f32_weighted writes for d_a_f32 with d_norm_weight (f16: norm_weight_dtype 0, f32: 1) and eps;
+ *   2: what m40llm_swiglu_f32 writes for gate = d_a_f32 and up = d_a2_f32, both [M][K];
+ * produced inside the pass that splits the rows into f16 planes, never written out as f32.  C_i [M][N_i] = rows x B_i (one
+ * to three f16 GGUF matrices, as m40llm_ext_gemm_f32xf16_gguf_f32_multi_async); with one matrix and d_R0_f32 [M][N0] not NULL
+ * C_0 = R_0 + product, what m40llm_residual_add_f32 gives (d_R0_f32 may be d_C0_f32).  Every result has the bits of
+ * that sequence of calls (element-wise call, m40llm_ext_gemm_f32xf16_gguf_f32_multi_async over the same matrices, residual add).  Returns 0 when enqueued on `stream_kind`, 1 when the shapes are not the many-row kernel's (M <= 32, K not
+ * a multiple of 32, an operand not 16-byte aligned) or its buffer cannot be provided -- nothing was enqueued and the caller
+ * issues the separate calls -- and -1 / -2 / -3 for a NULL, an argument out of range, a launch failure. */
+int m40llm_ext_prefill_gemm_fused_async(M40llmCudaContext* ctx, uint32_t source_kind, const void* d_a_f32, const void* d_a2_f32,
+                                        const void* d_norm_weight, uint32_t norm_weight_dtype, float eps, int M, int K,
+                                        int n_mats, const void* d_B0_f16, int N0, void* d_C0_f32, const void* d_R0_f32,
+                                        const void* d_B1_f16, int N1, void* d_C1_f32, const void* d_B2_f16, int N2,
+                                        void* d_C2_f32, uint32_t stream_kind);
 /* embedding rows of `rows` (<= 65535) token ids held on the device (f16 table [vocab][d_model]) -> f32 [rows][d_model];
  * the row form of m40llm_ext_embed_token_dev_async (src/infer/forward.rs:2241-2250 loads them one blocking call per
  * token).  Decode stream. */

@@ -156,6 +156,11 @@ int m40_launch_gemm_tiled(M40llmCudaContext* ctx, hipStream_t stream, uint32_t s
 // up to three weight matrices over the same activations in one launch; 1 = declined (no packing buffer), else 0 / -2
 int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, int M, int K,
                                 int n_mats, const uint16_t* const* B, const int* N, float* const* C);
+// the same with the rows of A produced by the packing pass (source_kind 0: A as it is, 1: RMSNorm of A with norm_w, 2:
+// SwiGLU of A (gate) and A2 (up)) and an optional residual per matrix added to the product (R[i] may be C[i])
+int m40_launch_gemm_tiled_fused(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int source_kind, const float* A,
+                                const float* A2, const void* norm_w, uint32_t norm_dtype, float eps, int M, int K, int n_mats,
+                                const uint16_t* const* B, const int* N, float* const* C, const float* const* R);
 bool m40_skinny_supported(const M40llmCudaContext* ctx, uint32_t stream_kind, int M, int N, int K, int fmt);
 int m40_launch_skinny(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int fmt, const float* A,
                       const float* up, const void* W0, float* C0, const void* W1, float* C1, int M, int N, int K);

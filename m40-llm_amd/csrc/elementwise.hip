@@ -45,6 +45,27 @@ __global__ __launch_bounds__(kThreads) void rms_norm_kernel(const float* __restr
 
     const uint16_t* w16 = reinterpret_cast<const uint16_t*>(weight);
     const float* w32 = reinterpret_cast<const float*>(weight);
+    if (vec && (!WEIGHTED || (weight_dtype == 0u ? (reinterpret_cast<uintptr_t>(weight) & 7u) == 0 : m40_aligned16(weight)))) {
+        // four elements per access (the same operations per element as the scalar form)
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+        float4* y4 = reinterpret_cast<float4*>(y);
+        for (uint32_t i = tid; i < dim / 4u; i += kThreads) {
+            const float4 a = x4[i];
+            float v[4] = {a.x * scale, a.y * scale, a.z * scale, a.w * scale};
+            if (WEIGHTED) {
+                if (weight_dtype == 0u) {
+                    const uint2 h = reinterpret_cast<const uint2*>(w16)[i];
+                    v[0] *= m40_h2f(static_cast<uint16_t>(h.x & 0xffffu)); v[1] *= m40_h2f(static_cast<uint16_t>(h.x >> 16));
+                    v[2] *= m40_h2f(static_cast<uint16_t>(h.y & 0xffffu)); v[3] *= m40_h2f(static_cast<uint16_t>(h.y >> 16));
+                } else {
+                    const float4 w = reinterpret_cast<const float4*>(w32)[i];
+                    v[0] *= w.x; v[1] *= w.y; v[2] *= w.z; v[3] *= w.w;
+                }
+            }
+            y4[i] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+        return;
+    }
     for (uint32_t i = tid; i < dim; i += kThreads) {
         float v = x[i] * scale;
         if (WEIGHTED) v = v * (weight_dtype == 0u ? m40_h2f(w16[i]) : w32[i]);
@@ -83,21 +104,55 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(float* __restrict__ a, f
     }
 }
 
-__global__ __launch_bounds__(kThreads) void residual_add_kernel(const float* __restrict__ a,
-                                                                const float* __restrict__ b,
-                                                                float* __restrict__ out, size_t n) {
+// Element-wise kernels over large arrays (the prefill's residual adds and SwiGLU: tens of MB per call): 16 bytes per lane
+// and access, four accesses in flight per thread; `out` may be one of the inputs (same index read, then written).  The
+// scalar form serves unaligned arrays and the last n % 4 elements.
+__global__ __launch_bounds__(kThreads) void residual_add_kernel(const float* a, const float* b, float* out, size_t n) {
     const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
     if (i < n) out[i] = a[i] + b[i];
 }
 
-__global__ __launch_bounds__(kThreads) void swiglu_kernel(const float* __restrict__ gate,
-                                                          const float* __restrict__ up,
-                                                          float* __restrict__ out, size_t n) {
+__global__ __launch_bounds__(kThreads) void residual_add4_kernel(const float4* a, const float4* b, float4* out, size_t n4) {
+    for (size_t base = (size_t)blockIdx.x * (4 * kThreads) + threadIdx.x; base < n4; base += (size_t)gridDim.x * (4 * kThreads)) {
+        float4 x[4], y[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t i = base + (size_t)u * kThreads;
+            if (i < n4) { x[u] = a[i]; y[u] = b[i]; }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t i = base + (size_t)u * kThreads;
+            if (i < n4) out[i] = make_float4(x[u].x + y[u].x, x[u].y + y[u].y, x[u].z + y[u].z, x[u].w + y[u].w);
+        }
+    }
+}
+
+__device__ __forceinline__ float swiglu_one(float g, float u) {
+    const float silu = g / (1.0f + expf(-g));
+    return silu * u;
+}
+
+__global__ __launch_bounds__(kThreads) void swiglu_kernel(const float* gate, const float* up, float* out, size_t n) {
     const size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
-    if (i < n) {
-        const float g = gate[i];
-        const float silu = g / (1.0f + expf(-g));
-        out[i] = silu * up[i];
+    if (i < n) out[i] = swiglu_one(gate[i], up[i]);
+}
+
+__global__ __launch_bounds__(kThreads) void swiglu4_kernel(const float4* gate, const float4* up, float4* out, size_t n4) {
+    for (size_t base = (size_t)blockIdx.x * (4 * kThreads) + threadIdx.x; base < n4; base += (size_t)gridDim.x * (4 * kThreads)) {
+        float4 g[4], v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t i = base + (size_t)u * kThreads;
+            if (i < n4) { g[u] = gate[i]; v[u] = up[i]; }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t i = base + (size_t)u * kThreads;
+            if (i < n4)
+                out[i] = make_float4(swiglu_one(g[u].x, v[u].x), swiglu_one(g[u].y, v[u].y), swiglu_one(g[u].z, v[u].z),
+                                     swiglu_one(g[u].w, v[u].w));
+        }
     }
 }
 
@@ -196,6 +251,11 @@ __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict
 }
 
 inline int blocks_for(size_t n) { return (int)((n + kThreads - 1) / kThreads); }
+// workgroups of the 16-byte forms: one pass of four accesses per thread, at most 8192 workgroups (then they loop)
+inline int wide_blocks_for(size_t n4) {
+    const size_t groups = (n4 + 4 * kThreads - 1) / (4 * kThreads);
+    return (int)(groups < 8192 ? groups : 8192);
+}
 
 }  // namespace
 
@@ -320,8 +380,18 @@ int m40llm_residual_add_f32_async(M40llmCudaContext* ctx, const void* d_a, const
     if (m40_ensure_device(ctx) != 0) return -2;
     if (n == 0) return 0;
     (void)hipGetLastError();
-    residual_add_kernel<<<blocks_for(n), kThreads, 0, ctx->decode_stream>>>(
-        static_cast<const float*>(d_a), static_cast<const float*>(d_b), static_cast<float*>(d_out), n);
+    const float* a = static_cast<const float*>(d_a);
+    const float* b = static_cast<const float*>(d_b);
+    float* out = static_cast<float*>(d_out);
+    size_t done = 0;
+    if (n >= 4096 && m40_aligned16(a) && m40_aligned16(b) && m40_aligned16(out)) {
+        const size_t n4 = n / 4;
+        residual_add4_kernel<<<wide_blocks_for(n4), kThreads, 0, ctx->decode_stream>>>(
+            reinterpret_cast<const float4*>(a), reinterpret_cast<const float4*>(b), reinterpret_cast<float4*>(out), n4);
+        done = 4 * n4;
+    }
+    if (done < n)
+        residual_add_kernel<<<blocks_for(n - done), kThreads, 0, ctx->decode_stream>>>(a + done, b + done, out + done, n - done);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -337,8 +407,18 @@ int m40llm_swiglu_f32_async(M40llmCudaContext* ctx, const void* d_gate, const vo
     if (m40_ensure_device(ctx) != 0) return -2;
     if (n == 0) return 0;
     (void)hipGetLastError();
-    swiglu_kernel<<<blocks_for(n), kThreads, 0, ctx->decode_stream>>>(
-        static_cast<const float*>(d_gate), static_cast<const float*>(d_up), static_cast<float*>(d_out), n);
+    const float* gate = static_cast<const float*>(d_gate);
+    const float* up = static_cast<const float*>(d_up);
+    float* out = static_cast<float*>(d_out);
+    size_t done = 0;
+    if (n >= 4096 && m40_aligned16(gate) && m40_aligned16(up) && m40_aligned16(out)) {
+        const size_t n4 = n / 4;
+        swiglu4_kernel<<<wide_blocks_for(n4), kThreads, 0, ctx->decode_stream>>>(
+            reinterpret_cast<const float4*>(gate), reinterpret_cast<const float4*>(up), reinterpret_cast<float4*>(out), n4);
+        done = 4 * n4;
+    }
+    if (done < n)
+        swiglu_kernel<<<blocks_for(n - done), kThreads, 0, ctx->decode_stream>>>(gate + done, up + done, out + done, n - done);
     return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

@@ -629,6 +629,38 @@ int m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(M40llmCudaContext* ctx, const v
     return launch_multi_f32xf16(ctx, stream, stream_kind, static_cast<const float*>(d_A_f32), M, K, n_mats, B, N, C);
 }
 
+int m40llm_ext_prefill_gemm_fused_async(M40llmCudaContext* ctx, uint32_t source_kind, const void* d_a_f32, const void* d_a2_f32,
+                                        const void* d_norm_weight, uint32_t norm_weight_dtype, float eps, int M, int K,
+                                        int n_mats, const void* d_B0_f16, int N0, void* d_C0_f32, const void* d_R0_f32,
+                                        const void* d_B1_f16, int N1, void* d_C1_f32, const void* d_B2_f16, int N2,
+                                        void* d_C2_f32, uint32_t stream_kind) {
+    if (!ctx || !d_a_f32) return -1;
+    if (source_kind > 2u || n_mats < 1 || n_mats > 3 || M <= 0 || K <= 0) return -2;
+    if (source_kind == 1u && (!d_norm_weight || norm_weight_dtype > 1u)) return -1;
+    if (source_kind == 2u && !d_a2_f32) return -1;
+    if (d_R0_f32 && n_mats != 1) return -2;
+    const uint16_t* B[3] = {static_cast<const uint16_t*>(d_B0_f16), static_cast<const uint16_t*>(d_B1_f16),
+                            static_cast<const uint16_t*>(d_B2_f16)};
+    float* C[3] = {static_cast<float*>(d_C0_f32), static_cast<float*>(d_C1_f32), static_cast<float*>(d_C2_f32)};
+    const float* R[3] = {static_cast<const float*>(d_R0_f32), nullptr, nullptr};
+    const int N[3] = {N0, N1, N2};
+    for (int i = 0; i < n_mats; ++i) {
+        if (!B[i] || !C[i]) return -1;
+        if (N[i] <= 0) return -2;
+    }
+    if (m40_ensure_device(ctx) != 0) return -2;
+    hipStream_t stream = m40_select_stream(ctx, stream_kind);
+    if (!stream) return -3;
+    const float* A = static_cast<const float*>(d_a_f32);
+    bool tiled = true;
+    for (int i = 0; i < n_mats && tiled; ++i) tiled = m40_gemm_tiled_supported(A, B[i], M, N[i], K);
+    if (source_kind == 1u) tiled = tiled && m40_aligned16(d_norm_weight);
+    if (source_kind == 2u) tiled = tiled && m40_aligned16(d_a2_f32);
+    if (!tiled) return 1;
+    return m40_launch_gemm_tiled_fused(ctx, stream, stream_kind, (int)source_kind, A, static_cast<const float*>(d_a2_f32),
+                                       d_norm_weight, norm_weight_dtype, eps, M, K, n_mats, B, N, C, R);
+}
+
 int m40llm_ext_gemm_f32xf16_gguf_f32_async(M40llmCudaContext* ctx, const void* d_A_f32, const void* d_B_f16,
                                            void* d_C_f32, int M, int N, int K, uint32_t stream_kind) {
     if (!ctx || !d_A_f32 || !d_B_f16 || !d_C_f32) return -1;

@@ -41,9 +41,22 @@ struct TiledMats {
     int n;
     const uint16_t* B[kMaxMats];
     float* C[kMaxMats];
+    const float* R[kMaxMats];       // not null: C = R + product (R may be C itself)
     int N[kMaxMats];
     int tile_start[kMaxMats + 1];   // first column tile of each matrix; [n] = total
 };
+
+// Where the rows of A come from: as they are, RMSNorm of the rows (what m40llm_rms_norm_f32_weighted writes: the same
+// sums in the same order, cuda/kernels.cu:770-807), or SwiGLU of two arrays (kernels.cu:869-880).  The packing pass
+// produces them on the fly, so the normalised / activated rows are never written out as f32 and read back.
+struct PackSource {
+    const float* a;
+    const float* a2;           // SwiGLU: the up array (a is gate)
+    const void* norm_w;        // RMSNorm weights
+    uint32_t norm_dtype;       // 0 f16, 1 f32
+    float eps;
+};
+enum { kPackPlain = 0, kPackNorm = 1, kPackSwiglu = 2 };
 
 struct StepRegs {   // one K step of one thread: rows lrow and lrow + 64, 16 bytes (8 halves) of each
     uint4 ah[2], al[2], b[2];
@@ -57,6 +70,12 @@ struct StepRegs {   // one K step of one thread: rows lrow and lrow + 64, 16 byt
 // out non-finite as the f32 arithmetic of the reference would give them (cuda/kernels.cu:5037-5052), never as a finite
 // value.
 constexpr int kPackChunks = 8;       // 8-element chunks a thread keeps in registers
+
+// SwiGLU of one element, the expression of swiglu_kernel (cuda/kernels.cu:869-880)
+__device__ __forceinline__ float tiled_swiglu(float g, float u) {
+    const float silu = g / (1.0f + expf(-g));
+    return silu * u;
+}
 
 __device__ __forceinline__ float pack_abs_or_inf(float v) { return fabsf(v) <= 3.402823466e+38f ? fabsf(v) : INFINITY; }
 
@@ -74,17 +93,61 @@ __device__ __forceinline__ void pack_split8(const float4& x0, const float4& x1, 
 }
 
 // ROW_THREADS = 64: a wave per row, four rows per workgroup, no barrier (K <= 4096 keeps the row in registers);
-// 256: a workgroup per row.
-template <int ROW_THREADS>
-__global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __restrict__ A, _Float16* __restrict__ hi,
+// 256: a workgroup per row (always for the RMSNorm source, whose sum of squares is formed with the thread layout and
+// order of rms_norm_kernel so that the fused form gives the bits of the two-launch form).
+template <int ROW_THREADS, int KIND>
+__global__ __launch_bounds__(256) void pack_hilo_planes_kernel(PackSource src_args, _Float16* __restrict__ hi,
                                                                _Float16* __restrict__ lo, float* __restrict__ row_scale,
                                                                int M, int K) {
+    static_assert(KIND != kPackNorm || ROW_THREADS == 256, "the norm's sums follow rms_norm_kernel's layout");
     __shared__ float wave_max[4];
+    __shared__ float wave_sums[4];
     constexpr int kRowsPerGroup = 256 / ROW_THREADS;
     const int row = (int)blockIdx.x * kRowsPerGroup + (int)threadIdx.x / ROW_THREADS, tid = (int)threadIdx.x % ROW_THREADS;
     if (ROW_THREADS == 64 && row >= M) return;          // whole waves: no barrier in this form
-    const float4* src = reinterpret_cast<const float4*>(A + (size_t)row * K);
+    const float4* src = reinterpret_cast<const float4*>(src_args.a + (size_t)row * K);
+    const float4* src2 = KIND == kPackSwiglu ? reinterpret_cast<const float4*>(src_args.a2 + (size_t)row * K) : nullptr;
     const int chunks = K >> 3;                     // K is a multiple of 32
+    float norm_scale = 1.0f;
+    if (KIND == kPackNorm) {
+        float ss = 0.0f;
+        for (int i = tid; i < K / 4; i += 256) {
+            const float4 v = src[i];
+            ss = fmaf(v.x, v.x, ss);
+            ss = fmaf(v.y, v.y, ss);
+            ss = fmaf(v.z, v.z, ss);
+            ss = fmaf(v.w, v.w, ss);
+        }
+        ss = m40_sum64(ss);
+        if ((tid & 63) == 0) wave_sums[tid >> 6] = ss;
+        __syncthreads();
+        float total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) total += wave_sums[w];
+        norm_scale = 1.0f / sqrtf(total / static_cast<float>(K) + src_args.eps);
+    }
+    // the eight source values of chunk c
+    auto load_chunk = [&](int c, float4& o0, float4& o1) {
+        o0 = src[2 * c];
+        o1 = src[2 * c + 1];
+        if (KIND == kPackSwiglu) {
+            const float4 u0 = src2[2 * c], u1 = src2[2 * c + 1];
+            o0 = make_float4(tiled_swiglu(o0.x, u0.x), tiled_swiglu(o0.y, u0.y), tiled_swiglu(o0.z, u0.z), tiled_swiglu(o0.w, u0.w));
+            o1 = make_float4(tiled_swiglu(o1.x, u1.x), tiled_swiglu(o1.y, u1.y), tiled_swiglu(o1.z, u1.z), tiled_swiglu(o1.w, u1.w));
+        }
+        if (KIND == kPackNorm) {
+            float w[8];
+            if (src_args.norm_dtype == 0u) {
+                m40_unpack8(reinterpret_cast<const uint4*>(src_args.norm_w)[c], w);
+            } else {
+                const float4 w0 = reinterpret_cast<const float4*>(src_args.norm_w)[2 * c], w1 = reinterpret_cast<const float4*>(src_args.norm_w)[2 * c + 1];
+                w[0] = w0.x; w[1] = w0.y; w[2] = w0.z; w[3] = w0.w; w[4] = w1.x; w[5] = w1.y; w[6] = w1.z; w[7] = w1.w;
+            }
+            // x * scale, then * weight: two roundings, as rms_norm_kernel has them
+            o0 = make_float4(o0.x * norm_scale * w[0], o0.y * norm_scale * w[1], o0.z * norm_scale * w[2], o0.w * norm_scale * w[3]);
+            o1 = make_float4(o1.x * norm_scale * w[4], o1.y * norm_scale * w[5], o1.z * norm_scale * w[6], o1.w * norm_scale * w[7]);
+        }
+    };
     const bool in_regs = chunks <= kPackChunks * ROW_THREADS;
     float4 x0[kPackChunks], x1[kPackChunks];
     float mx = 0.0f;
@@ -92,7 +155,7 @@ __global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __re
 #pragma unroll
         for (int i = 0; i < kPackChunks; ++i) {
             const int c = tid + ROW_THREADS * i;
-            if (c < chunks) { x0[i] = src[2 * c]; x1[i] = src[2 * c + 1]; }
+            if (c < chunks) load_chunk(c, x0[i], x1[i]);
         }
 #pragma unroll
         for (int i = 0; i < kPackChunks; ++i) {
@@ -103,7 +166,8 @@ __global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __re
         }
     } else {
         for (int c = tid; c < chunks; c += ROW_THREADS) {
-            const float4 a = src[2 * c], b = src[2 * c + 1];
+            float4 a, b;
+            load_chunk(c, a, b);
             mx = fmaxf(mx, fmaxf(fmaxf(pack_abs_or_inf(a.x), pack_abs_or_inf(a.y)), fmaxf(pack_abs_or_inf(a.z), pack_abs_or_inf(a.w))));
             mx = fmaxf(mx, fmaxf(fmaxf(pack_abs_or_inf(b.x), pack_abs_or_inf(b.y)), fmaxf(pack_abs_or_inf(b.z), pack_abs_or_inf(b.w))));
         }
@@ -140,8 +204,10 @@ __global__ __launch_bounds__(256) void pack_hilo_planes_kernel(const float* __re
         }
     } else {
         for (int c = tid; c < chunks; c += ROW_THREADS) {
+            float4 a, b;
+            load_chunk(c, a, b);
             half8 h, l;
-            pack_split8(src[2 * c], src[2 * c + 1], inv_scale, h, l);
+            pack_split8(a, b, inv_scale, h, l);
             hp[c] = h;
             lp[c] = l;
         }
@@ -280,20 +346,46 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_tiled_f32xf16_gguf_kernel(co
 
     // D fragment: lane holds rows 4 * (lane / 16) + r, column lane % 16 of each 16 x 16 tile
     const int out_col = lane & 15, out_row = (lane >> 4) * 4;
+    const float* R = k_splits == 1 ? mats.R[mat] : nullptr;      // a K split adds the residual when it adds the planes
+    // Two forms of the last step, chosen once per workgroup.  With a residual: per group of 16 rows its values first --
+    // unconditional loads from clamped addresses, no branch and no wait between them -- then the stores; a load that
+    // follows a store to memory it might alias is not moved ahead of it, and a load under a per-lane branch is awaited at
+    // the branch's end (measured with both mistakes in place: +10 us on a 65 us launch).
+    auto store_tile = [&](auto with_residual) {
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < 4; ++mt) {
+            float res[4][4];
+            if (decltype(with_residual)::value) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int row = m0 + wm * 64 + mt * 16 + out_row + r;
-            if (row >= M) continue;
-            const float sc = sc_all[mt][r];       // a power of two: partial sums of a K split scale exactly
+                for (int r = 0; r < 4; ++r) {
+                    const int row = m0 + wm * 64 + mt * 16 + out_row + r;
+                    const size_t row_off = (size_t)(row < M ? row : M - 1) * N;
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-                const int col = n0 + wn * 64 + nt * 16 + out_col;
-                if (col < N) C[((size_t)split * M + row) * N + col] = acc[mt][nt][r] * sc;
+                    for (int nt = 0; nt < 4; ++nt) {
+                        const int col = n0 + wn * 64 + nt * 16 + out_col;
+                        res[r][nt] = R[row_off + (col < N ? col : N - 1)];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = m0 + wm * 64 + mt * 16 + out_row + r;
+                if (row >= M) continue;
+                const float sc = sc_all[mt][r];       // a power of two: exact, also on the partial sums of a K split
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const int col = n0 + wn * 64 + nt * 16 + out_col;
+                    if (col < N) {
+                        const float v = acc[mt][nt][r] * sc;
+                        C[((size_t)split * M + row) * N + col] = decltype(with_residual)::value ? res[r][nt] + v : v;
+                    }
+                }
             }
         }
-    }
+    };
+    if (R) store_tile(std::true_type{});
+    else store_tile(std::false_type{});
 }
 
 // ---- wide tile: 128 x 256 per workgroup of four waves (wave tile 64 x 128), one workgroup per CU ---------------------------
@@ -473,31 +565,57 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_wide_kernel(const _Flo
     __builtin_amdgcn_s_waitcnt(vmcnt_only(0));      // no write into LDS may be outstanding when the workgroup ends
 
     const int out_col = lane & 15, out_row = (lane >> 4) * 4;
+    const float* R = mats.R[mat];
+    auto store_tile = [&](auto with_residual) {          // two forms, as in the kernel above
 #pragma unroll
-    for (int mt = 0; mt < kWideMT; ++mt) {
+        for (int mt = 0; mt < kWideMT; ++mt) {
+            float res[4][kWideNT];
+            if (decltype(with_residual)::value) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int row = m0 + wm * kWideWM + mt * 16 + out_row + r;
-            if (row >= M) continue;
-            const float sc = sc_all[mt][r];
+                for (int r = 0; r < 4; ++r) {
+                    const int row = m0 + wm * kWideWM + mt * 16 + out_row + r;
+                    const size_t row_off = (size_t)(row < M ? row : M - 1) * N;
 #pragma unroll
-            for (int nt = 0; nt < kWideNT; ++nt) {
-                const int col = n0 + wn * kWideWN + nt * 16 + out_col;
-                if (col < N) C[(size_t)row * N + col] = acc[mt][nt][r] * sc;
+                    for (int nt = 0; nt < kWideNT; ++nt) {
+                        const int col = n0 + wn * kWideWN + nt * 16 + out_col;
+                        res[r][nt] = R[row_off + (col < N ? col : N - 1)];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = m0 + wm * kWideWM + mt * 16 + out_row + r;
+                if (row >= M) continue;
+                const float sc = sc_all[mt][r];
+#pragma unroll
+                for (int nt = 0; nt < kWideNT; ++nt) {
+                    const int col = n0 + wn * kWideWN + nt * 16 + out_col;
+                    if (col < N) {
+                        const float v = acc[mt][nt][r] * sc;
+                        C[(size_t)row * N + col] = decltype(with_residual)::value ? res[r][nt] + v : v;
+                    }
+                }
             }
         }
-    }
+    };
+    if (R) store_tile(std::true_type{});
+    else store_tile(std::false_type{});
 }
 
-// out[i] = planes[0][i] + planes[1][i] + ... in that order (n4 float4 per plane)
-__global__ __launch_bounds__(256) void add_k_planes_kernel(const float4* __restrict__ planes, float4* __restrict__ out, size_t n4,
-                                                           int k_splits) {
+// out[i] = planes[0][i] + planes[1][i] + ... in that order (n4 float4 per plane), then residual[i] + that (residual may be out)
+__global__ __launch_bounds__(256) void add_k_planes_kernel(const float4* __restrict__ planes, const float4* residual, float4* out,
+                                                           size_t n4, int k_splits) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n4) return;
     float4 a = planes[i];
     for (int s = 1; s < k_splits; ++s) {
         const float4 b = planes[(size_t)s * n4 + i];
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    if (residual) {
+        const float4 r = residual[i];
+        a = make_float4(r.x + a.x, r.y + a.y, r.z + a.z, r.w + a.w);
     }
     out[i] = a;
 }
@@ -511,9 +629,12 @@ bool m40_gemm_tiled_supported(const void* A, const void* B, int M, int N, int K)
 
 // Returns 1 when the activations' packing buffer cannot be provided (the stream is being captured and the buffer is
 // too small, or the allocation fails): the caller then uses another kernel.
-int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, int M, int K,
-                                int n_mats, const uint16_t* const* B, const int* N, float* const* C) {
-    if (!ctx || stream_kind > 1u || n_mats < 1 || n_mats > kMaxMats) return -2;
+int m40_launch_gemm_tiled_fused(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, int source_kind, const float* A,
+                                const float* A2, const void* norm_w, uint32_t norm_dtype, float eps, int M, int K, int n_mats,
+                                const uint16_t* const* B, const int* N, float* const* C, const float* const* R) {
+    if (!ctx || stream_kind > 1u || n_mats < 1 || n_mats > kMaxMats || source_kind < kPackPlain || source_kind > kPackSwiglu) return -2;
+    if (source_kind == kPackSwiglu && (!A2 || !m40_aligned16(A2))) return -2;
+    if (source_kind == kPackNorm && (!norm_w || norm_dtype > 1u || !m40_aligned16(norm_w))) return -2;
     TiledMats mats{};
     mats.n = n_mats;
     long long tiles_n = 0;
@@ -521,6 +642,7 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
         if (!m40_gemm_tiled_supported(A, B[i], M, N[i], K) || !C[i]) return -2;
         mats.B[i] = B[i];
         mats.C[i] = C[i];
+        mats.R[i] = R ? R[i] : nullptr;
         mats.N[i] = N[i];
         mats.tile_start[i] = (int)tiles_n;
         tiles_n += (N[i] + kBN - 1) / kBN;
@@ -541,7 +663,7 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
     bool n4_ok = true;
     size_t out_floats = 0;
     for (int i = 0; i < n_mats; ++i) {
-        n4_ok = n4_ok && N[i] % 4 == 0 && m40_aligned16(C[i]);
+        n4_ok = n4_ok && N[i] % 4 == 0 && m40_aligned16(C[i]) && m40_aligned16(mats.R[i]);
         out_floats += (size_t)M * N[i];
     }
     if (n4_ok && tiles <= 128) {   // above that a split only adds a partial-sum pass (measured at 176 tiles)
@@ -569,10 +691,18 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
     _Float16* hi = static_cast<_Float16*>(sc.tiled_pack);
     _Float16* lo = hi + (size_t)M * K;
     float* row_scale = reinterpret_cast<float*>(static_cast<char*>(sc.tiled_pack) + (size_t)M * K * 4);
-    if (K <= kPackChunks * 64 * 8)
-        pack_hilo_planes_kernel<64><<<(unsigned)((M + 3) / 4), 256, 0, stream>>>(A, hi, lo, row_scale, M, K);
+    const PackSource source{A, A2, norm_w, norm_dtype, eps};
+    const bool wave_rows = K <= kPackChunks * 64 * 8;
+    if (source_kind == kPackNorm)
+        pack_hilo_planes_kernel<256, kPackNorm><<<(unsigned)M, 256, 0, stream>>>(source, hi, lo, row_scale, M, K);
+    else if (source_kind == kPackSwiglu && wave_rows)
+        pack_hilo_planes_kernel<64, kPackSwiglu><<<(unsigned)((M + 3) / 4), 256, 0, stream>>>(source, hi, lo, row_scale, M, K);
+    else if (source_kind == kPackSwiglu)
+        pack_hilo_planes_kernel<256, kPackSwiglu><<<(unsigned)M, 256, 0, stream>>>(source, hi, lo, row_scale, M, K);
+    else if (wave_rows)
+        pack_hilo_planes_kernel<64, kPackPlain><<<(unsigned)((M + 3) / 4), 256, 0, stream>>>(source, hi, lo, row_scale, M, K);
     else
-        pack_hilo_planes_kernel<256><<<(unsigned)M, 256, 0, stream>>>(A, hi, lo, row_scale, M, K);
+        pack_hilo_planes_kernel<256, kPackPlain><<<(unsigned)M, 256, 0, stream>>>(source, hi, lo, row_scale, M, K);
     float* partial = reinterpret_cast<float*>(static_cast<char*>(sc.tiled_pack) + (size_t)M * K * 4 + scale_bytes);
     TiledMats launch = mats;
     if (k_splits > 1) {
@@ -607,10 +737,16 @@ int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint
         for (int i = 0; i < n_mats; ++i) {
             const size_t n4 = (size_t)M * N[i] / 4;
             add_k_planes_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, stream>>>(reinterpret_cast<const float4*>(launch.C[i]),
+                                                                                  reinterpret_cast<const float4*>(mats.R[i]),
                                                                                   reinterpret_cast<float4*>(C[i]), n4, k_splits);
         }
     }
     return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+int m40_launch_gemm_tiled_multi(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, int M, int K,
+                                int n_mats, const uint16_t* const* B, const int* N, float* const* C) {
+    return m40_launch_gemm_tiled_fused(ctx, stream, stream_kind, kPackPlain, A, nullptr, nullptr, 0u, 0.0f, M, K, n_mats, B, N, C, nullptr);
 }
 
 int m40_launch_gemm_tiled(M40llmCudaContext* ctx, hipStream_t stream, uint32_t stream_kind, const float* A, const uint16_t* B,

@@ -558,7 +558,19 @@ int m40llm_ext_prefill_rope_append_async(M40llmCudaContext* ctx, M40llmKVCache* 
                                          const uint32_t* q_lens_host, const uint32_t* start_pos_host, uint32_t q_heads,
                                          float freq_base, float freq_scale, uint32_t rope_layout, const void* d_bq_f32,
                                          const void* d_bk_f32, const void* d_bv_f32) {
+    return m40llm_ext_prefill_rope_append_on_stream_async(ctx, kv, d_q_f32, d_k_f32, d_v_f32, batch, seq_slots_host, q_lens_host,
+                                                          start_pos_host, q_heads, freq_base, freq_scale, rope_layout, d_bq_f32,
+                                                          d_bk_f32, d_bv_f32, M40LLM_STREAM_DECODE);
+}
+
+int m40llm_ext_prefill_rope_append_on_stream_async(M40llmCudaContext* ctx, M40llmKVCache* kv, void* d_q_f32, void* d_k_f32,
+                                                   void* d_v_f32, uint32_t batch, const uint32_t* seq_slots_host,
+                                                   const uint32_t* q_lens_host, const uint32_t* start_pos_host,
+                                                   uint32_t q_heads, float freq_base, float freq_scale, uint32_t rope_layout,
+                                                   const void* d_bq_f32, const void* d_bk_f32, const void* d_bv_f32,
+                                                   uint32_t stream_kind) {
     if (!ctx || !kv || !d_q_f32 || !d_k_f32 || !d_v_f32 || !seq_slots_host || !q_lens_host) return -1;
+    if (stream_kind > 1u) return -2;
     const int n_bias = (d_bq_f32 != nullptr) + (d_bk_f32 != nullptr) + (d_bv_f32 != nullptr);
     if (n_bias != 0 && n_bias != 3) return -2;
     if (kv->compressed || !kv->d_k || !kv->d_v) return -9;
@@ -583,8 +595,8 @@ int m40llm_ext_prefill_rope_append_async(M40llmCudaContext* ctx, M40llmKVCache* 
         rows += q_lens_host[i];
         if (rows > 0x7fffffffull) return -2;
     }
-    hipStream_t stream = ctx->decode_stream;
-    const float* table = m40_rope_inv_freq_table(ctx, 1, stream, kv->head_dim, freq_base);
+    hipStream_t stream = stream_kind == M40LLM_STREAM_PREFILL ? ctx->prefill_stream : ctx->decode_stream;
+    const float* table = m40_rope_inv_freq_table(ctx, stream_kind, stream, kv->head_dim, freq_base);
     (void)hipGetLastError();
     prefill_rope_append_kernel<<<(unsigned)rows, kThreads, 0, stream>>>(
         static_cast<float*>(d_q_f32), static_cast<float*>(d_k_f32), static_cast<float*>(d_v_f32), kv->d_k, kv->d_v,

@@ -441,41 +441,68 @@ public:
         float* a = pws_.a.f32();
         float* b = pws_.b.f32();
         M40H_TRY(m40llm_ext_embed_rows_async(ctx_, tok_emb_, pws_.tokens.u32(), rows, cfg_.vocab, D, a));
+        M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
         std::vector<uint32_t> slots(batch);
         const uint32_t* d_off = pws_.offsets.u32();
         const uint32_t* d_len = pws_.lens.u32();
+        // Every launch of a layer goes to the prefill stream: RMSNorm and SwiGLU are produced inside the GEMMs' packing
+        // pass and the residual adds inside their last step (m40llm_ext_prefill_gemm_fused_async), so a layer is four
+        // projections, the RoPE + append launch and the attention, with no hop between streams.
         for (uint32_t l = 0; l < cfg_.n_layers; ++l) {
             const LayerWeights& w = layers_[l];
             for (uint32_t i = 0; i < batch; ++i) slots[i] = kv_slot(seq_ids[i], l);
-            M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, a, w.attn_norm, pws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
-            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(ctx_, pws_.xn.ptr(), (int)rows, (int)D, 3, w.wq, (int)D, pws_.q.ptr(),
-                                                                  w.wk, (int)KV, pws_.k.ptr(), w.wv, (int)KV, pws_.v.ptr(), PRE));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
-            M40H_TRY(m40llm_ext_prefill_rope_append_async(ctx_, kv_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), batch, slots.data(), lens,
-                                                          nullptr, cfg_.q_heads, cfg_.rope_base, cfg_.rope_scale, cfg_.rope_layout,
-                                                          cfg_.has_qkv_bias ? w.bq : nullptr, cfg_.has_qkv_bias ? w.bk : nullptr,
-                                                          cfg_.has_qkv_bias ? w.bv : nullptr));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            prefill_project(1, a, nullptr, w.attn_norm, pws_.xn.f32(), rows, D, 3, w.wq, D, pws_.q.f32(), w.wk, KV, pws_.k.f32(), w.wv, KV,
+                            pws_.v.f32(), nullptr);
+            M40H_TRY(m40llm_ext_prefill_rope_append_on_stream_async(ctx_, kv_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), batch, slots.data(),
+                                                                    lens, nullptr, cfg_.q_heads, cfg_.rope_base, cfg_.rope_scale,
+                                                                    cfg_.rope_layout, cfg_.has_qkv_bias ? w.bq : nullptr,
+                                                                    cfg_.has_qkv_bias ? w.bk : nullptr, cfg_.has_qkv_bias ? w.bv : nullptr,
+                                                                    PRE));
             M40H_TRY(m40llm_attention_prefill_f32_gqa_varlen_async(ctx_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), d_off, d_off, d_len, d_len,
                                                                    batch, cfg_.q_heads, cfg_.kv_heads, cfg_.head_dim, pws_.att.ptr()));
-            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx_, pws_.att.ptr(), w.wo, pws_.y.ptr(), (int)rows, (int)D, (int)D, PRE));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
-            M40H_TRY(m40llm_residual_add_f32_async(ctx_, a, pws_.y.ptr(), pws_.x1.ptr(), (size_t)rows * D));
-            M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, pws_.x1.ptr(), w.ffn_norm, pws_.xn.ptr(), rows, D, cfg_.rms_eps, cfg_.norm_weight_dtype));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
-            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(ctx_, pws_.xn.ptr(), (int)rows, (int)D, 2, w.wgate, (int)F,
-                                                                  pws_.gate.ptr(), w.wup, (int)F, pws_.up.ptr(), nullptr, 0, nullptr, PRE));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
-            M40H_TRY(m40llm_swiglu_f32_async(ctx_, pws_.gate.ptr(), pws_.up.ptr(), pws_.hid.ptr(), (size_t)rows * F));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
-            M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_async(ctx_, pws_.hid.ptr(), w.wdown, pws_.y.ptr(), (int)rows, (int)D, (int)F, PRE));
-            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
-            M40H_TRY(m40llm_residual_add_f32_async(ctx_, pws_.x1.ptr(), pws_.y.ptr(), b, (size_t)rows * D));
+            prefill_project(0, pws_.att.f32(), nullptr, nullptr, nullptr, rows, D, 1, w.wo, D, pws_.x1.f32(), nullptr, 0, nullptr, nullptr, 0,
+                            nullptr, a);
+            prefill_project(1, pws_.x1.f32(), nullptr, w.ffn_norm, pws_.xn.f32(), rows, D, 2, w.wgate, F, pws_.gate.f32(), w.wup, F,
+                            pws_.up.f32(), nullptr, 0, nullptr, nullptr);
+            prefill_project(2, pws_.gate.f32(), pws_.up.f32(), nullptr, pws_.hid.f32(), rows, F, 1, w.wdown, D, b, nullptr, 0, nullptr, nullptr,
+                            0, nullptr, pws_.x1.f32());
             std::swap(a, b);
         }
+        M40H_TRY(m40llm_stream_synchronize(ctx_, PRE));
         M40H_TRY(m40llm_stream_synchronize(ctx_, DEC));
         return a;
+    }
+
+    // One projection step of the packed prefill on the prefill stream: rows x B_i (up to three matrices), the rows being
+    // `x` (kind 0), RMSNorm(x) with norm_w (kind 1) or SwiGLU(x, x2) (kind 2), and C_0 = residual + product when a
+    // residual is given (one matrix).  One fused call; where that declines (few rows, odd shapes) the separate launches of
+    // forward.rs:2300-2530 with `tmp` holding the normalised / activated rows.
+    void prefill_project(uint32_t kind, const float* x, const float* x2, const void* norm_w, float* tmp, uint32_t rows, uint32_t K,
+                         int n_mats, const void* B0, uint32_t N0, float* C0, const void* B1, uint32_t N1, float* C1, const void* B2,
+                         uint32_t N2, float* C2, const float* residual) {
+        const uint32_t PRE = M40LLM_STREAM_PREFILL, DEC = M40LLM_STREAM_DECODE;
+        const int rc = m40llm_ext_prefill_gemm_fused_async(ctx_, kind, x, x2, norm_w, cfg_.norm_weight_dtype, cfg_.rms_eps, (int)rows, (int)K,
+                                                           n_mats, B0, (int)N0, C0, residual, B1, (int)N1, C1, B2, (int)N2, C2, PRE);
+        if (rc == 0) return;
+        if (rc != 1) M40H_TRY(rc);
+        const float* in = x;
+        if (kind != 0) {
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            if (kind == 1)
+                M40H_TRY(m40llm_rms_norm_f32_weighted_async(ctx_, x, norm_w, tmp, rows, K, cfg_.rms_eps, cfg_.norm_weight_dtype));
+            else
+                M40H_TRY(m40llm_swiglu_f32_async(ctx_, x, x2, tmp, (size_t)rows * K));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+            in = tmp;
+        }
+        float* out0 = residual ? pws_.y.f32() : C0;
+        M40H_TRY(m40llm_ext_gemm_f32xf16_gguf_f32_multi_async(ctx_, in, (int)rows, (int)K, n_mats, B0, (int)N0, out0, B1, (int)N1, C1, B2,
+                                                              (int)N2, C2, PRE));
+        if (residual) {
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, DEC, PRE));
+            M40H_TRY(m40llm_residual_add_f32_async(ctx_, residual, out0, C0, (size_t)rows * N0));
+            M40H_TRY(m40llm_stream_wait_for_stream(ctx_, PRE, DEC));
+        }
     }
 
     // Greedy decode of one sequence: prompt tokens from start_pos, then n_gen sampled tokens

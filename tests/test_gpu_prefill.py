@@ -154,3 +154,90 @@ def test_forward_prefill_matches_token_by_token_oracle_and_decode_continues(dev,
     with pytest.raises(RuntimeError, match="longer than max_seq_len"):
         dm.forward_prefill([0], [[1] * (S + 1)])
     dm.close()
+
+
+def _f16(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32).astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.parametrize("kind,M,K,Ns,residual,norm_dtype", [
+    (1, 300, 2048, (2048, 256, 256), False, 0),     # RMSNorm -> Q/K/V, 128 x 128 tiles, f16 norm weights
+    (1, 4100, 2048, (2048, 256, 256), False, 1),    # the same on the wide tile, f32 norm weights
+    (1, 40, 96, (136,), False, 0),                  # one matrix, three K steps
+    (0, 300, 2048, (2048,), True, 0),               # O projection + residual: K split, residual added with the partial sums
+    (0, 2100, 2048, (2048,), True, 0),              # no K split, 128 x 128 tiles: residual in the kernel's last step
+    (0, 4100, 2048, (2056,), True, 0),              # wide tile, ragged N
+    (2, 300, 5632, (2048,), True, 0),               # SwiGLU -> down projection + residual (a workgroup per row), K split
+    (2, 4100, 5632, (2048,), True, 0),              # the same on the wide tile
+    (2, 200, 256, (384, 64), False, 0),             # SwiGLU source, a wave per row, two matrices
+])
+def test_prefill_gemm_fused_equals_separate_calls(dev, kind, M, K, Ns, residual, norm_dtype):
+    # src/infer/forward.rs:2300-2345, 2440-2530 issue rms_norm / swiglu, the GEMMs and residual_add as separate launches; the
+    # fused call has to give the bits of rms_norm / swiglu -> the GEMM call over the same matrices -> residual_add, also with
+    # the result written over the residual
+    rng = np.random.default_rng(kind * 1000 + M + K)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    x[3] *= 1e-4
+    x[5, ::3] *= 300.0
+    x2 = rng.standard_normal((M, K)).astype(np.float32)
+    wn = (1.0 + 0.1 * rng.standard_normal(K)).astype(np.float32)
+    d_wn = dev.up(_f16(wn) if norm_dtype == 0 else wn)
+    Bs = [_f16(rng.standard_normal((n, K)) * 0.05) for n in Ns]
+    R = rng.standard_normal((M, Ns[0])).astype(np.float32)
+    dx, dx2, dB, dR = dev.up(x), dev.up(x2), [dev.up(b) for b in Bs], dev.up(R)
+    eps = 1e-5
+    # separate calls
+    rows = dev.zeros(M * K * 4)
+    if kind == 1:
+        dev.call("m40llm_rms_norm_f32_weighted_async", dx.ptr, d_wn.ptr, rows.ptr, M, K, eps, norm_dtype)
+    elif kind == 2:
+        dev.call("m40llm_swiglu_f32_async", dx.ptr, dx2.ptr, rows.ptr, M * K)
+    dev.sync()
+    src = rows if kind else dx
+    sep = [dev.zeros(M * n * 4) for n in Ns]
+    margs = []
+    for i in range(3):
+        margs += [dB[i].ptr, Ns[i], sep[i].ptr] if i < len(Ns) else [None, 0, None]
+    dev.call("m40llm_ext_gemm_f32xf16_gguf_f32_multi_async", src.ptr, M, K, len(Ns), *margs, 0)
+    dev.sync()
+    if residual:
+        dev.call("m40llm_residual_add_f32_async", dR.ptr, sep[0].ptr, sep[0].ptr, M * Ns[0])
+        dev.sync()
+    want = [sep[i].download(np.float32, (M, n)) for i, n in enumerate(Ns)]
+    # one fused call
+    outs = [dev.zeros(M * n * 4) for n in Ns]
+    args = []
+    for i in range(3):
+        if i == 0:
+            args += [dB[0].ptr, Ns[0], outs[0].ptr, dR.ptr if residual else None]
+        elif i < len(Ns):
+            args += [dB[i].ptr, Ns[i], outs[i].ptr]
+        else:
+            args += [None, 0, None]
+    dev.call("m40llm_ext_prefill_gemm_fused_async", kind, dx.ptr, dx2.ptr if kind == 2 else None, d_wn.ptr if kind == 1 else None,
+             norm_dtype, eps, M, K, len(Ns), *args, 0)
+    dev.sync()
+    for i, n in enumerate(Ns):
+        assert np.array_equal(outs[i].download(np.float32, (M, n)).view(np.uint32), want[i].view(np.uint32)), i
+    if residual:
+        # result over the residual
+        args[2] = dR.ptr
+        dev.call("m40llm_ext_prefill_gemm_fused_async", kind, dx.ptr, dx2.ptr if kind == 2 else None, d_wn.ptr if kind == 1 else None,
+                 norm_dtype, eps, M, K, len(Ns), *args, 0)
+        dev.sync()
+        assert np.array_equal(dR.download(np.float32, (M, Ns[0])).view(np.uint32), want[0].view(np.uint32))
+
+
+def test_prefill_gemm_fused_declines_and_checks(dev):
+    rng = np.random.default_rng(3)
+    M, K, N = 8, 256, 64
+    dx, dB, out = dev.up(rng.standard_normal((M, K)).astype(np.float32)), dev.up(_f16(rng.standard_normal((N, K)))), dev.zeros(M * N * 4)
+    tail = [None, 0, None, None, 0, None]
+    # few rows: not the many-row kernel's case -- nothing enqueued, the caller issues the separate calls
+    dev.call("m40llm_ext_prefill_gemm_fused_async", 0, dx.ptr, None, None, 0, 1e-5, M, K, 1, dB.ptr, N, out.ptr, None, *tail, 0, expect=1)
+    assert not out.download(np.float32, (M, N)).any()
+    dev.call("m40llm_ext_prefill_gemm_fused_async", 3, dx.ptr, None, None, 0, 1e-5, 64, K, 1, dB.ptr, N, out.ptr, None, *tail, 0, expect=-2)
+    dev.call("m40llm_ext_prefill_gemm_fused_async", 1, dx.ptr, None, None, 0, 1e-5, 64, K, 1, dB.ptr, N, out.ptr, None, *tail, 0, expect=-1)
+    dev.call("m40llm_ext_prefill_gemm_fused_async", 2, dx.ptr, None, None, 0, 1e-5, 64, K, 1, dB.ptr, N, out.ptr, None, *tail, 0, expect=-1)
+    dev.call("m40llm_ext_prefill_gemm_fused_async", 0, dx.ptr, None, None, 0, 1e-5, 64, K, 2, dB.ptr, N, out.ptr, out.ptr, dB.ptr, N, out.ptr,
+             None, 0, None, 0, expect=-2)     # a residual needs a single matrix
