@@ -70,6 +70,13 @@ __global__ __launch_bounds__(kThreads, 1) void rows_khalf_kernel(KHalfArgs p) {
     const int j = lane & 15, g = lane >> 4;
     const int tile = (int)blockIdx.x >> 1, half = (int)blockIdx.x & 1;
     const int n0 = tile * 16;
+    // The element this thread adds into `out` at the end (threads below 128: row tid / 16, column tid % 16), and its
+    // residual value, requested ahead of everything else: one unconditional load from a clamped address -- at the end it
+    // would be a round trip to memory with the whole workgroup waiting.
+    const int e_row = (tid >> 4) & 7, e_j = tid & 15;
+    const size_t e_off = (size_t)(e_row < p.rows ? e_row : 0) * p.N + (n0 + e_j < p.N ? n0 + e_j : p.N - 1);
+    const float e_res = *(p.residual ? p.residual + e_off : p.A);
+    __builtin_amdgcn_sched_barrier(0);
 
     // this wave's k-steps [ws0, ws1)
     const int KS = p.K >> 5;
@@ -190,16 +197,14 @@ __global__ __launch_bounds__(kThreads, 1) void rows_khalf_kernel(KHalfArgs p) {
     __syncthreads();
     // thread t < 128: element (row t / 16, column t % 16), the waves' sums in wave order
     if (tid < 128) {
-        const int e_row = tid >> 4, e_j = tid & 15;
         const int e_lane = 16 * (e_row >> 2) + e_j, e_r = e_row & 3;
         float v = red[e_r * 64 + e_lane];
 #pragma unroll
         for (int w = 1; w < kWaves; ++w) v += red[(w * 4 + e_r) * 64 + e_lane];
         const int col = n0 + e_j;
         if (e_row < p.rows && col < p.N) {
-            const size_t o = (size_t)e_row * p.N + col;
-            if (half == 0 && p.residual) v = p.residual[o] + v;
-            atomicAdd(p.out + o, v);
+            if (half == 0 && p.residual) v = e_res + v;
+            atomicAdd(p.out + (size_t)e_row * p.N + col, v);
         }
     }
 }
