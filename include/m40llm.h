@@ -343,6 +343,19 @@ int m40llm_attention_prefill_f32_gqa_varlen_async(M40llmCudaContext* ctx, const 
                                                   const uint32_t* kv_lens_dev, uint32_t batch_size, uint32_t q_heads,
                                                   uint32_t kv_heads, uint32_t head_dim, void* out_dev_f32);
 
+/* m40llm_attention_prefill_f32_gqa_varlen_async for a caller that also holds the key offsets and the lengths on the host
+ * (the same values as the device arrays, which the kernels read): validated from the host copies, so the call does not
+ * read the device arrays back -- each read-back waits for everything enqueued so far, once per layer of a prefill.  No
+ * counterpart in the reference (its launcher reads the lengths back).  Same codes; -1 also for a NULL host table. */
+int m40llm_ext_attention_prefill_f32_gqa_varlen_host_tables_async(M40llmCudaContext* ctx, const void* q_dev_f32,
+                                                                  const void* k_dev_f32, const void* v_dev_f32,
+                                                                  const uint32_t* q_offsets_dev, const uint32_t* kv_offsets_dev,
+                                                                  const uint32_t* q_lens_dev, const uint32_t* kv_lens_dev,
+                                                                  const uint32_t* kv_offsets_host, const uint32_t* q_lens_host,
+                                                                  const uint32_t* kv_lens_host, uint32_t batch_size,
+                                                                  uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                                                  void* out_dev_f32);
+
 /* raw views of the compressed cache for tests: which = 0 old_k, 1 q4_v, 2 q4_scale, 3 recent_k,
  * 4 recent_v, 5 seq_map; copies `bytes` from byte offset `offset` to the host */
 int m40llm_ext_kvcache_debug_read_raw(M40llmCudaContext* ctx, const M40llmKVCache* kv, uint32_t which,

@@ -296,15 +296,23 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
 
 int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const void* v, const uint32_t* q_offsets,
                  const uint32_t* kv_offsets, const uint32_t* q_lens, const uint32_t* kv_lens, uint32_t batch,
-                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, void* out, bool synchronize) {
+                 uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim, void* out, bool synchronize,
+                 const uint32_t* kv_offsets_host = nullptr, const uint32_t* q_lens_host = nullptr,
+                 const uint32_t* kv_lens_host = nullptr) {
     if (!ctx || !q || !k || !v || !q_offsets || !kv_offsets || !q_lens || !kv_lens || !out) return -1;
     if (batch == 0) return -2;
     if (q_heads == 0 || kv_heads == 0 || q_heads % kv_heads != 0) return -3;
     if (head_dim != 64 && head_dim != 128) return -9;
-    // the lengths are validated on the host before the launch, as the reference does (also in the _async form)
+    // the lengths are validated on the host before the launch, as the reference does (also in the _async form); a caller
+    // that holds the tables on the host passes them and spares the three blocking read-backs (each one drains the device)
+    const bool host_tables = kv_offsets_host && q_lens_host && kv_lens_host;
     std::vector<uint32_t> host(2 * (size_t)batch);
-    if (hipMemcpy(host.data(), q_lens, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
-    if (hipMemcpy(host.data() + batch, kv_lens, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
+    if (host_tables) {
+        for (uint32_t i = 0; i < batch; ++i) { host[i] = q_lens_host[i]; host[batch + i] = kv_lens_host[i]; }
+    } else {
+        if (hipMemcpy(host.data(), q_lens, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
+        if (hipMemcpy(host.data() + batch, kv_lens, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
+    }
     uint32_t max_q = 0, max_kv = 0;
     for (uint32_t i = 0; i < batch; ++i) {
         const uint32_t ql = host[i], kl = host[batch + i];
@@ -322,7 +330,8 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
     // layout needs the sequences' key ranges to lie one after the other (offsets non-decreasing with the batch index,
     // no overlap), which is how packed batches are built; anything else is refused.
     std::vector<uint32_t> offs(batch);
-    if (hipMemcpy(offs.data(), kv_offsets, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
+    if (host_tables) offs.assign(kv_offsets_host, kv_offsets_host + batch);
+    else if (hipMemcpy(offs.data(), kv_offsets, (size_t)batch * sizeof(uint32_t), hipMemcpyDeviceToHost) != hipSuccess) return -7;
     uint64_t end_prev = 0;
     for (uint32_t i = 0; i < batch; ++i) {
         if (offs[i] < end_prev) return -8;
@@ -380,6 +389,19 @@ int m40llm_attention_prefill_f32_gqa_varlen_async(M40llmCudaContext* ctx, const 
                                                   uint32_t kv_heads, uint32_t head_dim, void* out_dev_f32) {
     return prefill_impl(ctx, q_dev_f32, k_dev_f32, v_dev_f32, q_offsets_dev, kv_offsets_dev, q_lens_dev, kv_lens_dev,
                         batch_size, q_heads, kv_heads, head_dim, out_dev_f32, false);
+}
+
+int m40llm_ext_attention_prefill_f32_gqa_varlen_host_tables_async(M40llmCudaContext* ctx, const void* q_dev_f32,
+                                                                  const void* k_dev_f32, const void* v_dev_f32,
+                                                                  const uint32_t* q_offsets_dev, const uint32_t* kv_offsets_dev,
+                                                                  const uint32_t* q_lens_dev, const uint32_t* kv_lens_dev,
+                                                                  const uint32_t* kv_offsets_host, const uint32_t* q_lens_host,
+                                                                  const uint32_t* kv_lens_host, uint32_t batch_size,
+                                                                  uint32_t q_heads, uint32_t kv_heads, uint32_t head_dim,
+                                                                  void* out_dev_f32) {
+    if (!kv_offsets_host || !q_lens_host || !kv_lens_host) return -1;
+    return prefill_impl(ctx, q_dev_f32, k_dev_f32, v_dev_f32, q_offsets_dev, kv_offsets_dev, q_lens_dev, kv_lens_dev,
+                        batch_size, q_heads, kv_heads, head_dim, out_dev_f32, false, kv_offsets_host, q_lens_host, kv_lens_host);
 }
 
 }  // extern "C"

@@ -458,8 +458,10 @@ public:
                                                                     cfg_.rope_layout, cfg_.has_qkv_bias ? w.bq : nullptr,
                                                                     cfg_.has_qkv_bias ? w.bk : nullptr, cfg_.has_qkv_bias ? w.bv : nullptr,
                                                                     PRE));
-            M40H_TRY(m40llm_attention_prefill_f32_gqa_varlen_async(ctx_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), d_off, d_off, d_len, d_len,
-                                                                   batch, cfg_.q_heads, cfg_.kv_heads, cfg_.head_dim, pws_.att.ptr()));
+            M40H_TRY(m40llm_ext_attention_prefill_f32_gqa_varlen_host_tables_async(ctx_, pws_.q.ptr(), pws_.k.ptr(), pws_.v.ptr(), d_off, d_off,
+                                                                                   d_len, d_len, offsets.data(), lens, lens, batch,
+                                                                                   cfg_.q_heads, cfg_.kv_heads, cfg_.head_dim,
+                                                                                   pws_.att.ptr()));
             prefill_project(0, pws_.att.f32(), nullptr, nullptr, nullptr, rows, D, 1, w.wo, D, pws_.x1.f32(), nullptr, 0, nullptr, nullptr, 0,
                             nullptr, a);
             prefill_project(1, pws_.x1.f32(), nullptr, w.ffn_norm, pws_.xn.f32(), rows, D, 2, w.wgate, F, pws_.gate.f32(), w.wup, F,

@@ -871,6 +871,31 @@ def test_prefill_varlen_random_vs_oracle(dev, orc, qh, kvh, hd, ql, kl):
         assert np.all(np.abs(got[0] - want0) <= 2.0 ** -22 * np.abs(want0) + 2.0 ** -24)
 
 
+def test_prefill_varlen_host_tables_form_equals_device_tables_form(dev, orc):
+    # the form that validates from host copies of the tables (no read-back of the device arrays): the same bits, the same codes
+    rng = np.random.default_rng(21)
+    qh, kvh, hd, ql, kl = 8, 2, 128, [70, 33, 64], [70, 97, 64]
+    q = rng.standard_normal((sum(ql), qh, hd)).astype(np.float32)
+    k = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+    v = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+    want = _prefill_call(dev, orc, q, k, v, ql, kl, qh, kvh, hd, sync_form=False)
+    dq, dk, dv = dev.up(q), dev.up(k), dev.up(v)
+    h_qo, h_ko = orc.prefill_offsets(ql), orc.prefill_offsets(kl)
+    h_ql, h_kl = np.asarray(ql, dtype=np.uint32), np.asarray(kl, dtype=np.uint32)
+    dqo, dko, dql, dkl = dev.up(h_qo), dev.up(h_ko), dev.up(h_ql), dev.up(h_kl)
+    out = dev.zeros(q.nbytes)
+    name = "m40llm_ext_attention_prefill_f32_gqa_varlen_host_tables_async"
+    dev.call(name, dq.ptr, dk.ptr, dv.ptr, dqo.ptr, dko.ptr, dql.ptr, dkl.ptr, h_ko.ctypes.data, h_ql.ctypes.data, h_kl.ctypes.data,
+             len(ql), qh, kvh, hd, out.ptr)
+    dev.ctx.sync(0)
+    assert np.array_equal(out.download(np.float32, q.shape).view(np.uint32), want.view(np.uint32))
+    bad = np.asarray([70, 98, 64], dtype=np.uint32)          # more queries than keys in sequence 1
+    dev.call(name, dq.ptr, dk.ptr, dv.ptr, dqo.ptr, dko.ptr, dql.ptr, dkl.ptr, h_ko.ctypes.data, bad.ctypes.data, h_kl.ctypes.data,
+             len(ql), qh, kvh, hd, out.ptr, expect=-8)
+    dev.call(name, dq.ptr, dk.ptr, dv.ptr, dqo.ptr, dko.ptr, dql.ptr, dkl.ptr, None, h_ql.ctypes.data, h_kl.ctypes.data,
+             len(ql), qh, kvh, hd, out.ptr, expect=-1)
+
+
 def test_prefill_varlen_argument_checks(dev, orc):
     rng = np.random.default_rng(0)
     qh, kvh, hd, ql, kl = 4, 2, 64, [2, 3], [2, 5]
