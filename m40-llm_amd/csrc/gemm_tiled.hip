@@ -10,7 +10,7 @@
 // precision.  The global loads of the next three steps are in flight (three rotating register sets) while a step
 // computes from one LDS buffer and the following step's data moves into the other: one barrier per step.
 //
-// Large grids (at least one 128 x 256 tile per CU) take a second kernel built the same way round a wider tile and the
+// Larger grids (from 9/16 of a 128 x 256 tile per CU) take a second kernel built the same way round a wider tile and the
 // direct global-to-LDS loads of gfx950 (gemm_tiled_wide_kernel, below): what bounded the 128 x 128 kernel was not
 // arithmetic but the issue of its memory instructions, all of them between the barrier and the first matrix instruction.
 //
@@ -712,7 +712,8 @@ int m40_launch_gemm_tiled_fused(M40llmCudaContext* ctx, hipStream_t stream, uint
             at += (size_t)k_splits * M * N[i];
         }
     }
-    // the wide tile where it covers the CUs at least once (and element offsets fit the kernel's 32-bit arithmetic)
+    // the wide tile from 9/16 of a tile per CU on (measured at K 2048: 144 tiles 52 against 68 us for the 128 x 128 kernel, 180
+    // tiles 54 against 72 us; 120 tiles 51 against 48 us, 96 tiles 49 against 46 us), element offsets fitting its 32-bit arithmetic
     long long wide_tiles_n = 0;
     TiledMats wide = mats;
     bool wide_ok = k_splits == 1 && (long long)M * K < 0x7fffffffll;
@@ -722,7 +723,7 @@ int m40_launch_gemm_tiled_fused(M40llmCudaContext* ctx, hipStream_t stream, uint
         wide_ok = wide_ok && (long long)N[i] * K < 0x7fffffffll;
     }
     wide.tile_start[n_mats] = (int)wide_tiles_n;
-    if (wide_ok && tiles_m * wide_tiles_n >= ctx->num_cus) {
+    if (wide_ok && 16 * tiles_m * wide_tiles_n >= 9ll * ctx->num_cus) {
         static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_wide_kernel),
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds);
         wide_ok = attr == hipSuccess;

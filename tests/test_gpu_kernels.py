@@ -234,7 +234,7 @@ def test_gemm_many_rows_vs_oracle(dev, orc, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(2100, 4000, 96), (2100, 4000, 352), (4100, 2056, 2048)])
 def test_gemm_wide_tile_vs_float64_oracle_rows_and_narrow_kernel(dev, orc, M, N, K):
-    # Grids of at least one 128 x 256 tile per CU take the wide-tile kernel (direct global-to-LDS loads, five buffers):
+    # Grids from 9/16 of a 128 x 256 tile per CU on take the wide-tile kernel (direct global-to-LDS loads, five buffers):
     # fewer K steps than buffers, one turn of its ten-step ring plus a remainder, and many turns; ragged in M and N.
     # Per element within 1e-4 relative + 1e-5 absolute of the float64 product; the first rows also against the oracle's
     # f32 x f16 product (cuda/kernels.cu:5037-5052); and bit for bit what the 128 x 128 kernel gives for the same rows
