@@ -39,6 +39,7 @@ constexpr int key_tile_of(int hd) { return hd == 64 ? 64 : 32; }
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ m40_float4 mfma32(half8 a, half8 b, m40_float4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -232,14 +233,24 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         float x[4 * KB];
         const bool whole = key0 + (uint32_t)kKTile - 1u <= wave_first_end;      // every key of the tile visible to every query
         float mx = -INFINITY;
+        if (whole) {                      // the usual tile (a uniform branch): no per-key comparison
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
+            for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const bool visible = whole || key0 + 16u * kb + 4u * g + r <= row_end;
-                x[4 * kb + r] = visible ? sc[kb][r] * scale_log2 : -INFINITY;
-                mx = fmaxf(mx, x[4 * kb + r]);
-            }
+                for (int r = 0; r < 4; ++r) {
+                    x[4 * kb + r] = sc[kb][r] * scale_log2;
+                    mx = fmaxf(mx, x[4 * kb + r]);
+                }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const bool visible = key0 + 16u * kb + 4u * g + r <= row_end;
+                    x[4 * kb + r] = visible ? sc[kb][r] * scale_log2 : -INFINITY;
+                    mx = fmaxf(mx, x[4 * kb + r]);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float n = fmaxf(m_run, mx);
@@ -247,13 +258,14 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         half8 ph[KB / 2], pl[KB / 2];       // k-step t: slots 8 g + i = blocks 2 t (i < 4) and 2 t + 1 (i >= 4)
         float psum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4 * KB; ++i) {
-            const float pv = __builtin_amdgcn_exp2f(x[i] - n);               // a masked key: exp2(-inf) = 0
-            psum += pv;
-            _Float16 a, c;
-            split(pv, &a, &c);
-            ph[i >> 3][i & 7] = a;
-            pl[i >> 3][i & 7] = c;
+        for (int i = 0; i < 4 * KB; i += 2) {
+            // two weights at a time: the packed f32 -> f16 conversion of gfx950 halves the conversion instructions
+            const f32x2 pv = {__builtin_amdgcn_exp2f(x[i] - n), __builtin_amdgcn_exp2f(x[i + 1] - n)};   // a masked key: exp2(-inf) = 0
+            psum += pv.x + pv.y;
+            const half2v a = __builtin_convertvector(pv, half2v);
+            const half2v c = __builtin_convertvector(pv - __builtin_convertvector(a, f32x2), half2v);
+            ph[i >> 3][i & 7] = a.x; ph[i >> 3][(i & 7) + 1] = a.y;
+            pl[i >> 3][i & 7] = c.x; pl[i >> 3][(i & 7) + 1] = c.y;
         }
         if (__any(moved)) {               // sum and accumulators are only rescaled when some query's maximum rose
             // no maximum yet: the old state weighs nothing
