@@ -24,6 +24,12 @@
 // Reference: kernel cuda/kernels.cu:3749-3835; entry points, argument checks and their codes :4834-4977
 // (lengths are read back to the host and validated before the launch, also in the _async form).
 #include "common.hpp"
+#ifndef M40_PREFILL_QB64
+#define M40_PREFILL_QB64 2
+#endif
+#ifndef M40_PREFILL_QB128
+#define M40_PREFILL_QB128 1
+#endif
 
 #include <vector>
 
@@ -31,7 +37,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kQTile = 16 * kWaves;      // queries per workgroup
+constexpr int kQBlocks64 = M40_PREFILL_QB64, kQBlocks128 = M40_PREFILL_QB128;      // 16-query blocks per wave, by head_dim
 // keys per LDS tile (KT below): one or two k-steps of the P . V product; 64 where two planes of K and V^T fit the
 // static LDS limit (head_dim 64), 32 otherwise
 constexpr int key_tile_of(int hd) { return hd == 64 ? 64 : 32; }
@@ -107,7 +113,9 @@ __global__ __launch_bounds__(kThreads) void prefill_pack_kv_kernel(PrefillArgs p
     }
 }
 
-template <int HD>
+// QB: 16-query blocks per wave.  With two, every K and V fragment a wave reads from LDS serves 32 queries instead of 16:
+// the kernel's LDS traffic (each wave reads the whole K and V tile) was what it spent most of its time on.
+template <int HD, int QB>
 __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     constexpr int kKTile = key_tile_of(HD);
     constexpr int KB = kKTile / 16;        // 16-key score blocks of a tile
@@ -115,6 +123,8 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     constexpr int DT = HD / 16;            // 16-column output tiles
     constexpr int KSTR = HD + 8;           // LDS halves per K row: 16-byte fragment reads of 16 keys hit 64 distinct banks
     constexpr int VSTR = kKTile + 8;       // LDS halves per row of the transposed V tile [column][key]
+    constexpr int kQWave = 16 * QB;        // queries of a wave
+    constexpr int kQGroup = kQWave * kWaves;
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][kKTile * KSTR];   // [hi, lo][key][d]
     __shared__ __attribute__((aligned(16))) _Float16 v_lds[2][HD * VSTR];       // [hi, lo][d][key]
 
@@ -126,23 +136,29 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     // chip ran at a third of its occupancy.  Neighbouring workgroups are the q heads of one kv group on the same keys.
     const uint32_t b = blockIdx.z, h = blockIdx.x;
     const uint32_t q_len = p.q_lens[b], kv_len = p.kv_lens[b];
-    const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * kQTile;
+    const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * kQGroup;
     if (q0 >= q_len || q_len > kv_len) return;
     const uint32_t kvh = h / (p.q_heads / p.kv_heads);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int j = lane & 15, g = lane >> 4;
     const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
     const uint32_t shift = kv_len - q_len;                        // query q attends keys 0 .. shift + q
-    const uint32_t wg_last_q = q0 + kQTile - 1 < q_len - 1 ? q0 + kQTile - 1 : q_len - 1;
+    const uint32_t wg_last_q = q0 + kQGroup - 1 < q_len - 1 ? q0 + kQGroup - 1 : q_len - 1;
     const uint32_t n_tiles = (shift + wg_last_q) / kKTile + 1;    // key tiles this workgroup walks
 
-    // ---- this wave's 16 queries: A operand of the score product, lane (query j, k group g) holds
+    // ---- this wave's query blocks: A operand of the score product, lane (query j, k group g) of block qb holds
     //      Q[j][32 s + 8 g .. + 7] as a high and a low f16 part
-    const uint32_t wq0 = q0 + 16u * wave;                         // first query of the wave
+    const uint32_t wq0 = q0 + (uint32_t)kQWave * wave;            // first query of the wave
     const bool wave_live = wq0 < q_len;
-    const uint32_t my_q = wq0 + j < q_len ? wq0 + j : q_len - 1;  // a query past the end repeats the last one (not stored)
-    half8 qh[KS], ql[KS];
-    {
+    uint32_t row_end[QB];                                         // last key this lane's query of the block sees
+    uint32_t blk_end[QB];                                         // last key any query of the block sees
+    half8 qh[QB][KS], ql[QB][KS];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+        const uint32_t bq0 = wq0 + 16u * qb;
+        const uint32_t my_q = bq0 + j < q_len ? bq0 + j : q_len - 1;      // a query past the end repeats the last one (not stored)
+        row_end[qb] = shift + my_q;
+        blk_end[qb] = shift + (bq0 + 15u < q_len ? bq0 + 15u : q_len - 1);
         const float* qp = p.Q + ((size_t)(p.q_offsets[b] + my_q) * p.q_heads + h) * HD + 8 * g;
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -152,15 +168,13 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             for (int i = 0; i < 8; ++i) {
                 _Float16 a, c;
                 split(x[i], &a, &c);
-                qh[s][i] = a;
-                ql[s][i] = c;
+                qh[qb][s][i] = a;
+                ql[qb][s][i] = c;
             }
         }
     }
-    // this lane's query (all its scores, weights and accumulators belong to it) and its last visible key
-    const uint32_t row_end = shift + my_q;
     const uint32_t wave_first_end = shift + (wq0 < q_len ? wq0 : q_len - 1);          // last key the wave's first query sees
-    const uint32_t wave_end = shift + (wq0 + 15u < q_len ? wq0 + 15u : q_len - 1);    // last key any query of the wave sees
+    const uint32_t wave_end = blk_end[QB - 1];                                        // last key any query of the wave sees
 
     // ---- K / V tile loads: 16-byte pieces of the packed f16 planes (prefill_pack_kv_kernel), straight into LDS
     constexpr int PIECES = kKTile * HD / 8 / kThreads;           // per plane and thread: 1 (HD 64) or 2 (HD 128)
@@ -198,11 +212,16 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     // Products are formed transposed, S^T = K Q^T and O^T = V^T P^T, so that a lane (query j, group g) ends up with the
     // scores of ONE query for keys 4 g .. 4 g + 3 of both 16-key blocks, which are the k-slots 8 g .. 8 g + 7 of the
     // second product (key_of_slot): the weights never pass through LDS, and the running maximum, the sum and the
-    // rescaling factor are one value per lane.
-    float m_run = -INFINITY, l_run = 0.0f;   // maximum over the query's keys so far (equal in its four lanes); this lane's share of the sum
-    m40_float4 O[DT];                        // O^T[16 d + 4 g + r][query j]
+    // rescaling factor are one value per lane and query block.
+    float m_run[QB], l_run[QB];              // maximum over the query's keys so far (equal in its four lanes); this lane's share of the sum
+    m40_float4 O[QB][DT];                    // O^T[16 d + 4 g + r][query j] of the block
 #pragma unroll
-    for (int d = 0; d < DT; ++d) O[d] = m40_float4{0.f, 0.f, 0.f, 0.f};
+    for (int qb = 0; qb < QB; ++qb) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.0f;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) O[qb][d] = m40_float4{0.f, 0.f, 0.f, 0.f};
+    }
     const float scale_log2 = inv_sqrt * 1.4426950408889634f;     // scores in units of log2: weights are exp2(x - max)
 
     for (uint32_t tile = 0; tile < n_tiles; ++tile) {
@@ -212,12 +231,18 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         if (tile + 1 < n_tiles) issue(tile + 1);
         const uint32_t key0 = tile * kKTile;
         if (!wave_live || key0 > wave_end) continue;              // nothing of this tile is visible to the wave
+        // a block whose queries all end before this tile sits the tile out (only the first block can: later queries see more)
+        bool blk_on[QB];
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) blk_on[qb] = key0 <= blk_end[qb];
 
         // S^T of the tile's 16-key blocks: lane (query j, g) gets keys 16 kb + 4 g + r.  k . q = kh qh + kh ql + kl qh
-        // (the kl ql term is below 2^-22 of |q| |k|)
-        m40_float4 sc[KB];
+        // (the kl ql term is below 2^-22 of |q| |k|); a K fragment read serves every query block of the wave
+        m40_float4 sc[QB][KB];
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) sc[kb] = m40_float4{0.f, 0.f, 0.f, 0.f};
+        for (int qb = 0; qb < QB; ++qb)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) sc[qb][kb] = m40_float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             const int off = 32 * s + 8 * g;
@@ -225,84 +250,101 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
             for (int kb = 0; kb < KB; ++kb) {
                 const half8 kh = *reinterpret_cast<const half8*>(&k_lds[0][(16 * kb + j) * KSTR + off]);
                 const half8 kl = *reinterpret_cast<const half8*>(&k_lds[1][(16 * kb + j) * KSTR + off]);
-                sc[kb] = mfma32(kh, qh[s], sc[kb]);
-                sc[kb] = mfma32(kh, ql[s], sc[kb]);
-                sc[kb] = mfma32(kl, qh[s], sc[kb]);
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                    if (QB > 1 && !blk_on[qb]) continue;
+                    sc[qb][kb] = mfma32(kh, qh[qb][s], sc[qb][kb]);
+                    sc[qb][kb] = mfma32(kh, ql[qb][s], sc[qb][kb]);
+                    sc[qb][kb] = mfma32(kl, qh[qb][s], sc[qb][kb]);
+                }
             }
         }
-        float x[4 * KB];
         const bool whole = key0 + (uint32_t)kKTile - 1u <= wave_first_end;      // every key of the tile visible to every query
-        float mx = -INFINITY;
-        if (whole) {                      // the usual tile (a uniform branch): no per-key comparison
+        half8 ph[QB][KB / 2], pl[QB][KB / 2];       // k-step t: slots 8 g + i = blocks 2 t (i < 4) and 2 t + 1 (i >= 4)
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
+        for (int qb = 0; qb < QB; ++qb) {
+            if (QB > 1 && !blk_on[qb]) continue;
+            float x[4 * KB];
+            float mx = -INFINITY;
+            if (whole) {                      // the usual tile (a uniform branch): no per-key comparison
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    x[4 * kb + r] = sc[kb][r] * scale_log2;
-                    mx = fmaxf(mx, x[4 * kb + r]);
-                }
-        } else {
+                for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
+                    for (int r = 0; r < 4; ++r) {
+                        x[4 * kb + r] = sc[qb][kb][r] * scale_log2;
+                        mx = fmaxf(mx, x[4 * kb + r]);
+                    }
+            } else {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const bool visible = key0 + 16u * kb + 4u * g + r <= row_end;
-                    x[4 * kb + r] = visible ? sc[kb][r] * scale_log2 : -INFINITY;
-                    mx = fmaxf(mx, x[4 * kb + r]);
-                }
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const bool visible = key0 + 16u * kb + 4u * g + r <= row_end[qb];
+                        x[4 * kb + r] = visible ? sc[qb][kb][r] * scale_log2 : -INFINITY;
+                        mx = fmaxf(mx, x[4 * kb + r]);
+                    }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float n = fmaxf(m_run[qb], mx);
+            const bool moved = n != m_run[qb];
+            float psum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4 * KB; i += 2) {
+                // two weights at a time: the packed f32 -> f16 conversion of gfx950 halves the conversion instructions
+                const f32x2 pv = {__builtin_amdgcn_exp2f(x[i] - n), __builtin_amdgcn_exp2f(x[i + 1] - n)};   // a masked key: exp2(-inf) = 0
+                psum += pv.x + pv.y;
+                const half2v a = __builtin_convertvector(pv, half2v);
+                const half2v c = __builtin_convertvector(pv - __builtin_convertvector(a, f32x2), half2v);
+                ph[qb][i >> 3][i & 7] = a.x; ph[qb][i >> 3][(i & 7) + 1] = a.y;
+                pl[qb][i >> 3][i & 7] = c.x; pl[qb][i >> 3][(i & 7) + 1] = c.y;
+            }
+            if (__any(moved)) {               // sum and accumulators are only rescaled when some query's maximum rose
+                // no maximum yet: the old state weighs nothing
+                const float f = m_run[qb] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run[qb] - n);
+                l_run[qb] *= f;
+#pragma unroll
+                for (int d = 0; d < DT; ++d)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) O[qb][d][r] *= f;
+            }
+            m_run[qb] = n;
+            l_run[qb] += psum;
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float n = fmaxf(m_run, mx);
-        const bool moved = n != m_run;
-        half8 ph[KB / 2], pl[KB / 2];       // k-step t: slots 8 g + i = blocks 2 t (i < 4) and 2 t + 1 (i >= 4)
-        float psum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 4 * KB; i += 2) {
-            // two weights at a time: the packed f32 -> f16 conversion of gfx950 halves the conversion instructions
-            const f32x2 pv = {__builtin_amdgcn_exp2f(x[i] - n), __builtin_amdgcn_exp2f(x[i + 1] - n)};   // a masked key: exp2(-inf) = 0
-            psum += pv.x + pv.y;
-            const half2v a = __builtin_convertvector(pv, half2v);
-            const half2v c = __builtin_convertvector(pv - __builtin_convertvector(a, f32x2), half2v);
-            ph[i >> 3][i & 7] = a.x; ph[i >> 3][(i & 7) + 1] = a.y;
-            pl[i >> 3][i & 7] = c.x; pl[i >> 3][(i & 7) + 1] = c.y;
-        }
-        if (__any(moved)) {               // sum and accumulators are only rescaled when some query's maximum rose
-            // no maximum yet: the old state weighs nothing
-            const float f = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - n);
-            l_run *= f;
-#pragma unroll
-            for (int d = 0; d < DT; ++d)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) O[d][r] *= f;
-        }
-        m_run = n;
-        l_run += psum;
         // O^T += V^T . P^T, 32 keys per k-step: A = V^T[column 16 d + j][k-slots 32 t + 8 g .. + 7], B = this lane's
-        // eight weights of the step;  v p = vh ph + vh pl + vl ph
+        // eight weights of the step;  v p = vh ph + vh pl + vl ph; a V fragment read serves every query block
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
 #pragma unroll
             for (int t = 0; t < KB / 2; ++t) {
                 const half8 vh = *reinterpret_cast<const half8*>(&v_lds[0][(16 * d + j) * VSTR + 32 * t + 8 * g]);
                 const half8 vl = *reinterpret_cast<const half8*>(&v_lds[1][(16 * d + j) * VSTR + 32 * t + 8 * g]);
-                O[d] = mfma32(vh, ph[t], O[d]);
-                O[d] = mfma32(vh, pl[t], O[d]);
-                O[d] = mfma32(vl, ph[t], O[d]);
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                    if (QB > 1 && !blk_on[qb]) continue;
+                    O[qb][d] = mfma32(vh, ph[qb][t], O[qb][d]);
+                    O[qb][d] = mfma32(vh, pl[qb][t], O[qb][d]);
+                    O[qb][d] = mfma32(vl, ph[qb][t], O[qb][d]);
+                }
             }
         }
     }
 
     // ---- out = O / sum: this lane holds columns 16 d + 4 g .. + 3 of its query
     if (!wave_live) return;
-    float l = l_run + __shfl_xor(l_run, 16);
-    l += __shfl_xor(l, 32);
-    const float denom = l > 0.0f ? l : 1.0f;
-    if (wq0 + (uint32_t)j < q_len) {
-        float* op = p.Out + ((size_t)(p.q_offsets[b] + wq0 + j) * p.q_heads + h) * HD + 4 * g;
 #pragma unroll
-        for (int d = 0; d < DT; ++d)
-            *reinterpret_cast<float4*>(op + 16 * d) = make_float4(O[d][0] / denom, O[d][1] / denom, O[d][2] / denom, O[d][3] / denom);
+    for (int qb = 0; qb < QB; ++qb) {
+        float l = l_run[qb] + __shfl_xor(l_run[qb], 16);
+        l += __shfl_xor(l, 32);
+        const float denom = l > 0.0f ? l : 1.0f;
+        const uint32_t q = wq0 + 16u * qb + (uint32_t)j;
+        if (q < q_len) {
+            float* op = p.Out + ((size_t)(p.q_offsets[b] + q) * p.q_heads + h) * HD + 4 * g;
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+                *reinterpret_cast<float4*>(op + 16 * d) =
+                    make_float4(O[qb][d][0] / denom, O[qb][d][1] / denom, O[qb][d][2] / denom, O[qb][d][3] / denom);
+        }
     }
 }
 
@@ -368,13 +410,14 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
     a.plane_tiles = (uint32_t)plane_tiles;
     (void)hipGetLastError();
     const dim3 pack_grid((max_kv + kKTile - 1) / kKTile, kv_heads, batch);
-    const dim3 grid(q_heads, (max_q + kQTile - 1) / kQTile, batch);
+    const uint32_t q_group = 16u * kWaves * (uint32_t)(head_dim == 64 ? kQBlocks64 : kQBlocks128);     // queries per workgroup
+    const dim3 grid(q_heads, (max_q + q_group - 1) / q_group, batch);
     if (head_dim == 64) {
         prefill_pack_kv_kernel<64><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
-        prefill_attn_kernel<64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        prefill_attn_kernel<64, kQBlocks64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
     } else {
         prefill_pack_kv_kernel<128><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
-        prefill_attn_kernel<128><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        prefill_attn_kernel<128, kQBlocks128><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
     }
     if (hipGetLastError() != hipSuccess) return -4;
     if (synchronize && hipStreamSynchronize(ctx->prefill_stream) != hipSuccess) return -5;
