@@ -4,8 +4,8 @@
 // q_offsets[b] and kv_lens[b] keys from kv_offsets[b]; query q_idx attends keys 0 .. kv_len - q_len + q_idx.
 //
 // The reference walks every key once per (query, head) with one workgroup each (cuda/kernels.cu:3749-3835).  Here a
-// workgroup owns 64 consecutive queries of one q head (four waves x 16 queries) and streams the sequence's keys in
-// tiles of 32 through LDS, so a key row is fetched once per 64 queries.  Both products run on v_mfma_f32_16x16x32_f16
+// workgroup owns 64 or 128 consecutive queries of one q head (four waves x one or two blocks of 16 queries) and streams
+// the sequence's keys in tiles of 32 or 64 through LDS, so a key row is fetched once per 64 / 128 queries.  Both products run on v_mfma_f32_16x16x32_f16
 // with every f32 operand split exactly into an f16 high and an f16 low part (x = hi + lo to 2^-22): a product is
 // three instructions, hi hi + lo hi + hi lo (the lo lo term is below 2^-22 of the operands' magnitudes), which is
 // five times the rate of the f32 matrix instruction for the same product at f32-level accuracy:
@@ -24,12 +24,6 @@
 // Reference: kernel cuda/kernels.cu:3749-3835; entry points, argument checks and their codes :4834-4977
 // (lengths are read back to the host and validated before the launch, also in the _async form).
 #include "common.hpp"
-#ifndef M40_PREFILL_QB64
-#define M40_PREFILL_QB64 2
-#endif
-#ifndef M40_PREFILL_QB128
-#define M40_PREFILL_QB128 1
-#endif
 
 #include <vector>
 
@@ -37,7 +31,9 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-constexpr int kQBlocks64 = M40_PREFILL_QB64, kQBlocks128 = M40_PREFILL_QB128;      // 16-query blocks per wave, by head_dim
+// 16-query blocks per wave, by head_dim (measured at 4096 tokens: hd 64 one / two blocks 0.316 / 0.298 ms; hd 128 0.346 / 0.363 ms:
+// two blocks need more than 256 registers there)
+constexpr int kQBlocks64 = 2, kQBlocks128 = 1;
 // keys per LDS tile (KT below): one or two k-steps of the P . V product; 64 where two planes of K and V^T fit the
 // static LDS limit (head_dim 64), 32 otherwise
 constexpr int key_tile_of(int hd) { return hd == 64 ? 64 : 32; }
