@@ -24,7 +24,7 @@ HIP_SOURCES = ["context.hip", "elementwise.hip", "gemm.hip", "kvcache.hip", "att
 CPP_SOURCES = ["unavailable.cpp"]
 # per-file additions: matrix-instruction results straight into vector registers (the default form writes them to
 # accumulation registers and copies every element out again)
-HIP_FILE_FLAGS = {}
+HIP_FILE_FLAGS = {"prefill_attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _run(cmd):

@@ -31,9 +31,14 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-// 16-query blocks per wave, by head_dim (measured at 4096 tokens: hd 64 one / two blocks 0.316 / 0.298 ms; hd 128 0.346 / 0.363 ms:
-// two blocks need more than 256 registers there)
-constexpr int kQBlocks64 = 2, kQBlocks128 = 1;
+// 16-query blocks per wave: a K / V fragment read from LDS serves every block of the wave.  head_dim 64 always takes two
+// (one / two blocks at one sequence of 4096 tokens and 32 heads: 0.316 / 0.298 ms).  head_dim 128 takes two where long
+// sequences alone fill the chip four workgroups deep and one otherwise -- two blocks halve the workgroup count and double
+// the masked share of a short sequence's diagonal tiles (16 / 32 q heads, one against two blocks: 1 x 4096 tokens
+// 0.30 / 0.33 and 0.63 / 0.53 ms, 4 x 4096 1.17 / 1.02 and 2.13 / 1.85 ms, 16 x 300 0.069 / 0.077 and 0.099 / 0.112 ms).
+constexpr int kQBlocks64 = 2;
+constexpr uint32_t kTwoBlockMinQueries = 1024;      // a sequence counts as long from here
+constexpr int kTwoBlockMinGroupsPerCu = 4;
 // keys per LDS tile (KT below): one or two k-steps of the P . V product; 64 where two planes of K and V^T fit the
 // static LDS limit (head_dim 64), 32 otherwise
 constexpr int key_tile_of(int hd) { return hd == 64 ? 64 : 32; }
@@ -406,14 +411,20 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
     a.plane_tiles = (uint32_t)plane_tiles;
     (void)hipGetLastError();
     const dim3 pack_grid((max_kv + kKTile - 1) / kKTile, kv_heads, batch);
-    const uint32_t q_group = 16u * kWaves * (uint32_t)(head_dim == 64 ? kQBlocks64 : kQBlocks128);     // queries per workgroup
+    uint64_t long_groups = 0;           // two-block workgroups that the long sequences make
+    for (uint32_t i = 0; i < batch; ++i)
+        if (host[i] >= kTwoBlockMinQueries) long_groups += (uint64_t)((host[i] + 32u * kWaves - 1) / (32u * kWaves)) * q_heads;
+    const uint32_t blocks = head_dim == 64 ? (uint32_t)kQBlocks64
+                          : (long_groups >= (uint64_t)kTwoBlockMinGroupsPerCu * (uint64_t)ctx->num_cus ? 2u : 1u);
+    const uint32_t q_group = 16u * kWaves * blocks;     // queries per workgroup
     const dim3 grid(q_heads, (max_q + q_group - 1) / q_group, batch);
     if (head_dim == 64) {
         prefill_pack_kv_kernel<64><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
         prefill_attn_kernel<64, kQBlocks64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
     } else {
         prefill_pack_kv_kernel<128><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
-        prefill_attn_kernel<128, kQBlocks128><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        if (blocks == 2) prefill_attn_kernel<128, 2><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        else prefill_attn_kernel<128, 1><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
     }
     if (hipGetLastError() != hipSuccess) return -4;
     if (synchronize && hipStreamSynchronize(ctx->prefill_stream) != hipSuccess) return -5;

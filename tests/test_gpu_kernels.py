@@ -854,6 +854,9 @@ def test_prefill_varlen_reference_fixture(dev, orc, hd):
     (32, 4, 64, [300, 17], [300, 529]),                     # config-1 heads, several query tiles
     (3, 3, 128, [129], [1000]),                             # 871 cached keys ahead of the queries
     (16, 2, 128, [5, 5, 5, 5, 5], [8192, 5, 37, 64, 65]),   # the longest allowed key range
+    # head_dim 128 with enough long sequences for the form of two 16-query blocks per wave (1120 workgroups of 128
+    # queries from the four long ones), a short sequence and cached keys ahead of the queries in the same batch
+    (32, 4, 128, [1061, 1100, 50, 1024, 1030], [1161, 1100, 50, 1024, 1093]),
 ])
 def test_prefill_varlen_random_vs_oracle(dev, orc, qh, kvh, hd, ql, kl):
     rng = np.random.default_rng(len(ql) + hd)
