@@ -16,9 +16,13 @@
 // dimension the way the first product's accumulators hold them, so the softmax weights go from one matrix instruction
 // into the next inside the lane (no LDS round trip), and maximum, sum and rescaling factor are one value per lane.
 // V is stored transposed [d][key slot] so that a lane's eight key slots are one 16-byte read.
-// with a running maximum per query (the rows of a lane's accumulators are the same four queries in both products,
-// so the rescaling needs no exchange).  The result is the same softmax as the reference's three passes
-// (p = exp(s - max) / sum), within f32 rounding.  Operands beyond the f16 range (|x| > 65504) are not supported by the
+// The softmax is online, with a reference point per query in place of the running maximum: weights are
+// exp2(x - n) with n within 8 (log2 units) of the largest score so far, moved only when a tile holds a larger one
+// (the rows of a lane's accumulators are the same four queries in both products, so the rescaling needs no exchange).
+// The result is the same softmax as the reference's three passes (p = exp(s - max) / sum), within f32 rounding.
+// Two waves share a SIMD; a wave raises its priority for its matrix-instruction phases, so that the matrix pipe is
+// fed first and the other wave's vector work (exponentials, splits) fills the issue slots in between
+// (0.283 -> 0.252 ms for one 4096-token sequence at head_dim 64).  Operands beyond the f16 range (|x| > 65504) are not supported by the
 // split (none occur after RMSNorm-scaled projections; the decode-side attention has no such limit).
 //
 // Reference: kernel cuda/kernels.cu:3749-3835; entry points, argument checks and their codes :4834-4977
@@ -37,6 +41,7 @@ constexpr int kWaves = 4;
 // the masked share of a short sequence's diagonal tiles (16 / 32 q heads, one against two blocks: 1 x 4096 tokens
 // 0.30 / 0.33 and 0.63 / 0.53 ms, 4 x 4096 1.17 / 1.02 and 2.13 / 1.85 ms, 16 x 300 0.069 / 0.077 and 0.099 / 0.112 ms).
 constexpr int kQBlocks64 = 2;
+constexpr float kRefSlack = 8.0f;          // log2 units: weights stay below 256
 constexpr uint32_t kTwoBlockMinQueries = 1024;      // a sequence counts as long from here
 constexpr int kTwoBlockMinGroupsPerCu = 4;
 // keys per LDS tile (KT below): one or two k-steps of the P . V product; 64 where two planes of K and V^T fit the
@@ -50,6 +55,18 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ m40_float4 mfma32(half8 a, half8 b, m40_float4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+// Issue order of a phase of STEPS steps, each two 16-byte LDS fragment reads and PER matrix instructions that use them:
+// the reads run AHEAD steps in front of their instructions (left to itself the compiler reuses one register pair and
+// waits for every read right after issuing it).
+template <int STEPS, int PER, int AHEAD = 1>
+__device__ __forceinline__ void fragment_pipeline() {
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * (AHEAD < STEPS ? AHEAD : STEPS), 0);
+#pragma unroll
+    for (int i = 0; i < STEPS; ++i) {
+        if (i + AHEAD < STEPS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+    }
 }
 // x = hi + lo with both parts f16: exact to about 2^-22 relative for values inside the f16 range
 __device__ __forceinline__ void split(float x, _Float16* hi, _Float16* lo) {
@@ -126,6 +143,11 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     constexpr int VSTR = kKTile + 8;       // LDS halves per row of the transposed V tile [column][key]
     constexpr int kQWave = 16 * QB;        // queries of a wave
     constexpr int kQGroup = kQWave * kWaves;
+    // Two forms of the tile body, by measurement (one 4096-token sequence at 32 heads / eight sequences at 16 heads):
+    // head_dim 64 skips a first block that a tile lies wholly behind (branches around its matrix instructions) and
+    // leaves the order of fragment reads and matrix instructions to the compiler; head_dim 128 computes such a block
+    // masked and orders reads one step ahead of their instructions.  The other way round costs 5-6 % at either size.
+    constexpr bool kSkip = QB > 1 && HD == 64, kPipe = HD == 128;
     __shared__ __attribute__((aligned(16))) _Float16 k_lds[2][kKTile * KSTR];   // [hi, lo][key][d]
     __shared__ __attribute__((aligned(16))) _Float16 v_lds[2][HD * VSTR];       // [hi, lo][d][key]
 
@@ -140,7 +162,8 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
     const uint32_t q0 = (gridDim.y - 1u - blockIdx.y) * kQGroup;
     if (q0 >= q_len || q_len > kv_len) return;
     const uint32_t kvh = h / (p.q_heads / p.kv_heads);
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // as a scalar: tests on it branch without masks
     const int j = lane & 15, g = lane >> 4;
     const float inv_sqrt = HD == 64 ? 0.125f : 0.08838834764831845f;
     const uint32_t shift = kv_len - q_len;                        // query q attends keys 0 .. shift + q
@@ -232,11 +255,12 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         if (tile + 1 < n_tiles) issue(tile + 1);
         const uint32_t key0 = tile * kKTile;
         if (!wave_live || key0 > wave_end) continue;              // nothing of this tile is visible to the wave
-        // a block whose queries all end before this tile sits the tile out (only the first block can: later queries see more)
+        // a block whose queries all end before this tile (only the first can: later queries see more, and at most one
+        // tile per wave).  Computing it all the same changes nothing: every score is masked, and the weights are
+        // exp2(-inf - m) = 0 with the finite reference point that tile 0 has left (key 0 is visible to every query).
         bool blk_on[QB];
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) blk_on[qb] = key0 <= blk_end[qb];
-
+        for (int qb = 0; qb < QB; ++qb) blk_on[qb] = !kSkip || key0 <= blk_end[qb];
         // S^T of the tile's 16-key blocks: lane (query j, g) gets keys 16 kb + 4 g + r.  k . q = kh qh + kh ql + kl qh
         // (the kl ql term is below 2^-22 of |q| |k|); a K fragment read serves every query block of the wave
         m40_float4 sc[QB][KB];
@@ -244,6 +268,7 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
         for (int qb = 0; qb < QB; ++qb)
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) sc[qb][kb] = m40_float4{0.f, 0.f, 0.f, 0.f};
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             const int off = 32 * s + 8 * g;
@@ -253,18 +278,20 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
                 const half8 kl = *reinterpret_cast<const half8*>(&k_lds[1][(16 * kb + j) * KSTR + off]);
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) {
-                    if (QB > 1 && !blk_on[qb]) continue;
+                    if (kSkip && !blk_on[qb]) continue;
                     sc[qb][kb] = mfma32(kh, qh[qb][s], sc[qb][kb]);
                     sc[qb][kb] = mfma32(kh, ql[qb][s], sc[qb][kb]);
                     sc[qb][kb] = mfma32(kl, qh[qb][s], sc[qb][kb]);
                 }
             }
         }
+        if (kPipe) fragment_pipeline<KS * KB, 3 * QB>();
+        __builtin_amdgcn_s_setprio(0);
         const bool whole = key0 + (uint32_t)kKTile - 1u <= wave_first_end;      // every key of the tile visible to every query
         half8 ph[QB][KB / 2], pl[QB][KB / 2];       // k-step t: slots 8 g + i = blocks 2 t (i < 4) and 2 t + 1 (i >= 4)
 #pragma unroll
         for (int qb = 0; qb < QB; ++qb) {
-            if (QB > 1 && !blk_on[qb]) continue;
+            if (kSkip && !blk_on[qb]) continue;
             float x[4 * KB];
             float mx = -INFINITY;
             if (whole) {                      // the usual tile (a uniform branch): no per-key comparison
@@ -285,10 +312,25 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
                         mx = fmaxf(mx, x[4 * kb + r]);
                     }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float n = fmaxf(m_run[qb], mx);
-            const bool moved = n != m_run[qb];
+            // The weights are exp2(x - n) for a reference point n per query that need not be the maximum: any n within
+            // kRefSlack of it keeps the weights below 2^kRefSlack, far inside the range of the f16 split, and the softmax
+            // is the same.  The reference point moves (cross-lane maximum, rescaling of the sum and the accumulators)
+            // only when some lane of the wave sees a score more than kRefSlack above its query's: after the first tiles
+            // of a sequence that is rare, and the usual tile has no cross-lane exchange between its two products.
+            float n = m_run[qb];
+            if (__any(mx > n + kRefSlack)) {
+                mx = fmaxf(mx, __shfl_xor(mx, 16));
+                mx = fmaxf(mx, __shfl_xor(mx, 32));
+                n = fmaxf(n, mx);
+                // no reference point yet: the old state weighs nothing
+                const float f = m_run[qb] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run[qb] - n);
+                l_run[qb] *= f;
+#pragma unroll
+                for (int d = 0; d < DT; ++d)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) O[qb][d][r] *= f;
+                m_run[qb] = n;
+            }
             float psum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4 * KB; i += 2) {
@@ -300,20 +342,11 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
                 ph[qb][i >> 3][i & 7] = a.x; ph[qb][i >> 3][(i & 7) + 1] = a.y;
                 pl[qb][i >> 3][i & 7] = c.x; pl[qb][i >> 3][(i & 7) + 1] = c.y;
             }
-            if (__any(moved)) {               // sum and accumulators are only rescaled when some query's maximum rose
-                // no maximum yet: the old state weighs nothing
-                const float f = m_run[qb] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run[qb] - n);
-                l_run[qb] *= f;
-#pragma unroll
-                for (int d = 0; d < DT; ++d)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) O[qb][d][r] *= f;
-            }
-            m_run[qb] = n;
             l_run[qb] += psum;
         }
         // O^T += V^T . P^T, 32 keys per k-step: A = V^T[column 16 d + j][k-slots 32 t + 8 g .. + 7], B = this lane's
         // eight weights of the step;  v p = vh ph + vh pl + vl ph; a V fragment read serves every query block
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
 #pragma unroll
@@ -322,13 +355,15 @@ __global__ __launch_bounds__(kThreads) void prefill_attn_kernel(PrefillArgs p) {
                 const half8 vl = *reinterpret_cast<const half8*>(&v_lds[1][(16 * d + j) * VSTR + 32 * t + 8 * g]);
 #pragma unroll
                 for (int qb = 0; qb < QB; ++qb) {
-                    if (QB > 1 && !blk_on[qb]) continue;
+                    if (kSkip && !blk_on[qb]) continue;
                     O[qb][d] = mfma32(vh, ph[qb][t], O[qb][d]);
                     O[qb][d] = mfma32(vh, pl[qb][t], O[qb][d]);
                     O[qb][d] = mfma32(vl, ph[qb][t], O[qb][d]);
                 }
             }
         }
+        if (kPipe) fragment_pipeline<DT * (KB / 2), 3 * QB>();
+        __builtin_amdgcn_s_setprio(0);
     }
 
     // ---- out = O / sum: this lane holds columns 16 d + 4 g .. + 3 of its query

@@ -874,6 +874,30 @@ def test_prefill_varlen_random_vs_oracle(dev, orc, qh, kvh, hd, ql, kl):
         assert np.all(np.abs(got[0] - want0) <= 2.0 ** -22 * np.abs(want0) + 2.0 ** -24)
 
 
+@pytest.mark.parametrize("hd,qh,kvh", [(64, 8, 2), (128, 4, 2)])
+def test_prefill_varlen_scores_rising_along_the_keys(dev, orc, hd, qh, kvh):
+    # the kernel rescales its running state only when a tile holds a score well above the query's reference point: here the
+    # scores rise with the key index (every tile moves the reference point; the last visible keys carry the weight), fall
+    # again in a second sequence (the first tile fixes it for good), and a third holds one late key far above the rest
+    rng = np.random.default_rng(hd)
+    ql = kl = [700, 300, 260]
+    u = rng.standard_normal(hd).astype(np.float32)
+    u /= np.linalg.norm(u)
+    q = (u[None, None, :] * 6.0 + 0.3 * rng.standard_normal((sum(ql), qh, hd))).astype(np.float32)
+    k = (0.3 * rng.standard_normal((sum(kl), kvh, hd))).astype(np.float32)
+    ramp = np.concatenate([np.arange(700) * 0.05, (300 - np.arange(300)) * 0.08, np.zeros(260)]).astype(np.float32)
+    ramp[700 + 300 + 200] = 40.0
+    k += ramp[:, None, None] * u[None, None, :]
+    v = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+    rc, want = orc.attention_prefill(q, k, v, ql, kl, qh, kvh, hd)
+    assert rc == 0
+    got = _prefill_call(dev, orc, q, k, v, ql, kl, qh, kvh, hd, sync_form=False)
+    close(got, want)
+    # queries after the late key of the third sequence see (nearly) only it
+    late = got[700 + 300 + 230]
+    close(late, np.repeat(v[700 + 300 + 200], qh // kvh, axis=0), 1e-3, 1e-3)
+
+
 def test_prefill_varlen_host_tables_form_equals_device_tables_form(dev, orc):
     # the form that validates from host copies of the tables (no read-back of the device arrays): the same bits, the same codes
     rng = np.random.default_rng(21)
