@@ -338,7 +338,7 @@ def main():
                     help="-1 best available, 0 reference call sequence, 1 fused, 2 fused + graph")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (debug only; invalidates the metric)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-steps", type=int, default=8)
+    ap.add_argument("--cpu-steps", type=int, default=48)
     ap.add_argument("--kernel-reps", type=int, default=10)
     ap.add_argument("--no-b8", action="store_true", help="skip the batch-8 measurement reported in config.b8")
     ap.add_argument("--traffic-probe", action="store_true",

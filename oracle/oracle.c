@@ -78,7 +78,7 @@ uint16_t orc_f32_to_f16(float x) {
     return (uint16_t)(sign | half);
 }
 
-float orc_f16_to_f32(uint16_t h) {
+static float f16_to_f32_bits(uint16_t h) {
     const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
     uint32_t exp = (h >> 10) & 0x1fu;
     uint32_t mant = h & 0x3ffu;
@@ -102,11 +102,20 @@ float orc_f16_to_f32(uint16_t h) {
     return f;
 }
 
+/* Every f16 value's f32 image, filled from the routine above when the library is loaded: the conversions inside
+ * the GEMM and attention loops are one table read each (same bits, a few times faster than the branches). */
+static float f16_table[65536];
+__attribute__((constructor)) static void fill_f16_table(void) {
+    for (uint32_t h = 0; h < 65536u; ++h) f16_table[h] = f16_to_f32_bits((uint16_t)h);
+}
+static inline float h2f(uint16_t h) { return f16_table[h]; }
+float orc_f16_to_f32(uint16_t h) { return h2f(h); }
+
 void orc_f32_to_f16_n(const float* in, uint16_t* out, size_t n) {
     for (size_t i = 0; i < n; ++i) out[i] = orc_f32_to_f16(in[i]);
 }
 void orc_f16_to_f32_n(const uint16_t* in, float* out, size_t n) {
-    for (size_t i = 0; i < n; ++i) out[i] = orc_f16_to_f32(in[i]);
+    for (size_t i = 0; i < n; ++i) out[i] = h2f(in[i]);
 }
 
 /* ------------------------------------------------------------------------ */
@@ -153,7 +162,7 @@ int orc_rms_norm_weighted(const float* in, const void* weight, float* out,
         for (uint32_t i = 0; i < dim; ++i) ss += x[i] * x[i];
         const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
         for (uint32_t i = 0; i < dim; ++i) {
-            const float w = weight_dtype == 0 ? orc_f16_to_f32(w16[i]) : w32[i];
+            const float w = weight_dtype == 0 ? h2f(w16[i]) : w32[i];
             out[(size_t)r * dim + i] = x[i] * scale * w; /* order x*scale*w, kernels.cu:805 */
         }
     }
@@ -224,7 +233,7 @@ void orc_q80_to_f32(const uint8_t* in, float* out, size_t n) {
         const uint8_t* base = in + blk * 34;
         uint16_t dh;
         memcpy(&dh, base, 2);
-        const float d = orc_f16_to_f32(dh);
+        const float d = h2f(dh);
         const int8_t q = (int8_t)base[2 + idx];
         out[i] = d * (float)q;
     }
@@ -246,10 +255,10 @@ void orc_gemm_f32xf16_gguf(const float* A, const uint16_t* B, float* C, int M, i
             for (int c = 0; c < 4; ++c) b[c] = B + (size_t)(j0 + (c < nj ? c : 0)) * K;
             for (int kk = 0; kk < K; ++kk) {
                 const float av = a[kk];
-                acc[0] += av * orc_f16_to_f32(b[0][kk]);
-                acc[1] += av * orc_f16_to_f32(b[1][kk]);
-                acc[2] += av * orc_f16_to_f32(b[2][kk]);
-                acc[3] += av * orc_f16_to_f32(b[3][kk]);
+                acc[0] += av * h2f(b[0][kk]);
+                acc[1] += av * h2f(b[1][kk]);
+                acc[2] += av * h2f(b[2][kk]);
+                acc[3] += av * h2f(b[3][kk]);
             }
             for (int c = 0; c < nj; ++c) C[(size_t)i * N + j0 + c] = acc[c];
         }
@@ -261,7 +270,7 @@ void orc_gemm_f32xf16_rowmajor(const float* A, const uint16_t* B, float* C, int 
         for (int j = 0; j < N; ++j) {
             float acc = 0.0f;
             for (int kk = 0; kk < K; ++kk)
-                acc += A[(size_t)i * K + kk] * orc_f16_to_f32(B[(size_t)kk * N + j]);
+                acc += A[(size_t)i * K + kk] * h2f(B[(size_t)kk * N + j]);
             C[(size_t)i * N + j] = acc;
         }
 }
@@ -271,7 +280,7 @@ void orc_gemm_f16xf16_rowmajor(const uint16_t* A, const uint16_t* B, float* C, i
         for (int j = 0; j < N; ++j) {
             float acc = 0.0f;
             for (int kk = 0; kk < K; ++kk)
-                acc += orc_f16_to_f32(A[(size_t)i * K + kk]) * orc_f16_to_f32(B[(size_t)kk * N + j]);
+                acc += h2f(A[(size_t)i * K + kk]) * h2f(B[(size_t)kk * N + j]);
             C[(size_t)i * N + j] = acc;
         }
 }
@@ -291,7 +300,7 @@ void orc_gemm_f32xq80_gguf(const float* A, const uint8_t* B, float* C, int M, in
                 const uint8_t* base = col + (size_t)blk * 34;
                 uint16_t dh;
                 memcpy(&dh, base, 2);
-                const float d = orc_f16_to_f32(dh);
+                const float d = h2f(dh);
                 const int8_t* qs = (const int8_t*)(base + 2);
                 for (int t = 0; t < 32; ++t) {
                     const float x = d * (float)qs[t];
@@ -380,7 +389,7 @@ void orc_attention_last_token_gqa(const uint16_t* K, const uint16_t* V, uint32_t
         for (uint32_t t = 0; t < seq_len; ++t) {
             const size_t base = orc_kv_index(max_seq_len, kv_heads, head_dim, seq, t, kvh, 0);
             float dot = 0.0f;
-            for (uint32_t d = 0; d < head_dim; ++d) dot += qh[d] * orc_f16_to_f32(K[base + d]);
+            for (uint32_t d = 0; d < head_dim; ++d) dot += qh[d] * h2f(K[base + d]);
             const float s = dot * inv_sqrt;
             scores[t] = s;
             if (s > max_score) max_score = s;
@@ -394,7 +403,7 @@ void orc_attention_last_token_gqa(const uint16_t* K, const uint16_t* V, uint32_t
             for (uint32_t t = 0; t < seq_len; ++t) {
                 const size_t base = orc_kv_index(max_seq_len, kv_heads, head_dim, seq, t, kvh, 0);
                 const float p = expf(scores[t] - max_score) / denom;
-                acc += p * orc_f16_to_f32(V[base + d]);
+                acc += p * h2f(V[base + d]);
             }
             oh[d] = acc;
         }
@@ -529,12 +538,12 @@ size_t orc_ckv_bytes_q4_scale(const orc_ckv* c) {
  * byte = (q_even & 15) | ((q_odd & 15) << 4). */
 void orc_q4_quantize_row(const uint16_t* v_f16, uint32_t head_dim, uint8_t* packed, float* scale) {
     float max_v = 0.0f;
-    for (uint32_t d = 0; d < head_dim; ++d) max_v = fmaxf(max_v, fabsf(orc_f16_to_f32(v_f16[d])));
+    for (uint32_t d = 0; d < head_dim; ++d) max_v = fmaxf(max_v, fabsf(h2f(v_f16[d])));
     const float sc = max_v > 0.0f ? max_v / 7.0f : 1.0f / 7.0f;
     *scale = sc;
     for (uint32_t pair = 0; pair < head_dim / 2u; ++pair) {
-        const float a = orc_f16_to_f32(v_f16[2 * pair]);
-        const float b = orc_f16_to_f32(v_f16[2 * pair + 1]);
+        const float a = h2f(v_f16[2 * pair]);
+        const float b = h2f(v_f16[2 * pair + 1]);
         long qa = lrintf(a / sc), qb = lrintf(b / sc);
         if (qa < -7) qa = -7; if (qa > 7) qa = 7;
         if (qb < -7) qb = -7; if (qb > 7) qb = 7;
@@ -556,18 +565,18 @@ float orc_q4_unpack(uint8_t packed, uint32_t lane, float scale) {
  *   value = fmaf((float)q, d, m)  (one rounding, no pass through f16). */
 void orc_q4g32_quantize_row(const uint16_t* v_f16, uint32_t head_dim, uint8_t* packed, uint32_t* dm) {
     for (uint32_t g = 0; g < head_dim / 32u; ++g) {
-        float mn = orc_f16_to_f32(v_f16[32 * g]), mx = mn;
+        float mn = h2f(v_f16[32 * g]), mx = mn;
         for (uint32_t i = 1; i < 32u; ++i) {
-            const float v = orc_f16_to_f32(v_f16[32 * g + i]);
+            const float v = h2f(v_f16[32 * g + i]);
             mn = fminf(mn, v); mx = fmaxf(mx, v);
         }
         const uint16_t db = orc_f32_to_f16((mx - mn) / 15.0f), mb = orc_f32_to_f16(mn);
-        const float d = orc_f16_to_f32(db), m = orc_f16_to_f32(mb);
+        const float d = h2f(db), m = h2f(mb);
         dm[g] = (uint32_t)db | ((uint32_t)mb << 16);
         for (uint32_t pair = 0; pair < 16u; ++pair) {
             long q[2];
             for (int e = 0; e < 2; ++e) {
-                const float v = orc_f16_to_f32(v_f16[32 * g + 2 * pair + e]);
+                const float v = h2f(v_f16[32 * g + 2 * pair + e]);
                 q[e] = d > 0.0f ? lrintf((v - m) / d) : 0;
                 if (q[e] < 0) q[e] = 0;
                 if (q[e] > 15) q[e] = 15;
@@ -578,7 +587,7 @@ void orc_q4g32_quantize_row(const uint16_t* v_f16, uint32_t head_dim, uint8_t* p
 }
 float orc_q4g32_unpack(uint8_t packed, uint32_t lane, uint32_t dm) {
     const uint8_t nib = lane == 0u ? (packed & 0x0f) : ((packed >> 4) & 0x0f);
-    return fmaf((float)nib, orc_f16_to_f32((uint16_t)(dm & 0xffffu)), orc_f16_to_f32((uint16_t)(dm >> 16)));
+    return fmaf((float)nib, h2f((uint16_t)(dm & 0xffffu)), h2f((uint16_t)(dm >> 16)));
 }
 
 /* m40llm_kvcache_append_token_f32_rope_k_compressed_at_layout_async,
@@ -635,7 +644,7 @@ static uint32_t block_scores_impl(const uint16_t* kbase, uint32_t kv_heads, uint
             for (uint32_t t = start; t < end; ++t) {
                 const uint16_t* k = kbase + (size_t)t * ept + (size_t)kvh * head_dim;
                 for (uint32_t d = 0; d < head_dim; ++d)
-                    acc += (double)qh[d] * (double)orc_f16_to_f32(k[d]);
+                    acc += (double)qh[d] * (double)h2f(k[d]);
             }
             const double sc = acc / (double)(end - start) * (double)inv_sqrt;
             if (out_f64) out_f64[b] = sc;
@@ -647,7 +656,7 @@ static uint32_t block_scores_impl(const uint16_t* kbase, uint32_t kv_heads, uint
                 for (uint32_t t = start; t < end; ++t) {
                     const uint16_t* k = kbase + (size_t)t * ept + (size_t)kvh * head_dim;
                     for (uint32_t d = tid; d < head_dim; d += 128)
-                        part = fmaf(qh[d], orc_f16_to_f32(k[d]), part); /* nvcc contracts a*b+c */
+                        part = fmaf(qh[d], h2f(k[d]), part); /* nvcc contracts a*b+c */
                 }
                 red[tid] = part;
             }
@@ -663,7 +672,7 @@ static uint32_t block_scores_impl(const uint16_t* kbase, uint32_t kv_heads, uint
                 for (int j = 0; j < 8; ++j) sum[lane][j] = 0.0f;
                 for (uint32_t t = start + g; t < end; t += R) {
                     const uint16_t* k = kbase + (size_t)t * ept + (size_t)kvh * head_dim + 8u * c;
-                    for (int j = 0; j < 8; ++j) sum[lane][j] += orc_f16_to_f32(k[j]);
+                    for (int j = 0; j < 8; ++j) sum[lane][j] += h2f(k[j]);
                 }
             }
             for (uint32_t stride = R / 2u; stride > 0; stride >>= 1) { /* butterfly over g */
@@ -760,13 +769,13 @@ static float src_v(const kv_src* s, uint32_t t, uint32_t kvh, uint32_t d) {
                 return orc_q4g32_unpack(s->c->q4_v[q4_base + d / 2u], d & 1u,
                                         s->c->q4_dm[sc_idx * (s->head_dim / 32) + d / 32u]);
             const float v = orc_q4_unpack(s->c->q4_v[q4_base + d / 2u], d & 1u, s->c->q4_scale[sc_idx]);
-            return orc_f16_to_f32(orc_f32_to_f16(v)); /* rounded through f16, kernels.cu:3085-3086 */
+            return h2f(orc_f32_to_f16(v)); /* rounded through f16, kernels.cu:3085-3086 */
         }
         const size_t ept = (size_t)s->kv_heads * s->head_dim;
-        return orc_f16_to_f32(s->c->recent_v[((size_t)s->seq * s->recent_window + (t % s->recent_window)) * ept +
+        return h2f(s->c->recent_v[((size_t)s->seq * s->recent_window + (t % s->recent_window)) * ept +
                                              (size_t)kvh * s->head_dim + d]);
     }
-    return orc_f16_to_f32(s->V[orc_kv_index(s->max_seq_len, s->kv_heads, s->head_dim, s->seq, t, kvh, d)]);
+    return h2f(s->V[orc_kv_index(s->max_seq_len, s->kv_heads, s->head_dim, s->seq, t, kvh, d)]);
 }
 
 static void attend_token_list(const kv_src* s, const float* qh, uint32_t kvh, const uint32_t* tokens,
@@ -776,7 +785,7 @@ static void attend_token_list(const kv_src* s, const float* qh, uint32_t kvh, co
     for (uint32_t i = 0; i < n; ++i) {
         const uint16_t* k = src_k_row(s, tokens[i], kvh);
         float dot = 0.0f;
-        for (uint32_t d = 0; d < s->head_dim; ++d) dot += qh[d] * orc_f16_to_f32(k[d]);
+        for (uint32_t d = 0; d < s->head_dim; ++d) dot += qh[d] * h2f(k[d]);
         scores[i] = dot * inv_sqrt;
         if (scores[i] > max_score) max_score = scores[i];
     }
@@ -912,7 +921,7 @@ int orc_ckv_debug_select_old_blocks(const orc_ckv* c, uint32_t seq, const float*
         float score = 0.0f;
         for (uint32_t pos = start; pos < end; ++pos)
             for (uint32_t d = 0; d < hd; ++d)
-                score += q_head0[d] * orc_f16_to_f32(kbase[(size_t)pos * ept + d]);
+                score += q_head0[d] * h2f(kbase[(size_t)pos * ept + d]);
         score /= (float)(end - start);
         sc[b] = score * scale;
         idx[b] = b;
