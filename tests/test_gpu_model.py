@@ -363,11 +363,12 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
     """BASELINE config 3 at full depth: 36 layers (four distinct random layers repeated, every layer its own device
     copy, as the benchmark builds it), hidden 2048, 16 q / 2 kv heads, hd 128, FFN 11008, vocab 151936, biases, NeoX
     RoPE theta 1e6; batch 8, contexts U[256, 4096] pre-filled N(0,1), 64 greedy steps on the fused graph path.  The
-    oracle decodes the rows with the longest and the shortest context for all 64 steps and the other six rows for 8
-    (about a second of 16 threads per token); then 8 steps of all rows through the reference's row-batched call sequence."""
+    oracle decodes the rows with the longest and the shortest context for all 64 steps and the other six rows for 32
+    (about a third of a second of 16 threads per token); then 8 steps of all rows through the reference's row-batched
+    call sequence."""
     cfg = dict(syn.QWEN25_3B)
     W = syn.make_weights(cfg, seed=0, unique_layers=4, tie_embeddings=True)
-    B, steps, short_steps = 8, 64, 8
+    B, steps, short_steps, reference_steps = 8, 64, 32, 8
     S = 4096 + steps + 8
     L, KVH, HD = cfg["n_layers"], cfg["kv_heads"], cfg["head_dim"]
     rng = np.random.default_rng(0)
@@ -393,7 +394,7 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
                 slot = dm.H.m40host_model_kv_slot(dm.h, s, l)
                 m40.check(ctx.lib.m40llm_ext_kvcache_bulk_fill_f16(ctx.h, dm.kv_handle(), slot, dk.ptr, dv.ptr, int(lens[s])),
                           "m40llm_ext_kvcache_bulk_fill_f16")
-        run_steps = steps if mode == 2 else short_steps
+        run_steps = steps if mode == 2 else reference_steps
         ids, gaps = dm.decode_batch_greedy(np.arange(B), lens, toks, run_steps)
         for s in range(B):
             wid, wgap, wscale = want[s]
