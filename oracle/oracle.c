@@ -23,6 +23,8 @@
  *                           norm preservation and position 0 = identity
  *   greedy ................ reference literals ([0.1,-0.2,5,1]->2, [0,5,1]->1, NaN case)
  *   layer / model ......... float64 numpy restatement on a toy model; L=1 => context=V
+ *   packed prefill forward  float64 restatement without the f16 round trip of K / V (fits to 2e-5, the one with the
+ *                           round trip does not); batch == each prompt alone; layer-0 cache == the token path's
  */
 #include "oracle.h"
 
@@ -1100,6 +1102,71 @@ void orc_token_forward(const orc_model* m, orc_model_kv* kv, uint32_t seq, uint3
     }
     memcpy(hidden_out, a, sizeof(float) * D);
     free(a); free(b);
+}
+
+/* Packed prefill of several prompts: all tokens of all prompts as rows of one batch, layer by layer
+ * (src/infer/forward.rs:2153-2600).  Per layer: RMSNorm of every row, Q / K / V projections (+ bias), then per prompt
+ * and token the append of the rotated K and of V to the f16 cache at the token's position and the rotation of the f32
+ * Q and K rows in place (forward.rs:2349-2396); the packed causal attention runs on the f32 Q, K, V rows -- NOT on the
+ * f16 cache, which is where this path differs from the token-by-token one (forward.rs:2404-2415) -- then O projection +
+ * residual, RMSNorm, gate / up, SwiGLU, down + residual.  Every prompt starts at position 0.  hidden_out receives the
+ * rows [total][d_model] of the last layer.  Returns 0, or the attention's argument-check code. */
+int orc_prefill_forward(const orc_model* m, orc_model_kv* kv, const uint32_t* seq_ids, const uint32_t* lens,
+                        const uint32_t* tokens, uint32_t batch, float* hidden_out) {
+    const uint32_t D = m->d_model, kv_dim = m->kv_heads * m->head_dim, F = m->ffn;
+    size_t rows = 0;
+    uint32_t* offsets = (uint32_t*)malloc(sizeof(uint32_t) * (batch ? batch : 1));
+    for (uint32_t i = 0; i < batch; ++i) { offsets[i] = (uint32_t)rows; rows += lens[i]; }
+    float* a = (float*)malloc(sizeof(float) * rows * D);
+    float* b = (float*)malloc(sizeof(float) * rows * D);
+    float* xn = (float*)malloc(sizeof(float) * rows * D);
+    float* q = (float*)malloc(sizeof(float) * rows * D);
+    float* k = (float*)malloc(sizeof(float) * rows * kv_dim);
+    float* v = (float*)malloc(sizeof(float) * rows * kv_dim);
+    float* att = (float*)malloc(sizeof(float) * rows * D);
+    float* y = (float*)malloc(sizeof(float) * rows * D);
+    float* x1 = (float*)malloc(sizeof(float) * rows * D);
+    float* gate = (float*)malloc(sizeof(float) * rows * F);
+    float* up = (float*)malloc(sizeof(float) * rows * F);
+    int rc = 0;
+    for (size_t r = 0; r < rows; ++r) orc_f16_to_f32_n(m->tok_emb + (size_t)tokens[r] * D, a + r * D, D);
+    for (uint32_t l = 0; l < m->n_layers && rc == 0; ++l) {
+        orc_rms_norm_weighted(a, m->attn_norm[l], xn, (uint32_t)rows, D, m->rms_eps, 1);
+        orc_gemm_f32xf16_gguf(xn, m->wq[l], q, (int)rows, (int)D, (int)D);
+        orc_gemm_f32xf16_gguf(xn, m->wk[l], k, (int)rows, (int)kv_dim, (int)D);
+        orc_gemm_f32xf16_gguf(xn, m->wv[l], v, (int)rows, (int)kv_dim, (int)D);
+        if (m->has_qkv_bias)
+            for (size_t r = 0; r < rows; ++r) {
+                orc_residual_add(q + r * D, m->bq[l], q + r * D, D);
+                orc_residual_add(k + r * kv_dim, m->bk[l], k + r * kv_dim, kv_dim);
+                orc_residual_add(v + r * kv_dim, m->bv[l], v + r * kv_dim, kv_dim);
+            }
+        for (uint32_t i = 0; i < batch; ++i) {
+            const uint32_t slot = seq_ids[i] * m->n_layers + l;
+            for (uint32_t t = 0; t < lens[i]; ++t) {
+                const size_t r = (size_t)offsets[i] + t;
+                orc_kv_append_f32_rope_k(kv->K, kv->V, kv->max_seq_len, m->kv_heads, m->head_dim, slot, t, k + r * kv_dim,
+                                         v + r * kv_dim, m->rope_base, m->rope_scale, m->rope_layout);
+                orc_rope_inplace(q + r * D, 1, m->q_heads, m->head_dim, t, m->rope_base, m->rope_scale, m->rope_layout);
+                orc_rope_inplace(k + r * kv_dim, 1, m->kv_heads, m->head_dim, t, m->rope_base, m->rope_scale, m->rope_layout);
+            }
+        }
+        rc = orc_attention_prefill_gqa_varlen(q, k, v, offsets, offsets, lens, lens, batch, m->q_heads, m->kv_heads,
+                                              m->head_dim, att);
+        if (rc != 0) break;
+        orc_gemm_f32xf16_gguf(att, m->wo[l], y, (int)rows, (int)D, (int)D);
+        orc_residual_add(a, y, x1, rows * D);
+        orc_rms_norm_weighted(x1, m->ffn_norm[l], xn, (uint32_t)rows, D, m->rms_eps, 1);
+        orc_gemm_f32xf16_gguf(xn, m->wgate[l], gate, (int)rows, (int)F, (int)D);
+        orc_gemm_f32xf16_gguf(xn, m->wup[l], up, (int)rows, (int)F, (int)D);
+        orc_swiglu(gate, up, gate, rows * F);
+        orc_gemm_f32xf16_gguf(gate, m->wdown[l], y, (int)rows, (int)D, (int)F);
+        orc_residual_add(x1, y, b, rows * D);
+        float* t = a; a = b; b = t;
+    }
+    if (rc == 0) memcpy(hidden_out, a, sizeof(float) * rows * D);
+    free(offsets); free(a); free(b); free(xn); free(q); free(k); free(v); free(att); free(y); free(x1); free(gate); free(up);
+    return rc;
 }
 
 void orc_logits(const orc_model* m, const float* hidden, float* logits) {

@@ -198,6 +198,10 @@ void orc_layer_forward(const orc_model* m, orc_model_kv* kv, uint32_t layer, uin
                        uint32_t pos, const float* x, float* out);
 void orc_token_forward(const orc_model* m, orc_model_kv* kv, uint32_t seq, uint32_t pos,
                        uint32_t token_id, float* hidden_out);
+/* packed prefill of several prompts as one batch of rows (src/infer/forward.rs:2153-2600): the attention runs on the
+ * f32 K / V rows, the f16 cache is written on the side; hidden_out = [sum of lens][d_model] */
+int  orc_prefill_forward(const orc_model* m, orc_model_kv* kv, const uint32_t* seq_ids, const uint32_t* lens,
+                         const uint32_t* tokens, uint32_t batch, float* hidden_out);
 void orc_logits(const orc_model* m, const float* hidden, float* logits);
 /* prompt then n_gen greedy tokens; ids_out holds n_prompt+n_gen ids; gaps_out
  * (may be NULL) holds the top-1/top-2 logit gap of each generated token */

@@ -124,6 +124,7 @@ def lib() -> C.CDLL:
     sig("orc_model_kv_destroy", None, C.POINTER(OrcModelKv))
     sig("orc_layer_forward", None, C.POINTER(OrcModel), C.POINTER(OrcModelKv), u32, u32, u32, vp, vp)
     sig("orc_token_forward", None, C.POINTER(OrcModel), C.POINTER(OrcModelKv), u32, u32, u32, vp)
+    sig("orc_prefill_forward", C.c_int, C.POINTER(OrcModel), C.POINTER(OrcModelKv), vp, vp, vp, u32, vp)
     sig("orc_logits", None, C.POINTER(OrcModel), vp, vp)
     sig("orc_decode_greedy", None, C.POINTER(OrcModel), C.POINTER(OrcModelKv), u32, vp, u32, u32,
         u32, vp, vp)
@@ -470,6 +471,16 @@ class Model:
     def token_forward(self, seq, pos, token_id):
         out = np.empty(self.cfg["d_model"], dtype=np.float32)
         lib().orc_token_forward(C.byref(self.m), self.kv, seq, pos, int(token_id), ptr(out))
+        return out
+
+    def prefill_forward(self, seq_ids, prompts):
+        """Packed prefill of several prompts (each from position 0 of its sequence): hidden rows [sum of lens][d_model]."""
+        ids = np.ascontiguousarray(seq_ids, dtype=np.uint32)
+        lens = np.ascontiguousarray([len(p) for p in prompts], dtype=np.uint32)
+        toks = np.ascontiguousarray(np.concatenate([np.asarray(p, dtype=np.uint32) for p in prompts]))
+        out = np.empty((int(lens.sum()), self.cfg["d_model"]), dtype=np.float32)
+        rc = lib().orc_prefill_forward(C.byref(self.m), self.kv, ptr(ids), ptr(lens), ptr(toks), len(ids), ptr(out))
+        assert rc == 0, rc
         return out
 
     def logits(self, hidden):

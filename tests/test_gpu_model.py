@@ -359,6 +359,57 @@ def test_tinyllama_full_depth_greedy_ids_graph_mode(ctx, orc, heartbeat):
     dm.close()
 
 
+def test_tinyllama_full_depth_packed_prefill_vs_oracle(ctx, orc, heartbeat):
+    """The packed prefill forward at the full BASELINE config-2 shape (22 layers): two prompts of 700 and 330 tokens as
+    one batch of 1030 rows -- the gate / up projection runs on the 128 x 256-tile GEMM, the others on the 128 x 128 one,
+    the attention with two query blocks per wave -- against the oracle's packed prefill (src/infer/forward.rs:2153-2600:
+    the attention reads the f32 K / V rows): last hidden state and logits of each prompt inside the float bar of the
+    decode tests, the same next token.  The token-by-token paths (the device's and the oracle's), whose attention reads K
+    and V back from the f16 cache, agree within the reference's own whole-model tolerance (5e-3,
+    tests/forward_parity_toy.rs:389).  The 16 greedy tokens that the graph path then decodes from the cache the prefill
+    wrote equal the oracle's from its own prefill's cache (up to a listed tie)."""
+    cfg = dict(syn.TINYLLAMA_1B)
+    W = syn.make_weights(cfg, seed=0)
+    lens, n_gen = (700, 330), 16
+    S = max(lens) + n_gen + 8
+    rng = np.random.default_rng(4)
+    prompts = [rng.integers(0, cfg["vocab"], size=n).astype(np.uint32) for n in lens]
+    om = _oracle_model(orc, cfg, W, S, 2)
+    orc.set_threads(16)
+    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=2)
+    dm.set_mode(2)
+    hid, log = dm.forward_prefill([0, 1], [p.tolist() for p in prompts])
+    heartbeat()
+    want_rows = om.prefill_forward([0, 1], [p.tolist() for p in prompts])         # about a minute of 16 threads
+    heartbeat()
+    one = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=1)      # the per-token device path (fused kernels)
+    one.set_mode(1)
+    end = np.cumsum(lens) - 1
+    for s, p in enumerate(prompts):
+        want_h = want_rows[end[s]]
+        wl = om.logits(want_h)
+        dh, dl = float(np.abs(hid[s] - want_h).max()), float(np.abs(log[s] - wl).max())
+        print(f"[tinyllama-22L prefill, prompt of {len(p)}] hidden deviation {dh:.3e} (largest |hidden| {np.abs(want_h).max():.3e}), "
+              f"logit deviation {dl:.3e} = {dl / (1e-3 * np.abs(wl).max() + 1e-4):.3f} of the bar")
+        # a fifth of the float bar (measured: a hundredth of it -- 1e-5 of the largest element)
+        assert dh <= 2e-4 * np.abs(want_h).max() + 1e-4, (s, dh)
+        assert dl <= 2e-4 * np.abs(wl).max() + 1e-4, (s, dl)
+        for pos, t in enumerate(p):
+            th, tl = one.forward_token(0, pos, int(t), want_hidden=pos == len(p) - 1, want_logits=pos == len(p) - 1)
+        dth = float(np.abs(hid[s] - th).max())
+        print(f"[tinyllama-22L prefill, prompt of {len(p)}] against the device's token-by-token forward (K / V through f16): hidden {dth:.3e}")
+        assert dth <= 5e-3 * np.abs(th).max(), (s, dth)
+        first = int(orc.greedy_topk1(wl))
+        top2 = np.partition(wl, -2)[-2:]
+        if int(np.argmax(log[s])) != first:
+            assert float(top2[1] - top2[0]) <= _tie_bound(float(np.abs(wl).max())), s
+            continue                     # a tie at the first pick: the two runs are different sequences from here
+        want, wgap, wscale = _oracle_greedy_with_logits(orc, om, s, [first], n_gen, start_pos=len(p), beat=heartbeat)
+        got, _ = dm.decode_greedy(s, [first], n_gen, start_pos=len(p))
+        _assert_ids_equal_up_to_legitimate_tie(got[1:], want[1:], wgap, wscale, f"tinyllama-22L decode after a prefill of {len(p)}")
+    dm.close(); one.close()
+
+
 def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
     """BASELINE config 3 at full depth: 36 layers (four distinct random layers repeated, every layer its own device
     copy, as the benchmark builds it), hidden 2048, 16 q / 2 kv heads, hd 128, FFN 11008, vocab 151936, biases, NeoX

@@ -601,8 +601,10 @@ def make_toy_model(rng, qkv_bias, rope_layout, n_layers=2, d_model=64, q_heads=4
     return cfg, W
 
 
-def f64_model_logits(cfg, W, ids):
-    """Independent float64 restatement of the decoder (full-sequence causal attention), last-token logits."""
+def f64_model_logits(cfg, W, ids, kv_through_f16=True, want_hidden=False):
+    """Independent float64 restatement of the decoder (full-sequence causal attention), last-token logits.
+    kv_through_f16: K and V pass through the f16 cache (the token-by-token path); False = the packed prefill, whose
+    attention reads the f32 rows."""
     f = lambda a: a.view(np.float16).astype(np.float64)
     D, H, KVH, hd = cfg["d_model"], cfg["q_heads"], cfg["kv_heads"], cfg["head_dim"]
     T = len(ids)
@@ -624,7 +626,7 @@ def f64_model_logits(cfg, W, ids):
             a, b = t[..., : hd // 2].copy(), t[..., hd // 2:].copy()
             t[..., : hd // 2], t[..., hd // 2:] = a * c - b * s, a * s + b * c
         return t
-    h16 = lambda a: a.astype(np.float16).astype(np.float64)
+    h16 = (lambda a: a.astype(np.float16).astype(np.float64)) if kv_through_f16 else (lambda a: a)
     for l in range(cfg["n_layers"]):
         xn = norm(x, W["attn_norm"][l])
         q = xn @ f(W["wq"][l]).T; k = xn @ f(W["wk"][l]).T; v = xn @ f(W["wv"][l]).T
@@ -641,6 +643,8 @@ def f64_model_logits(cfg, W, ids):
         xn = norm(x, W["ffn_norm"][l])
         g = xn @ f(W["wgate"][l]).T; u = xn @ f(W["wup"][l]).T
         x = x + (g / (1 + np.exp(-g)) * u) @ f(W["wdown"][l]).T
+    if want_hidden:
+        return x
     return norm(x[-1:], W["out_norm"]) @ f(W["lm_head"]).T
 
 
@@ -662,6 +666,44 @@ def test_model_decode_vs_float64(orc, qkv_bias, layout):
     out_ids, gaps = m.decode_greedy(0, ids, 4)
     assert list(out_ids[: len(ids)]) == ids and out_ids[len(ids)] == int(np.argmax(want))
     assert (gaps >= 0).all()
+
+
+@pytest.mark.parametrize("qkv_bias,layout", [(False, 0), (True, 1)])
+def test_packed_prefill_forward_vs_float64_and_token_by_token(orc, qkv_bias, layout):
+    # src/infer/forward.rs:2153-2600: the packed prefill's attention reads the f32 K / V rows, the f16 cache is written on
+    # the side.  The float64 restatement without the f16 round trip must fit tightly, the one with it must not (the bound
+    # tells the two apart); the token-by-token path agrees within the reference's own whole-model tolerance
+    # (tests/forward_parity_toy.rs:389); a batch of prompts equals each prompt alone; and the cache the prefill leaves
+    # serves the decode that follows.
+    rng = np.random.default_rng(53 + layout)
+    cfg, W = make_toy_model(rng, qkv_bias, layout, n_layers=3, d_model=256, ffn=160)      # head_dim 64: the packed attention takes 64 or 128
+    prompts = [[3, 17, 42, 8, 8, 29, 11, 2, 40], [5], [7, 7, 30, 1]]
+    m = orc.Model(cfg, W)
+    m.alloc_kv(16, 3)
+    rows = m.prefill_forward([2, 0, 1], prompts)
+    off = np.concatenate([[0], np.cumsum([len(p) for p in prompts])])
+    for i, p in enumerate(prompts):
+        got = rows[off[i]:off[i + 1]]
+        want = f64_model_logits(cfg, W, np.array(p), kv_through_f16=False, want_hidden=True)
+        rounded = f64_model_logits(cfg, W, np.array(p), kv_through_f16=True, want_hidden=True)
+        scale = np.abs(want).max()
+        assert np.abs(got - want).max() <= 2e-5 * scale, (i, np.abs(got - want).max() / scale)
+        if len(p) > 1:      # one token: softmax over one key, the rounding of K has no effect and that of V is below the bound
+            assert np.abs(got - rounded).max() > 2e-5 * scale, (i, np.abs(got - rounded).max() / scale)
+        alone = orc.Model(cfg, W)
+        alone.alloc_kv(16, 1)
+        assert np.array_equal(alone.prefill_forward([0], [p]).view(np.uint32), got.view(np.uint32))
+        tok = orc.Model(cfg, W)
+        tok.alloc_kv(16, 1)
+        for pos, t in enumerate(p):
+            h = tok.token_forward(0, pos, t)
+        assert np.abs(got[-1] - h).max() <= 5e-3 * max(1.0, np.abs(h).max())
+        # layer 0 sees the same rows in both paths: its cache entries are the same bits
+        Kp, Vp = alone.kv_views(); Kt, Vt = tok.kv_views()
+        assert np.array_equal(Kp[0, :len(p)], Kt[0, :len(p)]) and np.array_equal(Vp[0, :len(p)], Vt[0, :len(p)])
+    # the decode that follows a prefill continues from its cache
+    ids, _ = m.decode_greedy(2, [int(np.argmax(m.logits(rows[off[1] - 1])))], 3, start_pos=len(prompts[0]))
+    assert len(ids) == 4
 
 
 def test_layer_single_token_context_is_v(orc):
