@@ -30,11 +30,11 @@ def _toy_cfg(layout, bias, hd=64):
                 rope_base=10000.0 if layout == 0 else 1e6, rope_scale=1.0, rope_layout=layout, qkv_bias=bias)
 
 
-def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0, beat=None):
+def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0, beat=None, hidden=None):
     """orc_decode_greedy's loop (oracle/oracle.c) driven from here so that every pick's logits row is seen:
-    returns ids (prompt + picks), the top-1 / top-2 gap and the largest |logit| of every pick."""
+    returns ids (prompt + picks), the top-1 / top-2 gap and the largest |logit| of every pick.  `hidden`: the state the
+    first pick is made from when the prompt has already been run (a packed prefill up to start_pos)."""
     pos = start_pos
-    hidden = None
     for t in prompt:
         hidden = om.token_forward(seq, pos, int(t)); pos += 1
     ids, gaps, scale = [int(t) for t in prompt], [], []

@@ -8,6 +8,7 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 from gpu_common import m40  # noqa: E402
+from test_gpu_model import _assert_ids_equal_up_to_legitimate_tie, _oracle_greedy_with_logits  # noqa: E402
 
 syn = importlib.import_module("m40-llm_amd.synthetic")
 sch = importlib.import_module("m40-llm_amd.scheduler")
@@ -48,5 +49,44 @@ def test_scheduler_outputs_equal_oracle_greedy_per_request(ctx, orc, mode, hd):
         assert s.state(rids[i]) == "complete", s.error(rids[i])
         assert s.generated(rids[i]) == want[len(prompt):].tolist(), (i, float(gaps.min()))
     assert s.available_slots() == 3
+    s.close()
+    dm.close()
+
+
+def test_scheduler_full_depth_tinyllama_requests_equal_oracle(ctx, orc, heartbeat):
+    """The scheduler at the full BASELINE config-2 shape (22 layers): six requests with prompts of 40-150 tokens on four
+    slots, arrivals spread over the ticks, so that packed prefills of one to three prompts, batched decode steps of one to
+    four rows with device-side picks, and reused slots all occur.  Each request's tokens equal what the oracle generates
+    for it alone -- its prompt through the oracle's packed prefill, as the scheduler runs prompts
+    (src/server.rs:420-560 -> forward.rs:2153-2600), then token by token -- up to a listed tie."""
+    cfg = dict(syn.TINYLLAMA_1B)
+    W = syn.make_weights(cfg, seed=0)
+    S, n_new = 192, 12
+    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=4)
+    dm.set_mode(2)
+    om = orc.Model(dict(cfg, qkv_bias=False), W)
+    orc.set_threads(16)
+    rng = np.random.default_rng(11)
+    specs = [rng.integers(0, cfg["vocab"], size=n).tolist() for n in (150, 40, 97, 64, 120, 41)]
+    s = sch.Scheduler.for_model(dm)
+    rids, pending, ticks = {}, list(enumerate(specs)), 0
+    while pending or s.active():
+        # three arrivals at the start (one packed prefill of three prompts), later ones as slots free up, two at a time
+        burst = 3 if ticks == 0 else 2
+        while pending and s.available_slots() and burst and (ticks == 0 or ticks % 5 == 0):
+            i, prompt = pending.pop(0)
+            rids[i] = s.submit(prompt, max_tokens=n_new)
+            burst -= 1
+        s.tick()
+        ticks += 1
+        assert ticks < 400
+    for i, prompt in enumerate(specs):
+        assert s.state(rids[i]) == "complete", s.error(rids[i])
+        om.alloc_kv(S, 1)
+        hidden = om.prefill_forward([0], [prompt])[-1]
+        want, wgap, wscale = _oracle_greedy_with_logits(orc, om, 0, [], n_new, start_pos=len(prompt), hidden=hidden)
+        heartbeat()
+        _assert_ids_equal_up_to_legitimate_tie(s.generated(rids[i]), want, wgap, wscale, f"scheduler, 22 layers, request {i} (prompt of {len(prompt)})")
+    assert s.available_slots() == 4
     s.close()
     dm.close()
