@@ -35,14 +35,14 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
-// 16-query blocks per wave: a K / V fragment read from LDS serves every block of the wave.  head_dim 64 always takes two
-// (one / two blocks at one sequence of 4096 tokens and 32 heads: 0.316 / 0.298 ms).  head_dim 128 takes two where long
-// sequences alone fill the chip four workgroups deep and one otherwise -- two blocks halve the workgroup count and double
-// the masked share of a short sequence's diagonal tiles (16 / 32 q heads, one against two blocks: 1 x 4096 tokens
-// 0.30 / 0.33 and 0.63 / 0.53 ms, 4 x 4096 1.17 / 1.02 and 2.13 / 1.85 ms, 16 x 300 0.069 / 0.077 and 0.099 / 0.112 ms).
-constexpr int kQBlocks64 = 2;
+// 16-query blocks per wave: a K / V fragment read from LDS serves every block of the wave.  Two blocks where long
+// sequences alone fill the chip four workgroups deep, one otherwise -- two blocks halve the workgroup count and double
+// the masked share of a short sequence's diagonal tiles.  One against two blocks, head_dim 128 at 16 / 32 q heads:
+// 1 x 4096 tokens 0.30 / 0.33 and 0.63 / 0.53 ms, 4 x 4096 1.17 / 1.02 and 2.13 / 1.85 ms, 16 x 300 0.069 / 0.077 and
+// 0.099 / 0.112 ms; head_dim 64 at 32 q heads: 1 x 1024 48 / 52 us, 1 x 2048 94 / 102 us, 16 x 300 59 / 69 us,
+// 1 x 4096 0.260 / 0.240 ms, 2 x 4096 0.58 / 0.51 ms.
 constexpr float kRefSlack = 8.0f;          // log2 units: weights stay below 256
-constexpr uint32_t kTwoBlockMinQueries = 1024;      // a sequence counts as long from here
+constexpr uint32_t kTwoBlockMinQueries = 2048;      // a sequence counts as long from here
 constexpr int kTwoBlockMinGroupsPerCu = 4;
 // keys per LDS tile (KT below): one or two k-steps of the P . V product; 64 where two planes of K and V^T fit the
 // static LDS limit (head_dim 64), 32 otherwise
@@ -449,13 +449,13 @@ int prefill_impl(M40llmCudaContext* ctx, const void* q, const void* k, const voi
     uint64_t long_groups = 0;           // two-block workgroups that the long sequences make
     for (uint32_t i = 0; i < batch; ++i)
         if (host[i] >= kTwoBlockMinQueries) long_groups += (uint64_t)((host[i] + 32u * kWaves - 1) / (32u * kWaves)) * q_heads;
-    const uint32_t blocks = head_dim == 64 ? (uint32_t)kQBlocks64
-                          : (long_groups >= (uint64_t)kTwoBlockMinGroupsPerCu * (uint64_t)ctx->num_cus ? 2u : 1u);
+    const uint32_t blocks = long_groups >= (uint64_t)kTwoBlockMinGroupsPerCu * (uint64_t)ctx->num_cus ? 2u : 1u;
     const uint32_t q_group = 16u * kWaves * blocks;     // queries per workgroup
     const dim3 grid(q_heads, (max_q + q_group - 1) / q_group, batch);
     if (head_dim == 64) {
         prefill_pack_kv_kernel<64><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
-        prefill_attn_kernel<64, kQBlocks64><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        if (blocks == 2) prefill_attn_kernel<64, 2><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
+        else prefill_attn_kernel<64, 1><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);
     } else {
         prefill_pack_kv_kernel<128><<<pack_grid, kThreads, 0, ctx->prefill_stream>>>(a);
         if (blocks == 2) prefill_attn_kernel<128, 2><<<grid, kThreads, 0, ctx->prefill_stream>>>(a);

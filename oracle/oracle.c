@@ -383,8 +383,14 @@ void orc_attention_last_token_gqa(const uint16_t* K, const uint16_t* V, uint32_t
                                   const float* q, uint32_t q_heads, uint32_t seq_len, float* out) {
     const uint32_t group = q_heads / kv_heads;
     const float inv_sqrt = orc_inv_sqrt_head_dim(head_dim);
-    float* scores = (float*)malloc(sizeof(float) * (seq_len ? seq_len : 1));
+    /* Heads are independent and spread over threads (when this call is not itself inside a parallel loop).  The weight
+     * of a key, expf(score - max) / denom, is the same number for every output column: it is computed once per key, and
+     * the weighted sum walks the keys in the outer loop with one accumulator per column -- every column's own sum still
+     * adds its keys in ascending order, so the results are the reference's bit for bit. */
+#pragma omp parallel for schedule(dynamic) if ((size_t)seq_len * q_heads >= 4096)
     for (uint32_t h = 0; h < q_heads; ++h) {
+        float* scores = (float*)malloc(sizeof(float) * ((size_t)(seq_len ? seq_len : 1) + head_dim));
+        float* acc = scores + (seq_len ? seq_len : 1);
         const uint32_t kvh = h / group;
         const float* qh = q + (size_t)h * head_dim;
         float max_score = -INFINITY;
@@ -399,18 +405,16 @@ void orc_attention_last_token_gqa(const uint16_t* K, const uint16_t* V, uint32_t
         float denom = 0.0f;
         for (uint32_t t = 0; t < seq_len; ++t) denom += expf(scores[t] - max_score);
         if (!(denom > 0.0f)) denom = 1.0f;
-        float* oh = out + (size_t)h * head_dim;
-        for (uint32_t d = 0; d < head_dim; ++d) {
-            float acc = 0.0f;
-            for (uint32_t t = 0; t < seq_len; ++t) {
-                const size_t base = orc_kv_index(max_seq_len, kv_heads, head_dim, seq, t, kvh, 0);
-                const float p = expf(scores[t] - max_score) / denom;
-                acc += p * h2f(V[base + d]);
-            }
-            oh[d] = acc;
+        for (uint32_t d = 0; d < head_dim; ++d) acc[d] = 0.0f;
+        for (uint32_t t = 0; t < seq_len; ++t) {
+            const size_t base = orc_kv_index(max_seq_len, kv_heads, head_dim, seq, t, kvh, 0);
+            const float p = expf(scores[t] - max_score) / denom;
+            for (uint32_t d = 0; d < head_dim; ++d) acc[d] += p * h2f(V[base + d]);
         }
+        float* oh = out + (size_t)h * head_dim;
+        for (uint32_t d = 0; d < head_dim; ++d) oh[d] = acc[d];
+        free(scores);
     }
-    free(scores);
 }
 
 /* Reference: cuda/kernels.cu:1740-1823 (one row per batch entry, rows with
@@ -450,10 +454,14 @@ int orc_attention_prefill_gqa_varlen(const float* q, const float* k, const float
         if (q_lens[b] == 0 || kv_lens[b] == 0 || q_lens[b] > kv_lens[b] || kv_lens[b] > 8192) return -8;
     const uint32_t group = q_heads / kv_heads;
     const float inv_sqrt = orc_inv_sqrt_head_dim(head_dim);
-#pragma omp parallel for schedule(dynamic) if (batch > 1)
+    /* queries are independent and spread over threads; a key's weight is computed once and the weighted sum keeps one
+     * accumulator per column with the keys in the outer loop (each column's sum in ascending key order, as in the
+     * reference: the same bits) */
     for (uint32_t b = 0; b < batch; ++b) {
-        float* scores = (float*)malloc(sizeof(float) * kv_lens[b]);
+#pragma omp parallel for schedule(dynamic, 4)
         for (uint32_t qi = 0; qi < q_lens[b]; ++qi) {
+            float* scores = (float*)malloc(sizeof(float) * ((size_t)kv_lens[b] + head_dim));
+            float* acc = scores + kv_lens[b];
             const uint32_t causal_end = kv_lens[b] - q_lens[b] + qi;
             for (uint32_t h = 0; h < q_heads; ++h) {
                 const uint32_t kvh = h / group;
@@ -470,18 +478,17 @@ int orc_attention_prefill_gqa_varlen(const float* q, const float* k, const float
                 float denom = 0.0f;
                 for (uint32_t t = 0; t <= causal_end; ++t) denom += expf(scores[t] - max_score);
                 if (!(denom > 0.0f)) denom = 1.0f;
-                float* oh = out + ((size_t)(q_offsets[b] + qi) * q_heads + h) * head_dim;
-                for (uint32_t d = 0; d < head_dim; ++d) {
-                    float acc = 0.0f;
-                    for (uint32_t t = 0; t <= causal_end; ++t) {
-                        const float* vh = v + ((size_t)(kv_offsets[b] + t) * kv_heads + kvh) * head_dim;
-                        acc += (expf(scores[t] - max_score) / denom) * vh[d];
-                    }
-                    oh[d] = acc;
+                for (uint32_t d = 0; d < head_dim; ++d) acc[d] = 0.0f;
+                for (uint32_t t = 0; t <= causal_end; ++t) {
+                    const float* vh = v + ((size_t)(kv_offsets[b] + t) * kv_heads + kvh) * head_dim;
+                    const float p = expf(scores[t] - max_score) / denom;
+                    for (uint32_t d = 0; d < head_dim; ++d) acc[d] += p * vh[d];
                 }
+                float* oh = out + ((size_t)(q_offsets[b] + qi) * q_heads + h) * head_dim;
+                for (uint32_t d = 0; d < head_dim; ++d) oh[d] = acc[d];
             }
+            free(scores);
         }
-        free(scores);
     }
     return 0;
 }

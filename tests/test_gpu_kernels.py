@@ -854,9 +854,10 @@ def test_prefill_varlen_reference_fixture(dev, orc, hd):
     (32, 4, 64, [300, 17], [300, 529]),                     # config-1 heads, several query tiles
     (3, 3, 128, [129], [1000]),                             # 871 cached keys ahead of the queries
     (16, 2, 128, [5, 5, 5, 5, 5], [8192, 5, 37, 64, 65]),   # the longest allowed key range
-    # head_dim 128 with enough long sequences for the form of two 16-query blocks per wave (1120 workgroups of 128
-    # queries from the four long ones), a short sequence and cached keys ahead of the queries in the same batch
-    (32, 4, 128, [1061, 1100, 50, 1024, 1030], [1161, 1100, 50, 1024, 1093]),
+    # enough long sequences (2048 queries and more) for the form of two 16-query blocks per wave -- 1088 and 1056
+    # workgroups of 128 queries -- with a short sequence and cached keys ahead of the queries in the same batch
+    (32, 4, 128, [2061, 2100, 50], [2161, 2100, 50]),
+    (32, 4, 64, [2100, 2050, 70], [2133, 2050, 70]),
 ])
 def test_prefill_varlen_random_vs_oracle(dev, orc, qh, kvh, hd, ql, kl):
     rng = np.random.default_rng(len(ql) + hd)
