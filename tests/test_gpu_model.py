@@ -413,13 +413,12 @@ def test_tinyllama_full_depth_packed_prefill_vs_oracle(ctx, orc, heartbeat):
 def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
     """BASELINE config 3 at full depth: 36 layers (four distinct random layers repeated, every layer its own device
     copy, as the benchmark builds it), hidden 2048, 16 q / 2 kv heads, hd 128, FFN 11008, vocab 151936, biases, NeoX
-    RoPE theta 1e6; batch 8, contexts U[256, 4096] pre-filled N(0,1), 64 greedy steps on the fused graph path.  The
-    oracle decodes the rows with the longest and the shortest context for all 64 steps and the other six rows for 32
-    (about a third of a second of 16 threads per token); then 8 steps of all rows through the reference's row-batched
-    call sequence."""
+    RoPE theta 1e6; batch 8, contexts U[256, 4096] pre-filled N(0,1), 64 greedy steps on the fused graph path, every
+    row against the oracle's decode of that row alone (512 picks); then 8 steps of all rows through the reference's
+    row-batched call sequence."""
     cfg = dict(syn.QWEN25_3B)
     W = syn.make_weights(cfg, seed=0, unique_layers=4, tie_embeddings=True)
-    B, steps, short_steps, reference_steps = 8, 64, 32, 8
+    B, steps, reference_steps = 8, 64, 8
     S = 4096 + steps + 8
     L, KVH, HD = cfg["n_layers"], cfg["kv_heads"], cfg["head_dim"]
     rng = np.random.default_rng(0)
@@ -433,8 +432,7 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
         for l in range(L):           # every (sequence, layer) slot holds the first lens[s] rows of the same K / V
             Ko[s * L + l, :lens[s]] = k16[:lens[s]]; Vo[s * L + l, :lens[s]] = v16[:lens[s]]
     orc.set_threads(16)
-    deep = {int(np.argmax(lens)), int(np.argmin(lens))}
-    n_steps = [steps if s in deep else short_steps for s in range(B)]
+    n_steps = [steps] * B
     want = [_oracle_greedy_with_logits(orc, om, s, [toks[s]], n_steps[s], start_pos=int(lens[s]), beat=heartbeat) for s in range(B)]
     dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=B)
     dk, dv = ctx.to_device(k16), ctx.to_device(v16)
