@@ -30,16 +30,19 @@ def _toy_cfg(layout, bias, hd=64):
                 rope_base=10000.0 if layout == 0 else 1e6, rope_scale=1.0, rope_layout=layout, qkv_bias=bias)
 
 
-def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0, beat=None, hidden=None):
+def _oracle_greedy_with_logits(orc, om, seq, prompt, n_gen, start_pos=0, beat=None, hidden=None, keep=None):
     """orc_decode_greedy's loop (oracle/oracle.c) driven from here so that every pick's logits row is seen:
     returns ids (prompt + picks), the top-1 / top-2 gap and the largest |logit| of every pick.  `hidden`: the state the
-    first pick is made from when the prompt has already been run (a packed prefill up to start_pos)."""
+    first pick is made from when the prompt has already been run (a packed prefill up to start_pos); `keep`: a list
+    that receives every pick's logits row."""
     pos = start_pos
     for t in prompt:
         hidden = om.token_forward(seq, pos, int(t)); pos += 1
     ids, gaps, scale = [int(t) for t in prompt], [], []
     for g in range(n_gen):
         wl = om.logits(hidden)
+        if keep is not None:
+            keep.append(wl)
         nxt = int(orc.greedy_topk1(wl))
         top2 = np.partition(wl, -2)[-2:]
         gaps.append(float(top2[1] - top2[0])); scale.append(float(np.abs(wl).max()))
@@ -415,7 +418,9 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
     copy, as the benchmark builds it), hidden 2048, 16 q / 2 kv heads, hd 128, FFN 11008, vocab 151936, biases, NeoX
     RoPE theta 1e6; batch 8, contexts U[256, 4096] pre-filled N(0,1), 64 greedy steps on the fused graph path, every
     row against the oracle's decode of that row alone (512 picks); then 8 steps of all rows through the reference's
-    row-batched call sequence."""
+    row-batched call sequence; and teacher-forced along the oracle's own sequences (fused kernels, one batched step per
+    position with the oracle's tokens), the logits of all 512 picks stay inside the float bar and pick the same token
+    unless the oracle's top-2 gap is inside the tie bound -- which carries the comparison past a row's first tie."""
     cfg = dict(syn.QWEN25_3B)
     W = syn.make_weights(cfg, seed=0, unique_layers=4, tie_embeddings=True)
     B, steps, reference_steps = 8, 64, 8
@@ -433,7 +438,9 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
             Ko[s * L + l, :lens[s]] = k16[:lens[s]]; Vo[s * L + l, :lens[s]] = v16[:lens[s]]
     orc.set_threads(16)
     n_steps = [steps] * B
-    want = [_oracle_greedy_with_logits(orc, om, s, [toks[s]], n_steps[s], start_pos=int(lens[s]), beat=heartbeat) for s in range(B)]
+    oracle_logits = [[] for _ in range(B)]
+    want = [_oracle_greedy_with_logits(orc, om, s, [toks[s]], n_steps[s], start_pos=int(lens[s]), beat=heartbeat, keep=oracle_logits[s])
+            for s in range(B)]
     dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=S, max_sequences=B)
     dk, dv = ctx.to_device(k16), ctx.to_device(v16)
     for mode in (2, 0):
@@ -451,6 +458,22 @@ def test_qwen_full_depth_batched_greedy_ids_graph_mode(ctx, orc, heartbeat):
             _assert_ids_equal_up_to_legitimate_tie(ids[s][:n], wid[1:1 + n], wgap[:n], wscale[:n],
                                                    f"qwen-36L B=8 mode {mode} row {s} ({n} steps, context {int(lens[s])})")
         print(f"[qwen-36L B=8 mode {mode}] min device top-2 gap over {B * run_steps} picks: {gaps.min():.3e}")
+    # teacher-forced: step g feeds every row the oracle's token g at position lens + g (rows past lens are rewritten)
+    dm.set_mode(1)
+    worst, ties = 0.0, 0
+    for g in range(steps):
+        _, gl = dm.forward_batched(np.arange(B), lens + g, [int(want[s][0][g]) for s in range(B)])
+        for s in range(B):
+            wl, (wid, wgap, wscale) = oracle_logits[s][g], want[s]
+            delta = float(np.abs(gl[s] - wl).max())
+            worst = max(worst, delta / (1e-3 * wscale[g] + 1e-4))
+            assert delta <= 1e-3 * wscale[g] + 1e-4, (s, g, delta, wscale[g])
+            if int(np.argmax(gl[s])) != int(wid[g + 1]):
+                ties += 1
+                assert wgap[g] <= _tie_bound(wscale[g]), (s, g, wgap[g])
+        if g % 8 == 7:
+            heartbeat()
+    print(f"[qwen-36L B=8 teacher-forced] largest logit deviation = {worst:.3f} of the bar over {B * steps} picks; {ties} picks inside the tie bound differ")
     dk.free(); dv.free()
     dm.close()
 
