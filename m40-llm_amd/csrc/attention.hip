@@ -179,10 +179,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_partial_kernel(AttnParam
     for (int h = 0; h < G; ++h) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            float v = acc[h][j];
-#pragma unroll
-            for (int o = LPT; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
-            acc[h][j] = v;
+            acc[h][j] = m40_sum_lanes_from<LPT>(acc[h][j]);
         }
         const float ssum = m40_sum64(lsum[h]);
         if (lane == 0) wsum[wave][h] = ssum;

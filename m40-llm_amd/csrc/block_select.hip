@@ -485,10 +485,7 @@ __global__ __launch_bounds__(kBsThreads, 3) void bs_attend_kernel(BsMulti multi)
     // ---- join the lanes of a wave, then the waves ------------------------------------------------------------------
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        float v = st.acc[j];
-#pragma unroll
-        for (int o = LPT; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
-        st.acc[j] = v;
+        st.acc[j] = m40_sum_lanes_from<LPT>(st.acc[j]);
     }
     const float lsum = m40_sum64(st.l);
     if (lane == 0) { wmax[wave] = st.m; wsum[wave] = lsum; }

@@ -263,15 +263,46 @@ __device__ __forceinline__ float m40_sum16(float x) {  // over rows of 16 lanes
     x += m40_dpp_f<M40_DPP_MIRROR>(x);
     return x;
 }
+// The xor-16 and xor-32 steps on the vector ALU: v_permlane16_swap (v_permlane32_swap) exchanges the odd rows of 16 (32)
+// lanes of its first operand with the even rows of its second; with both operands holding x, one register ends with
+// the even rows' values in every lane and the other with the odd rows', and their sum or maximum is the butterfly
+// step -- the same two numbers in either order as lane l joining lane l ^ 16 (l ^ 32), hence the same bits as the
+// ds_bpermute form (__shfl_xor), which pays an LDS round trip per step (36 ns against 21 ns in a dependent chain).
+// The s_nop covers the wait states between a vector write of an operand and the swap.  All 64 lanes must be active.
+__device__ __forceinline__ void m40_swap_rows16(float& a, float& b) { asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void m40_swap_rows32(float& a, float& b) { asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ float m40_add_xor16(float x) { float a = x, b = x; m40_swap_rows16(a, b); return a + b; }
+__device__ __forceinline__ float m40_add_xor32(float x) { float a = x, b = x; m40_swap_rows32(a, b); return a + b; }
+__device__ __forceinline__ float m40_max_xor16(float x) { float a = x, b = x; m40_swap_rows16(a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float m40_max_xor32(float x) { float a = x, b = x; m40_swap_rows32(a, b); return fmaxf(a, b); }
+// Butterfly sum over the lanes that differ in the bits FROM, 2 FROM, ... 32 (lanes equal in the bits below FROM keep
+// separate sums): xor 8 is a rotation of the row of 16 by 8, xor 16 and 32 the swaps above -- the partner of every
+// step and the order of the steps are those of  for (o = FROM; o < 64; o <<= 1) v += __shfl_xor(v, o).
+#define M40_DPP_ROW_ROR8 0x128
+template <int FROM>
+__device__ __forceinline__ float m40_sum_lanes_from(float v) {
+    static_assert(FROM == 8 || FROM == 16 || FROM == 32, "steps below 8 have no single-instruction form here");
+    if (FROM <= 8) v += m40_dpp_f<M40_DPP_ROW_ROR8>(v);
+    if (FROM <= 16) v = m40_add_xor16(v);
+    return m40_add_xor32(v);
+}
 __device__ __forceinline__ float m40_sum64(float x) {  // whole wave
     x = m40_sum16(x);
-    x += __shfl_xor(x, 16, 64);
-    x += __shfl_xor(x, 32, 64);
+    x = m40_add_xor16(x);
+    x = m40_add_xor32(x);
+    return x;
+}
+__device__ __forceinline__ float m40_max16(float x) {  // over rows of 16 lanes
+    x = fmaxf(x, m40_dpp_f<M40_DPP_XOR1>(x));
+    x = fmaxf(x, m40_dpp_f<M40_DPP_XOR2>(x));
+    x = fmaxf(x, m40_dpp_f<M40_DPP_HALF_MIRROR>(x));      // quads hold their maximum: the mirrors join 4 + 4 and 8 + 8
+    x = fmaxf(x, m40_dpp_f<M40_DPP_MIRROR>(x));
     return x;
 }
 __device__ __forceinline__ float m40_max64(float x) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+    x = m40_max16(x);
+    x = m40_max_xor16(x);
+    x = m40_max_xor32(x);
     return x;
 }
 

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(1024) void gemm_mfma_f32xf16_gguf_kernel(
     // lane (j, g) holds D[4g + r][j], r = 0..3
     if (STACKED) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], 32, 64);  // hi rows + lo rows
+        for (int r = 0; r < 4; ++r) acc[r] = m40_add_xor32(acc[r]);  // hi rows + lo rows
     }
     float* my = red + ((size_t)(s * T + t_in) * 256);
     if (!STACKED || g < 2) {

@@ -547,7 +547,7 @@ __global__ __launch_bounds__(64 * WAVES, 2) void q80i8_gemm_kernel(Q80I8Args p) 
 #pragma unroll
         for (int t = 0; t < T; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[t][r] += __shfl_xor(acc[t][r], 32, 64);
+            for (int r = 0; r < 4; ++r) acc[t][r] = m40_add_xor32(acc[t][r]);
     }
     if (STACK) {
         // lane (j, g) holds digit g of rows r: the three sums meet in the lanes g = 0

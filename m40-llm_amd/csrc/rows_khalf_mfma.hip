@@ -126,8 +126,8 @@ __global__ __launch_bounds__(kThreads, 1) void rows_khalf_kernel(KHalfArgs p) {
             mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
         }
         mx = fmaxf(mx, __builtin_bit_cast(float, from_partner8(__builtin_bit_cast(uint32_t, mx))));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = m40_max_xor16(mx);
+        mx = m40_max_xor32(mx);
         float scale = 1.0f, inv_scale = 1.0f;
         if (mx > 0.0f && mx < INFINITY) {
             int ex;
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kThreads, 1) void rows_khalf_kernel(KHalfArgs p) {
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        acc[r] += __shfl_xor(acc[r], 32, 64);          // hi rows (g 0, 1) + lo rows (g 2, 3)
+        acc[r] = m40_add_xor32(acc[r]);          // hi rows (g 0, 1) + lo rows (g 2, 3)
         red[(wave * 4 + r) * 64 + lane] = acc[r];
     }
     __syncthreads();

@@ -267,11 +267,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
                 if (!live) v[c][e] = 0.0f;
                 mx = fmaxf(mx, fabsf(v[c][e]));
             }
-#pragma unroll
-        for (int o = 1; o < kRowThreads; o <<= 1) {
-            sq += __shfl_xor(sq, o, 64);
-            mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        }
+        // over the row's lanes (an aligned group of 16, 32 or 64): the bits of the xor butterfly 1, 2, ..., on the vector ALU
+        static_assert(kRowThreads == 16 || kRowThreads == 32 || kRowThreads == 64, "a row is 16, 32 or 64 lanes");
+        sq = m40_sum16(sq);
+        mx = m40_max16(mx);
+        if (kRowThreads >= 32) { sq = m40_add_xor16(sq); mx = m40_max_xor16(mx); }
+        if (kRowThreads >= 64) { sq = m40_add_xor32(sq); mx = m40_max_xor32(mx); }
         float scale = 1.0f, inv_scale = 1.0f;
         if (mx > 0.0f && mx < INFINITY) {
             int ex;
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void rows_mfma_kernel(RowsMfmaArgs p
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            acc[r] += __shfl_xor(acc[r], 32, 64);       // hi rows (g 0, 1) + lo rows (g 2, 3)
+            acc[r] = m40_add_xor32(acc[r]);       // hi rows (g 0, 1) + lo rows (g 2, 3)
             red_s[parity][wave][r][lane] = acc[r];
         }
     };

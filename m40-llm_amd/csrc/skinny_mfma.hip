@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kThreads, 2) void skinny_mfma_kernel(SkinnyArgs p) 
     // lane (j, g) holds rows 4g + r of column j
     if (STACKED) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[r] += __shfl_xor(acc[r], 32, 64);  // hi rows + lo rows
+        for (int r = 0; r < 4; ++r) acc[r] = m40_add_xor32(acc[r]);  // hi rows + lo rows
     }
     if (!tile_live || n0 + j >= N) return;
     if (STACKED && g >= 2) return;
