@@ -303,6 +303,22 @@ def measure_b8(pkg, syn, ctx, steps=32, warmup=4):
     return rec, (cfg, W, lens, k16h, v16h, first)
 
 
+def measure_prefill(syn, ctx, cfg, W, tokens=4096, reps=3):
+    """The step before decode, reported beside the metric (never folded into value): one prompt of `tokens` ids through
+    the packed prefill forward of the same model (all layers, last-token logits), host clock around the blocking call."""
+    dm = syn.DeviceModel(ctx, cfg, W, max_seq_len=tokens + 8, max_sequences=1)
+    dm.set_mode(2)
+    prompt = np.random.default_rng(1).integers(0, cfg["vocab"], size=tokens).tolist()
+    dm.forward_prefill([0], [prompt])
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        dm.forward_prefill([0], [prompt])
+    ms = (time.perf_counter() - t0) * 1e3 / reps
+    dm.close()
+    return {"workload": f"one prompt of {tokens} tokens, packed prefill forward of the same {cfg['n_layers']}-layer model, "
+                        "last-token logits included", "prompt_tokens": tokens, "ms": ms, "tok_s": tokens / (ms * 1e-3), "runs_timed": reps}
+
+
 def plain_read_yardstick(pkg, ctx, nbytes):
     """Fastest of a few workgroup counts for a plain one-launch read of nbytes (rotating over cold buffers): what a
     bandwidth-bound kernel of this size can reach on this box, launch ramp and tail included."""
@@ -341,6 +357,7 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=48)
     ap.add_argument("--kernel-reps", type=int, default=10)
     ap.add_argument("--no-b8", action="store_true", help="skip the batch-8 measurement reported in config.b8")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the packed-prefill measurement reported in config.prefill")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy through the library (calibrates rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings against a transfer of known size)")
@@ -437,6 +454,11 @@ def main():
     }
     out["config"]["host_sampler_fallback"] = dm.last_timed_host_fallback()
     dm.close()
+    if not args.no_prefill and not args.layers:
+        try:
+            out["config"]["prefill"] = measure_prefill(syn, ctx, cfg, W)
+        except Exception as e:
+            out["config"]["prefill"] = {"error": repr(e)}
     b8_state = None
     if not args.no_b8 and not args.layers:
         try:
