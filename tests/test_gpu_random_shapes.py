@@ -1,0 +1,115 @@
+"""Seeded sweep over odd shapes: the entry points of the path against the oracle at sizes drawn around the kernels'
+tile, chunk and wave boundaries (rows 1-1030, columns 1-5632, K from 8, contexts from 1 token, query blocks of 15-17 and
+63-65 and 127-129 queries, cached keys ahead of the queries).  Products are measured in units of the element's own terms
+S = sum |a| |w| (2e-6 S: the bound of test_gpu_error_bounds.py with room for the oracle's own rounding), attention
+outputs absolutely (|out| <= max |v| ~ 4)."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+sys.path.insert(0, os.path.dirname(__file__))
+from gpu_common import Dev, f16bits, m40  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return Dev()
+
+
+def _pick(rng, choices):
+    return int(choices[rng.integers(0, len(choices))])
+
+
+def test_f16_products_at_random_shapes(dev, orc):
+    rng = np.random.default_rng(101)
+    orc.set_threads(16)
+    done = 0
+    while done < 60:
+        M = _pick(rng, [1, 1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 33, 100, 129, 300, 513, 1030])
+        N = _pick(rng, [1, 2, 7, 64, 100, 255, 256, 257, 1000, 2048, 2560, 4097, 5632])
+        K = _pick(rng, [8, 16, 24, 32, 64, 72, 256, 1000, 2048, 2056, 4096, 5632])
+        if M * N * K > 3e9:
+            continue
+        A = (rng.standard_normal((M, K)) * (10.0 ** rng.integers(-3, 4))).astype(np.float32)
+        B = f16bits(rng.standard_normal((N, K)) * 0.05)
+        want = orc.gemm("f32xf16_gguf", A, B, M, N, K)
+        got = dev.gemm_gguf(A, B, M, N, K)
+        S = np.abs(A).astype(np.float64) @ np.abs(B.view(np.float16).astype(np.float64)).T
+        err = float((np.abs(got.astype(np.float64) - want) / (S + 1e-30)).max())
+        assert err <= 2e-6, (M, N, K, err)
+        done += 1
+
+
+def test_q80_products_at_random_shapes(dev, orc):
+    rng = np.random.default_rng(102)
+    orc.set_threads(16)
+    done = 0
+    while done < 30:
+        M = _pick(rng, [1, 2, 3, 4, 5, 8, 9, 16])
+        N = _pick(rng, [32, 100, 1000, 4096, 14336])
+        K = _pick(rng, [32, 64, 256, 4096, 14336])
+        if M * N * K > 1e9:
+            continue
+        w = np.empty((N, K // 32, 34), dtype=np.uint8)
+        w[:, :, :2] = rng.uniform(0.001, 0.01, size=(N, K // 32)).astype(np.float16).view(np.uint8).reshape(N, K // 32, 2)
+        w[:, :, 2:] = rng.integers(-127, 128, size=(N, K // 32, 32)).astype(np.int8).view(np.uint8)
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        want = orc.gemm("f32xq80_gguf", A, w, M, N, K)
+        dx, dw, dC = dev.up(A), dev.up(w), dev.zeros(M * N * 4)
+        dev.call("m40llm_ext_gemm_f32xq80_gguf_f32", dx.ptr, dw.ptr, dC.ptr, M, N, K)
+        got = dC.download(np.float32, (M, N))
+        W = (w[:, :, :2].copy().view(np.float16).astype(np.float64) * w[:, :, 2:].view(np.int8).astype(np.float64)).reshape(N, -1)
+        S = np.abs(A).astype(np.float64) @ np.abs(W).T
+        err = float((np.abs(got.astype(np.float64) - want) / (S + 1e-30)).max())
+        assert err <= 2e-6, (M, N, K, err)
+        done += 1
+
+
+def test_dense_attention_at_random_shapes(dev, orc):
+    rng = np.random.default_rng(103)
+    orc.set_threads(16)
+    for _ in range(40):
+        hd, kvh, g = _pick(rng, [64, 128]), _pick(rng, [1, 2, 4, 8]), _pick(rng, [1, 2, 4, 8])
+        qh = kvh * g
+        L = _pick(rng, [1, 2, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 513, 1000, 2049, 4096, 5000])
+        K16 = f16bits(rng.standard_normal((L, kvh, hd))).reshape(L, kvh, hd)
+        V16 = f16bits(rng.standard_normal((L, kvh, hd))).reshape(L, kvh, hd)
+        q = rng.standard_normal(qh * hd).astype(np.float32)
+        kv = m40.KVCache(dev.ctx, L, 1, kvh, hd)
+        dev.fill_dense(kv, 0, K16, V16)
+        got = dev.attention(kv, 0, q, qh, L)
+        want = orc.attention(K16[None].copy(), V16[None].copy(), L, kvh, hd, 0, q, qh, L)
+        err = float(np.abs(got - want).max())
+        assert err <= 2e-5, (qh, kvh, hd, L, err)
+
+
+def test_packed_prefill_attention_at_random_shapes(dev, orc):
+    rng = np.random.default_rng(104)
+    orc.set_threads(16)
+    done = 0
+    while done < 40:
+        hd, kvh, g = _pick(rng, [64, 128]), _pick(rng, [1, 2, 4]), _pick(rng, [1, 2, 4, 8])
+        qh = kvh * g
+        ql = [_pick(rng, [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 200, 300, 600]) for _ in range(_pick(rng, [1, 2, 3, 5]))]
+        kl = [x + _pick(rng, [0, 0, 1, 31, 64, 100]) for x in ql]
+        if sum(x * y for x, y in zip(ql, kl)) * qh > 3e7:
+            continue
+        Q = rng.standard_normal((sum(ql), qh, hd)).astype(np.float32)
+        Kf = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+        Vf = rng.standard_normal((sum(kl), kvh, hd)).astype(np.float32)
+        rc, want = orc.attention_prefill(Q, Kf, Vf, ql, kl, qh, kvh, hd)
+        assert rc == 0
+        dq, dk, dv = dev.up(Q), dev.up(Kf), dev.up(Vf)
+        dqo, dko = dev.up(orc.prefill_offsets(ql)), dev.up(orc.prefill_offsets(kl))
+        dql, dkl = dev.up(np.asarray(ql, dtype=np.uint32)), dev.up(np.asarray(kl, dtype=np.uint32))
+        out = dev.zeros(Q.nbytes)
+        dev.call("m40llm_attention_prefill_f32_gqa_varlen", dq.ptr, dk.ptr, dv.ptr, dqo.ptr, dko.ptr, dql.ptr, dkl.ptr, len(ql), qh, kvh,
+                 hd, out.ptr)
+        got = out.download(np.float32, Q.shape)
+        err = float(np.abs(got - want).max())
+        assert err <= 2e-5, (qh, kvh, hd, ql, kl, err)
+        done += 1
