@@ -3,6 +3,7 @@ tile, chunk and wave boundaries (rows 1-1030, columns 1-5632, K from 8, contexts
 63-65 and 127-129 queries, cached keys ahead of the queries).  Products are measured in units of the element's own terms
 S = sum |a| |w| (2e-6 S: the bound of test_gpu_error_bounds.py with room for the oracle's own rounding), attention
 outputs absolutely (|out| <= max |v| ~ 4)."""
+import importlib
 import os
 import sys
 
@@ -11,6 +12,9 @@ import pytest
 
 sys.path.insert(0, os.path.dirname(__file__))
 from gpu_common import Dev, f16bits, m40  # noqa: E402
+from test_gpu_model import _oracle_greedy_with_logits, _tie_bound  # noqa: E402
+
+syn = importlib.import_module("m40-llm_amd.synthetic")
 
 pytestmark = pytest.mark.gpu
 
@@ -112,4 +116,62 @@ def test_packed_prefill_attention_at_random_shapes(dev, orc):
         got = out.download(np.float32, Q.shape)
         err = float(np.abs(got - want).max())
         assert err <= 2e-5, (qh, kvh, hd, ql, kl, err)
+        done += 1
+
+
+def _ids_equal_or_tie(got, want, gaps, scale):
+    diff = np.flatnonzero(np.asarray(got) != np.asarray(want))
+    return diff.size == 0 or gaps[int(diff[0])] <= _tie_bound(scale[int(diff[0])])
+
+
+def test_random_model_configurations_through_every_host_mode(dev, orc):
+    # small decoders of random shape (head_dim 16-128, 1-32 heads, FFN 64-5632, vocabulary 50-5000, 1-3 layers, either
+    # RoPE layout, with and without biases, 1-5 sequences with prompts of 1-40 tokens) in the three host modes: greedy
+    # decode of every prompt, then the packed prefill of all prompts (where the head size has one) with logits inside the
+    # float bar and the batched decode from its cache -- ids equal to the oracle's, or parting at a pick inside the tie bound
+    rng = np.random.default_rng(105)
+    pick = lambda c: c[int(rng.integers(0, len(c)))]
+    orc.set_threads(16)
+    done = 0
+    while done < 24:
+        hd, kvh, g = pick([16, 32, 64, 128]), pick([1, 2, 4]), pick([1, 2, 4, 8])
+        qh = kvh * g
+        if qh * hd > 2048:
+            continue
+        cfg = dict(n_layers=pick([1, 2, 3]), d_model=qh * hd, q_heads=qh, kv_heads=kvh, head_dim=hd,
+                   ffn=pick([64, 256, 384, 1000, 1536, 2048, 5632]), vocab=pick([50, 300, 1000, 5000]), rms_eps=1e-5,
+                   rope_base=pick([10000.0, 1e6]), rope_scale=1.0, rope_layout=pick([0, 1]), qkv_bias=bool(pick([0, 1])))
+        W = syn.make_weights(cfg, seed=int(rng.integers(0, 1000)), std=0.08, emb_std=1.0)
+        S, B, n_gen = 80, pick([1, 2, 3, 5]), 5
+        prompts = [rng.integers(0, cfg["vocab"], size=pick([1, 2, 7, 33, 40])).tolist() for _ in range(B)]
+        lens = np.array([len(p) for p in prompts], dtype=np.uint32)
+        om = orc.Model(dict(cfg), W)
+        om.alloc_kv(S, B)
+        want = [_oracle_greedy_with_logits(orc, om, s, p, n_gen) for s, p in enumerate(prompts)]
+        om2 = orc.Model(dict(cfg), W)
+        om2.alloc_kv(S, B)
+        packed = hd in (64, 128)
+        if packed:
+            rows = om2.prefill_forward(list(range(B)), prompts)
+            wl = [om2.logits(rows[e]) for e in np.cumsum(lens) - 1]
+            firsts = [int(orc.greedy_topk1(l)) for l in wl]
+            cont = [_oracle_greedy_with_logits(orc, om2, s, [firsts[s]], n_gen, start_pos=int(lens[s])) for s in range(B)]
+        for mode in (0, 1, 2):
+            dm = syn.DeviceModel(dev.ctx, cfg, W, max_seq_len=S, max_sequences=B)
+            dm.set_mode(mode)
+            for s, p in enumerate(prompts):
+                got, _ = dm.decode_greedy(s, p, n_gen)
+                assert _ids_equal_or_tie(got[len(p):], want[s][0][len(p):], want[s][1], want[s][2]), (cfg, mode, s)
+            dm.close()
+            if not packed:
+                continue
+            dm = syn.DeviceModel(dev.ctx, cfg, W, max_seq_len=S, max_sequences=B)
+            dm.set_mode(mode)
+            _, log = dm.forward_prefill(list(range(B)), prompts)
+            for s in range(B):
+                assert float(np.abs(log[s] - wl[s]).max()) <= 1e-3 * np.abs(wl[s]).max() + 1e-4, (cfg, mode, s)
+            ids, _ = dm.decode_batch_greedy(np.arange(B), lens, firsts, n_gen)
+            for s in range(B):
+                assert _ids_equal_or_tie(ids[s], cont[s][0][1:], cont[s][1], cont[s][2]), (cfg, mode, s)
+            dm.close()
         done += 1
