@@ -11,7 +11,8 @@ import numpy as np
 import pytest
 
 sys.path.insert(0, os.path.dirname(__file__))
-from gpu_common import Dev, f16bits, m40  # noqa: E402
+from gpu_common import Dev, close, f16bits, m40  # noqa: E402
+from test_gpu_block_select import _block_select_case  # noqa: E402
 from test_gpu_model import _oracle_greedy_with_logits, _tie_bound  # noqa: E402
 
 syn = importlib.import_module("m40-llm_amd.synthetic")
@@ -174,4 +175,25 @@ def test_random_model_configurations_through_every_host_mode(dev, orc):
             for s in range(B):
                 assert _ids_equal_or_tie(ids[s], cont[s][0][1:], cont[s][1], cont[s][2]), (cfg, mode, s)
             dm.close()
+        done += 1
+
+
+def test_block_select_at_random_geometries(dev, orc):
+    # contexts of 1-3000 tokens, windows of 1-1024, blocks of 1-100 tokens, 1-64 listed blocks, both old-V formats:
+    # the listed block ids are the reference order's bit for bit, the output inside the float bar
+    rng = np.random.default_rng(106)
+    pick = lambda c: c[int(rng.integers(0, len(c)))]
+    done = 0
+    while done < 60:
+        hd, kvh, g = pick([64, 128]), pick([1, 2, 4, 8]), pick([1, 2, 4, 8])
+        qh = kvh * g
+        L = pick([1, 2, 5, 17, 64, 65, 100, 300, 777, 1025, 2100, 3000])
+        W, bs, top = pick([1, 2, 4, 16, 32, 100, 512, 1024]), pick([1, 2, 4, 16, 32, 48, 64, 100]), pick([1, 2, 3, 8, 17, 64])
+        if qh * L * hd > 3e7:
+            continue
+        r = _block_select_case(dev, orc, qh, kvh, hd, L, W, bs, top, seed=int(rng.integers(0, 1000)), backing=pick([2, 2, 3]))
+        case = (qh, kvh, hd, L, W, bs, top)
+        assert np.array_equal(r["cnt"], r["wcnt"]), case
+        assert np.array_equal(r["sel"], r["wsel"]), case
+        close(r["got"], r["want"])
         done += 1
