@@ -16,6 +16,7 @@ from test_gpu_block_select import _block_select_case  # noqa: E402
 from test_gpu_model import _oracle_greedy_with_logits, _tie_bound  # noqa: E402
 
 syn = importlib.import_module("m40-llm_amd.synthetic")
+sch = importlib.import_module("m40-llm_amd.scheduler")
 
 pytestmark = pytest.mark.gpu
 
@@ -197,3 +198,56 @@ def test_block_select_at_random_geometries(dev, orc):
         assert np.array_equal(r["sel"], r["wsel"]), case
         close(r["got"], r["want"])
         done += 1
+
+
+def test_scheduler_random_request_streams(dev, orc):
+    # small decoders of random shape behind the scheduler: 1-4 slots, 3-10 requests with prompts of 1-31 tokens and 1-9
+    # new tokens arriving over the first dozen ticks, one in seven cancelled two ticks after its arrival, any host mode.
+    # Every request completes (or stays cancelled) and its tokens are the oracle's for that request alone -- the prompt
+    # through the oracle's packed prefill where the scheduler packs prompts -- or part at a pick inside the tie bound.
+    rng = np.random.default_rng(107)
+    pick = lambda c: c[int(rng.integers(0, len(c)))]
+    orc.set_threads(16)
+    for _ in range(40):
+        hd, kvh, g = pick([16, 64, 128]), pick([1, 2]), pick([1, 2, 4])
+        qh = kvh * g
+        cfg = dict(n_layers=pick([1, 2]), d_model=qh * hd, q_heads=qh, kv_heads=kvh, head_dim=hd, ffn=pick([128, 512, 1000]),
+                   vocab=pick([60, 300, 2000]), rms_eps=1e-5, rope_base=10000.0, rope_scale=1.0, rope_layout=pick([0, 1]),
+                   qkv_bias=bool(pick([0, 1])))
+        W = syn.make_weights(cfg, seed=int(rng.integers(0, 1000)), std=0.08, emb_std=1.0)
+        S, slots, mode = 64, pick([1, 2, 3, 4]), pick([0, 1, 2])
+        dm = syn.DeviceModel(dev.ctx, cfg, W, max_seq_len=S, max_sequences=slots)
+        dm.set_mode(mode)
+        s = sch.Scheduler.for_model(dm)
+        specs = [(rng.integers(0, cfg["vocab"], size=pick([1, 2, 9, 20, 31])).tolist(), pick([1, 2, 5, 9]), int(rng.integers(0, 12)),
+                  bool(rng.random() < 0.15)) for _ in range(pick([3, 6, 10]))]
+        rids, cancel_at, tick = {}, {}, 0
+        pending = sorted(range(len(specs)), key=lambda i: specs[i][2])
+        while pending or s.active():
+            while pending and specs[pending[0]][2] <= tick and s.available_slots():
+                i = pending.pop(0)
+                rids[i] = s.submit(specs[i][0], max_tokens=specs[i][1])
+                if specs[i][3]:
+                    cancel_at[i] = tick + 2
+            for i in [i for i, t in cancel_at.items() if t == tick]:
+                s.cancel(rids[i])
+                del cancel_at[i]
+            s.tick()
+            tick += 1
+            assert tick < 500
+        for i, (prompt, gen, _, _) in enumerate(specs):
+            om = orc.Model(dict(cfg), W)
+            om.alloc_kv(S, 1)
+            if hd in (64, 128):
+                hidden = om.prefill_forward([0], [prompt])[-1]
+                want, gaps, scale = _oracle_greedy_with_logits(orc, om, 0, [], gen, start_pos=len(prompt), hidden=hidden)
+            else:
+                want, gaps, scale = _oracle_greedy_with_logits(orc, om, 0, prompt, gen)
+                want = want[len(prompt):]
+            got, state = s.generated(rids[i]), s.state(rids[i])
+            assert state in ("complete", "cancelled"), (cfg, i, state, s.error(rids[i]))
+            assert state == "cancelled" or len(got) == gen, (cfg, i, got)
+            assert _ids_equal_or_tie(got, want[:len(got)], gaps, scale), (cfg, mode, i, got, want)
+        assert s.available_slots() == slots
+        s.close()
+        dm.close()
