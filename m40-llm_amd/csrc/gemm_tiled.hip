@@ -603,21 +603,30 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tiled_wide_kernel(const _Flo
     else store_tile(std::false_type{});
 }
 
-// out[i] = planes[0][i] + planes[1][i] + ... in that order (n4 float4 per plane), then residual[i] + that (residual may be out)
-__global__ __launch_bounds__(256) void add_k_planes_kernel(const float4* __restrict__ planes, const float4* residual, float4* out,
-                                                           size_t n4, int k_splits) {
+// out[i] = planes[0][i] + planes[1][i] + ... in that order (n4 float4 per plane), then residual[i] + that (residual may be
+// out); blockIdx.y = matrix, so the up to three matrices of a launch are summed by one launch as well
+struct KPlaneSet {
+    const float4* planes[kMaxMats];
+    const float4* residual[kMaxMats];
+    float4* out[kMaxMats];
+    size_t n4[kMaxMats];
+};
+__global__ __launch_bounds__(256) void add_k_planes_kernel(KPlaneSet set, int k_splits) {
+    const int m = blockIdx.y;
+    const size_t n4 = set.n4[m];
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n4) return;
+    const float4* planes = set.planes[m];
     float4 a = planes[i];
     for (int s = 1; s < k_splits; ++s) {
         const float4 b = planes[(size_t)s * n4 + i];
         a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
     }
-    if (residual) {
-        const float4 r = residual[i];
+    if (set.residual[m]) {
+        const float4 r = set.residual[m][i];
         a = make_float4(r.x + a.x, r.y + a.y, r.z + a.z, r.w + a.w);
     }
-    out[i] = a;
+    set.out[m][i] = a;
 }
 
 }  // namespace
@@ -735,12 +744,16 @@ int m40_launch_gemm_tiled_fused(M40llmCudaContext* ctx, hipStream_t stream, uint
     else
         gemm_tiled_f32xf16_gguf_kernel<<<(unsigned)(tiles * k_splits), kThreads, lds_bytes, stream>>>(hi, lo, row_scale, launch, M, K, k_splits);
     if (k_splits > 1) {
+        KPlaneSet set{};
+        size_t blocks = 0;
         for (int i = 0; i < n_mats; ++i) {
-            const size_t n4 = (size_t)M * N[i] / 4;
-            add_k_planes_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, stream>>>(reinterpret_cast<const float4*>(launch.C[i]),
-                                                                                  reinterpret_cast<const float4*>(mats.R[i]),
-                                                                                  reinterpret_cast<float4*>(C[i]), n4, k_splits);
+            set.planes[i] = reinterpret_cast<const float4*>(launch.C[i]);
+            set.residual[i] = reinterpret_cast<const float4*>(mats.R[i]);
+            set.out[i] = reinterpret_cast<float4*>(C[i]);
+            set.n4[i] = (size_t)M * N[i] / 4;
+            blocks = blocks > (set.n4[i] + 255) / 256 ? blocks : (set.n4[i] + 255) / 256;
         }
+        add_k_planes_kernel<<<dim3((unsigned)blocks, (unsigned)n_mats), 256, 0, stream>>>(set, k_splits);
     }
     return hipGetLastError() == hipSuccess ? 0 : -2;
 }
